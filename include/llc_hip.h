@@ -1,0 +1,231 @@
+/*
+ * llc_hip.h -- C-ABI of the gfx950 (MI355X) kernel library behind LLCompiler's compiled-op path.
+ *
+ * The reference lowers LLH ops to CPU loop nests inside a generated `main(void**)`; its runtime
+ * op library is an empty placeholder (ops/cpu/ops.h, 0 bytes).  This header is the `ops/hip`
+ * sibling: one entry point per LLH op (or per fused group the reference's pipeline forms), plus
+ * the model-level entry that keeps the reference's packed-pointer convention.
+ *
+ * Conventions
+ *  - plain C: pointers, sizes, no C++ or torch types.
+ *  - every `data`/`base` pointer is a DEVICE pointer; `size`/`stride` arrays and attribute structs
+ *    live on the host.  Strides are in ELEMENTS, like the reference's Tensor
+ *    (include/llcompiler/Compiler/Tensor.h:36-48).
+ *  - the caller owns every input and output buffer (Tensor.h:35: the descriptor allocates nothing).
+ *  - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Calls only enqueue
+ *    work; the caller synchronises.
+ *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
+ *    llc_hip_last_error() (thread local).  The reference only logs on failure
+ *    (include/llcompiler/Support/Logger.h:132-134); returning a status is a deliberate tightening.
+ */
+#ifndef LLC_HIP_H_
+#define LLC_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLC_HIP_ABI_VERSION 1
+#define LLC_MAX_RANK 8
+
+/* Element type codes.  0-6 are the reference's `enum Type` (Tensor.h:25-33, and the Python map
+ * llcompiler/executor/engine.py:11); 7 and 8 are new. */
+typedef enum llc_dtype {
+  LLC_INT8 = 0,
+  LLC_INT16 = 1,
+  LLC_INT32 = 2,
+  LLC_INT64 = 3,
+  LLC_FLOAT32 = 4,
+  LLC_DOUBLE64 = 5,
+  LLC_INT1 = 6, /* one byte per element, 0 or 1 (torch.bool) */
+  LLC_BFLOAT16 = 7,
+  LLC_FLOAT16 = 8
+} llc_dtype;
+
+/* Non-owning tensor descriptor; same fields in the same order as the reference's
+ * `struct Tensor` (Tensor.h:42-47) with the two std::vectors flattened to rank + pointers.
+ * The element at index (i0, i1, ...) is at  data + (offset + sum_k i_k * stride[k]) elements. */
+typedef struct llc_tensor {
+  void* data;
+  void* base;
+  size_t type;   /* llc_dtype */
+  size_t offset; /* elements */
+  size_t rank;
+  const size_t* size;
+  const size_t* stride;
+} llc_tensor;
+
+typedef enum llc_status {
+  LLC_OK = 0,
+  LLC_ERR_BAD_ARG = -1,     /* null pointer, bad enum value */
+  LLC_ERR_DTYPE = -2,       /* unsupported or mismatched element types */
+  LLC_ERR_SHAPE = -3,       /* rank / extent mismatch between operands */
+  LLC_ERR_LAYOUT = -4,      /* strides the kernel cannot address */
+  LLC_ERR_UNSUPPORTED = -5, /* attribute combination not implemented */
+  LLC_ERR_HIP = -6,         /* a HIP runtime call failed */
+  LLC_ERR_NO_DEVICE = -7,
+  LLC_ERR_TOO_LARGE = -8
+} llc_status;
+
+/* ---- library ---- */
+int llc_hip_abi_version(void);
+/* Selects the device and checks that it is a gfx950 part. */
+int llc_hip_init(int device);
+const char* llc_hip_last_error(void);
+const char* llc_hip_status_string(int status);
+
+/* ---- fused epilogue of the contractions.  The reference's pipeline fuses the elementwise
+ * consumers of a linalg op into it (linalg-fuse-elementwise-ops,
+ * include/llcompiler/TransformLibrary/linalg_include.mlir:50-53); here the same chain
+ *   out = act(alpha * acc + bias + residual)
+ * is applied to the accumulator tile before it is stored. ---- */
+typedef enum llc_activation { LLC_ACT_NONE = 0, LLC_ACT_RELU = 1, LLC_ACT_GELU = 2 } llc_activation;
+typedef struct llc_epilogue {
+  float alpha;                /* applied to the fp32 accumulator; 1.0f = none */
+  const llc_tensor* bias;     /* rank 1, one value per output column / filter; may be NULL */
+  const llc_tensor* residual; /* same shape as the output, contiguous; may be NULL */
+  int act;                    /* llc_activation */
+} llc_epilogue;
+
+/* llh.matmul (include/llcompiler/Dialect/LLH/IR/LLHOps.td:438-444; lowered at
+ * src/Conversion/LLHToHLO/LLHToHLO.cpp:485): out[m,n] = sum_k lhs[m,k] * rhs[k,n], rank 2,
+ * fp32 accumulate.  f32, bf16 or f16 operands (all three the same type).  Either operand may be a
+ * transposed view (stride[0] == 1), which is how llh.transpose{perms=[1,0]} of a weight
+ * (llcompiler/importer/fx_op_translate/transpose.py:39-48) is consumed without a copy.
+ * `epi` may be NULL. */
+int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+                   void* stream);
+
+/* llh.batch_matmul (LLHOps.td:446-452; LLHToHLO.cpp:363-382: batch dims {0}/{0}, contracting lhs
+ * dim 2 with rhs dim 1): rank 3.  The two inner dims of each operand may be a transposed view. */
+int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+                         void* stream);
+
+/* llh.conv / llh.conv_bias attributes (LLHOps.td:407-436).  NCHW x FCHW -> NCHW.
+ * pad = {h_lo, w_lo, h_hi, w_hi}: the order the shape rule reads
+ * (src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:257-268) and the importer writes
+ * (llcompiler/importer/fx_op_translate/conv.py:48-70). */
+typedef struct llc_conv_attrs {
+  int64_t dilation[2];
+  int64_t kernel_shape[2];
+  int64_t pad[4];
+  int64_t stride[2];
+  int64_t group;
+} llc_conv_attrs;
+/* Cross-correlation as implicit GEMM (LLHToHLO.cpp:214-270).  conv_bias is `epi->bias`. */
+int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* attrs, const llc_epilogue* epi,
+                   llc_tensor* out, void* stream);
+
+/* ---- fused elementwise chain.  One launch evaluates a whole chain of LLH elementwise ops, the
+ * unit the reference forms with linalg-fuse-elementwise-ops (linalg_include.mlir:50-53,94).
+ * Unary abs/sqrt/exp/relu/rsqrt (LLHOps.td:345-355), binary add/sub/mul/div/max/min/pow
+ * (LLHOps.td:357-393), compare (LLHOps.td:395-405), where (LLHOps.td:509-517), convert_to
+ * (LLHOps.td:329-335); neg/gelu/tanh/erf/sigmoid/log/recip are added for the nodes the
+ * reference leaves to torch eager.  llh.broadcast_to (LLHOps.td:206-217) is never materialised:
+ * an input whose extent is 1 where the output's is not is read with stride 0. ---- */
+typedef enum llc_ew_opcode {
+  LLC_EW_ABS = 0, LLC_EW_SQRT = 1, LLC_EW_EXP = 2, LLC_EW_RELU = 3, LLC_EW_RSQRT = 4, LLC_EW_NEG = 5,
+  LLC_EW_GELU = 6, LLC_EW_TANH = 7, LLC_EW_ERF = 8, LLC_EW_SIGMOID = 9, LLC_EW_LOG = 10, LLC_EW_RECIP = 11,
+  LLC_EW_MOV = 15,
+  LLC_EW_ADD = 16, LLC_EW_SUB = 17, LLC_EW_MUL = 18, LLC_EW_DIV = 19, LLC_EW_MAX = 20, LLC_EW_MIN = 21,
+  LLC_EW_POW = 22,
+  /* 32 + the reference's CompareKind value (include/llcompiler/Dialect/LLH/IR/LLHEnums.td:111-116) */
+  LLC_EW_CMP_EQ = 33, LLC_EW_CMP_GE = 34, LLC_EW_CMP_LE = 35, LLC_EW_CMP_GT = 36, LLC_EW_CMP_LT = 37,
+  LLC_EW_CMP_NE = 38,
+  LLC_EW_WHERE = 48 /* dst = a != 0 ? b : c */
+} llc_ew_opcode;
+/* operand selectors: 0..LLC_EW_MAX_REGS-1 = register, LLC_EW_IN0 + k = input k, LLC_EW_IMM = imm */
+#define LLC_EW_MAX_REGS 4
+#define LLC_EW_MAX_INPUTS 6
+#define LLC_EW_MAX_INSTS 24
+#define LLC_EW_IN0 16
+#define LLC_EW_IMM 64
+typedef struct llc_ew_inst {
+  int32_t op;  /* llc_ew_opcode */
+  int32_t dst; /* register written */
+  int32_t a, b, c;
+  float imm;
+} llc_ew_inst;
+typedef struct llc_ew_program {
+  int32_t n_insts;
+  int32_t result; /* register holding the chain's value */
+  int32_t integer; /* 0: compute in fp32; 1: compute in int64 (imm is rounded to an integer) */
+  llc_ew_inst insts[LLC_EW_MAX_INSTS];
+} llc_ew_program;
+/* Every input must have the output's rank with each extent equal to the output's or 1.  The
+ * output is contiguous. */
+int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor* const* inputs, size_t n_inputs,
+                        llc_tensor* out, void* stream);
+
+/* llh.reduce_sum / reduce_max / reduce_min {axis} (LLHOps.td:528-553; LLHToHLO.cpp:81-171,
+ * 448-464): init 0 / -inf / +inf, the result drops the reduced axes
+ * (LLHinfersymbolShape.cpp:185-212).  The reduced axes must be adjacent. */
+typedef enum llc_reduce_kind { LLC_REDUCE_SUM = 0, LLC_REDUCE_MAX = 1, LLC_REDUCE_MIN = 2 } llc_reduce_kind;
+int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
+                   void* stream);
+
+/* softmax over the last dim: the amax -> sub -> exp -> sum -> div group that ATen `_softmax`
+ * decomposes to (llcompiler/compiler/torch_compile_config.py:24), as one kernel.  fp32
+ * statistics for every storage type. */
+int llc_hip_softmax(const llc_tensor* x, llc_tensor* out, void* stream);
+
+/* llh.layer_norm{epsilon, axis} (LLHOps.td:454-463) over the last dim; biased variance, fp32
+ * statistics; scale / bias may be NULL. */
+int llc_hip_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_tensor* bias, double epsilon,
+                       llc_tensor* out, void* stream);
+
+/* llh.max_pool (LLHOps.td:495-507; LLHToHLO.cpp:295-339), NCHW, ceil_mode false.
+ * init_zero = 1 reproduces the reference's reduce_window init value 0 (LLHToHLO.cpp:313-314);
+ * init_zero = 0 is torch's -inf padding. */
+typedef struct llc_pool_attrs {
+  int64_t dilation[2];
+  int64_t kernel_shape[2];
+  int64_t pad[4]; /* h_lo, w_lo, h_hi, w_hi */
+  int64_t stride[2];
+  int32_t init_zero;
+} llc_pool_attrs;
+int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* attrs, llc_tensor* out, void* stream);
+
+/* llh.adaptive_average_pool{out_size=(1,1)} (LLHOps.td:337-339; shape rule
+ * LLHinfersymbolShape.cpp:587-613): [N,C,H,W] -> [N,C] (or [N,C,1,1]). */
+int llc_hip_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream);
+
+/* ---- data movement, bit exact for every element size (1, 2, 4, 8 bytes) ---- */
+/* llh.transpose{perms} (LLHOps.td:343; LLHToHLO.td:24-26): out.size[i] = x.size[perms[i]] */
+int llc_hip_transpose(const llc_tensor* x, const int64_t* perms, llc_tensor* out, void* stream);
+/* llh.stride_slice (LLHOps.td:261-269; LLHToHLO.cpp:341-361;
+ * src/Conversion/StablehlotoLinalgExtension/StablehlotoLinalgExtension.cpp:64-118):
+ * out.size[d] = ceildiv(end[d] - start[d], step[d]).  llh.extract (LLHOps.td:252-259) is the
+ * rank-dropping special case and is expressed by the caller through `out`'s descriptor. */
+int llc_hip_stride_slice(const llc_tensor* x, const int64_t* start, const int64_t* end, const int64_t* step,
+                         llc_tensor* out, void* stream);
+/* llh.broadcast_to (LLHOps.td:206-217; LLHToHLO.cpp:191-212), materialised: same rank, input
+ * extents 1 are repeated. */
+int llc_hip_broadcast_to(const llc_tensor* x, llc_tensor* out, void* stream);
+/* Strided -> contiguous copy of any view (the materialising half of reshape, LLHOps.td:281-289). */
+int llc_hip_copy(const llc_tensor* x, llc_tensor* out, void* stream);
+/* Row gather along dim 0 with int64 indices (aten.embedding / index_select, left to torch eager
+ * by the reference): out[i, ...] = table[idx[i], ...]. */
+int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream);
+/* llh.convert_to (LLHOps.td:329-335; LLHToHLO.cpp:489) between f32, bf16, f16, i64, i32, i1. */
+int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* stream);
+
+/* ---- model-level entry: the reference's `main(void** params)` convention
+ * (src/Compiler/Execution.cpp:21-66; unpacked by
+ * src/Dialect/LLVMExtension/Transforms/AdaptEntryParmsForEngine.cpp:188-284):
+ *   params[0]            int64_t* symbols, or NULL
+ *   then per input, then per output, five slots:
+ *     base*, data*, size_t* offset, size_t* size[rank], size_t* stride[rank]
+ * llc_hip_unpack_params turns that array into descriptors (ranks are known to the plan, as they
+ * are baked into the reference's compiled prologue).  `types` gives the element type of each
+ * tensor.  Returns the number of slots consumed, or a negative llc_status. */
+int llc_hip_unpack_params(void* const* params, size_t n_tensors, const size_t* ranks, const size_t* types,
+                          llc_tensor* tensors_out, const int64_t** symbols_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLC_HIP_H_ */

@@ -1,0 +1,99 @@
+// Host-side plumbing shared by every entry point of the kernel library: status/error reporting,
+// descriptor validation, dtype helpers and launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "llc_hip.h"
+
+namespace llc {
+
+int set_error(int status, const char* fmt, ...);
+
+inline size_t dtype_size(size_t t) {
+  switch (t) {
+    case LLC_INT8: case LLC_INT1: return 1;
+    case LLC_INT16: case LLC_BFLOAT16: case LLC_FLOAT16: return 2;
+    case LLC_INT32: case LLC_FLOAT32: return 4;
+    case LLC_INT64: case LLC_DOUBLE64: return 8;
+  }
+  return 0;
+}
+inline bool is_float_dtype(size_t t) { return t == LLC_FLOAT32 || t == LLC_BFLOAT16 || t == LLC_FLOAT16; }
+
+// Validated view of an llc_tensor: extents/strides as int64, data pointer with `offset` applied.
+struct View {
+  char* ptr = nullptr;
+  int dtype = -1;
+  int rank = 0;
+  int64_t size[LLC_MAX_RANK];
+  int64_t stride[LLC_MAX_RANK];
+  int64_t numel() const {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= size[i];
+    return n;
+  }
+  bool contiguous() const {
+    int64_t s = 1;
+    for (int i = rank - 1; i >= 0; --i) {
+      if (size[i] != 1 && stride[i] != s) return false;
+      s *= size[i];
+    }
+    return true;
+  }
+  size_t esize() const { return dtype_size((size_t)dtype); }
+};
+
+// Fills `v` from `t`; returns LLC_OK or sets the error (naming `what`).
+int make_view(const llc_tensor* t, const char* what, View* v);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+int check_launch(const char* kernel);
+
+#define LLC_TRY(expr)              \
+  do {                             \
+    int _st = (expr);              \
+    if (_st != LLC_OK) return _st; \
+  } while (0)
+
+#define LLC_HIP_TRY(expr)                                                                       \
+  do {                                                                                          \
+    hipError_t _e = (expr);                                                                     \
+    if (_e != hipSuccess) return ::llc::set_error(LLC_ERR_HIP, "%s: %s", #expr, hipGetErrorString(_e)); \
+  } while (0)
+
+// ---- device helpers ----
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+// round to nearest even; NaN stays a quiet NaN
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+
+// exact erf-based GELU: 0.5 x (1 + erf(x / sqrt 2))
+__device__ __forceinline__ float gelu_exact(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+}  // namespace llc

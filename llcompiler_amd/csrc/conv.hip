@@ -1,0 +1,299 @@
+// llh.conv / llh.conv_bias as implicit GEMM on the matrix cores (NCHW x FCHW -> NCHW).
+//
+//   Y[n, f, oh, ow] = act(alpha * sum_{c,kh,kw} W[f, c, kh, kw] * X[n, c, ih, iw] + bias[f] + residual)
+//   ih = oh*stride_h - pad_h + kh*dil_h,  iw = ow*stride_w - pad_w + kw*dil_w   (zero outside)
+//
+// GEMM view per group: rows = filters (FCHW weights are already [F, K] with k = (c,kh,kw)
+// contiguous), columns = output pixels of the whole batch (n, oh, ow), K = C/g*KH*KW.  Pixels are
+// the column dim because they are the contiguous dim of the NCHW output: for a fixed accumulator
+// register 32 lanes store 32 consecutive pixels of one filter plane.
+//
+// The im2col matrix is never materialised.  Each lane owns one pixel column of the tile and a run
+// of consecutive k; it walks (c, kh, kw) incrementally, gathers X with bounds checks (lanes of a
+// wave read consecutive pixels, so loads coalesce for stride 1) and writes its run k-contiguous
+// into the same padded LDS tile layout the matmul kernel uses.  Weights go through the shared
+// vector loader.  fp32 tensors use the fp32 MFMA, bf16/f16 the 16-bit MFMA; accumulation is fp32.
+#include "gemm_core.hpp"
+
+namespace llc {
+using namespace gemm;
+namespace {
+
+struct ConvParams {
+  const char* X;
+  const char* W;
+  char* Y;
+  const char* bias;      // [F] or null
+  const char* residual;  // same layout as Y or null
+  int32_t N, C, H, Wd, F, KH, KW, OH, OW;
+  int32_t ph, pw, sh, sw, dh, dw;
+  int32_t Cg, Fg;   // channels / filters per group
+  int32_t Kdim;     // Cg*KH*KW
+  int32_t ncols;    // N*OH*OW
+  float alpha;
+  int32_t act;
+  int32_t tiles_m, tiles_n;
+};
+
+// Gathers this lane's run of k for one pixel column of the im2col matrix.
+template <typename T, int BN>
+struct Im2colLoader {
+  static constexpr int BK = kRowBytes / sizeof(T);
+  static constexpr int KPT = BK * BN / 256;   // consecutive k per lane
+  static constexpr int kParts = 256 / BN;     // lanes sharing one column
+  static_assert(KPT * sizeof(T) % 16 == 0, "a lane's run must be whole 16-byte vectors");
+  T v[KPT];
+  const T* plane0;  // X + (n*C + g*Cg)*H*W for this lane's pixel
+  int ih0, iw0;
+  bool valid;
+
+  __device__ __forceinline__ void init(const ConvParams& p, int g, int col0) {
+    const int j = threadIdx.x % BN;
+    const int col = col0 + j;
+    valid = col < p.ncols;
+    const int ohw = p.OH * p.OW;
+    const int n = valid ? col / ohw : 0;
+    const int pix = valid ? col % ohw : 0;
+    const int oh = pix / p.OW, ow = pix % p.OW;
+    ih0 = oh * p.sh - p.ph;
+    iw0 = ow * p.sw - p.pw;
+    plane0 = (const T*)p.X + ((int64_t)n * p.C + (int64_t)g * p.Cg) * p.H * p.Wd;
+  }
+
+  __device__ __forceinline__ void load(const ConvParams& p, int k0) {
+    const int kpart = threadIdx.x / BN;
+    int k = k0 + kpart * KPT;
+    const int khw = p.KH * p.KW;
+    int c = k / khw;
+    int r = k - c * khw;
+    int kh = r / p.KW;
+    int kw = r - kh * p.KW;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      T z = static_cast<T>(0.0f);
+      const int ih = ih0 + kh * p.dh, iw = iw0 + kw * p.dw;
+      if (valid && k < p.Kdim && ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd)
+        z = plane0[((int64_t)c * p.H + ih) * p.Wd + iw];
+      v[i] = z;
+      ++k;
+      if (++kw == p.KW) {
+        kw = 0;
+        if (++kh == p.KH) {
+          kh = 0;
+          ++c;
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(char* lds) const {
+    const int j = threadIdx.x % BN, kpart = threadIdx.x / BN;
+    char* dst = lds + j * kRowStride + kpart * KPT * (int)sizeof(T);
+    constexpr int EPV = 16 / sizeof(T);
+#pragma unroll
+    for (int q = 0; q < KPT / EPV; ++q) {
+      struct alignas(16) Pack { T e[EPV]; } pk;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) pk.e[e] = v[q * EPV + e];
+      *(Pack*)(dst + q * 16) = pk;
+    }
+  }
+};
+
+template <typename T, int BM, int BN, int LA>
+__global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
+  constexpr int BK = kRowBytes / sizeof(T);
+  constexpr int WTM = BM / 2, WTN = BN / 2;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int kABytes = BM * kRowStride, kBBytes = BN * kRowStride;
+  constexpr int kBufBytes = kABytes + kBBytes;
+  extern __shared__ __align__(16) char smem[];
+
+  int tile_m, tile_n;
+  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int g = blockIdx.z;
+  const T* Wg = (const T*)p.W + (int64_t)g * p.Fg * p.Kdim;
+
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int wm = wave / 2, wn = wave % 2;
+  const int li = lane % 32, lh = lane / 32;
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  TileLoader<T, BM, LA> la;
+  Im2colLoader<T, BN> lb;
+  lb.init(p, g, n0);
+  const int nk = (p.Kdim + BK - 1) / BK;
+  la.load(Wg, m0, p.Fg, 0, p.Kdim, p.Kdim, 1);
+  lb.load(p, 0);
+  la.store(smem);
+  lb.store(smem + kABytes);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+      la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
+      lb.load(p, (kt + 1) * BK);
+    }
+    const char* sa = smem + cur * kBufBytes + (wm * WTM + li) * kRowStride + lh * 16;
+    const char* sb = smem + cur * kBufBytes + kABytes + (wn * WTN + li) * kRowStride + lh * 16;
+    mma_tile<T, TM, TN>(sa, sb, acc);
+    if (kt + 1 < nk) {
+      la.store(smem + (cur ^ 1) * kBufBytes);
+      lb.store(smem + (cur ^ 1) * kBufBytes + kABytes);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: column = pixel (n, oh*OW+ow), row = filter of this group ----
+  T* Y = (T*)p.Y;
+  const int ohw = p.OH * p.OW;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * WTN + j * 32 + li;
+    if (col >= p.ncols) continue;
+    const int n = col / ohw, pix = col - n * ohw;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+        if (row >= p.Fg) continue;
+        const int f = g * p.Fg + row;
+        const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, f) : 0.0f;
+        epilogue_store<T>(Y, ((int64_t)n * p.F + f) * ohw + pix, acc[i][j][r], p.alpha, bv, p.residual, p.act);
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int LA>
+int launch_cfg(const ConvParams& p0, int groups, hipStream_t s) {
+  ConvParams p = p0;
+  p.tiles_m = (p.Fg + BM - 1) / BM;
+  p.tiles_n = (p.ncols + BN - 1) / BN;
+  const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
+  auto kern = conv_kernel<T, BM, BN, LA>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles > 0x7fffffff || groups > 65535) return set_error(LLC_ERR_TOO_LARGE, "conv: grid too large");
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1, (unsigned)groups), dim3(256), lds, s, p);
+  return check_launch("conv_kernel");
+}
+
+template <typename T, int LA>
+int launch_tiles(const ConvParams& p, int groups, hipStream_t s) {
+  const int64_t t128 = (int64_t)((p.Fg + 127) / 128) * ((p.ncols + 127) / 128) * groups;
+  if (p.Fg > 64 && t128 >= 128) return launch_cfg<T, 128, 128, LA>(p, groups, s);
+  if (p.Fg > 64) return launch_cfg<T, 128, 64, LA>(p, groups, s);
+  if ((int64_t)((p.ncols + 127) / 128) * groups >= 128) return launch_cfg<T, 64, 128, LA>(p, groups, s);
+  return launch_cfg<T, 64, 64, LA>(p, groups, s);
+}
+
+template <typename T>
+int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
+  constexpr int EPV = 16 / sizeof(T);
+  const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
+  if (w_vec) return launch_tiles<T, kLoadKVec>(p, groups, s);
+  return launch_tiles<T, kLoadGeneric>(p, groups, s);
+}
+
+}  // namespace
+}  // namespace llc
+
+using namespace llc;
+
+extern "C" int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* at, const llc_epilogue* epi,
+                              llc_tensor* out, void* stream) {
+  View a, k, o;
+  LLC_TRY(make_view(x, "conv input", &a));
+  LLC_TRY(make_view(w, "conv weight", &k));
+  LLC_TRY(make_view(out, "conv output", &o));
+  if (!at) return set_error(LLC_ERR_BAD_ARG, "conv: null attributes");
+  if (a.dtype != k.dtype || a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "conv: operand types differ");
+  if (a.dtype != LLC_FLOAT32 && a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16)
+    return set_error(LLC_ERR_DTYPE, "conv: element type %d (LLH_FloatTensor expected)", a.dtype);
+  if (a.rank != 4 || k.rank != 4 || o.rank != 4) return set_error(LLC_ERR_SHAPE, "conv: NCHW x FCHW -> NCHW expected");
+  if (!a.contiguous() || !k.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "conv: contiguous tensors expected");
+  const int64_t group = at->group;
+  for (int i = 0; i < 2; ++i)
+    if (at->stride[i] <= 0 || at->dilation[i] <= 0 || at->pad[i] < 0 || at->pad[i + 2] < 0)
+      return set_error(LLC_ERR_BAD_ARG, "conv: bad window attributes");
+  if (group <= 0 || a.size[1] % group || k.size[0] % group || k.size[1] * group != a.size[1])
+    return set_error(LLC_ERR_SHAPE, "conv: C=%lld, weight [%lld,%lld,..], group=%lld do not agree", (long long)a.size[1],
+                     (long long)k.size[0], (long long)k.size[1], (long long)group);
+  if (at->kernel_shape[0] != k.size[2] || at->kernel_shape[1] != k.size[3])
+    return set_error(LLC_ERR_SHAPE, "conv: kernel_shape attribute does not match the weight");
+  // LLHinfersymbolShape.cpp:257-268
+  const int64_t OH = (a.size[2] + at->pad[0] + at->pad[2] - at->dilation[0] * (k.size[2] - 1) - 1) / at->stride[0] + 1;
+  const int64_t OW = (a.size[3] + at->pad[1] + at->pad[3] - at->dilation[1] * (k.size[3] - 1) - 1) / at->stride[1] + 1;
+  if (o.size[0] != a.size[0] || o.size[1] != k.size[0] || o.size[2] != OH || o.size[3] != OW)
+    return set_error(LLC_ERR_SHAPE, "conv: output is %lldx%lldx%lldx%lld, expected %lldx%lldx%lldx%lld", (long long)o.size[0],
+                     (long long)o.size[1], (long long)o.size[2], (long long)o.size[3], (long long)a.size[0],
+                     (long long)k.size[0], (long long)OH, (long long)OW);
+  if (o.numel() == 0) return LLC_OK;
+  if (a.numel() >= (int64_t)1 << 31 || o.numel() >= (int64_t)1 << 31 || k.numel() >= (int64_t)1 << 31)
+    return set_error(LLC_ERR_TOO_LARGE, "conv: tensors of 2^31 elements or more");
+  ConvParams p{};
+  p.X = a.ptr;
+  p.W = k.ptr;
+  p.Y = o.ptr;
+  p.N = (int)a.size[0];
+  p.C = (int)a.size[1];
+  p.H = (int)a.size[2];
+  p.Wd = (int)a.size[3];
+  p.F = (int)k.size[0];
+  p.KH = (int)k.size[2];
+  p.KW = (int)k.size[3];
+  p.OH = (int)OH;
+  p.OW = (int)OW;
+  p.ph = (int)at->pad[0];
+  p.pw = (int)at->pad[1];
+  p.sh = (int)at->stride[0];
+  p.sw = (int)at->stride[1];
+  p.dh = (int)at->dilation[0];
+  p.dw = (int)at->dilation[1];
+  p.Cg = (int)(a.size[1] / group);
+  p.Fg = (int)(k.size[0] / group);
+  p.Kdim = p.Cg * p.KH * p.KW;
+  p.ncols = (int)(a.size[0] * OH * OW);
+  p.alpha = 1.0f;
+  p.act = LLC_ACT_NONE;
+  if (epi) {
+    p.alpha = epi->alpha;
+    if (epi->act < LLC_ACT_NONE || epi->act > LLC_ACT_GELU) return set_error(LLC_ERR_BAD_ARG, "conv: activation %d", epi->act);
+    p.act = epi->act;
+    if (epi->bias) {
+      View b;
+      LLC_TRY(make_view(epi->bias, "conv bias", &b));
+      if (b.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "conv: bias type differs from output");
+      if (b.numel() != p.F || !b.contiguous()) return set_error(LLC_ERR_SHAPE, "conv: bias must hold %d contiguous values", p.F);
+      p.bias = b.ptr;
+    }
+    if (epi->residual) {
+      View r;
+      LLC_TRY(make_view(epi->residual, "conv residual", &r));
+      if (r.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "conv: residual type differs from output");
+      if (r.numel() != o.numel() || !r.contiguous()) return set_error(LLC_ERR_SHAPE, "conv: residual must match the output and be contiguous");
+      p.residual = r.ptr;
+    }
+  }
+  hipStream_t s = as_stream(stream);
+  switch (a.dtype) {
+    case LLC_FLOAT32: return launch_loaders<float>(p, (int)group, s);
+    case LLC_BFLOAT16: return launch_loaders<__bf16>(p, (int)group, s);
+    default: return launch_loaders<_Float16>(p, (int)group, s);
+  }
+}

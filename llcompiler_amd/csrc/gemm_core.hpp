@@ -1,0 +1,205 @@
+// Building blocks shared by the matrix-core kernels (matmul / batch_matmul / conv2d): LDS tile
+// geometry, global->LDS operand staging, the MFMA step and the fused epilogue.
+#pragma once
+#include "common.hpp"
+
+namespace llc {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+namespace gemm {
+
+constexpr int kRowBytes = 128;   // bytes of k per LDS tile row
+constexpr int kRowStride = 144;  // padded row pitch in LDS
+constexpr int kXcds = 8;
+
+enum Loader { kLoadKVec = 0, kLoadRVec = 1, kLoadGeneric = 2 };
+
+template <typename T> struct Elem;
+template <> struct Elem<float> { static constexpr int kDtype = LLC_FLOAT32; };
+template <> struct Elem<__bf16> { static constexpr int kDtype = LLC_BFLOAT16; };
+template <> struct Elem<_Float16> { static constexpr int kDtype = LLC_FLOAT16; };
+
+// ---- one MFMA step on a 16-byte A fragment and a 16-byte B fragment ----
+template <typename T>
+__device__ __forceinline__ void mfma_step(const u32x4_t& a, const u32x4_t& b, f32x16_t& acc) {
+  if constexpr (sizeof(T) == 4) {
+    // k slots inside an 8-k chunk are permuted identically for A and B (lane half h owns k = 4h..4h+3)
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
+  } else if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc,
+                                                  0, 0, 0);
+  } else {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), acc, 0,
+                                                 0, 0);
+  }
+}
+
+// ---- global -> register staging of one operand tile: ROWS rows x 128 bytes of k ----
+// kLoadKVec : unit stride along k.  Each lane moves 16-byte vectors (one row, 8 or 4 consecutive k).
+// kLoadRVec : unit stride along the row index.  Each lane owns a 4(k) x EPV(rows) block, transposed
+//             in registers before it is written to LDS.
+// kLoadGeneric : element-wise with arbitrary strides.
+template <typename T, int ROWS, int MODE>
+struct TileLoader {
+  static constexpr int EPV = 16 / sizeof(T);       // elements per 16 bytes
+  static constexpr int BK = kRowBytes / sizeof(T);  // k extent of a tile
+  static constexpr int kVecs = ROWS * 8;            // 16-byte vectors per tile
+  static constexpr int kIters = (kVecs + 255) / 256;
+  // kLoadRVec: blocks of 4 k x EPV rows
+  static constexpr int kRBlocksPerK = ROWS / EPV;
+  static constexpr int kRBlocks = (BK / 4) * kRBlocksPerK;
+  static constexpr int kRIters = (kRBlocks + 255) / 256;
+  static constexpr int kGenElems = ROWS * BK / 256;
+
+  u32x4_t v[MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * 4 : 1)];
+  T g[MODE == kLoadGeneric ? kGenElems : 1];
+
+  // rows: valid row count of the operand; row0/k0: tile origin; s_r / s_k: element strides
+  __device__ __forceinline__ void load(const T* base, int row0, int rows, int k0, int K, int64_t s_r, int64_t s_k) {
+    const int tid = threadIdx.x;
+    if constexpr (MODE == kLoadKVec) {
+#pragma unroll
+      for (int i = 0; i < kIters; ++i) {
+        const int vid = i * 256 + tid;
+        const int r = vid >> 3, kv = vid & 7;
+        const int gr = row0 + r, gk = k0 + kv * EPV;
+        u32x4_t z = {0, 0, 0, 0};
+        if ((kVecs % 256 == 0 || vid < kVecs) && gr < rows && gk < K) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
+        v[i] = z;
+      }
+    } else if constexpr (MODE == kLoadRVec) {
+#pragma unroll
+      for (int i = 0; i < kRIters; ++i) {
+        const int bid = i * 256 + tid;
+        const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
+        const int gr = row0 + rb * EPV;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const int gk = k0 + kb * 4 + kk;
+          u32x4_t z = {0, 0, 0, 0};
+          if ((kRBlocks % 256 == 0 || bid < kRBlocks) && gr < rows && gk < K) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
+          v[i * 4 + kk] = z;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kGenElems; ++i) {
+        const int e = i * 256 + tid;
+        const int r = e / BK, k = e % BK;
+        const int gr = row0 + r, gk = k0 + k;
+        T z = static_cast<T>(0.0f);
+        if (gr < rows && gk < K) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
+        g[i] = z;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(char* lds) const {
+    const int tid = threadIdx.x;
+    if constexpr (MODE == kLoadKVec) {
+#pragma unroll
+      for (int i = 0; i < kIters; ++i) {
+        const int vid = i * 256 + tid;
+        if (kVecs % 256 == 0 || vid < kVecs) *(u32x4_t*)(lds + (vid >> 3) * kRowStride + (vid & 7) * 16) = v[i];
+      }
+    } else if constexpr (MODE == kLoadRVec) {
+#pragma unroll
+      for (int i = 0; i < kRIters; ++i) {
+        const int bid = i * 256 + tid;
+        if (!(kRBlocks % 256 == 0 || bid < kRBlocks)) continue;
+        const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
+        char* dst = lds + (rb * EPV) * kRowStride + kb * 4 * (int)sizeof(T);
+        const u32x4_t r0 = v[i * 4 + 0], r1 = v[i * 4 + 1], r2 = v[i * 4 + 2], r3 = v[i * 4 + 3];
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x4_t o = {r0[j], r1[j], r2[j], r3[j]};
+            *(u32x4_t*)(dst + j * kRowStride) = o;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            // 16-bit element j of each k-row: low halves for even j, high halves for odd j
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            uint2 o;
+            o.x = __builtin_amdgcn_perm(r1[j >> 1], r0[j >> 1], sel);
+            o.y = __builtin_amdgcn_perm(r3[j >> 1], r2[j >> 1], sel);
+            *(uint2*)(dst + j * kRowStride) = o;
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kGenElems; ++i) {
+        const int e = i * 256 + tid;
+        *(T*)(lds + (e / BK) * kRowStride + (e % BK) * (int)sizeof(T)) = g[i];
+      }
+    }
+  }
+};
+
+
+__device__ __forceinline__ float load_as_f32(const char* p, int dtype, int64_t i) {
+  if (dtype == LLC_FLOAT32) return ((const float*)p)[i];
+  if (dtype == LLC_BFLOAT16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+  return f16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+
+// XCD-aware workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8
+// XCDs by the hardware, so ids are first regrouped per XCD, then walked in column-grouped order
+// (8 tile rows per group): each XCD's L2 sees a compact patch of the output.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  int id = blockIdx.x;
+  if (total % kXcds == 0) id = (id % kXcds) * (total / kXcds) + id / kXcds;
+  const int G = 8;
+  const int per_group = G * tiles_n;
+  const int group = id / per_group;
+  const int first_m = group * G;
+  const int gsize = (tiles_m - first_m) < G ? (tiles_m - first_m) : G;
+  const int in_group = id % per_group;
+  tm = first_m + in_group % gsize;
+  tn = in_group / gsize;
+}
+
+// MFMAs of one LDS tile pair for one wave: TM x TN fragments of 32x32, four 16-byte k-chunks pairs.
+// sa / sb point at this lane's first fragment row (+ lane-half chunk offset) inside the A / B tile.
+template <typename T, int TM, int TN>
+__device__ __forceinline__ void mma_tile(const char* sa, const char* sb, f32x16_t (&acc)[TM][TN]) {
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    u32x4_t fa[TM], fb[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = *(const u32x4_t*)(sa + i * 32 * kRowStride + s * 32);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = *(const u32x4_t*)(sb + j * 32 * kRowStride + s * 32);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) mfma_step<T>(fa[i], fb[j], acc[i][j]);
+  }
+}
+
+// act(alpha * acc + bias + residual) -> storage type, one element
+template <typename T>
+__device__ __forceinline__ void epilogue_store(T* C, int64_t o, float acc, float alpha, float bias, const char* res,
+                                               int act) {
+  constexpr int dt = Elem<T>::kDtype;
+  float v = acc * alpha + bias;
+  if (res) v += load_as_f32(res, dt, o);
+  if (act == LLC_ACT_RELU) v = (v > 0.0f || v != v) ? v : 0.0f;
+  else if (act == LLC_ACT_GELU) v = gelu_exact(v);
+  if constexpr (dt == LLC_FLOAT32) C[o] = v;
+  else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o] = f32_to_bf16_bits(v);
+  else ((uint16_t*)C)[o] = f32_to_f16_bits(v);
+}
+
+}  // namespace gemm
+}  // namespace llc

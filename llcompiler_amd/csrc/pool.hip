@@ -1,0 +1,100 @@
+// llh.max_pool over NCHW.  One lane per output element, lanes consecutive along OW so that window
+// rows are read as contiguous (stride-`stride_w`) runs; overlapping windows are served by L1/L2, so
+// HBM traffic stays at input once + output once.
+#include "common.hpp"
+
+namespace llc {
+namespace {
+
+struct PoolParams {
+  const char* x;
+  char* y;
+  int32_t dtype;
+  int32_t H, W, OH, OW;
+  int32_t KH, KW, ph, pw, sh, sw, dh, dw;
+  int32_t init_zero;
+  int64_t total;  // N*C*OH*OW
+};
+
+
+template <int DT>
+__global__ __launch_bounds__(256) void max_pool_kernel(const PoolParams p) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= p.total) return;
+  const int ow = (int)(o % p.OW);
+  int64_t t = o / p.OW;
+  const int oh = (int)(t % p.OH);
+  const int64_t nc = t / p.OH;
+  const int64_t plane = nc * p.H * p.W;
+  float acc = p.init_zero ? 0.0f : -INFINITY;
+  for (int kh = 0; kh < p.KH; ++kh) {
+    const int ih = oh * p.sh - p.ph + kh * p.dh;
+    if (ih < 0 || ih >= p.H) continue;
+    for (int kw = 0; kw < p.KW; ++kw) {
+      const int iw = ow * p.sw - p.pw + kw * p.dw;
+      if (iw < 0 || iw >= p.W) continue;
+      const int64_t i = plane + (int64_t)ih * p.W + iw;
+      float v;
+      if constexpr (DT == LLC_FLOAT32) v = ((const float*)p.x)[i];
+      else if constexpr (DT == LLC_BFLOAT16) v = bf16_bits_to_f32(((const uint16_t*)p.x)[i]);
+      else v = f16_bits_to_f32(((const uint16_t*)p.x)[i]);
+      acc = (v > acc || v != v) ? v : acc;  // NaN propagates, like stablehlo.maximum / torch
+    }
+  }
+  if constexpr (DT == LLC_FLOAT32) ((float*)p.y)[o] = acc;
+  else if constexpr (DT == LLC_BFLOAT16) ((uint16_t*)p.y)[o] = f32_to_bf16_bits(acc);
+  else ((uint16_t*)p.y)[o] = f32_to_f16_bits(acc);
+}
+
+}  // namespace
+}  // namespace llc
+
+using namespace llc;
+
+extern "C" int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* at, llc_tensor* out, void* stream) {
+  View a, o;
+  LLC_TRY(make_view(x, "max_pool input", &a));
+  LLC_TRY(make_view(out, "max_pool output", &o));
+  if (!at) return set_error(LLC_ERR_BAD_ARG, "max_pool: null attributes");
+  if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "max_pool: input and output types differ");
+  if (a.dtype != LLC_FLOAT32 && a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16)
+    return set_error(LLC_ERR_DTYPE, "max_pool: element type %d", a.dtype);
+  if (a.rank != 4 || o.rank != 4) return set_error(LLC_ERR_SHAPE, "max_pool: NCHW tensors expected");
+  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "max_pool: contiguous tensors expected");
+  for (int i = 0; i < 2; ++i)
+    if (at->kernel_shape[i] <= 0 || at->stride[i] <= 0 || at->dilation[i] <= 0 || at->pad[i] < 0 || at->pad[i + 2] < 0)
+      return set_error(LLC_ERR_BAD_ARG, "max_pool: bad window attributes");
+  // LLHinfersymbolShape.cpp:257-268 (the pooling rule shares the convolution formula)
+  const int64_t OH = (a.size[2] + at->pad[0] + at->pad[2] - at->dilation[0] * (at->kernel_shape[0] - 1) - 1) / at->stride[0] + 1;
+  const int64_t OW = (a.size[3] + at->pad[1] + at->pad[3] - at->dilation[1] * (at->kernel_shape[1] - 1) - 1) / at->stride[1] + 1;
+  if (o.size[0] != a.size[0] || o.size[1] != a.size[1] || o.size[2] != OH || o.size[3] != OW)
+    return set_error(LLC_ERR_SHAPE, "max_pool: output is %lldx%lldx%lldx%lld, expected %lldx%lldx%lldx%lld",
+                     (long long)o.size[0], (long long)o.size[1], (long long)o.size[2], (long long)o.size[3],
+                     (long long)a.size[0], (long long)a.size[1], (long long)OH, (long long)OW);
+  PoolParams p{};
+  p.x = a.ptr;
+  p.y = o.ptr;
+  p.dtype = a.dtype;
+  p.H = (int)a.size[2];
+  p.W = (int)a.size[3];
+  p.OH = (int)OH;
+  p.OW = (int)OW;
+  p.KH = (int)at->kernel_shape[0];
+  p.KW = (int)at->kernel_shape[1];
+  p.ph = (int)at->pad[0];
+  p.pw = (int)at->pad[1];
+  p.sh = (int)at->stride[0];
+  p.sw = (int)at->stride[1];
+  p.dh = (int)at->dilation[0];
+  p.dw = (int)at->dilation[1];
+  p.init_zero = at->init_zero;
+  p.total = o.numel();
+  if (p.total == 0) return LLC_OK;
+  const int64_t blocks = (p.total + 255) / 256;
+  if (blocks > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "max_pool: output too large");
+  hipStream_t s = as_stream(stream);
+  if (a.dtype == LLC_FLOAT32) hipLaunchKernelGGL((max_pool_kernel<LLC_FLOAT32>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+  else if (a.dtype == LLC_BFLOAT16) hipLaunchKernelGGL((max_pool_kernel<LLC_BFLOAT16>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((max_pool_kernel<LLC_FLOAT16>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+  return check_launch("max_pool_kernel");
+}

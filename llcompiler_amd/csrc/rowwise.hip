@@ -1,0 +1,492 @@
+// Row-wise kernels over the last (contiguous) dim: softmax, layer_norm and reduce_sum/max/min.
+//
+// A row is read from HBM exactly once: TPR lanes share a row, each lane keeps ITEMS vectors of VEC
+// elements in registers, statistics are reduced with wave64 cross-lane shuffles (and one LDS hop
+// when a row spans several waves), and the result is written once.  Statistics are always fp32.
+// Algorithmic traffic is therefore read + write of the tensor, which is what these kernels are
+// measured against.
+#include "common.hpp"
+
+namespace llc {
+namespace {
+
+enum RowOp { kSoftmax = 0, kLayerNorm = 1, kReduce = 2 };
+
+struct RowParams {
+  const char* x;
+  char* y;
+  const char* gamma;  // layer_norm scale (may be null)
+  const char* beta;   // layer_norm bias (may be null)
+  int32_t dtype;      // storage type of x / y / gamma / beta
+  int32_t kind;       // llc_reduce_kind for kReduce
+  int64_t rows;
+  int32_t cols;
+  float eps;
+  float scale;  // kReduce: result multiplied by this (1/HW for average pooling)
+};
+
+template <int VEC>
+__device__ __forceinline__ void load_row_vec(const char* base, int dtype, int64_t off, float* dst) {
+  if (dtype == LLC_FLOAT32) {
+    struct alignas(4 * VEC) P { float v[VEC]; };
+    P p = *(const P*)(base + off * 4);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) dst[j] = p.v[j];
+  } else {
+    struct alignas(2 * VEC) P { uint16_t v[VEC]; };
+    P p = *(const P*)(base + off * 2);
+    if (dtype == LLC_BFLOAT16) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) dst[j] = bf16_bits_to_f32(p.v[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) dst[j] = f16_bits_to_f32(p.v[j]);
+    }
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void store_row_vec(char* base, int dtype, int64_t off, const float* src) {
+  if (dtype == LLC_FLOAT32) {
+    struct alignas(4 * VEC) P { float v[VEC]; } p;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) p.v[j] = src[j];
+    *(P*)(base + off * 4) = p;
+  } else {
+    struct alignas(2 * VEC) P { uint16_t v[VEC]; } p;
+    if (dtype == LLC_BFLOAT16) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_bf16_bits(src[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_f16_bits(src[j]);
+    }
+    *(P*)(base + off * 2) = p;
+  }
+}
+
+__device__ __forceinline__ float nmax(float a, float b) { return (a > b || a != a) ? a : b; }
+__device__ __forceinline__ float nmin(float a, float b) { return (a < b || a != a) ? a : b; }
+
+enum Combine { kAdd = 0, kMax = 1, kMin = 2 };
+template <int C> __device__ __forceinline__ float combine(float a, float b) {
+  if constexpr (C == kAdd) return a + b;
+  else if constexpr (C == kMax) return nmax(a, b);
+  else return nmin(a, b);
+}
+
+// Reduction over the TPR lanes that share a row.  TPR <= 64: xor-shuffles inside the wave.
+// TPR == 256: the whole block is one row; wave results meet in LDS.
+template <int TPR, int C>
+__device__ __forceinline__ float row_reduce(float v, float* smem) {
+  constexpr int W = TPR < kWave ? TPR : kWave;
+#pragma unroll
+  for (int o = W / 2; o > 0; o >>= 1) v = combine<C>(v, __shfl_xor(v, o, kWave));
+  if constexpr (TPR > kWave) {
+    constexpr int NW = TPR / kWave;
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();  // smem reuse across successive reductions
+    if ((threadIdx.x & (kWave - 1)) == 0) smem[wave] = v;
+    __syncthreads();
+    v = smem[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) v = combine<C>(v, smem[w]);
+  }
+  return v;
+}
+
+template <int OP, int VEC, int TPR, int ITEMS>
+__global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
+  __shared__ float smem[4];
+  constexpr int RPB = 256 / TPR;  // rows per block
+  const int lane = threadIdx.x % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const bool row_ok = row < p.rows;
+  const int64_t base = row * p.cols;
+
+  float v[ITEMS][VEC];
+  bool ok[ITEMS];
+  const float fill = (OP == kSoftmax) ? -INFINITY
+                     : (OP == kReduce) ? (p.kind == LLC_REDUCE_SUM ? 0.0f : (p.kind == LLC_REDUCE_MAX ? -INFINITY : INFINITY))
+                                       : 0.0f;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int col = (it * TPR + lane) * VEC;
+    ok[it] = row_ok && col < p.cols;
+    if (ok[it]) load_row_vec<VEC>(p.x, p.dtype, base + col, v[it]);
+    else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[it][j] = fill;
+    }
+  }
+
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) m = nmax(m, v[it][j]);
+    m = row_reduce<TPR, kMax>(m, smem);
+    float s = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        // masked lanes hold -inf: exp(-inf - m) = 0 for finite m; keep them out when m is -inf too
+        float e = ok[it] ? expf(v[it][j] - m) : 0.0f;
+        v[it][j] = e;
+        s += e;
+      }
+    s = row_reduce<TPR, kAdd>(s, smem);
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      if (ok[it]) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[it][j] *= inv;
+        store_row_vec<VEC>(p.y, p.dtype, base + (it * TPR + lane) * VEC, v[it]);
+      }
+    }
+  } else if constexpr (OP == kLayerNorm) {
+    float s = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s += v[it][j];
+    s = row_reduce<TPR, kAdd>(s, smem);
+    const float mean = s / (float)p.cols;
+    float q = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float d = ok[it] ? v[it][j] - mean : 0.0f;
+        v[it][j] = d;
+        q += d * d;
+      }
+    q = row_reduce<TPR, kAdd>(q, smem);
+    const float rstd = 1.0f / sqrtf(q / (float)p.cols + p.eps);
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      if (ok[it]) {
+        const int col = (it * TPR + lane) * VEC;
+        float g[VEC], b[VEC];
+        if (p.gamma) load_row_vec<VEC>(p.gamma, p.dtype, col, g);
+        if (p.beta) load_row_vec<VEC>(p.beta, p.dtype, col, b);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          float t = v[it][j] * rstd;
+          if (p.gamma) t *= g[j];
+          if (p.beta) t += b[j];
+          v[it][j] = t;
+        }
+        store_row_vec<VEC>(p.y, p.dtype, base + col, v[it]);
+      }
+    }
+  } else {
+    float r;
+    if (p.kind == LLC_REDUCE_SUM) {
+      r = 0.0f;
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) r += v[it][j];
+      r = row_reduce<TPR, kAdd>(r, smem) * p.scale;
+    } else if (p.kind == LLC_REDUCE_MAX) {
+      r = -INFINITY;
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) r = nmax(r, v[it][j]);
+      r = row_reduce<TPR, kMax>(r, smem);
+    } else {
+      r = INFINITY;
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) r = nmin(r, v[it][j]);
+      r = row_reduce<TPR, kMin>(r, smem);
+    }
+    if (row_ok && lane == 0) {
+      float one[1] = {r};
+      store_row_vec<1>(p.y, p.dtype, row, one);
+    }
+  }
+}
+
+// Rows too long for registers: one block per row, three strided sweeps over the row (the second
+// and third hit L2).  Correctness path for rare shapes, not a tuned one.
+template <int OP>
+__global__ __launch_bounds__(256) void row_loop_kernel(const RowParams p) {
+  __shared__ float smem[4];
+  const int64_t row = blockIdx.x;
+  const int64_t base = row * p.cols;
+  float one[1];
+  if constexpr (OP == kSoftmax) {
+    float m = -INFINITY;
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      m = nmax(m, one[0]);
+    }
+    m = row_reduce<256, kMax>(m, smem);
+    float s = 0.0f;
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      s += expf(one[0] - m);
+    }
+    s = row_reduce<256, kAdd>(s, smem);
+    const float inv = 1.0f / s;
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      one[0] = expf(one[0] - m) * inv;
+      store_row_vec<1>(p.y, p.dtype, base + c, one);
+    }
+  } else if constexpr (OP == kLayerNorm) {
+    float s = 0.0f;
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      s += one[0];
+    }
+    s = row_reduce<256, kAdd>(s, smem);
+    const float mean = s / (float)p.cols;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      float d = one[0] - mean;
+      q += d * d;
+    }
+    q = row_reduce<256, kAdd>(q, smem);
+    const float rstd = 1.0f / sqrtf(q / (float)p.cols + p.eps);
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      float t = (one[0] - mean) * rstd;
+      float g[1], b[1];
+      if (p.gamma) { load_row_vec<1>(p.gamma, p.dtype, c, g); t *= g[0]; }
+      if (p.beta) { load_row_vec<1>(p.beta, p.dtype, c, b); t += b[0]; }
+      one[0] = t;
+      store_row_vec<1>(p.y, p.dtype, base + c, one);
+    }
+  } else {
+    float r = p.kind == LLC_REDUCE_SUM ? 0.0f : (p.kind == LLC_REDUCE_MAX ? -INFINITY : INFINITY);
+    for (int c = threadIdx.x; c < p.cols; c += 256) {
+      load_row_vec<1>(p.x, p.dtype, base + c, one);
+      r = p.kind == LLC_REDUCE_SUM ? r + one[0] : (p.kind == LLC_REDUCE_MAX ? nmax(r, one[0]) : nmin(r, one[0]));
+    }
+    if (p.kind == LLC_REDUCE_SUM) r = row_reduce<256, kAdd>(r, smem) * p.scale;
+    else if (p.kind == LLC_REDUCE_MAX) r = row_reduce<256, kMax>(r, smem);
+    else r = row_reduce<256, kMin>(r, smem);
+    if (threadIdx.x == 0) {
+      one[0] = r;
+      store_row_vec<1>(p.y, p.dtype, row, one);
+    }
+  }
+}
+
+// Reduction over a middle dim: x viewed as [outer, R, inner], inner > 1.  One lane per output
+// element, lanes consecutive along `inner` so every load is coalesced; R is walked sequentially.
+__global__ __launch_bounds__(256) void mid_reduce_kernel(const RowParams p, int64_t outer, int64_t R, int64_t inner) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= outer * inner) return;
+  const int64_t i = o % inner, b = o / inner;
+  float r = p.kind == LLC_REDUCE_SUM ? 0.0f : (p.kind == LLC_REDUCE_MAX ? -INFINITY : INFINITY);
+  float one[1];
+  for (int64_t k = 0; k < R; ++k) {
+    load_row_vec<1>(p.x, p.dtype, (b * R + k) * inner + i, one);
+    r = p.kind == LLC_REDUCE_SUM ? r + one[0] : (p.kind == LLC_REDUCE_MAX ? nmax(r, one[0]) : nmin(r, one[0]));
+  }
+  if (p.kind == LLC_REDUCE_SUM) r *= p.scale;
+  one[0] = r;
+  store_row_vec<1>(p.y, p.dtype, o, one);
+}
+
+template <int OP, int VEC, int TPR>
+void launch_items(const RowParams& p, int items, hipStream_t s) {
+  const int rpb = 256 / TPR;
+  const unsigned blocks = (unsigned)((p.rows + rpb - 1) / rpb);
+  switch (items) {
+    case 1: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 1>), dim3(blocks), dim3(256), 0, s, p); break;
+    case 2: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 2>), dim3(blocks), dim3(256), 0, s, p); break;
+    case 4: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 4>), dim3(blocks), dim3(256), 0, s, p); break;
+    default: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 8>), dim3(blocks), dim3(256), 0, s, p); break;
+  }
+}
+
+template <int OP, int VEC>
+bool launch_tpr(const RowParams& p, hipStream_t s) {
+  // smallest register tile that holds a row; ties go to fewer lanes per row (no LDS hop)
+  const int tprs[3] = {16, 64, 256};
+  const int items[4] = {1, 2, 4, 8};
+  int best_t = 0, best_i = 0;
+  int64_t best_cap = -1;
+  for (int t : tprs)
+    for (int i : items) {
+      int64_t cap = (int64_t)t * i * VEC;
+      if (cap >= p.cols && (best_cap < 0 || cap < best_cap)) {
+        best_cap = cap;
+        best_t = t;
+        best_i = i;
+      }
+    }
+  if (best_cap < 0) return false;
+  if (best_t == 16) launch_items<OP, VEC, 16>(p, best_i, s);
+  else if (best_t == 64) launch_items<OP, VEC, 64>(p, best_i, s);
+  else launch_items<OP, VEC, 256>(p, best_i, s);
+  return true;
+}
+
+template <int OP>
+int launch_rows(const RowParams& p, hipStream_t s) {
+  if (p.rows == 0 || p.cols == 0) return LLC_OK;
+  if (p.rows > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "row kernel: %lld rows", (long long)p.rows);
+  const int es = p.dtype == LLC_FLOAT32 ? 4 : 2;
+  const int wide = 16 / es;
+  auto al = [&](const void* q) { return q == nullptr || ((uintptr_t)q % 16) == 0; };
+  bool vec_ok = (p.cols % wide) == 0 && al(p.x) && (OP == kReduce || al(p.y)) && al(p.gamma) && al(p.beta);
+  bool done = false;
+  if (vec_ok) done = es == 4 ? launch_tpr<OP, 4>(p, s) : launch_tpr<OP, 8>(p, s);
+  if (!done && p.cols <= 2048) done = launch_tpr<OP, 1>(p, s);
+  if (!done) hipLaunchKernelGGL((row_loop_kernel<OP>), dim3((unsigned)p.rows), dim3(256), 0, s, p);
+  return check_launch("row_kernel");
+}
+
+int row_dtype_ok(const View& v, const char* what) {
+  if (v.dtype != LLC_FLOAT32 && v.dtype != LLC_BFLOAT16 && v.dtype != LLC_FLOAT16)
+    return set_error(LLC_ERR_DTYPE, "%s: element type %d (f32, bf16 or f16 expected)", what, v.dtype);
+  return LLC_OK;
+}
+
+}  // namespace
+}  // namespace llc
+
+using namespace llc;
+
+extern "C" int llc_hip_softmax(const llc_tensor* x, llc_tensor* out, void* stream) {
+  View a, o;
+  LLC_TRY(make_view(x, "softmax input", &a));
+  LLC_TRY(make_view(out, "softmax output", &o));
+  LLC_TRY(row_dtype_ok(a, "softmax"));
+  if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "softmax: input and output types differ");
+  if (a.rank < 1 || a.rank != o.rank) return set_error(LLC_ERR_SHAPE, "softmax: rank mismatch");
+  for (int d = 0; d < a.rank; ++d)
+    if (a.size[d] != o.size[d]) return set_error(LLC_ERR_SHAPE, "softmax: extent mismatch at dim %d", d);
+  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "softmax: contiguous tensors expected");
+  RowParams p{};
+  p.x = a.ptr;
+  p.y = o.ptr;
+  p.dtype = a.dtype;
+  p.cols = (int32_t)a.size[a.rank - 1];
+  if (a.size[a.rank - 1] >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "softmax: row too long");
+  p.rows = p.cols ? a.numel() / p.cols : 0;
+  return launch_rows<kSoftmax>(p, as_stream(stream));
+}
+
+extern "C" int llc_hip_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_tensor* bias, double epsilon,
+                                  llc_tensor* out, void* stream) {
+  View a, o, g, b;
+  LLC_TRY(make_view(x, "layer_norm input", &a));
+  LLC_TRY(make_view(out, "layer_norm output", &o));
+  LLC_TRY(row_dtype_ok(a, "layer_norm"));
+  if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "layer_norm: input and output types differ");
+  if (a.rank < 1 || a.rank != o.rank) return set_error(LLC_ERR_SHAPE, "layer_norm: rank mismatch");
+  for (int d = 0; d < a.rank; ++d)
+    if (a.size[d] != o.size[d]) return set_error(LLC_ERR_SHAPE, "layer_norm: extent mismatch at dim %d", d);
+  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "layer_norm: contiguous tensors expected");
+  RowParams p{};
+  const int64_t cols = a.size[a.rank - 1];
+  if (cols >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "layer_norm: row too long");
+  if (scale) {
+    LLC_TRY(make_view(scale, "layer_norm scale", &g));
+    if (g.dtype != a.dtype) return set_error(LLC_ERR_DTYPE, "layer_norm: scale type differs from input");
+    if (g.numel() != cols || !g.contiguous()) return set_error(LLC_ERR_SHAPE, "layer_norm: scale must hold %lld contiguous values", (long long)cols);
+    p.gamma = g.ptr;
+  }
+  if (bias) {
+    LLC_TRY(make_view(bias, "layer_norm bias", &b));
+    if (b.dtype != a.dtype) return set_error(LLC_ERR_DTYPE, "layer_norm: bias type differs from input");
+    if (b.numel() != cols || !b.contiguous()) return set_error(LLC_ERR_SHAPE, "layer_norm: bias must hold %lld contiguous values", (long long)cols);
+    p.beta = b.ptr;
+  }
+  p.x = a.ptr;
+  p.y = o.ptr;
+  p.dtype = a.dtype;
+  p.cols = (int32_t)cols;
+  p.rows = cols ? a.numel() / cols : 0;
+  p.eps = (float)epsilon;
+  return launch_rows<kLayerNorm>(p, as_stream(stream));
+}
+
+namespace llc {
+// [outer, R, inner] reduction used by llc_hip_reduce and the global average pool.
+int reduce_3d(const View& a, const View& o, int kind, int64_t outer, int64_t R, int64_t inner, float scale,
+              hipStream_t s) {
+  RowParams p{};
+  p.x = a.ptr;
+  p.y = o.ptr;
+  p.dtype = a.dtype;
+  p.kind = kind;
+  p.scale = scale;
+  if (outer * inner == 0) return LLC_OK;
+  if (R >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "reduce: %lld reduced elements", (long long)R);
+  if (inner == 1) {
+    p.rows = outer;
+    p.cols = (int32_t)R;
+    if (R == 0) {  // empty reduction: the init value
+      p.cols = 0;
+    }
+    return launch_rows<kReduce>(p, s);
+  }
+  const int64_t n = outer * inner;
+  if ((n + 255) / 256 > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "reduce: too many outputs");
+  hipLaunchKernelGGL(mid_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, outer, R, inner);
+  return check_launch("mid_reduce_kernel");
+}
+}  // namespace llc
+
+extern "C" int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
+                              void* stream) {
+  View a, o;
+  LLC_TRY(make_view(x, "reduce input", &a));
+  LLC_TRY(make_view(out, "reduce output", &o));
+  LLC_TRY(row_dtype_ok(a, "reduce"));
+  if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "reduce: input and output types differ");
+  if (kind < LLC_REDUCE_SUM || kind > LLC_REDUCE_MIN) return set_error(LLC_ERR_BAD_ARG, "reduce: kind %d", kind);
+  if (n_axes == 0 || !axes) return set_error(LLC_ERR_BAD_ARG, "reduce: no axes");
+  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "reduce: contiguous tensors expected");
+  bool red[LLC_MAX_RANK] = {false};
+  for (size_t i = 0; i < n_axes; ++i) {
+    int64_t ax = axes[i] < 0 ? axes[i] + a.rank : axes[i];
+    if (ax < 0 || ax >= a.rank) return set_error(LLC_ERR_BAD_ARG, "reduce: axis %lld out of range", (long long)axes[i]);
+    red[ax] = true;
+  }
+  int first = -1, last = -1;
+  for (int d = 0; d < a.rank; ++d)
+    if (red[d]) {
+      if (first < 0) first = d;
+      last = d;
+    }
+  int64_t outer = 1, R = 1, inner = 1, kept = 1;
+  for (int d = 0; d < a.rank; ++d) {
+    if (d < first) outer *= a.size[d];
+    else if (d <= last) {
+      // a kept dim of extent 1 between reduced dims does not break adjacency
+      if (!red[d] && a.size[d] != 1) return set_error(LLC_ERR_UNSUPPORTED, "reduce: reduced axes must be adjacent");
+      R *= a.size[d];
+    } else inner *= a.size[d];
+    if (!red[d]) kept *= a.size[d];
+  }
+  if (o.numel() != kept) return set_error(LLC_ERR_SHAPE, "reduce: output holds %lld elements, expected %lld", (long long)o.numel(), (long long)kept);
+  return reduce_3d(a, o, kind, outer, R, inner, 1.0f, as_stream(stream));
+}
+
+extern "C" int llc_hip_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream) {
+  View a, o;
+  LLC_TRY(make_view(x, "global_avg_pool input", &a));
+  LLC_TRY(make_view(out, "global_avg_pool output", &o));
+  LLC_TRY(row_dtype_ok(a, "global_avg_pool"));
+  if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "global_avg_pool: input and output types differ");
+  if (a.rank != 4) return set_error(LLC_ERR_SHAPE, "global_avg_pool: NCHW input expected");
+  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "global_avg_pool: contiguous tensors expected");
+  const int64_t nc = a.size[0] * a.size[1], hw = a.size[2] * a.size[3];
+  if (o.numel() != nc) return set_error(LLC_ERR_SHAPE, "global_avg_pool: output holds %lld elements, expected %lld", (long long)o.numel(), (long long)nc);
+  if (hw == 0) return set_error(LLC_ERR_SHAPE, "global_avg_pool: empty window");
+  return reduce_3d(a, o, LLC_REDUCE_SUM, nc, hw, 1, 1.0f / (float)hw, as_stream(stream));
+}

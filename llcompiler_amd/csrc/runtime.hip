@@ -1,0 +1,104 @@
+// Library-level entry points: version, device selection, error text, descriptor validation and
+// the unpacking of the reference's packed `main(void**)` parameter array.
+#include <cstring>
+
+#include "common.hpp"
+
+namespace llc {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int make_view(const llc_tensor* t, const char* what, View* v) {
+  if (!t) return set_error(LLC_ERR_BAD_ARG, "%s: null tensor descriptor", what);
+  if (t->rank > LLC_MAX_RANK) return set_error(LLC_ERR_SHAPE, "%s: rank %zu > %d", what, t->rank, LLC_MAX_RANK);
+  size_t es = dtype_size(t->type);
+  if (es == 0) return set_error(LLC_ERR_DTYPE, "%s: unknown element type code %zu", what, t->type);
+  if (t->rank > 0 && (!t->size || !t->stride)) return set_error(LLC_ERR_BAD_ARG, "%s: null size/stride array", what);
+  v->dtype = (int)t->type;
+  v->rank = (int)t->rank;
+  int64_t n = 1;
+  for (size_t i = 0; i < t->rank; ++i) {
+    v->size[i] = (int64_t)t->size[i];
+    v->stride[i] = (int64_t)t->stride[i];
+    if (v->size[i] < 0) return set_error(LLC_ERR_SHAPE, "%s: negative extent", what);
+    n *= v->size[i];
+  }
+  if (n > 0 && !t->data) return set_error(LLC_ERR_BAD_ARG, "%s: null data pointer", what);
+  v->ptr = (char*)t->data + t->offset * es;
+  return LLC_OK;
+}
+
+int check_launch(const char* kernel) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(LLC_ERR_HIP, "launch of %s failed: %s", kernel, hipGetErrorString(e));
+  return LLC_OK;
+}
+
+}  // namespace llc
+
+using namespace llc;
+
+extern "C" int llc_hip_abi_version(void) { return LLC_HIP_ABI_VERSION; }
+
+extern "C" const char* llc_hip_last_error(void) { return g_err; }
+
+extern "C" const char* llc_hip_status_string(int status) {
+  switch (status) {
+    case LLC_OK: return "ok";
+    case LLC_ERR_BAD_ARG: return "bad argument";
+    case LLC_ERR_DTYPE: return "unsupported or mismatched element type";
+    case LLC_ERR_SHAPE: return "shape mismatch";
+    case LLC_ERR_LAYOUT: return "unsupported strides";
+    case LLC_ERR_UNSUPPORTED: return "unsupported attribute combination";
+    case LLC_ERR_HIP: return "HIP runtime error";
+    case LLC_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case LLC_ERR_TOO_LARGE: return "tensor too large for this kernel";
+  }
+  return "unknown status";
+}
+
+extern "C" int llc_hip_init(int device) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return set_error(LLC_ERR_NO_DEVICE, "no HIP device visible");
+  if (device < 0 || device >= n) return set_error(LLC_ERR_BAD_ARG, "device %d out of range (0..%d)", device, n - 1);
+  LLC_HIP_TRY(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  LLC_HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return set_error(LLC_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device,
+                     prop.gcnArchName);
+  return LLC_OK;
+}
+
+extern "C" int llc_hip_unpack_params(void* const* params, size_t n_tensors, const size_t* ranks, const size_t* types,
+                                     llc_tensor* tensors_out, const int64_t** symbols_out) {
+  if (!params || (n_tensors && (!ranks || !types || !tensors_out)))
+    return set_error(LLC_ERR_BAD_ARG, "unpack_params: null argument");
+  if (symbols_out) *symbols_out = (const int64_t*)params[0];
+  size_t slot = 1;
+  for (size_t i = 0; i < n_tensors; ++i) {
+    llc_tensor* t = &tensors_out[i];
+    if (ranks[i] > LLC_MAX_RANK) return set_error(LLC_ERR_SHAPE, "unpack_params: tensor %zu has rank %zu", i, ranks[i]);
+    t->base = params[slot + 0];
+    t->data = params[slot + 1];
+    const size_t* off = (const size_t*)params[slot + 2];
+    if (!off) return set_error(LLC_ERR_BAD_ARG, "unpack_params: tensor %zu has a null offset slot", i);
+    t->offset = *off;
+    t->type = types[i];
+    t->rank = ranks[i];
+    t->size = (const size_t*)params[slot + 3];
+    t->stride = (const size_t*)params[slot + 4];
+    if (ranks[i] && (!t->size || !t->stride))
+      return set_error(LLC_ERR_BAD_ARG, "unpack_params: tensor %zu has null size/stride slots", i);
+    slot += 5;
+  }
+  return (int)slot;
+}

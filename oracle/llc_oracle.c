@@ -30,8 +30,8 @@ enum {
   LLC_U_LOG = 10, LLC_U_RECIP = 11
 };
 enum { LLC_B_ADD = 0, LLC_B_SUB = 1, LLC_B_MUL = 2, LLC_B_DIV = 3, LLC_B_MAX = 4, LLC_B_MIN = 5, LLC_B_POW = 6 };
-/* LLHEnums.td:86-100 CompareKind order */
-enum { LLC_C_EQ = 0, LLC_C_LE = 1, LLC_C_LT = 2, LLC_C_GE = 3, LLC_C_GT = 4, LLC_C_NE = 5 };
+/* CompareKind values of include/llcompiler/Dialect/LLH/IR/LLHEnums.td:111-116 */
+enum { LLC_C_EQ = 1, LLC_C_GE = 2, LLC_C_LE = 3, LLC_C_GT = 4, LLC_C_LT = 5, LLC_C_NE = 6 };
 enum { LLC_R_SUM = 0, LLC_R_MAX = 1, LLC_R_MIN = 2 };
 
 /* ---- bf16 helpers: round-to-nearest-even, NaN kept quiet ---- */

@@ -17,7 +17,7 @@ _LIB_PATH = os.path.join(_HERE, "libllc_oracle.so")
 UNARY = {"abs": 0, "sqrt": 1, "exp": 2, "relu": 3, "rsqrt": 4, "neg": 5, "gelu": 6, "tanh": 7,
          "erf": 8, "sigmoid": 9, "log": 10, "recip": 11}
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "max": 4, "min": 5, "pow": 6}
-COMPARE = {"EQ": 0, "LE": 1, "LT": 2, "GE": 3, "GT": 4, "NE": 5}
+COMPARE = {"EQ": 1, "GE": 2, "LE": 3, "GT": 4, "LT": 5, "NE": 6}
 REDUCE = {"sum": 0, "max": 1, "min": 2}
 
 

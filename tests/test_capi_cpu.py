@@ -1,0 +1,83 @@
+"""CPU-side checks of the boundary: the library loads, exports every symbol the header declares,
+and the argument validation that needs no GPU reports errors instead of crashing."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from llcompiler_amd import _capi as C
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "llc_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(llc_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols() == sorted(C.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(C.LIB_PATH), "build the library first: python -m llcompiler_amd.build"
+    L = ctypes.CDLL(C.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(L, name), name
+    assert L.llc_hip_abi_version() == 1
+
+
+def test_status_strings_and_null_argument_errors():
+    L = C.lib()
+    assert L.llc_hip_status_string(0) == b"ok"
+    assert b"shape" in L.llc_hip_status_string(-3)
+    st = L.llc_hip_softmax(None, None, None)
+    assert st == -1
+    assert b"null" in L.llc_hip_last_error()
+    with pytest.raises(C.LlcHipError):
+        C.check(st)
+
+
+def test_descriptor_layout_matches_reference_tensor_field_order():
+    # include/llcompiler/Compiler/Tensor.h:42-47: data, base, type, offset, size, stride
+    names = [f[0] for f in C.LlcTensor._fields_]
+    assert names == ["data", "base", "type", "offset", "rank", "size", "stride"]
+    # type codes 0-6 are the reference's enum (Tensor.h:25-33; engine.py:11 maps f32->4, i64->3, bool->6)
+    import torch
+    assert C.TORCH_DTYPE_TO_TYPE[torch.float32] == 4
+    assert C.TORCH_DTYPE_TO_TYPE[torch.int64] == 3
+    assert C.TORCH_DTYPE_TO_TYPE[torch.bool] == 6
+
+
+def test_unpack_params_follows_execution_run_layout():
+    # src/Compiler/Execution.cpp:21-41: [symbols|NULL] then per tensor base, data, &offset, size*, stride*
+    L = C.lib()
+    sizes = (ctypes.c_size_t * 2)(3, 5)
+    strides = (ctypes.c_size_t * 2)(5, 1)
+    off = ctypes.c_size_t(7)
+    syms = (ctypes.c_int64 * 1)(42)
+    params = (ctypes.c_void_p * 6)(ctypes.addressof(syms), 0x1000, 0x1040, ctypes.addressof(off),
+                                   ctypes.addressof(sizes), ctypes.addressof(strides))
+    ranks = (ctypes.c_size_t * 1)(2)
+    types = (ctypes.c_size_t * 1)(C.FLOAT32)
+    out = (C.LlcTensor * 1)()
+    sym_out = ctypes.POINTER(ctypes.c_int64)()
+    used = L.llc_hip_unpack_params(params, 1, ranks, types, out, ctypes.byref(sym_out))
+    assert used == 6
+    t = out[0]
+    assert (t.base, t.data, t.offset, t.rank, t.type) == (0x1000, 0x1040, 7, 2, C.FLOAT32)
+    assert [t.size[i] for i in range(2)] == [3, 5] and [t.stride[i] for i in range(2)] == [5, 1]
+    assert sym_out[0] == 42
+    # no symbols: slot 0 is NULL (Execution.cpp:24) and still consumed
+    params[0] = None
+    used = L.llc_hip_unpack_params(params, 1, ranks, types, out, ctypes.byref(sym_out))
+    assert used == 6 and not sym_out
+
+
+def test_cpu_tensor_is_refused_not_computed():
+    import torch
+    from llcompiler_amd import ops
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.softmax(torch.zeros(2, 3))

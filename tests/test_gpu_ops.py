@@ -1,0 +1,374 @@
+"""GPU parity of every kernel entry point against the CPU oracle, called through the C-ABI.
+
+Tolerances are the north star's: fp32 rtol 1e-4 / atol 1e-5, bf16 rtol 2e-2, data movement bit
+exact.  Inputs are seeded numpy arrays copied to the device, so oracle and kernel see the same bits.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import (assert_close_bf16, assert_close_f32, bf16_round, dev, host, rng)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from llcompiler_amd import ops as _ops
+    return _ops
+
+
+# --------------------------------------------------------------------------- elementwise
+def test_add_relu_f32_and_bf16(ops, oracle):
+    r = rng(1)
+    for shape in [(4, 1024, 256), (7, 33), (5,), (3, 1, 17)]:
+        a = r.uniform(-1, 1, shape).astype(np.float32)
+        b = r.uniform(-1, 1, shape).astype(np.float32)
+        prog = ops.make_program([("add", "r0", "in0", "in1"), ("relu", "r0", "r0")], "r0")
+        want = oracle.unary("relu", oracle.binary("add", a, b))
+        got = ops.elementwise(prog, [dev(a), dev(b)], shape, torch.float32)
+        np.testing.assert_array_equal(host(got), want, err_msg=str(shape))  # add and max are exactly rounded
+        ab, bb = bf16_round(a), bf16_round(b)
+        wantb = bf16_round(oracle.unary("relu", oracle.binary("add", ab, bb)))
+        gotb = ops.elementwise(prog, [dev(a, torch.bfloat16), dev(b, torch.bfloat16)], shape, torch.bfloat16)
+        np.testing.assert_array_equal(host(gotb), wantb, err_msg=str(shape))
+
+
+def test_fused_chain_with_immediates(ops, oracle):
+    # ElewiseFusion1 of the reference's notes: x+x; -3; /2; relu; * y
+    r = rng(2)
+    x = r.standard_normal((3, 3, 56, 56)).astype(np.float32)
+    y = r.standard_normal((3, 3, 56, 56)).astype(np.float32)
+    prog = ops.make_program([("add", "r0", "in0", "in0"), ("sub", "r0", "r0", 3.0), ("div", "r0", "r0", 2.0),
+                             ("relu", "r0", "r0"), ("mul", "r1", "r0", "in1")], "r1")
+    t = oracle.binary("add", x, x)
+    t = oracle.binary("sub", t, np.full_like(t, 3.0))
+    t = oracle.binary("div", t, np.full_like(t, 2.0))
+    want = oracle.binary("mul", oracle.unary("relu", t), y)
+    got = ops.elementwise(prog, [dev(x), dev(y)], x.shape, torch.float32)
+    np.testing.assert_array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("name", ["abs", "sqrt", "exp", "relu", "rsqrt", "neg", "gelu", "tanh", "erf", "sigmoid", "log", "recip"])
+def test_unary_ops(ops, oracle, name):
+    r = rng(3)
+    x = r.uniform(-4, 4, (63, 130)).astype(np.float32)
+    if name in ("sqrt", "rsqrt", "log", "recip"):
+        x = np.abs(x) + 0.1
+    prog = ops.make_program([(name, "r0", "in0")], "r0")
+    got = ops.elementwise(prog, [dev(x)], x.shape, torch.float32)
+    assert_close_f32(host(got), oracle.unary(name, x), name)
+
+
+@pytest.mark.parametrize("name", ["add", "sub", "mul", "div", "max", "min", "pow"])
+def test_binary_ops(ops, oracle, name):
+    r = rng(4)
+    a = r.uniform(0.1, 2, (17, 257)).astype(np.float32) * (1 if name == "pow" else r.choice([-1, 1], (17, 257)))
+    a = a.astype(np.float32)
+    b = r.uniform(0.5, 2, (17, 257)).astype(np.float32)
+    prog = ops.make_program([(name, "r0", "in0", "in1")], "r0")
+    got = ops.elementwise(prog, [dev(a), dev(b)], a.shape, torch.float32)
+    assert_close_f32(host(got), oracle.binary(name, a, b), name)
+
+
+def test_nan_propagation_in_relu_and_max(ops):
+    x = np.array([np.nan, -1.0, 2.0, -0.0], np.float32)
+    prog = ops.make_program([("relu", "r0", "in0")], "r0")
+    got = host(ops.elementwise(prog, [dev(x)], x.shape, torch.float32))
+    assert np.isnan(got[0]) and list(got[1:]) == [0.0, 2.0, 0.0]
+
+
+def test_broadcast_patterns(ops, oracle):
+    r = rng(5)
+    # bias over the last dim, per-channel NCHW, attention mask [B,1,1,S] -> [B,H,S,S], scalar tensor<1>
+    cases = [((6, 40), (40,)), ((2, 5, 7, 8), (1, 5, 1, 1)), ((2, 3, 8, 8), (2, 1, 1, 8)), ((4, 9), (1,)),
+             ((3, 4, 5), (3, 1, 5)), ((3, 4, 6), (4, 1))]
+    for full, small in cases:
+        a = r.standard_normal(full).astype(np.float32)
+        b = r.standard_normal(small).astype(np.float32)
+        prog = ops.make_program([("add", "r0", "in0", "in1")], "r0")
+        got = ops.elementwise(prog, [dev(a), dev(b)], full, torch.float32)
+        np.testing.assert_array_equal(host(got), a + b, err_msg=str((full, small)))
+        # the same through the oracle's explicit broadcast_to
+        bb = b.reshape((1,) * (len(full) - b.ndim) + b.shape)
+        np.testing.assert_array_equal(host(got), oracle.binary("add", a, oracle.broadcast_to(bb, full)))
+
+
+def test_compare_where_convert(ops, oracle):
+    r = rng(6)
+    a = r.integers(-3, 4, (11, 50)).astype(np.float32)
+    b = r.integers(-3, 4, (11, 50)).astype(np.float32)
+    for name, kind in [("eq", "EQ"), ("ne", "NE"), ("ge", "GE"), ("gt", "GT"), ("le", "LE"), ("lt", "LT")]:
+        prog = ops.make_program([(name, "r0", "in0", "in1")], "r0")
+        got = ops.elementwise(prog, [dev(a), dev(b)], a.shape, torch.bool)
+        np.testing.assert_array_equal(host(got), oracle.compare(kind, a, b), err_msg=name)
+    pred = a > b
+    prog = ops.make_program([("where", "r0", "in0", "in1", "in2")], "r0")
+    got = ops.elementwise(prog, [dev(pred), dev(a), dev(b)], a.shape, torch.float32)
+    np.testing.assert_array_equal(host(got), oracle.where(pred, a, b))
+    f = np.array([1.9, -1.9, 3.0, 100.5], np.float32)
+    np.testing.assert_array_equal(host(ops.convert(dev(f), torch.int64)), oracle.convert(f, np.int64))
+    i = np.array([3, -4, 1 << 20], np.int64)
+    np.testing.assert_array_equal(host(ops.convert(dev(i), torch.float32)), oracle.convert(i, np.float32))
+    np.testing.assert_array_equal(host(ops.convert(dev(f), torch.bfloat16)), bf16_round(f))
+    big = np.array([(1 << 40) + 3, -(1 << 35)], np.int64)
+    np.testing.assert_array_equal(host(ops.convert(dev(big), torch.int32)), big.astype(np.int32))
+
+
+def test_int64_elementwise(ops, oracle):
+    r = rng(7)
+    a = r.integers(0, 1 << 40, (5, 33)).astype(np.int64)
+    b = r.integers(1, 1000, (5, 33)).astype(np.int64)
+    for name in ["add", "sub", "mul", "div", "max", "min"]:
+        prog = ops.make_program([(name, "r0", "in0", "in1")], "r0", integer=True)
+        got = ops.elementwise(prog, [dev(a), dev(b)], a.shape, torch.int64)
+        np.testing.assert_array_equal(host(got), oracle.binary(name, a, b), err_msg=name)
+
+
+def test_elementwise_empty_and_errors(ops):
+    prog = ops.make_program([("relu", "r0", "in0")], "r0")
+    out = ops.elementwise(prog, [torch.empty(0, 4, device="cuda")], (0, 4), torch.float32)
+    assert out.shape == (0, 4)
+    from llcompiler_amd._capi import LlcHipError
+    with pytest.raises(LlcHipError):
+        ops.elementwise(prog, [torch.zeros(3, 4, device="cuda")], (3, 5), torch.float32)
+
+
+# --------------------------------------------------------------------------- row kernels
+@pytest.mark.parametrize("shape", [(37, 129), (64, 128), (9, 512), (5, 4096), (3, 5000), (2, 20000), (4, 12, 64, 64), (1, 1)])
+def test_softmax(ops, oracle, shape):
+    r = rng(8)
+    x = (r.standard_normal(shape) * 3).astype(np.float32)
+    got = ops.softmax(dev(x))
+    assert_close_f32(host(got), oracle.softmax_lastdim(x), "softmax f32 %s" % (shape,))
+    xb = bf16_round(x)
+    gotb = ops.softmax(dev(x, torch.bfloat16))
+    assert_close_bf16(host(gotb), bf16_round(oracle.softmax_lastdim(xb)), "softmax bf16 %s" % (shape,))
+
+
+def test_softmax_masked_rows(ops, oracle):
+    # additive -1e4 padding tails as in the BERT config; plus a row of equal values
+    x = np.zeros((3, 64), np.float32)
+    x[0, 40:] = -1e4
+    x[1, :] = 7.0
+    x[2, 1:] = -1e4
+    got = host(ops.softmax(dev(x)))
+    assert_close_f32(got, oracle.softmax_lastdim(x))
+    np.testing.assert_allclose(got.sum(-1), 1.0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(19, 96), (32, 768), (8, 1024), (5, 100), (2, 9000), (3, 7, 64)])
+def test_layer_norm(ops, oracle, shape):
+    r = rng(9)
+    x = (r.standard_normal(shape) * 2 + 1).astype(np.float32)
+    g = r.uniform(-1, 1, shape[-1]).astype(np.float32)
+    b = r.uniform(-1, 1, shape[-1]).astype(np.float32)
+    got = ops.layer_norm(dev(x), dev(g), dev(b), 1e-5)
+    assert_close_f32(host(got), oracle.layernorm_lastdim(x, g, b, 1e-5), "layernorm f32 %s" % (shape,))
+    got = ops.layer_norm(dev(x), None, None, 1e-5)
+    assert_close_f32(host(got), oracle.layernorm_lastdim(x, None, None, 1e-5), "layernorm plain %s" % (shape,))
+    xb, gb, bb = bf16_round(x), bf16_round(g), bf16_round(b)
+    gotb = ops.layer_norm(dev(x, torch.bfloat16), dev(g, torch.bfloat16), dev(b, torch.bfloat16), 1e-5)
+    assert_close_bf16(host(gotb), bf16_round(oracle.layernorm_lastdim(xb, gb, bb, 1e-5)), "layernorm bf16 %s" % (shape,))
+
+
+@pytest.mark.parametrize("shape,axes", [((3, 4, 5, 6), [3]), ((3, 4, 5, 6), [1, 2]), ((3, 4, 5, 6), [0]), ((3, 4, 5, 6), [2, 3]),
+                                        ((3, 4, 5, 6), [0, 1, 2, 3]), ((16, 4096), [1]), ((7, 300, 9), [1]), ((2, 3000), [-1])])
+def test_reduce(ops, oracle, shape, axes):
+    r = rng(10)
+    x = r.standard_normal(shape).astype(np.float32)
+    for kind in ["sum", "max", "min"]:
+        got = ops.reduce(kind, dev(x), axes)
+        want = oracle.reduce(kind, x, axes)
+        if kind == "sum":
+            assert_close_f32(host(got), want, "reduce_sum %s %s" % (shape, axes))
+        else:
+            np.testing.assert_array_equal(host(got), want)
+    neg = -np.abs(x) - 1  # init is -inf, not 0 (LLHToHLO.cpp:81-133)
+    assert host(ops.reduce("max", dev(neg), axes)).max() < 0
+
+
+def test_reduce_rejects_split_axes(ops):
+    from llcompiler_amd._capi import LlcHipError
+    with pytest.raises(LlcHipError, match="adjacent"):
+        ops.reduce("sum", torch.zeros(2, 3, 4, 5, device="cuda"), [0, 2])
+
+
+# --------------------------------------------------------------------------- data movement (bit exact)
+@pytest.mark.parametrize("dtype", [np.float32, np.int64, np.float16, np.int8])
+def test_transpose_bit_exact(ops, oracle, dtype):
+    r = rng(11)
+    x = r.integers(0, 127, (4, 6, 70, 66)).astype(dtype)
+    for perms in [(0, 2, 1, 3), (3, 2, 1, 0), (1, 0, 2, 3), (0, 1, 3, 2), (2, 3, 0, 1), (0, 1, 2, 3)]:
+        got = ops.transpose(dev(x), perms)
+        np.testing.assert_array_equal(host(got), oracle.transpose(x, perms), err_msg=str(perms))
+    m = r.integers(0, 127, (129, 257)).astype(dtype)
+    np.testing.assert_array_equal(host(ops.transpose(dev(m), (1, 0))), m.T)
+
+
+def test_attention_head_split_and_merge(ops, oracle):
+    r = rng(12)
+    x = r.standard_normal((2, 16, 4, 64)).astype(np.float32)  # [B,S,heads,64]
+    t = ops.transpose(dev(x), (0, 2, 1, 3))
+    np.testing.assert_array_equal(host(t), oracle.transpose(x, (0, 2, 1, 3)))
+    back = ops.transpose(t, (0, 2, 1, 3))
+    np.testing.assert_array_equal(host(back), x)
+    xb = dev(x, torch.bfloat16)
+    np.testing.assert_array_equal(host(ops.transpose(ops.transpose(xb, (0, 2, 1, 3)), (0, 2, 1, 3))), host(xb))
+
+
+def test_slice_extract_broadcast_copy_gather(ops, oracle):
+    r = rng(13)
+    z = r.integers(0, 1 << 30, (6, 5, 8, 12)).astype(np.int64)
+    got = ops.stride_slice(dev(z), (0, 1, 0, 1), (6, 3, 8, 11), (1, 1, 2, 3))
+    np.testing.assert_array_equal(host(got), oracle.stride_slice(z, (0, 1, 0, 1), (6, 3, 8, 11), (1, 1, 2, 3)))
+    assert got.shape == (6, 2, 4, 4)
+    f = r.standard_normal((7, 3, 16)).astype(np.float32)
+    np.testing.assert_array_equal(host(ops.stride_slice(dev(f), (2, 0, 4), (5, 3, 12), (1, 1, 1))), f[2:5, :, 4:12])
+    np.testing.assert_array_equal(host(ops.extract(dev(f), 2)), oracle.extract(f, 2))
+    np.testing.assert_array_equal(host(ops.extract(dev(f), -1)), oracle.extract(f, -1))
+    b = r.standard_normal((3, 1, 5, 1)).astype(np.float32)
+    np.testing.assert_array_equal(host(ops.broadcast_to(dev(b), (3, 4, 5, 6))), oracle.broadcast_to(b, (3, 4, 5, 6)))
+    view = dev(f).permute(2, 0, 1)[::2]
+    np.testing.assert_array_equal(host(ops.copy(view)), np.ascontiguousarray(f.transpose(2, 0, 1)[::2]))
+    table = r.standard_normal((11, 6)).astype(np.float32)
+    table8 = r.standard_normal((50, 768)).astype(np.float32)
+    idx = np.array([[0, 10, 3], [3, 3, 7]], np.int64)
+    np.testing.assert_array_equal(host(ops.gather_rows(dev(table), dev(idx))), oracle.gather_rows(table, idx))
+    idx2 = r.integers(0, 50, (4, 9)).astype(np.int64)
+    np.testing.assert_array_equal(host(ops.gather_rows(dev(table8), dev(idx2))), oracle.gather_rows(table8, idx2))
+    # empty and ragged
+    assert ops.stride_slice(dev(f), (3, 0, 0), (3, 3, 16), (1, 1, 1)).shape == (0, 3, 16)
+
+
+# --------------------------------------------------------------------------- contractions
+MM_SHAPES = [(1, 1, 1), (3, 3, 3), (4, 512, 784), (4, 10, 512), (33, 65, 129), (128, 128, 128), (256, 384, 96),
+             (200, 72, 264), (130, 250, 36)]
+
+
+@pytest.mark.parametrize("M,N,K", MM_SHAPES)
+def test_matmul_f32(ops, oracle, M, N, K):
+    r = rng(M * 7 + N * 3 + K)
+    a = r.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = r.uniform(-1, 1, (K, N)).astype(np.float32)
+    want = oracle.matmul(a, b, "mkn")
+    assert_close_f32(host(ops.matmul(dev(a), dev(b))), want, "NN %s" % ((M, N, K),))
+    # rhs as a transposed view of an [N,K] weight (llh.transpose folded into the operand)
+    bt = dev(np.ascontiguousarray(b.T))
+    assert_close_f32(host(ops.matmul(dev(a), bt.t())), want, "NT %s" % ((M, N, K),))
+    at = dev(np.ascontiguousarray(a.T))
+    assert_close_f32(host(ops.matmul(at.t(), dev(b))), want, "TN %s" % ((M, N, K),))
+
+
+@pytest.mark.parametrize("M,N,K", MM_SHAPES)
+def test_matmul_bf16(ops, oracle, M, N, K):
+    r = rng(M * 7 + N * 3 + K + 1)
+    a = bf16_round(r.uniform(-1, 1, (M, K)))
+    b = bf16_round(r.uniform(-1, 1, (K, N)))
+    want = bf16_round(oracle.matmul(a, b, "mkn"))
+    got = ops.matmul(dev(a, torch.bfloat16), dev(b, torch.bfloat16))
+    assert_close_bf16(host(got), want, "NN bf16 %s" % ((M, N, K),))
+    bt = dev(np.ascontiguousarray(b.T), torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(dev(a, torch.bfloat16), bt.t())), want, "NT bf16 %s" % ((M, N, K),))
+    goth = ops.matmul(dev(a, torch.float16), dev(b, torch.float16))
+    assert_close_bf16(host(goth), oracle.matmul(a, b, "mkn"), "NN f16 %s" % ((M, N, K),))
+
+
+def test_matmul_epilogue(ops, oracle):
+    r = rng(21)
+    M, N, K = 70, 136, 200
+    a = r.standard_normal((M, K)).astype(np.float32) * 0.2
+    b = r.standard_normal((K, N)).astype(np.float32) * 0.2
+    bias = r.standard_normal(N).astype(np.float32)
+    res = r.standard_normal((M, N)).astype(np.float32)
+    base = oracle.matmul(a, b, "mkn")
+    for act, alpha in [("none", 1.0), ("relu", 1.0), ("gelu", 0.125)]:
+        want = base * np.float32(alpha) + bias[None, :] + res
+        if act != "none":
+            want = oracle.unary(act, want)
+        epi = ops.Epilogue(alpha=alpha, bias=dev(bias), residual=dev(res), act=act)
+        assert_close_f32(host(ops.matmul(dev(a), dev(b), epi)), want, "epilogue " + act)
+
+
+@pytest.mark.parametrize("B,M,N,K", [(3, 9, 4, 6), (4, 64, 64, 64), (6, 128, 128, 64), (5, 100, 64, 100), (2, 130, 70, 36)])
+def test_batch_matmul(ops, oracle, B, M, N, K):
+    r = rng(B + M + N + K)
+    a = r.uniform(-1, 1, (B, M, K)).astype(np.float32)
+    b = r.uniform(-1, 1, (B, K, N)).astype(np.float32)
+    want = oracle.batch_matmul(a, b, "mkn")
+    assert_close_f32(host(ops.batch_matmul(dev(a), dev(b))), want, "bmm f32")
+    # QK^T form: rhs is the transposed view of [B,N,K]
+    bt = dev(np.ascontiguousarray(b.transpose(0, 2, 1)))
+    assert_close_f32(host(ops.batch_matmul(dev(a), bt.transpose(1, 2))), want, "bmm f32 NT")
+    ab, bb = bf16_round(a), bf16_round(b)
+    gotb = ops.batch_matmul(dev(ab, torch.bfloat16), dev(bb, torch.bfloat16))
+    assert_close_bf16(host(gotb), bf16_round(oracle.batch_matmul(ab, bb, "mkn")), "bmm bf16")
+
+
+def test_matmul_shape_errors(ops):
+    from llcompiler_amd._capi import LlcHipError
+    with pytest.raises(LlcHipError, match="matmul"):
+        ops.matmul(torch.zeros(3, 4, device="cuda"), torch.zeros(5, 6, device="cuda"), out=torch.zeros(3, 6, device="cuda"))
+    with pytest.raises(LlcHipError):
+        ops.matmul(torch.zeros(3, 4, device="cuda"), torch.zeros(4, 6, device="cuda", dtype=torch.bfloat16),
+                   out=torch.zeros(3, 6, device="cuda"))
+
+
+CONV_CASES = [
+    # N, C, H, W, F, KH, KW, pad(h,w), stride, dil, group
+    (2, 3, 9, 11, 4, 3, 3, (1, 1), (1, 1), (1, 1), 1),
+    (1, 3, 33, 29, 64, 7, 7, (3, 3), (2, 2), (1, 1), 1),   # stem-like, K = 147
+    (2, 4, 10, 12, 6, 3, 2, (2, 0), (2, 1), (1, 2), 2),
+    (1, 6, 8, 8, 6, 3, 3, (1, 2), (1, 3), (2, 1), 6),
+    (2, 64, 14, 14, 128, 1, 1, (0, 0), (2, 2), (1, 1), 1),  # 1x1 stride-2 downsample
+    (3, 3, 12, 12, 2, 5, 5, (2, 2), (1, 1), (1, 1), 1),
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),   # basic-block conv
+    (2, 128, 7, 7, 256, 3, 3, (1, 1), (2, 2), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d(ops, oracle, case):
+    N, C, H, W, Fo, KH, KW, p, s, d, g = case
+    r = rng(sum(case[:7]))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    fan = (C // g) * KH * KW
+    w = (r.standard_normal((Fo, C // g, KH, KW)) / np.sqrt(fan)).astype(np.float32)
+    b = r.standard_normal(Fo).astype(np.float32)
+    pad = (p[0], p[1], p[0], p[1])
+    want = oracle.conv2d(x, w, None, pad=pad, stride=s, dilation=d, group=g)
+    got = ops.conv2d(dev(x), dev(w), pad=pad, stride=s, dilation=d, group=g)
+    assert_close_f32(host(got), want, "conv %s" % (case,))
+    # conv_bias + relu + residual epilogue (a ResNet basic block tail)
+    res = r.standard_normal(want.shape).astype(np.float32)
+    want2 = oracle.unary("relu", oracle.conv2d(x, w, b, pad=pad, stride=s, dilation=d, group=g) + res)
+    epi = ops.Epilogue(bias=dev(b), residual=dev(res), act="relu")
+    assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s, dilation=d, group=g, epilogue=epi)), want2,
+                     "conv+bias+res+relu %s" % (case,))
+    xb, wb = bf16_round(x), bf16_round(w)
+    gotb = ops.conv2d(dev(xb, torch.bfloat16), dev(wb, torch.bfloat16), pad=pad, stride=s, dilation=d, group=g)
+    assert_close_bf16(host(gotb), bf16_round(oracle.conv2d(xb, wb, None, pad=pad, stride=s, dilation=d, group=g)),
+                      "conv bf16 %s" % (case,))
+
+
+def test_conv2d_asymmetric_pad(ops, oracle):
+    r = rng(31)
+    x = r.standard_normal((1, 2, 6, 7)).astype(np.float32)
+    w = r.standard_normal((3, 2, 3, 3)).astype(np.float32)
+    pad = (2, 0, 1, 3)
+    assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad)), oracle.conv2d(x, w, None, pad=pad))
+
+
+def test_max_pool_and_avg_pool(ops, oracle):
+    r = rng(32)
+    x = r.standard_normal((2, 3, 23, 27)).astype(np.float32)
+    for k, p, s, d in [((3, 3), (1, 1), (2, 2), (1, 1)), ((5, 5), (2, 2), (1, 1), (2, 2)), ((2, 3), (1, 0), (2, 1), (2, 1)),
+                       ((7, 7), (3, 1), (2, 2), (2, 1))]:
+        pad = (p[0], p[1], p[0], p[1])
+        for iz in (False, True):
+            got = ops.max_pool(dev(x), k, pad=pad, stride=s, dilation=d, init_zero=iz)
+            np.testing.assert_array_equal(host(got), oracle.maxpool2d(x, k, pad=pad, stride=s, dilation=d, init_zero=iz))
+    y = r.standard_normal((4, 6, 7, 7)).astype(np.float32)
+    assert_close_f32(host(ops.global_avg_pool(dev(y))), oracle.global_avgpool(y))
