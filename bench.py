@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Headline benchmark: the single-op suite (matmul, batch_matmul, fused add+relu, softmax,
+layernorm; fp32 and bf16) run through the C-ABI kernel library on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one pass over all ten ops with their inputs already resident in HBM.  Prints ONE JSON
+line: whole-suite latency per pass, the roofline of the kernel that dominates the pass (and of
+every other kernel under "kernels"), and the CPU oracle timed on a bounded sample of the same
+workload on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+
+WORKLOAD = "single-op suite fp32+bf16: matmul 2048^3, batch_matmul [32,512,64]x[32,64,512], add+relu [64,1024,1024], softmax [4096,4096], layernorm [8192,1024]"
+
+
+def _uniform(shape, dtype, gen, device):
+    # values ~U(-1,1), generated on the CPU so that every run sees the same bits
+    t = torch.rand(shape, generator=gen, dtype=torch.float32) * 2 - 1
+    return t.to(dtype).to(device)
+
+
+class Case:
+    """One op of the suite with `sets` rotating operand sets (so HBM-bound kernels cannot live in
+    the 256 MB last-level cache) and its algorithmic work."""
+
+    def __init__(self, name, dtype_name, bound, flops, bytes_, make, run, sets):
+        self.name, self.dtype_name, self.bound, self.flops, self.bytes = name, dtype_name, bound, flops, bytes_
+        # descriptors are built once per operand set; a timed call only crosses the C-ABI
+        self.calls = [run(*make()) for _ in range(sets)]
+        self.sets = sets
+
+    def run(self, i):
+        self.calls[i % self.sets].launch()
+
+
+def build_cases(ops, device):
+    gen = torch.Generator().manual_seed(0)
+    cases = []
+    for dt_name, dt, es in (("f32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+        M = N = K = 2048
+        cases.append(Case("matmul", dt_name, "mfma", 2.0 * M * N * K, (M * K + K * N + M * N) * es,
+                          lambda: (_uniform((M, K), dt, gen, device), _uniform((K, N), dt, gen, device),
+                                   torch.empty((M, N), dtype=dt, device=device)),
+                          lambda a, b, o: ops.matmul(a, b, out=o, defer=True), 1))
+        B, m, k, n = 32, 512, 64, 512
+        nbytes = (B * m * k + B * k * n + B * m * n) * es
+        cases.append(Case("batch_matmul", dt_name, "hbm", 2.0 * B * m * n * k, nbytes,
+                          lambda: (_uniform((B, m, k), dt, gen, device), _uniform((B, k, n), dt, gen, device),
+                                   torch.empty((B, m, n), dtype=dt, device=device)),
+                          lambda a, b, o: ops.batch_matmul(a, b, out=o, defer=True), max(1, int(1.2e9 // nbytes))))
+        shape = (64, 1024, 1024)
+        numel = 64 * 1024 * 1024
+        prog = ops.make_program([("add", "r0", "in0", "in1"), ("relu", "r0", "r0")], "r0")
+        cases.append(Case("add_relu", dt_name, "hbm", 0.0, 3 * numel * es,
+                          lambda: (_uniform(shape, dt, gen, device), _uniform(shape, dt, gen, device),
+                                   torch.empty(shape, dtype=dt, device=device)),
+                          lambda a, b, o, prog=prog, shape=shape, dt=dt: ops.elementwise(prog, [a, b], shape, dt, out=o, defer=True), 2))
+        cases.append(Case("softmax", dt_name, "hbm", 0.0, 2 * 4096 * 4096 * es,
+                          lambda: (_uniform((4096, 4096), dt, gen, device), torch.empty((4096, 4096), dtype=dt, device=device)),
+                          lambda x, o: ops.softmax(x, out=o, defer=True), 8))
+        cases.append(Case("layernorm", dt_name, "hbm", 0.0, (2 * 8192 * 1024 + 2 * 1024) * es,
+                          lambda: (_uniform((8192, 1024), dt, gen, device), torch.ones(1024, dtype=dt, device=device),
+                                   torch.zeros(1024, dtype=dt, device=device), torch.empty((8192, 1024), dtype=dt, device=device)),
+                          lambda x, g, b, o: ops.layer_norm(x, g, b, 1e-5, out=o, defer=True), 16))
+    return cases
+
+
+def time_gpu(fn, steps, warmup):
+    """Average milliseconds per call of fn(i), HIP events on the stream the kernels are launched on."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def roofline_of(case, ms):
+    if case.bound == "mfma":
+        achieved = case.flops / (ms * 1e-3) / 1e12
+        peak = PEAK_MFMA_TFLOPS[case.dtype_name]
+        unit = "TFLOP/s"
+    else:
+        achieved = case.bytes / (ms * 1e-3) / 1e9
+        peak = PEAK_HBM_GBS
+        unit = "GB/s"
+    return {"kernel": "%s_%s" % (case.name, case.dtype_name), "bound": case.bound, "achieved": round(achieved, 2),
+            "peak": peak, "unit": unit, "frac": round(achieved / peak, 4), "traffic": None, "avg_ms": round(ms, 5)}
+
+
+def cpu_baseline():
+    """The CPU oracle (the reference's loop nests restated in C, one thread) on a bounded sample of
+    each fp32 op of the suite, extrapolated linearly to the full op; about 10-30 s of CPU work."""
+    from oracle import ref
+    r = np.random.default_rng(0)
+    parts = {}
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    a = r.uniform(-1, 1, (48, 2048)).astype(np.float32)
+    b = r.uniform(-1, 1, (2048, 2048)).astype(np.float32)
+    parts["matmul"] = timed(lambda: ref.matmul(a, b, "mnk")) * (2048 / 48)
+    a3 = r.uniform(-1, 1, (4, 512, 64)).astype(np.float32)
+    b3 = r.uniform(-1, 1, (4, 64, 512)).astype(np.float32)
+    parts["batch_matmul"] = timed(lambda: ref.batch_matmul(a3, b3, "mnk")) * (32 / 4)
+    x = r.uniform(-1, 1, (8, 1024, 1024)).astype(np.float32)
+    y = r.uniform(-1, 1, (8, 1024, 1024)).astype(np.float32)
+    parts["add_relu"] = timed(lambda: ref.unary("relu", ref.binary("add", x, y))) * (64 / 8)
+    s = r.uniform(-1, 1, (1024, 4096)).astype(np.float32)
+    parts["softmax"] = timed(lambda: ref.softmax_lastdim(s)) * (4096 / 1024)
+    l = r.uniform(-1, 1, (2048, 1024)).astype(np.float32)
+    g = np.ones(1024, np.float32)
+    parts["layernorm"] = timed(lambda: ref.layernorm_lastdim(l, g, np.zeros(1024, np.float32))) * (8192 / 2048)
+    total_ms = sum(parts.values()) * 1e3
+    return {"value": round(total_ms, 1), "unit": "ms", "cores": 1, "kind": "port",
+            "sample": "fp32 half of the suite on the C oracle, 1 thread: matmul 48 of 2048 rows, batch_matmul 4 of 32 "
+                      "batches, add+relu 8 of 64 slabs, softmax 1024 of 4096 rows, layernorm 2048 of 8192 rows; each "
+                      "extrapolated linearly and summed (the bf16 half has no CPU path in the reference)",
+            "per_op_ms": {k: round(v * 1e3, 1) for k, v in parts.items()}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU; there is no CPU fallback")
+    from llcompiler_amd import ops
+    device = torch.device("cuda", 0)
+    cases = build_cases(ops, device)
+
+    def step(i):
+        for c in cases:
+            c.run(i)
+
+    torch.cuda.synchronize()
+    ms_per_step = time_gpu(step, args.steps, args.warmup)
+    # per-kernel average durations, each in its own timed loop
+    kernels = [roofline_of(c, time_gpu(c.run, args.steps, args.warmup)) for c in cases]
+    dominant = max(kernels, key=lambda k: k["avg_ms"])
+    out = {
+        "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32+bf16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": WORKLOAD, "values": "U(-1,1), seed 0", "ops_per_step": len(cases)},
+        "roofline": {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "dominant_kernel": dominant["kernel"],
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

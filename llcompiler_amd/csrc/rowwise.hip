@@ -312,13 +312,14 @@ void launch_items(const RowParams& p, int items, hipStream_t s) {
 
 template <int OP, int VEC>
 bool launch_tpr(const RowParams& p, hipStream_t s) {
-  // smallest register tile that holds a row; ties go to fewer lanes per row (no LDS hop)
+  // smallest register tile that holds a row; among equal capacities prefer 4 then 2 vectors per
+  // lane (enough loads in flight per lane, rows spread over many lanes), then 8, then 1
   const int tprs[3] = {16, 64, 256};
-  const int items[4] = {1, 2, 4, 8};
+  const int items[4] = {4, 2, 8, 1};
   int best_t = 0, best_i = 0;
   int64_t best_cap = -1;
-  for (int t : tprs)
-    for (int i : items) {
+  for (int i : items)
+    for (int t : tprs) {
       int64_t cap = (int64_t)t * i * VEC;
       if (cap >= p.cols && (best_cap < 0 || cap < best_cap)) {
         best_cap = cap;

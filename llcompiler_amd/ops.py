@@ -2,6 +2,8 @@
 
 Each function allocates the output with torch (device memory only), builds the descriptors and
 enqueues the kernel on torch's current HIP stream.  No arithmetic happens in Python or in torch.
+With defer=True a function returns a `Call` whose launch() only crosses the C-ABI, for callers
+that issue the same call many times on fixed buffers (plans, benchmarks).
 """
 import ctypes
 
@@ -15,6 +17,27 @@ def _dev(t):
         raise RuntimeError("llcompiler_amd kernels run on the GPU only; got a %s tensor (no CPU fallback)" % t.device)
     C.init(t.device.index or 0)
     return t.device
+
+
+class Call:
+    """A kernel call with its descriptors already built."""
+
+    __slots__ = ("fn", "args", "keep", "out", "device")
+
+    def __init__(self, fn, args, keep, out, device):
+        self.fn, self.args, self.keep, self.out, self.device = fn, args, keep, out, device
+
+    def launch(self):
+        st = self.fn(*self.args, C.current_stream(self.device))
+        if st != 0:
+            C.check(st)
+        return self.out
+
+
+def _launch(fn, args, keep, out, device, defer):
+    """args: everything but the trailing stream argument."""
+    call = Call(fn, args, keep, out, device)
+    return call if defer else call.launch()
 
 
 def window_out(n, pad_lo, pad_hi, dil, k, stride):
@@ -31,7 +54,7 @@ class Epilogue:
 
     def build(self):
         self._b = C.tensor_ref(self.bias)
-        self._r = C.tensor_ref(self.residual.contiguous()) if self.residual is not None else None
+        self._r = C.tensor_ref(self.residual) if self.residual is not None else None
         self._s = C.LlcEpilogue(self.alpha, self._b.ptr if self._b else None, self._r.ptr if self._r else None,
                                 self.act)
         return ctypes.pointer(self._s)
@@ -41,25 +64,25 @@ def _epi(e):
     return e.build() if e is not None else None
 
 
-def matmul(a, b, epilogue=None, out=None):
+def matmul(a, b, epilogue=None, out=None, defer=False):
     dev = _dev(a)
     if out is None:
         out = torch.empty((a.shape[0], b.shape[1]), dtype=a.dtype, device=dev)
     ra, rb, ro = C.tensor_ref(a), C.tensor_ref(b), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_matmul(ra.ptr, rb.ptr, _epi(epilogue), ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_matmul, (ra.ptr, rb.ptr, _epi(epilogue), ro.ptr), (ra, rb, ro, epilogue), out, dev,
+                   defer)
 
 
-def batch_matmul(a, b, epilogue=None, out=None):
+def batch_matmul(a, b, epilogue=None, out=None, defer=False):
     dev = _dev(a)
     if out is None:
         out = torch.empty((a.shape[0], a.shape[1], b.shape[2]), dtype=a.dtype, device=dev)
     ra, rb, ro = C.tensor_ref(a), C.tensor_ref(b), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_batch_matmul(ra.ptr, rb.ptr, _epi(epilogue), ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_batch_matmul, (ra.ptr, rb.ptr, _epi(epilogue), ro.ptr), (ra, rb, ro, epilogue), out,
+                   dev, defer)
 
 
-def conv2d(x, w, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), group=1, epilogue=None, out=None):
+def conv2d(x, w, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), group=1, epilogue=None, out=None, defer=False):
     """pad = (h_lo, w_lo, h_hi, w_hi), the LLH attribute order."""
     dev = _dev(x)
     N, _, H, W = x.shape
@@ -71,13 +94,12 @@ def conv2d(x, w, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), group=1, epil
     attrs = C.LlcConvAttrs((ctypes.c_int64 * 2)(*dilation), (ctypes.c_int64 * 2)(KH, KW), (ctypes.c_int64 * 4)(*pad),
                            (ctypes.c_int64 * 2)(*stride), group)
     rx, rw, ro = C.tensor_ref(x), C.tensor_ref(w), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_conv2d(rx.ptr, rw.ptr, ctypes.byref(attrs), _epi(epilogue), ro.ptr,
-                                   C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_conv2d, (rx.ptr, rw.ptr, ctypes.pointer(attrs), _epi(epilogue), ro.ptr),
+                   (rx, rw, ro, attrs, epilogue), out, dev, defer)
 
 
 def make_program(insts, result=0, integer=False):
-    """insts: list of (op, dst, a[, b[, c]][, imm=...]) with operands 'r0'..'r3', 'in0'..'in5' or a number."""
+    """insts: list of (op, dst, a[, b[, c]]) with operands 'r0'..'r3', 'in0'..'in5' or one number (the immediate)."""
     prog = C.LlcEwProgram()
     if len(insts) > C.EW_MAX_INSTS:
         raise ValueError("elementwise chain of %d instructions (max %d)" % (len(insts), C.EW_MAX_INSTS))
@@ -101,7 +123,7 @@ def make_program(insts, result=0, integer=False):
     return prog
 
 
-def elementwise(prog, inputs, out_shape, out_dtype, out=None):
+def elementwise(prog, inputs, out_shape, out_dtype, out=None, defer=False):
     dev = _dev(inputs[0])
     if out is None:
         out = torch.empty(tuple(out_shape), dtype=out_dtype, device=dev)
@@ -113,41 +135,39 @@ def elementwise(prog, inputs, out_shape, out_dtype, out=None):
         refs.append(C.tensor_ref(t, (1,) * pad + tuple(t.shape), (0,) * pad + tuple(t.stride())))
     arr = (ctypes.POINTER(C.LlcTensor) * max(len(refs), 1))(*[r.ptr for r in refs])
     ro = C.tensor_ref(out)
-    C.check(C.lib().llc_hip_elementwise(ctypes.byref(prog), arr, len(refs), ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_elementwise, (ctypes.pointer(prog), arr, len(refs), ro.ptr), (prog, refs, arr, ro),
+                   out, dev, defer)
 
 
-def reduce(kind, x, axes, out=None):
+def reduce(kind, x, axes, out=None, defer=False):
     dev = _dev(x)
     axes = [a % x.dim() for a in axes]
     if out is None:
         out = torch.empty([s for d, s in enumerate(x.shape) if d not in axes], dtype=x.dtype, device=dev)
     code = {"sum": C.REDUCE_SUM, "max": C.REDUCE_MAX, "min": C.REDUCE_MIN}[kind]
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_reduce(code, rx.ptr, C.i64_array(axes), len(axes), ro.ptr, C.current_stream(dev)))
-    return out
+    ax = C.i64_array(axes)
+    return _launch(C.lib().llc_hip_reduce, (code, rx.ptr, ax, len(axes), ro.ptr), (rx, ro, ax), out, dev, defer)
 
 
-def softmax(x, out=None):
+def softmax(x, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty_like(x)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_softmax(rx.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_softmax, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
 
 
-def layer_norm(x, scale=None, bias=None, eps=1e-5, out=None):
+def layer_norm(x, scale=None, bias=None, eps=1e-5, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty_like(x)
     rx, ro, rs, rb = C.tensor_ref(x), C.tensor_ref(out), C.tensor_ref(scale), C.tensor_ref(bias)
-    C.check(C.lib().llc_hip_layer_norm(rx.ptr, rs.ptr if rs else None, rb.ptr if rb else None, float(eps), ro.ptr,
-                                       C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_layer_norm, (rx.ptr, rs.ptr if rs else None, rb.ptr if rb else None, float(eps),
+                                                ro.ptr), (rx, ro, rs, rb), out, dev, defer)
 
 
-def max_pool(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), init_zero=False, out=None):
+def max_pool(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), init_zero=False, out=None, defer=False):
     dev = _dev(x)
     N, Cc, H, W = x.shape
     OH = window_out(H, pad[0], pad[2], dilation[0], kernel[0], stride[0])
@@ -157,87 +177,80 @@ def max_pool(x, kernel, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), init_z
     attrs = C.LlcPoolAttrs((ctypes.c_int64 * 2)(*dilation), (ctypes.c_int64 * 2)(*kernel), (ctypes.c_int64 * 4)(*pad),
                            (ctypes.c_int64 * 2)(*stride), 1 if init_zero else 0)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_max_pool(rx.ptr, ctypes.byref(attrs), ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_max_pool, (rx.ptr, ctypes.pointer(attrs), ro.ptr), (rx, ro, attrs), out, dev, defer)
 
 
-def global_avg_pool(x, keepdim=False, out=None):
+def global_avg_pool(x, keepdim=False, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         shape = (x.shape[0], x.shape[1], 1, 1) if keepdim else (x.shape[0], x.shape[1])
         out = torch.empty(shape, dtype=x.dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_global_avg_pool(rx.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_global_avg_pool, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
 
 
-def transpose(x, perms, out=None):
+def transpose(x, perms, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty([x.shape[p] for p in perms], dtype=x.dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_transpose(rx.ptr, C.i64_array(perms), ro.ptr, C.current_stream(dev)))
-    return out
+    pm = C.i64_array(perms)
+    return _launch(C.lib().llc_hip_transpose, (rx.ptr, pm, ro.ptr), (rx, ro, pm), out, dev, defer)
 
 
-def stride_slice(x, start, end, step, out=None):
+def stride_slice(x, start, end, step, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty([max(0, -(-(e - s) // st)) for s, e, st in zip(start, end, step)], dtype=x.dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_stride_slice(rx.ptr, C.i64_array(start), C.i64_array(end), C.i64_array(step), ro.ptr,
-                                         C.current_stream(dev)))
-    return out
+    a, b, c = C.i64_array(start), C.i64_array(end), C.i64_array(step)
+    return _launch(C.lib().llc_hip_stride_slice, (rx.ptr, a, b, c, ro.ptr), (rx, ro, a, b, c), out, dev, defer)
 
 
-def extract(x, index):
+def extract(x, index, out=None, defer=False):
     """llh.extract: row `index` of dim 0 with the dim dropped; a negative index counts from the end
     (src/Dialect/LLH/IR/LLHCanonicalize.cpp:337-354)."""
+    dev = _dev(x)
     if index < 0:
         index += x.shape[0]
-    out = torch.empty(tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+    if out is None:
+        out = torch.empty(tuple(x.shape[1:]), dtype=x.dtype, device=dev)
     start = [index] + [0] * (x.dim() - 1)
     end = [index + 1] + list(x.shape[1:])
-    ro = C.tensor_ref(out, (1,) + tuple(out.shape), (out.numel(),) + tuple(out.stride()))
+    ro = C.tensor_ref(out, (1,) + tuple(out.shape), (max(out.numel(), 1),) + tuple(out.stride()))
     rx = C.tensor_ref(x)
-    dev = _dev(x)
-    C.check(C.lib().llc_hip_stride_slice(rx.ptr, C.i64_array(start), C.i64_array(end), C.i64_array([1] * x.dim()),
-                                         ro.ptr, C.current_stream(dev)))
-    return out
+    a, b, c = C.i64_array(start), C.i64_array(end), C.i64_array([1] * x.dim())
+    return _launch(C.lib().llc_hip_stride_slice, (rx.ptr, a, b, c, ro.ptr), (rx, ro, a, b, c), out, dev, defer)
 
 
-def broadcast_to(x, shape, out=None):
+def broadcast_to(x, shape, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty(tuple(shape), dtype=x.dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_broadcast_to(rx.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_broadcast_to, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
 
 
-def copy(x, out=None):
+def copy(x, out=None, defer=False):
     """Materialises any strided view into a contiguous tensor."""
     dev = _dev(x)
     if out is None:
         out = torch.empty(tuple(x.shape), dtype=x.dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_copy(rx.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_copy, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
 
 
-def gather_rows(table, idx, out=None):
+def gather_rows(table, idx, out=None, defer=False):
     dev = _dev(table)
     if out is None:
         out = torch.empty(tuple(idx.shape) + tuple(table.shape[1:]), dtype=table.dtype, device=dev)
     rt, ri, ro = C.tensor_ref(table), C.tensor_ref(idx), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_gather_rows(rt.ptr, ri.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_gather_rows, (rt.ptr, ri.ptr, ro.ptr), (rt, ri, ro), out, dev, defer)
 
 
-def convert(x, dtype, out=None):
+def convert(x, dtype, out=None, defer=False):
     dev = _dev(x)
     if out is None:
         out = torch.empty(tuple(x.shape), dtype=dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
-    C.check(C.lib().llc_hip_convert(rx.ptr, ro.ptr, C.current_stream(dev)))
-    return out
+    return _launch(C.lib().llc_hip_convert, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
