@@ -1,0 +1,102 @@
+"""torch.compile backend: the counterpart of llcompiler/compiler/compiler.py.
+
+    model = torch.compile(model, backend=LLCompiler(mode="inference", target="gfx950", pipeline="hip"))
+
+Flow (reference: compiler.py:84-168): dynamo + AOT-autograd hand over an ATen graph; supported
+nodes are carved into fused submodules by CapabilityBasedPartitioner; each submodule is imported
+into an LLH graph, run through the LLH pipeline, planned into kernel calls and replaced by a
+Torch_ExecutionEngine.  Unsupported nodes stay in torch eager.  Nothing is shelled out to and no
+shared library is generated per model: the "compiled artefact" is the kernel plan.
+"""
+from typing import Any, List
+
+import torch
+import torch.fx
+from torch._decomp import get_decompositions
+from torch._dynamo.backends.common import aot_autograd
+from torch.fx.passes.infra.partitioner import CapabilityBasedPartitioner
+
+from ..executor.engine import Torch_ExecutionEngine
+from ..importer.fx_importer import torch_translate_to_llh_graph
+from ..llh.passes import run_llh_pipeline
+from .torch_compile_config import LLC_DECOMPOSITIONS, LLCOperatorSupport
+
+TARGETS = ("gfx950",)
+PIPELINES = ("hip",)
+
+
+class LLCompiler:
+    """
+    example:
+        compiler = LLCompiler()
+        opt = torch.compile(model, backend=compiler)
+        out = opt(*inputs)
+    """
+
+    def __init__(self, mode: str = "inference", target: str = "gfx950", pipeline: str = "hip", index_bit_width: int = 64,
+                 symbol_infer=True, target_layout="NCHW", vebose_first_ir=False, log_root: str = "", log_level: str = "debug",
+                 log_llvm: bool = True, cpu="", mtriple="", **kwargs) -> None:
+        # the reference accepts x86 / x86_64 and the "transform" pipeline only
+        # (include/llcompiler/Support/Enums.td:28-34, src/Compiler/Compiler.cpp:144-148)
+        if target not in TARGETS:
+            raise ValueError("target %r: this backend generates code for %s only" % (target, ", ".join(TARGETS)))
+        if pipeline not in PIPELINES:
+            raise ValueError("pipeline %r: only %s is available" % (pipeline, ", ".join(PIPELINES)))
+        if target_layout != "NCHW":
+            raise ValueError("target_layout %r: NCHW only" % (target_layout,))
+        if mode not in ("inference", "training"):
+            raise ValueError("mode %r" % (mode,))
+        self.mode, self.target, self.pipeline = mode, target, pipeline
+        self.vebose_first_ir = vebose_first_ir
+        self.log_root, self.log_level = log_root, log_level
+        self.target_layout = target_layout
+        self.compile_count = 0
+        self.engines = []
+
+    def _process_fx(self, model: torch.fx.GraphModule, inputs: List[torch.Tensor], **kwargs):
+        partition = CapabilityBasedPartitioner(model, LLCOperatorSupport(), allows_single_node_partition=True)
+        return partition.partition_and_fuse()
+
+    def not_compile(self, model: Any, inputs: List[torch.Tensor], **kwargs):
+        return model
+
+    def importer(self, model: torch.fx.GraphModule):
+        return torch_translate_to_llh_graph(model)
+
+    def compiler_fx(self, model: torch.fx.GraphModule, inputs: List[torch.Tensor], **kwargs):
+        model = self._process_fx(model, inputs, **kwargs)
+        for name, submodule in dict(model._modules).items():
+            if not isinstance(submodule, torch.fx.GraphModule):
+                continue
+            executor = self.compiler_fx_submodule(submodule)
+            model.delete_submodule(name)
+            setattr(model, name, executor)
+        return model.forward
+
+    def compiler_fx_submodule(self, model: torch.fx.GraphModule, **kwargs):
+        graph = self.importer(model)
+        run_llh_pipeline(graph)
+        if self.vebose_first_ir:
+            print(graph.dump())
+        self.compile_count += 1
+        executor = _EngineModule(Torch_ExecutionEngine(graph))
+        self.engines.append(executor.engine)
+        return executor
+
+    def __call__(self, model, inputs: List[torch.Tensor]) -> Any:
+        if not isinstance(model, torch.fx.GraphModule):
+            raise ValueError("Unsupported")
+        bw_compiler = self.not_compile if self.mode == "inference" else self.compiler_fx
+        return aot_autograd(fw_compiler=self.compiler_fx, bw_compiler=bw_compiler, inference_compiler=self.compiler_fx,
+                            decompositions=get_decompositions(LLC_DECOMPOSITIONS))(model, inputs)
+
+
+class _EngineModule(torch.nn.Module):
+    """Lets an engine sit where the fused submodule was (GraphModule children must be Modules)."""
+
+    def __init__(self, engine):
+        super().__init__()
+        self.engine = engine
+
+    def forward(self, *args):
+        return self.engine.run(*args)

@@ -1,0 +1,420 @@
+"""Run-time side of a compiled LLH graph: device buffers, symbolic-shape dispatch and the call
+convention of the reference's executor.
+
+`Torch_ExecutionEngine.run(*args)` keeps the reference's convention
+(llcompiler/executor/engine.py:56-78): tensors positional, Python ints are symbol values, the
+result is a tensor or a list.  What changes underneath:
+
+  * output shapes come from evaluating the graph's symbolic extents with the bound symbols, not
+    from re-tracing the FX graph with FakeTensorProp on every call
+    (llcompiler/executor/out_put_call.py:154-170);
+  * for every distinct binding (symbol values + input layouts) the plan is specialised once into an
+    `Instance`: concrete shapes, intermediate device buffers (reused by liveness), and prepared
+    kernel calls.  Later calls with the same binding only patch the input/output pointers into the
+    descriptors and launch;
+  * tensors live on the GPU; nothing is copied to the host.
+"""
+import ctypes
+
+import torch
+
+from .. import _capi as C
+from .. import ops
+from ..llh.expr import Expr, evaluate
+from ..llh.graph import Value
+from .planner import make_plan
+
+# same codes as the reference's map (engine.py:11), extended with bf16 / f16 / i32
+TORCH_DTYPE_TO_TYPE = C.TORCH_DTYPE_TO_TYPE
+
+
+def _concrete(shape, env):
+    return tuple(evaluate(d, env) if isinstance(d, Expr) else int(d) for d in shape)
+
+
+class _Pool:
+    """Intermediate device buffers, reused once their last reader has been enqueued (all kernels of
+    an instance run in order on one stream, so reuse needs no further synchronisation)."""
+
+    def __init__(self, device):
+        self.device = device
+        self.free = {}
+        self.all = []
+
+    def take(self, nbytes):
+        size = max(256, (nbytes + 255) // 256 * 256)
+        lst = self.free.get(size)
+        if lst:
+            return lst.pop()
+        buf = torch.empty(size, dtype=torch.uint8, device=self.device)
+        self.all.append(buf)
+        return buf
+
+    def give(self, buf):
+        self.free.setdefault(buf.numel(), []).append(buf)
+
+
+class Instance:
+    """A plan specialised to concrete extents: a flat list of prepared kernel calls."""
+
+    def __init__(self, graph, steps, env, inputs, device):
+        self.graph, self.env, self.device = graph, env, device
+        self.calls = []
+        self.patches = []          # (TensorRef, "in"|"out", index, byte offset from that tensor's data_ptr)
+        self.keep = []
+        self._roots = {}           # storage data_ptr -> ("in"|"out", index, base data_ptr)
+        self.out_meta = []         # (shape, dtype) of every tensor output
+        self.example_outputs = []
+        self._build(steps, inputs)
+
+    # ---- bookkeeping of per-call storages ----
+    def _register_root(self, kind, index, t):
+        self._roots.setdefault(t.untyped_storage().data_ptr(), (kind, index, t.data_ptr()))
+
+    def _launch_later(self, call):
+        # every descriptor the call holds is checked against the per-call storages
+        for item in call.keep:
+            self._scan(item)
+        self.calls.append(call)
+
+    def _scan(self, item):
+        if isinstance(item, C.TensorRef):
+            t = item._keep
+            if isinstance(t, torch.Tensor):
+                root = self._roots.get(t.untyped_storage().data_ptr())
+                if root is not None:
+                    self.patches.append((item, root[0], root[1], t.data_ptr() - root[2]))
+        elif isinstance(item, ops.Epilogue):
+            for r in (getattr(item, "_b", None), getattr(item, "_r", None)):
+                if r is not None:
+                    self._scan(r)
+        elif isinstance(item, (list, tuple)):
+            for x in item:
+                self._scan(x)
+
+    # ---- building ----
+    def _build(self, steps, inputs):
+        g = self.graph
+        dev = self.device
+        val = {}
+        for i, (v, t) in enumerate(zip(g.inputs, inputs)):
+            val[id(v)] = t
+            self._register_root("in", i, t)
+        out_ids = {}
+        for k, o in enumerate(g.outputs):
+            if isinstance(o, Value):
+                out_ids.setdefault(id(o), []).append(k)
+        # liveness per backing buffer: a value and every view derived from it share one root; the
+        # root's buffer returns to the pool after the last step that reads any of them
+        root_of = {}
+        for st in steps:
+            if st.kind == "view":
+                src = id(st.inputs[0])
+                root_of[id(st.output)] = root_of.get(src, src)
+        last_use = {}
+        for si, st in enumerate(steps):
+            reads = list(st.inputs)
+            e = st.attrs.get("epilogue") if isinstance(st.attrs, dict) else None
+            if e:
+                reads += [x for x in (e.get("bias"), e.get("residual")) if x is not None]
+            for r in reads:
+                rid = root_of.get(id(r), id(r))
+                last_use[rid] = si
+        for o in g.outputs:
+            if isinstance(o, Value):
+                last_use[root_of.get(id(o), id(o))] = len(steps)  # read by the output copy at the end
+        pool = _Pool(dev)
+        self.pool = pool
+        owner = {}      # id(root value) -> pool buffer backing it
+        temps = []      # staging copies made for the current step
+        n_out_bufs = 0
+
+        def new_tensor(v, shape=None):
+            nonlocal n_out_bufs
+            shape = _concrete(v.shape if shape is None else shape, self.env)
+            if id(v) in out_ids:
+                t = torch.empty(shape, dtype=v.dtype, device=dev)
+                self._register_root("out", n_out_bufs, t)
+                self.out_buffers.append(t)
+                n_out_bufs += 1
+                return t
+            n = 1
+            for d in shape:
+                n *= d
+            buf = pool.take(n * v.dtype.itemsize)
+            owner[id(v)] = buf
+            return buf[: n * v.dtype.itemsize].view(v.dtype).view(shape)
+
+        self.out_buffers = []
+
+        def contiguous(t):
+            if t.is_contiguous():
+                return t
+            n = t.numel()
+            buf = pool.take(n * t.dtype.itemsize)
+            temps.append(buf)
+            c = buf[: n * t.dtype.itemsize].view(t.dtype).view(tuple(t.shape))
+            if n:
+                self._launch_later(ops.copy(t, out=c, defer=True))
+            return c
+
+        for si, st in enumerate(steps):
+            k = st.kind
+            ins = [val[id(v)] for v in st.inputs]
+            if k == "view":
+                before = len(temps)
+                val[id(st.output)] = self._view(st, ins[0], contiguous)
+                if len(temps) > before:
+                    # the reshape needed a contiguous copy: the view now lives in that copy, which stays
+                    # private to this instance (later views of it are not tracked for reuse)
+                    self.keep.append(temps.pop())
+            elif k == "constant":
+                c = torch.full((1,), st.attrs["value"], dtype=st.output.dtype, device=dev)
+                self.keep.append(c)
+                val[id(st.output)] = c
+            elif k == "ew":
+                out = new_tensor(st.output)
+                prog = ops.make_program(st.attrs["insts"], st.attrs["result"], st.attrs["integer"])
+                if out.numel():
+                    self._launch_later(ops.elementwise(prog, ins, tuple(out.shape), out.dtype, out=out, defer=True))
+                val[id(st.output)] = out
+            elif k in ("matmul", "batch_matmul", "conv"):
+                e = st.attrs["epilogue"]
+                out = new_tensor(st.output)
+                natural = _concrete(st.attrs["natural_shape"], self.env)
+                bias = val[id(e["bias"])] if e["bias"] is not None else None
+                res = val[id(e["residual"])] if e["residual"] is not None else None
+                if bias is not None:
+                    bias = contiguous(bias.reshape(-1) if bias.is_contiguous() else bias).reshape(-1)
+                if res is not None:
+                    res = contiguous(res)
+                epi = None
+                if bias is not None or res is not None or e["act"] or e["alpha"] != 1.0:
+                    epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=res, act=e["act"] or "none")
+                o = out.view(natural)
+                if k == "matmul":
+                    call = ops.matmul(ins[0], ins[1], epi, out=o, defer=True)
+                elif k == "batch_matmul":
+                    call = ops.batch_matmul(ins[0], ins[1], epi, out=o, defer=True)
+                else:
+                    call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],
+                                      dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi, out=o, defer=True)
+                if out.numel():
+                    self._launch_later(call)
+                val[id(st.output)] = out
+            elif k == "softmax":
+                out = new_tensor(st.output)
+                if out.numel():
+                    self._launch_later(ops.softmax(contiguous(ins[0]), out=out, defer=True))
+                val[id(st.output)] = out
+            elif k == "layer_norm":
+                out = new_tensor(st.output)
+                rest = ins[1:]
+                scale = contiguous(rest.pop(0)) if st.attrs.get("has_scale", True) and rest else None
+                bias = contiguous(rest.pop(0)) if st.attrs.get("has_bias", True) and rest else None
+                if out.numel():
+                    self._launch_later(ops.layer_norm(contiguous(ins[0]), scale, bias, st.attrs["epsilon"], out=out, defer=True))
+                val[id(st.output)] = out
+            elif k == "reduce":
+                out = new_tensor(st.output)
+                x = contiguous(ins[0])
+                axes = sorted(a % x.dim() for a in st.attrs["axis"])
+                self._reduce(st.attrs["kind"], x, axes, out, pool)
+                val[id(st.output)] = out
+            elif k == "max_pool":
+                out = new_tensor(st.output)
+                a = st.attrs
+                if out.numel():
+                    self._launch_later(ops.max_pool(contiguous(ins[0]), a["kernel_shape"], pad=a["pad"], stride=a["stride"],
+                                                    dilation=a["dilation"], init_zero=False, out=out, defer=True))
+                val[id(st.output)] = out
+            elif k == "avg_pool":
+                out = new_tensor(st.output)
+                if out.numel():
+                    self._launch_later(ops.global_avg_pool(contiguous(ins[0]), out=out, defer=True))
+                val[id(st.output)] = out
+            elif k == "gather":
+                out = new_tensor(st.output)
+                if out.numel():
+                    self._launch_later(ops.gather_rows(contiguous(ins[0]), contiguous(ins[1]), out=out, defer=True))
+                val[id(st.output)] = out
+            else:
+                raise NotImplementedError(k)
+            # buffers whose last reader has now been enqueued go back to the pool
+            for buf in temps:
+                pool.give(buf)
+            del temps[:]
+            for rid in [r for r in owner if last_use.get(r, si) <= si]:
+                pool.give(owner.pop(rid))
+        # graph outputs
+        self.output_plan = []
+        for o in g.outputs:
+            if isinstance(o, Value):
+                t = val[id(o)]
+                root = self._roots.get(t.untyped_storage().data_ptr())
+                if root is None or root[0] != "out" or not t.is_contiguous():
+                    # an output that aliases an input or an intermediate view: materialise it per call
+                    fresh = torch.empty(tuple(t.shape), dtype=t.dtype, device=dev)
+                    self._register_root("out", n_out_bufs, fresh)
+                    self.out_buffers.append(fresh)
+                    if fresh.numel():
+                        self._launch_later(ops.copy(t, out=fresh, defer=True))
+                    self.output_plan.append(("tensor", n_out_bufs, tuple(fresh.shape), tuple(fresh.stride()), 0))
+                    n_out_bufs += 1
+                else:
+                    off = (t.data_ptr() - root[2]) // t.dtype.itemsize
+                    self.output_plan.append(("tensor", root[1], tuple(t.shape), tuple(t.stride()), off))
+            elif isinstance(o, Expr):
+                self.output_plan.append(("int", evaluate(o, self.env)))
+            else:
+                self.output_plan.append(("const", o))
+        self.out_specs = [(tuple(b.shape), b.dtype) for b in self.out_buffers]
+        self._first = True
+
+    def _view(self, st, t, contiguous):
+        a = st.attrs
+        op = a["op"]
+        if op in ("identity",):
+            return t
+        if op in ("reshape", "flatten"):
+            shape = _concrete(st.output.shape, self.env)
+            try:
+                return t.view(shape)
+            except RuntimeError:
+                return contiguous(t).view(shape)
+        if op == "transpose":
+            return t.permute(*a["perms"])
+        if op == "broadcast_to":
+            return t.expand(*_concrete(st.output.shape, self.env))
+        if op == "stride_slice":
+            idx = tuple(slice(evaluate(s, self.env) if isinstance(s, Expr) else s, evaluate(e, self.env) if isinstance(e, Expr) else e,
+                              st_) for s, e, st_ in zip(a["start"], a["end"], a["stride"]))
+            return t[idx]
+        if op == "extract":
+            return t[a["index"]]
+        raise NotImplementedError(op)
+
+    def _reduce(self, kind, x, axes, out, pool):
+        """The kernel reduces one run of adjacent axes; split axes are reduced run by run, innermost first."""
+        runs = []
+        for a in axes:
+            if runs and runs[-1][-1] == a - 1:
+                runs[-1].append(a)
+            else:
+                runs.append([a])
+        cur = x
+        for i, run in enumerate(reversed(runs)):
+            last = i == len(runs) - 1
+            shape = [s for d, s in enumerate(cur.shape) if d not in run]
+            if last:
+                dst = out.view(shape) if out.numel() else out
+            else:
+                n = 1
+                for s in shape:
+                    n *= s
+                buf = pool.take(n * x.dtype.itemsize)
+                self.keep.append(buf)  # partial results stay private to this step
+                dst = buf[: n * x.dtype.itemsize].view(x.dtype).view(shape)
+            if dst.numel():
+                self._launch_later(ops.reduce(kind, cur, run, out=dst, defer=True))
+            cur = dst
+
+    # ---- execution ----
+    def run(self, inputs):
+        if self._first:
+            outs = self.out_buffers
+            self._first = False
+        else:
+            outs = [torch.empty(s, dtype=d, device=self.device) for s, d in self.out_specs]
+        in_ptrs = [t.data_ptr() for t in inputs]
+        out_ptrs = [t.data_ptr() for t in outs]
+        for ref, kind, idx, delta in self.patches:
+            p = (in_ptrs[idx] if kind == "in" else out_ptrs[idx]) + delta
+            ref.desc.data = p
+            ref.desc.base = p
+        for c in self.calls:
+            c.launch()
+        results = []
+        for spec in self.output_plan:
+            if spec[0] == "tensor":
+                _, idx, shape, stride, off = spec
+                t = outs[idx]
+                results.append(t if (tuple(t.shape) == shape and off == 0) else t.as_strided(shape, stride, off))
+            else:
+                results.append(spec[1])
+        return results
+
+
+class ExecutionEngine:
+    """Base of the reference's engines (engine.py:15-26): holds the compiled artefact, is callable."""
+
+    def __init__(self, graph):
+        self.graph = graph
+        self.steps = make_plan(graph)
+        self.instances = {}
+
+    def run(self, *args):
+        raise NotImplementedError
+
+    def __call__(self, *args):
+        return self.run(*args)
+
+
+class Torch_ExecutionEngine(ExecutionEngine):
+    def trans_to_tensor(self, *args):
+        """The reference wraps every torch tensor in its C++ Tensor descriptor here (engine.py:34-54);
+        this build keeps the torch tensor and builds descriptors once per specialised instance."""
+        inputs = []
+        for arg in args:
+            if isinstance(arg, torch.Tensor):
+                if arg.dtype not in TORCH_DTYPE_TO_TYPE:
+                    raise TypeError("Unsupported type: %s" % arg.dtype)
+                inputs.append(arg)
+            elif isinstance(arg, int) or arg is None:
+                pass
+            else:
+                raise TypeError("Unsupported type: %s" % type(arg))
+        return inputs
+
+    def bind_symbols(self, args, inputs):
+        g = self.graph
+        env = {}
+        ints = [a for a in args if isinstance(a, int) and not isinstance(a, bool)]
+        if len(ints) != len(g.symbol_args):
+            raise ValueError("expected %d symbol values (python ints), got %d" % (len(g.symbol_args), len(ints)))
+        for name, v in zip(g.symbol_args, ints):
+            env[name] = v
+        for name, (i, d) in g.symbol_sources.items():
+            env.setdefault(name, inputs[i].shape[d])
+        return env
+
+    def run(self, *args):
+        # ([inputs...]) case, as in the reference
+        if len(args) == 1 and isinstance(args[0], (list, tuple)):
+            args = tuple(args[0])
+        inputs = self.trans_to_tensor(*args)
+        g = self.graph
+        if len(inputs) != len(g.inputs):
+            raise ValueError("expected %d tensors, got %d" % (len(g.inputs), len(inputs)))
+        env = self.bind_symbols(args, inputs)
+        device = None
+        for t in inputs:
+            if not t.is_cuda:
+                raise RuntimeError("llcompiler_amd executes on the GPU only; got a %s tensor (no CPU fallback)" % t.device)
+            device = t.device
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        for v, t in zip(g.inputs, inputs):
+            want = _concrete(v.shape, env)
+            if tuple(t.shape) != want or t.dtype != v.dtype:
+                raise ValueError("input %s: expected %s %s, got %s %s" % (v.name, want, v.dtype, tuple(t.shape), t.dtype))
+        key = (tuple(sorted(env.items())), tuple((tuple(t.shape), tuple(t.stride())) for t in inputs), device.index)
+        inst = self.instances.get(key)
+        if inst is None:
+            C.init(device.index or 0)
+            inst = Instance(g, self.steps, env, inputs, device)
+            self.instances[key] = inst
+        results = inst.run(inputs)
+        if getattr(g, "single_output", len(results) == 1) and len(results) == 1:
+            return results[0]
+        return results

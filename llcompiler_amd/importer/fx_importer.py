@@ -1,0 +1,515 @@
+"""FX graph (ATen / prims ops after AOT decomposition) -> LLH graph.
+
+Counterpart of the reference's importer (llcompiler/importer/fx_translate.py:289-521 and
+fx_op_translate/*.py): one translator per ATen/prims target, registered in
+TORCH_FUNCTION_TRANSLATE, producing the same LLH ops and attributes (conv attrs as in conv.py:48-70,
+negative reduce axes normalised and keepdim expressed as reduce + reshape as in
+reduce_ops.py:56-82, scalars as tensor<1xT> constants as in fx_translate.py:274-282).
+Differences, all on purpose: bf16/f16 are accepted; `where` passes on_false (the reference passes
+on_true twice, where.py:48-49); gelu, softmax, layer_norm, embedding and the extra unary ops
+are translated instead of being left to torch eager.
+"""
+import operator
+
+import torch
+
+from ..llh.expr import Expr, from_sympy
+from ..llh.graph import Graph, Value
+
+aten = torch.ops.aten
+prims = torch.ops.prims
+
+TORCH_FUNCTION_TRANSLATE = {}
+_SUPPORT_CHECKS = {}
+
+
+def TORCH_FUNCTION_TRANSLATE_REGISTER(*targets, check=None):
+    def deco(fn):
+        for t in targets:
+            TORCH_FUNCTION_TRANSLATE[t] = fn
+            if check is not None:
+                _SUPPORT_CHECKS[t] = check
+        return fn
+    return deco
+
+
+def dim_of(d):
+    if isinstance(d, int):
+        return d
+    if isinstance(d, torch.SymInt):
+        e = d.node.expr
+        if e.is_number:
+            return int(e)
+        return from_sympy(e)
+    raise TypeError("extent %r" % (d,))
+
+
+def meta_shape(node_or_val):
+    val = node_or_val.meta["val"] if isinstance(node_or_val, torch.fx.Node) else node_or_val
+    return tuple(dim_of(d) for d in val.shape)
+
+
+class Ctx:
+    def __init__(self, graph):
+        self.g = graph
+        self.env = {}  # fx node -> Value | tuple of Values | None (symbolic ints)
+
+    def val(self, a):
+        return self.env[a] if isinstance(a, torch.fx.Node) else a
+
+    def tensor_or_const(self, a, like):
+        """Python scalars become tensor<1xT> constants of the other operand's element type."""
+        if isinstance(a, torch.fx.Node):
+            v = self.env[a]
+            if isinstance(v, Value):
+                return v
+            raise NotImplementedError("symbolic scalar operand %s" % a)
+        dt = like.dtype if like is not None else torch.float32
+        if isinstance(a, float) and not dt.is_floating_point:
+            dt = torch.float32
+        return self.g.constant(a, dt)
+
+
+def _out_shape(node):
+    return meta_shape(node)
+
+
+def _out_dtype(node):
+    return node.meta["val"].dtype
+
+
+def _reshape_to(ctx, x, shape):
+    if tuple(x.shape) == tuple(shape):
+        return x
+    return ctx.g.add_op("reshape", [x], {"shape": tuple(shape)}, shapes=[tuple(shape)], dtypes=[x.dtype])
+
+
+# ---------------------------------------------------------------- contractions
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.mm.default)
+def _mm(ctx, node):
+    return ctx.g.add_op("matmul", [ctx.val(node.args[0]), ctx.val(node.args[1])])
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.bmm.default)
+def _bmm(ctx, node):
+    return ctx.g.add_op("batch_matmul", [ctx.val(node.args[0]), ctx.val(node.args[1])])
+
+
+def _conv_ok(node):
+    a = node.args
+    return (not a[6]) and len(a[3]) == 2 and all(int(p) == 0 for p in a[7])
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.convolution.default, check=_conv_ok)
+def _conv(ctx, node):
+    x, w, b, stride, padding, dilation, transposed, output_padding, groups = node.args
+    xv, wv = ctx.val(x), ctx.val(w)
+    attrs = {"dilation": tuple(dilation), "kernel_shape": tuple(wv.shape[-2:]),
+             "pad": (padding[0], padding[1], padding[0], padding[1]), "stride": tuple(stride), "group": int(groups),
+             "layout": "NCHW"}
+    if b is None:
+        return ctx.g.add_op("conv", [xv, wv], attrs)
+    return ctx.g.add_op("conv_bias", [xv, wv, ctx.val(b)], attrs)
+
+
+# ---------------------------------------------------------------- views
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.t.default)
+def _t(ctx, node):
+    x = ctx.val(node.args[0])
+    if x.rank < 2:
+        return x
+    return ctx.g.add_op("transpose", [x], {"perms": (1, 0)})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.permute.default)
+def _permute(ctx, node):
+    x = ctx.val(node.args[0])
+    perms = tuple(p % x.rank for p in node.args[1])
+    return ctx.g.add_op("transpose", [x], {"perms": perms})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.transpose.int)
+def _transpose_int(ctx, node):
+    x = ctx.val(node.args[0])
+    a, b = node.args[1] % x.rank, node.args[2] % x.rank
+    perms = list(range(x.rank))
+    perms[a], perms[b] = perms[b], perms[a]
+    return ctx.g.add_op("transpose", [x], {"perms": tuple(perms)})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.view.default, aten.reshape.default, aten._unsafe_view.default,
+                                   aten.unsqueeze.default, aten.squeeze.dim, aten.squeeze.dims, aten.squeeze.default,
+                                   prims.squeeze.default, aten.flatten.using_ints)
+def _view(ctx, node):
+    return _reshape_to(ctx, ctx.val(node.args[0]), _out_shape(node))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.clone.default, aten.contiguous.default, aten.alias.default,
+                                   aten.detach.default, aten.lift_fresh_copy.default, aten._to_copy.default,
+                                   prims.convert_element_type.default)
+def _identity_or_convert(ctx, node):
+    x = ctx.val(node.args[0])
+    dt = _out_dtype(node)
+    if dt != x.dtype:
+        return ctx.g.add_op("convert_to", [x], {"dtype": dt})
+    return ctx.g.add_op("identity", [x])
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(prims.broadcast_in_dim.default)
+def _broadcast_in_dim(ctx, node):
+    x = ctx.val(node.args[0])
+    shape = _out_shape(node)
+    dims = list(node.args[2])
+    aligned = [1] * len(shape)
+    for i, d in enumerate(dims):
+        aligned[d] = x.shape[i]
+    x = _reshape_to(ctx, x, aligned)
+    if tuple(aligned) == tuple(shape):
+        return x
+    return ctx.g.add_op("broadcast_to", [x], {"shape": shape, "cast_dims": tuple(range(len(shape)))})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.expand.default)
+def _expand(ctx, node):
+    x = ctx.val(node.args[0])
+    shape = _out_shape(node)
+    aligned = (1,) * (len(shape) - x.rank) + tuple(x.shape)
+    x = _reshape_to(ctx, x, aligned)
+    if tuple(aligned) == tuple(shape):
+        return x
+    return ctx.g.add_op("broadcast_to", [x], {"shape": shape, "cast_dims": tuple(range(len(shape)))})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.select.int)
+def _select(ctx, node):
+    x = ctx.val(node.args[0])
+    dim, index = node.args[1] % x.rank, node.args[2]
+    if dim == 0:
+        return ctx.g.add_op("extract", [x], {"index": int(index)})
+    if index < 0:
+        index += x.shape[dim]
+    start = [0] * x.rank
+    end = list(x.shape)
+    start[dim], end[dim] = index, index + 1
+    s = ctx.g.add_op("stride_slice", [x], {"start": tuple(start), "end": tuple(end), "stride": (1,) * x.rank})
+    return _reshape_to(ctx, s, _out_shape(node))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.slice.Tensor)
+def _slice(ctx, node):
+    x = ctx.val(node.args[0])
+    args = list(node.args) + [None] * (5 - len(node.args))
+    dim = (args[1] or 0) % x.rank
+    size = x.shape[dim]
+    start = args[2] or 0
+    end = size if args[3] is None else args[3]
+    step = 1 if args[4] is None else args[4]
+    if isinstance(size, int):
+        if start < 0:
+            start += size
+        if isinstance(end, int):
+            if end < 0:
+                end += size
+            end = min(end, size)
+    st = [0] * x.rank
+    en = list(x.shape)
+    sp = [1] * x.rank
+    st[dim], en[dim], sp[dim] = start, end, step
+    if st[dim] == 0 and en[dim] == size and step == 1:
+        return x
+    return ctx.g.add_op("stride_slice", [x], {"start": tuple(st), "end": tuple(en), "stride": tuple(sp)},
+                        shapes=[_out_shape(node)], dtypes=[x.dtype])
+
+
+# ---------------------------------------------------------------- elementwise
+def _binary(name):
+    def tr(ctx, node):
+        a, b = node.args[0], node.args[1]
+        av = ctx.tensor_or_const(a, ctx.val(b) if isinstance(b, torch.fx.Node) else None)
+        bv = ctx.tensor_or_const(b, av)
+        if not isinstance(a, torch.fx.Node):
+            av = ctx.tensor_or_const(a, bv)
+        alpha = node.kwargs.get("alpha", 1)
+        if alpha != 1:
+            bv = ctx.g.add_op("mul", [bv, ctx.g.constant(alpha, bv.dtype)])
+        out = ctx.g.add_op(name, [av, bv])
+        dt = _out_dtype(node)
+        if out.dtype != dt:
+            out = ctx.g.add_op("convert_to", [out], {"dtype": dt})
+        return out
+    return tr
+
+
+for _name, _targets in {
+    "add": (aten.add.Tensor, aten.add.Scalar, prims.add.default),
+    "sub": (aten.sub.Tensor, aten.sub.Scalar, prims.sub.default),
+    "mul": (aten.mul.Tensor, aten.mul.Scalar, prims.mul.default),
+    "div": (aten.div.Tensor, aten.div.Scalar, prims.div.default),
+    "max": (aten.maximum.default, prims.maximum.default),
+    "min": (aten.minimum.default, prims.minimum.default),
+    "pow": (aten.pow.Tensor_Scalar, aten.pow.Tensor_Tensor, prims.pow.default),
+}.items():
+    TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_binary(_name))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.rsub.Scalar, aten.rsub.Tensor)
+def _rsub(ctx, node):
+    a = ctx.val(node.args[0])
+    b = ctx.tensor_or_const(node.args[1], a)
+    return ctx.g.add_op("sub", [b, a])
+
+
+def _unary(name):
+    def tr(ctx, node):
+        return ctx.g.add_op(name, [ctx.val(node.args[0])])
+    return tr
+
+
+for _name, _targets in {
+    "relu": (aten.relu.default,), "abs": (aten.abs.default, prims.abs.default), "exp": (aten.exp.default, prims.exp.default),
+    "sqrt": (aten.sqrt.default, prims.sqrt.default), "rsqrt": (aten.rsqrt.default, prims.rsqrt.default),
+    "neg": (aten.neg.default, prims.neg.default), "tanh": (aten.tanh.default, prims.tanh.default),
+    "erf": (aten.erf.default, prims.erf.default), "sigmoid": (aten.sigmoid.default,),
+    "log": (aten.log.default, prims.log.default), "recip": (aten.reciprocal.default, prims.reciprocal.default),
+}.items():
+    TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_unary(_name))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.gelu.default, check=lambda n: n.kwargs.get("approximate", "none") == "none")
+def _gelu(ctx, node):
+    return ctx.g.add_op("gelu", [ctx.val(node.args[0])])
+
+
+def _compare(kind):
+    def tr(ctx, node):
+        a = ctx.val(node.args[0])
+        b = ctx.tensor_or_const(node.args[1], a)
+        return ctx.g.add_op("compare", [a, b], {"kind": kind})
+    return tr
+
+
+for _kind, _targets in {
+    "EQ": (aten.eq.Tensor, aten.eq.Scalar, prims.eq.default), "NE": (aten.ne.Tensor, aten.ne.Scalar, prims.ne.default),
+    "GE": (aten.ge.Tensor, aten.ge.Scalar, prims.ge.default), "GT": (aten.gt.Tensor, aten.gt.Scalar, prims.gt.default),
+    "LE": (aten.le.Tensor, aten.le.Scalar, prims.le.default), "LT": (aten.lt.Tensor, aten.lt.Scalar, prims.lt.default),
+}.items():
+    TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_compare(_kind))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(prims.where.default, aten.where.self)
+def _where(ctx, node):
+    pred = ctx.val(node.args[0])
+    t, f = node.args[1], node.args[2]
+    like = ctx.val(t) if isinstance(t, torch.fx.Node) else (ctx.val(f) if isinstance(f, torch.fx.Node) else None)
+    tv = ctx.tensor_or_const(t, like)
+    fv = ctx.tensor_or_const(f, tv)
+    out = ctx.g.add_op("where", [pred, tv, fv])
+    dt = _out_dtype(node)
+    if out.dtype != dt:
+        out = ctx.g.add_op("convert_to", [out], {"dtype": dt})
+    return out
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.scalar_tensor.default, aten.full.default)
+def _full(ctx, node):
+    if node.target is aten.scalar_tensor.default:
+        value = node.args[0]
+    else:
+        value = node.args[1]
+    dt = _out_dtype(node)
+    c = ctx.g.constant(value, dt)
+    shape = _out_shape(node)
+    if len(shape) == 0:
+        return _reshape_to(ctx, c, ())
+    c = _reshape_to(ctx, c, (1,) * len(shape))
+    if all(isinstance(d, int) and d == 1 for d in shape):
+        return c
+    return ctx.g.add_op("broadcast_to", [c], {"shape": shape, "cast_dims": tuple(range(len(shape)))})
+
+
+# ---------------------------------------------------------------- reductions / normalisation / pooling
+def _reduce(name):
+    def tr(ctx, node):
+        x = ctx.val(node.args[0])
+        dims = node.args[1] if len(node.args) > 1 else list(range(x.rank))
+        if isinstance(dims, int):
+            dims = [dims]
+        axes = tuple(sorted(d % x.rank for d in dims)) if len(dims) else tuple(range(x.rank))
+        keepdim = node.args[2] if len(node.args) > 2 else False
+        r = ctx.g.add_op(name, [x], {"axis": axes})
+        if keepdim:
+            r = _reshape_to(ctx, r, _out_shape(node))
+        return r
+    return tr
+
+
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amax.default)(_reduce("reduce_max"))
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amin.default)(_reduce("reduce_min"))
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.sum.dim_IntList)(_reduce("reduce_sum"))
+
+
+def _mean_ok(node):
+    shape = node.args[0].meta["val"].shape
+    dims = node.args[1]
+    return all(isinstance(shape[d], int) for d in dims)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.mean.dim, check=_mean_ok)
+def _mean(ctx, node):
+    x = ctx.val(node.args[0])
+    dims = tuple(sorted(d % x.rank for d in node.args[1]))
+    keepdim = node.args[2] if len(node.args) > 2 else False
+    if x.rank == 4 and dims == (2, 3):
+        r = ctx.g.add_op("adaptive_average_pool", [x], {"out_size": (1, 1)})
+        return r if keepdim else _reshape_to(ctx, r, _out_shape(node))
+    count = 1
+    for d in dims:
+        count *= x.shape[d]
+    r = ctx.g.add_op("reduce_sum", [x], {"axis": dims})
+    r = ctx.g.add_op("div", [r, ctx.g.constant(float(count), x.dtype)])
+    return _reshape_to(ctx, r, _out_shape(node)) if keepdim else r
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._adaptive_avg_pool2d.default, aten.adaptive_avg_pool2d.default,
+                                   check=lambda n: list(n.args[1]) == [1, 1])
+def _adaptive_avg_pool(ctx, node):
+    return ctx.g.add_op("adaptive_average_pool", [ctx.val(node.args[0])], {"out_size": (1, 1)})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._softmax.default,
+                                   check=lambda n: n.args[1] % n.args[0].meta["val"].dim() == n.args[0].meta["val"].dim() - 1)
+def _softmax(ctx, node):
+    x = ctx.val(node.args[0])
+    return ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm.default, check=lambda n: len(n.args[1]) == 1)
+def _layer_norm(ctx, node):
+    x, shape, w, b, eps = node.args
+    ops = [ctx.val(x)] + [ctx.val(t) for t in (w, b) if t is not None]
+    attrs = {"epsilon": float(eps), "axis": -1, "has_scale": w is not None, "has_bias": b is not None}
+    y = ctx.g.add_op("layer_norm", ops, attrs)
+    return (y, None, None)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._native_batch_norm_legit_no_training.default)
+def _batch_norm(ctx, node):
+    x, w, b, mean, var, momentum, eps = node.args
+    xv = ctx.val(x)
+    c = xv.shape[1]
+    wv = ctx.val(w) if w is not None else _ones_like_channels(ctx, c, xv.dtype, 1.0)
+    bv = ctx.val(b) if b is not None else _ones_like_channels(ctx, c, xv.dtype, 0.0)
+    y = ctx.g.add_op("batch_norm_inference", [xv, wv, bv, ctx.val(mean), ctx.val(var)],
+                     {"epsilon": float(eps), "momentum": float(momentum), "feature_index": 1})
+    return (y, None, None)
+
+
+def _ones_like_channels(ctx, c, dtype, value):
+    k = ctx.g.constant(value, dtype)
+    return ctx.g.add_op("broadcast_to", [k], {"shape": (c,), "cast_dims": (0,)})
+
+
+def _maxpool_ok(node):
+    a = list(node.args) + [None] * 6
+    return not a[5]  # ceil_mode
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.max_pool2d_with_indices.default, check=_maxpool_ok)
+def _max_pool(ctx, node):
+    a = list(node.args) + [None] * (6 - len(node.args))
+    x, k = ctx.val(a[0]), tuple(a[1])
+    if len(k) == 1:
+        k = (k[0], k[0])
+    stride = tuple(a[2]) if a[2] else k
+    pad = tuple(a[3]) if a[3] else (0, 0)
+    dil = tuple(a[4]) if a[4] else (1, 1)
+    def two(t): return t if len(t) == 2 else (t[0], t[0])
+    stride, pad, dil = two(stride), two(pad), two(dil)
+    y = ctx.g.add_op("max_pool", [x], {"ceil_mode": False, "dilation": dil, "kernel_shape": k,
+                                        "pad": (pad[0], pad[1], pad[0], pad[1]), "stride": stride, "layout": "NCHW"})
+    return (y, None)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.embedding.default)
+def _embedding(ctx, node):
+    return ctx.g.add_op("gather", [ctx.val(node.args[0]), ctx.val(node.args[1])])
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(operator.getitem)
+def _getitem(ctx, node):
+    src = ctx.env[node.args[0]]
+    return src[node.args[1]]
+
+
+# symbolic integer arithmetic feeds shapes only; extents are taken from each node's fake value
+_SYMBOLIC_TARGETS = {aten.sym_size.int, aten.sym_numel.default, operator.mul, operator.add, operator.sub,
+                     operator.floordiv, operator.truediv, operator.neg, operator.pow}
+if hasattr(torch, "_sym_sqrt"):
+    _SYMBOLIC_TARGETS.add(torch._sym_sqrt)
+if hasattr(torch, "sym_float"):
+    _SYMBOLIC_TARGETS.add(torch.sym_float)
+
+
+def is_supported(node):
+    """Whether a call_function node can be compiled (the reference's LLC_SUPPORT_DICT lookup,
+    llcompiler/compiler/torch_compile_config.py:29-132, extended with per-node attribute checks)."""
+    if node.target in _SYMBOLIC_TARGETS:
+        return True
+    if node.target not in TORCH_FUNCTION_TRANSLATE:
+        return False
+    chk = _SUPPORT_CHECKS.get(node.target)
+    try:
+        return True if chk is None else bool(chk(node))
+    except Exception:
+        return False
+
+
+def torch_translate_to_llh_graph(gm):
+    """Counterpart of torch_translate_to_mlir_module (llcompiler/importer/fx_translate.py:517-521)."""
+    g = Graph()
+    ctx = Ctx(g)
+    for node in gm.graph.nodes:
+        if node.op == "placeholder":
+            val = node.meta.get("val", node.meta.get("example_value"))
+            if isinstance(val, torch.Tensor):
+                ctx.env[node] = g.add_input(meta_shape(val), val.dtype, name=node.name)
+            elif isinstance(val, (torch.SymInt, int)):
+                # dynamo passes SymInts as leading int arguments (fx_translate.py:373-406)
+                e = dim_of(val)
+                name = e.args[0] if isinstance(e, Expr) and e.kind == "sym" else str(e)
+                g.add_symbol_arg(name)
+                ctx.env[node] = None
+            elif val is None:
+                g.arg_kinds.append(("none", None))
+                ctx.env[node] = None
+            else:
+                raise TypeError("Unsupported type: %s" % type(val))
+        elif node.op == "call_function":
+            if node.target in _SYMBOLIC_TARGETS:
+                ctx.env[node] = None
+                continue
+            tr = TORCH_FUNCTION_TRANSLATE.get(node.target)
+            if tr is None:
+                raise NotImplementedError("no LLH translation for %s" % (node.target,))
+            ctx.env[node] = tr(ctx, node)
+        elif node.op == "output":
+            outs = node.args[0]
+            single = not isinstance(outs, (tuple, list))
+            seq = [outs] if single else list(outs)
+            res = []
+            for o in seq:
+                if o is None:
+                    res.append(None)
+                elif isinstance(o, torch.fx.Node):
+                    v = ctx.env[o]
+                    if v is None:  # a symbolic int result
+                        res.append(dim_of(o.meta["val"]))
+                    else:
+                        res.append(v)
+                else:
+                    res.append(o)
+            g.set_outputs(res)
+            g.single_output = single
+        else:
+            raise NotImplementedError("fx node kind %s" % node.op)
+    return g

@@ -1,0 +1,149 @@
+"""Symbolic extents: small integer expression trees over named symbols ("s0", "s1", ...).
+
+This is the host-side stand-in for the reference's symbol system (SymEngine expressions attached
+to tensor dims, src/Dialect/LLH/SymbolInfer/): every dynamic dim of a graph value is an `Expr`,
+and the executor evaluates it with the symbol values bound at call time.  The node kinds are the
+ones the reference's run-time evaluator handles (llcompiler/executor/out_put_call.py:21-48: Add,
+Mul, FloorDiv, Pow, Symbol, Number) plus CeilDiv (the affine maps of
+src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:281-288), Sub, Max and Min.
+"""
+from functools import reduce as _reduce
+
+
+class Expr:
+    __slots__ = ("kind", "args")
+
+    def __init__(self, kind, args):
+        self.kind, self.args = kind, tuple(args)
+
+    # ---- construction ----
+    @staticmethod
+    def sym(name):
+        return Expr("sym", (name,))
+
+    def _bin(self, kind, other, swap=False):
+        a, b = (other, self) if swap else (self, other)
+        return simplify(Expr(kind, (a, b)))
+
+    def __add__(self, o): return self._bin("add", o)
+    def __radd__(self, o): return self._bin("add", o, True)
+    def __sub__(self, o): return self._bin("sub", o)
+    def __rsub__(self, o): return self._bin("sub", o, True)
+    def __mul__(self, o): return self._bin("mul", o)
+    def __rmul__(self, o): return self._bin("mul", o, True)
+    def __floordiv__(self, o): return self._bin("floordiv", o)
+    def __rfloordiv__(self, o): return self._bin("floordiv", o, True)
+
+    def __eq__(self, other):
+        if isinstance(other, Expr):
+            return self.kind == other.kind and self.args == other.args
+        return False
+
+    def __hash__(self):
+        return hash((self.kind, self.args))
+
+    def __repr__(self):
+        if self.kind == "sym":
+            return self.args[0]
+        op = {"add": "+", "sub": "-", "mul": "*", "floordiv": "//"}.get(self.kind)
+        if op:
+            return "(%r %s %r)" % (self.args[0], op, self.args[1])
+        return "%s(%s)" % (self.kind, ", ".join(repr(a) for a in self.args))
+
+    def symbols(self):
+        if self.kind == "sym":
+            return {self.args[0]}
+        out = set()
+        for a in self.args:
+            if isinstance(a, Expr):
+                out |= a.symbols()
+        return out
+
+
+def ceildiv(a, b):
+    if isinstance(a, int) and isinstance(b, int):
+        return -(-a // b)
+    return simplify(Expr("ceildiv", (a, b)))
+
+
+def emax(a, b):
+    if isinstance(a, int) and isinstance(b, int):
+        return max(a, b)
+    return a if a == b else Expr("max", (a, b))
+
+
+def simplify(e):
+    if not isinstance(e, Expr) or e.kind == "sym":
+        return e
+    a = [simplify(x) for x in e.args]
+    if all(isinstance(x, int) for x in a):
+        return evaluate(Expr(e.kind, a), {})
+    k = e.kind
+    if k == "add":
+        if a[0] == 0: return a[1]
+        if a[1] == 0: return a[0]
+    if k == "sub" and a[1] == 0:
+        return a[0]
+    if k == "sub" and a[0] == a[1]:
+        return 0
+    if k == "mul":
+        if a[0] == 1: return a[1]
+        if a[1] == 1: return a[0]
+        if a[0] == 0 or a[1] == 0: return 0
+    if k in ("floordiv", "ceildiv") and a[1] == 1:
+        return a[0]
+    return Expr(k, a)
+
+
+def evaluate(e, env):
+    """Integer value of `e` with symbols bound by `env` (name -> int)."""
+    if isinstance(e, int):
+        return e
+    k, a = e.kind, e.args
+    if k == "sym":
+        try:
+            return int(env[a[0]])
+        except KeyError:
+            raise KeyError("symbol %s is not bound by any input of this call" % a[0])
+    x = evaluate(a[0], env)
+    if k == "pow":
+        return x ** int(a[1])
+    y = evaluate(a[1], env)
+    if k == "add": return x + y
+    if k == "sub": return x - y
+    if k == "mul": return x * y
+    if k == "floordiv": return x // y
+    if k == "ceildiv": return -(-x // y)
+    if k == "max": return max(x, y)
+    if k == "min": return min(x, y)
+    raise NotImplementedError(k)
+
+
+def product(dims):
+    return _reduce(lambda x, y: x * y, dims, 1)
+
+
+def from_sympy(expr):
+    """Converts the sympy expression behind a torch SymInt (the same node kinds as
+    llcompiler/executor/out_put_call.py:21-48)."""
+    import sympy
+    if isinstance(expr, (int,)):
+        return expr
+    if isinstance(expr, sympy.Integer):
+        return int(expr)
+    if isinstance(expr, sympy.Symbol):
+        return Expr.sym(expr.name)
+    name = type(expr).__name__
+    if isinstance(expr, sympy.Add):
+        return _reduce(lambda x, y: x + y, [from_sympy(a) for a in expr.args])
+    if isinstance(expr, sympy.Mul):
+        return _reduce(lambda x, y: x * y, [from_sympy(a) for a in expr.args])
+    if name in ("FloorDiv", "CleanDiv", "PythonFloorDiv", "IntTrueDiv"):
+        return from_sympy(expr.args[0]) // from_sympy(expr.args[1])
+    if name == "CeilDiv":
+        return ceildiv(from_sympy(expr.args[0]), from_sympy(expr.args[1]))
+    if isinstance(expr, sympy.Pow) and isinstance(expr.args[1], sympy.Integer) and int(expr.args[1]) >= 0:
+        return simplify(Expr("pow", (from_sympy(expr.args[0]), int(expr.args[1]))))
+    if name == "Max":
+        return _reduce(emax, [from_sympy(a) for a in expr.args])
+    raise NotImplementedError("symbolic extent %r (%s)" % (expr, name))

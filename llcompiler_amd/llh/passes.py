@@ -1,0 +1,154 @@
+"""LLH-level rewrites run before kernel planning.  Counterparts of the reference's
+src/Dialect/LLH/Transforms passes and canonicalisers, on the Python graph:
+
+  canonicalize           no-op reshape / broadcast / convert / identity folds, x*1, x+0
+                         (LLHCanonicalize.cpp:378-455, LLHFolder.cpp:33-330)
+  decompose_batch_norm   batch_norm_inference -> add, sqrt, reshape, broadcast_to x4, sub, mul, div, add
+                         (DecomposeOps.cpp:110-148; op order pinned by test/Dialect/LLH/decompose_ops.mlir:10-20)
+  fuse_softmax           reduce_max -> sub -> exp -> reduce_sum -> div  ==>  softmax
+                         (the group ATen _softmax decomposes to, torch_compile_config.py:24)
+"""
+import torch
+
+from .graph import BINARY_OPS, Value
+
+
+def _is_const(v, value=None):
+    if not isinstance(v, Value) or v.const is None:
+        return False
+    return value is None or float(v.const) == float(value)
+
+
+def _through_broadcast(v):
+    """Looks through reshape / broadcast_to of a one-element constant."""
+    while v.producer is not None and v.producer.name in ("reshape", "broadcast_to") and v.const is None:
+        v = v.producer.operands[0]
+    return v
+
+
+def canonicalize(g):
+    changed = True
+    while changed:
+        changed = False
+        for op in list(g.ops):
+            r = op.results[0]
+            rep = None
+            if op.name == "identity":
+                rep = op.operands[0]
+            elif op.name == "convert_to" and op.attrs["dtype"] == op.operands[0].dtype:
+                rep = op.operands[0]
+            elif op.name in ("reshape", "broadcast_to") and tuple(op.operands[0].shape) == tuple(r.shape):
+                rep = op.operands[0]
+            elif op.name == "reshape" and op.operands[0].producer is not None and op.operands[0].producer.name == "reshape":
+                # reshape(reshape(x)) -> reshape(x)
+                src = op.operands[0].producer.operands[0]
+                op.operands[0].users.remove(op)
+                op.operands[0] = src
+                src.users.append(op)
+                changed = True
+                continue
+            elif op.name == "transpose" and tuple(op.attrs["perms"]) == tuple(range(r.rank)):
+                rep = op.operands[0]
+            elif op.name in ("mul", "div") and _is_const(_through_broadcast(op.operands[1]), 1.0) and \
+                    tuple(op.operands[0].shape) == tuple(r.shape) and op.operands[0].dtype == r.dtype:
+                rep = op.operands[0]
+            elif op.name == "mul" and _is_const(_through_broadcast(op.operands[0]), 1.0) and \
+                    tuple(op.operands[1].shape) == tuple(r.shape) and op.operands[1].dtype == r.dtype:
+                rep = op.operands[1]
+            elif op.name in ("add", "sub") and _is_const(_through_broadcast(op.operands[1]), 0.0) and \
+                    tuple(op.operands[0].shape) == tuple(r.shape) and op.operands[0].dtype == r.dtype:
+                rep = op.operands[0]
+            if rep is not None:
+                g.replace_all_uses(r, rep)
+                g.erase(op)
+                changed = True
+        g.dead_code_eliminate()
+    return g
+
+
+def decompose_batch_norm(g):
+    """scale * (input - mean) / sqrt(var + eps) + bias with per-channel reshape + broadcast_to."""
+    for op in list(g.ops):
+        if op.name != "batch_norm_inference":
+            continue
+        x, scale, bias, mean, var = op.operands
+        idx = g.ops.index(op)
+        tail = g.ops[idx:]
+        del g.ops[idx:]
+        feature = op.attrs.get("feature_index", 1)
+        eps = g.constant(op.attrs["epsilon"], var.dtype)
+        fined = g.add_op("add", [var, eps])
+        stddev = g.add_op("sqrt", [fined])
+        aligned = tuple(x.shape[d] if d == feature else 1 for d in range(x.rank))
+
+        def expand(v):
+            r = g.add_op("reshape", [v], {"shape": aligned}, shapes=[aligned], dtypes=[v.dtype])
+            return g.add_op("broadcast_to", [r], {"shape": tuple(x.shape), "cast_dims": tuple(range(x.rank))})
+
+        m, s, b, sd = expand(mean), expand(scale), expand(bias), expand(stddev)
+        res = g.add_op("sub", [x, m])
+        res = g.add_op("mul", [res, s])
+        res = g.add_op("div", [res, sd])
+        res = g.add_op("add", [res, b])
+        g.ops += [t for t in tail if t is not op]
+        g.replace_all_uses(op.results[0], res)
+        for o in op.operands:
+            if op in o.users:
+                o.users.remove(op)
+    return g
+
+
+def _strip_keepdim(v, full_shape):
+    """v is (reduce result) possibly followed by reshape (keepdim) and broadcast_to back to full_shape."""
+    chain = []
+    while v.producer is not None and v.producer.name in ("reshape", "broadcast_to"):
+        chain.append(v.producer)
+        v = v.producer.operands[0]
+    return v, chain
+
+
+def fuse_softmax(g):
+    for op in list(g.ops):
+        if op.name != "div" or op not in g.ops:
+            continue
+        e, denom = op.operands
+        if e.producer is None or e.producer.name != "exp":
+            continue
+        s, _ = _strip_keepdim(denom, e.shape)
+        if s.producer is None or s.producer.name != "reduce_sum" or s.producer.operands[0] is not e:
+            continue
+        rank = e.rank
+        if tuple(a % rank for a in s.producer.attrs["axis"]) != (rank - 1,):
+            continue
+        sub = e.producer.operands[0].producer
+        if sub is None or sub.name != "sub":
+            continue
+        x, mx = sub.operands
+        m, _ = _strip_keepdim(mx, x.shape)
+        if m.producer is None or m.producer.name != "reduce_max" or m.producer.operands[0] is not x:
+            continue
+        if tuple(a % rank for a in m.producer.attrs["axis"]) != (rank - 1,):
+            continue
+        if tuple(x.shape) != tuple(op.results[0].shape):
+            continue
+        # every intermediate must be private to the pattern
+        if len(e.users) != 2 or len(sub.results[0].users) != 1 or len(x.users) < 2:
+            continue
+        idx = g.ops.index(op)
+        tail = g.ops[idx:]
+        del g.ops[idx:]
+        y = g.add_op("softmax", [x], {"axis": rank - 1})
+        g.ops += tail
+        g.replace_all_uses(op.results[0], y)
+        g.dead_code_eliminate()
+    return g
+
+
+def run_llh_pipeline(g):
+    """Order follows the reference's pipeline (src/Pipeline/TransformPipeline.cpp:103-128):
+    legalise/remove-redundant, decompose, canonicalise."""
+    canonicalize(g)
+    decompose_batch_norm(g)
+    fuse_softmax(g)
+    canonicalize(g)
+    return g
