@@ -1,0 +1,61 @@
+"""Ahead-of-time entry: compile a whole torch module into ONE engine with symbolic extents.
+
+torch.compile guards re-specialise extents 0 and 1, so a batch-1 call would get a plan of its own.
+`compile_module` exports the module once (torch.export with the given dynamic dims), runs the
+same decompositions, importer and LLH pipeline as the torch.compile backend and returns a callable
+whose single plan serves every value of the symbolic dims, batch 1 included.  Every node must be
+translatable: there is no eager fallback on this entry.
+"""
+import torch
+from torch._decomp import get_decompositions
+
+from ..executor.engine import Torch_ExecutionEngine
+from ..importer.fx_importer import torch_translate_to_llh_graph
+from ..llh.passes import run_llh_pipeline
+from .torch_compile_config import LLC_DECOMPOSITIONS
+
+
+class CompiledModule:
+    def __init__(self, engine, lifted, n_user):
+        self.engine, self.lifted, self.n_user = engine, lifted, n_user
+
+    def __call__(self, *args):
+        if len(args) != self.n_user:
+            raise ValueError("expected %d inputs, got %d" % (self.n_user, len(args)))
+        out = self.engine.run(*self.lifted, *args)
+        # export always returns a tuple; a single result is handed back bare, like the module would
+        if isinstance(out, (list, tuple)) and len(out) == 1:
+            return out[0]
+        return out
+
+
+def compile_module(model, example_args, dynamic_shapes=None, verbose=False):
+    model = model.eval()
+    with torch.no_grad():
+        ep = torch.export.export(model, tuple(example_args), dynamic_shapes=dynamic_shapes)
+        # export keeps composite ops (layer_norm, linear, softmax.int ...) that AOT-autograd would already
+        # have taken apart: start from the core-ATen table, then apply the backend's own set on top
+        table = torch.export.default_decompositions()
+        for k, v in get_decompositions(LLC_DECOMPOSITIONS).items():
+            table[k] = v
+        ep = ep.run_decompositions(table)
+    gm = ep.graph_module
+    sig = ep.graph_signature
+    state = dict(ep.state_dict)
+    state.update(getattr(ep, "constants", {}) or {})
+    lifted = []
+    n_user = 0
+    for spec in sig.input_specs:
+        kind = spec.kind.name
+        if kind == "USER_INPUT":
+            n_user += 1
+        else:
+            t = state[spec.target]
+            lifted.append(t.detach() if isinstance(t, torch.Tensor) else t)
+    if any(s.kind.name != "USER_INPUT" for s in sig.input_specs[len(lifted):]):
+        raise NotImplementedError("lifted inputs must precede user inputs")
+    graph = torch_translate_to_llh_graph(gm)
+    run_llh_pipeline(graph)
+    if verbose:
+        print(graph.dump())
+    return CompiledModule(Torch_ExecutionEngine(graph), lifted, n_user)

@@ -34,6 +34,9 @@ LLC_DECOMPOSITIONS = {
     aten.linear,
     aten.matmul,
     aten.t,
+    # the GPU dispatch of eval-mode batch norm; both decompose to aten.native_batch_norm
+    aten.miopen_batch_norm,
+    aten.cudnn_batch_norm,
 }
 LLC_DECOMPOSITIONS.discard(aten.t)  # aten.t is translated directly (llh.transpose perms [1,0])
 

@@ -397,6 +397,10 @@ class Torch_ExecutionEngine(ExecutionEngine):
         if len(inputs) != len(g.inputs):
             raise ValueError("expected %d tensors, got %d" % (len(g.inputs), len(inputs)))
         env = self.bind_symbols(args, inputs)
+        for v, t in zip(g.inputs, inputs):
+            want = _concrete(v.shape, env)
+            if tuple(t.shape) != want or t.dtype != v.dtype:
+                raise ValueError("input %s: expected %s %s, got %s %s" % (v.name, want, v.dtype, tuple(t.shape), t.dtype))
         device = None
         for t in inputs:
             if not t.is_cuda:
@@ -404,10 +408,6 @@ class Torch_ExecutionEngine(ExecutionEngine):
             device = t.device
         if device is None:
             device = torch.device("cuda", torch.cuda.current_device())
-        for v, t in zip(g.inputs, inputs):
-            want = _concrete(v.shape, env)
-            if tuple(t.shape) != want or t.dtype != v.dtype:
-                raise ValueError("input %s: expected %s %s, got %s %s" % (v.name, want, v.dtype, tuple(t.shape), t.dtype))
         key = (tuple(sorted(env.items())), tuple((tuple(t.shape), tuple(t.stride())) for t in inputs), device.index)
         inst = self.instances.get(key)
         if inst is None:

@@ -102,6 +102,8 @@ class Planner:
         absorbed, reshaped, last = [], False, op
         while len(v.users) == 1 and id(v) not in self.outputs:
             u = v.users[0]
+            if id(u) in self.absorbed:
+                break  # already the epilogue of an earlier contraction (e.g. the other branch of a residual add)
             if u.name == "reshape" and epi["act"] is None:
                 # a reshape of the contiguous result keeps the linear element order
                 nxt = u.results[0]

@@ -404,6 +404,25 @@ def _batch_norm(ctx, node):
     return (y, None, None)
 
 
+def _bn_eval_only(node):
+    return node.args[5] is False
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_batch_norm.default, aten._native_batch_norm_legit.default,
+                                   aten.miopen_batch_norm.default, aten.cudnn_batch_norm.default, check=_bn_eval_only)
+def _batch_norm_native(ctx, node):
+    """The batch-norm entry points a GPU module dispatches to in eval mode; all share the signature
+    (input, weight, bias, running_mean, running_var, training=False, momentum, eps)."""
+    x, w, b, mean, var, training, momentum, eps = node.args
+    xv = ctx.val(x)
+    c = xv.shape[1]
+    wv = ctx.val(w) if w is not None else _ones_like_channels(ctx, c, xv.dtype, 1.0)
+    bv = ctx.val(b) if b is not None else _ones_like_channels(ctx, c, xv.dtype, 0.0)
+    y = ctx.g.add_op("batch_norm_inference", [xv, wv, bv, ctx.val(mean), ctx.val(var)],
+                     {"epsilon": float(eps), "momentum": float(momentum), "feature_index": 1})
+    return (y, None, None)
+
+
 def _ones_like_channels(ctx, c, dtype, value):
     k = ctx.g.constant(value, dtype)
     return ctx.g.add_op("broadcast_to", [k], {"shape": (c,), "cast_dims": (0,)})

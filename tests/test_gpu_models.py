@@ -1,0 +1,167 @@
+"""The five benchmark configurations end to end: torch module -> (torch.compile backend | export
+entry) -> LLH graph -> kernel plan -> HIP kernels, compared with torch eager on the CPU, which is
+the comparator of the reference's own python tests (llcompiler/test_models/utility.py:18-28), and for
+the MLP also with the C oracle.  Tolerances: fp32 rtol 1e-4 / atol 1e-5; bf16 rtol 2e-2."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from tests.util import BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+
+
+def _compile(model, dynamic=False):
+    from llcompiler_amd import LLCompiler
+    torch._dynamo.reset()
+    comp = LLCompiler(mode="inference", target="gfx950", pipeline="hip")
+    return torch.compile(copy.deepcopy(model).eval().cuda(), backend=comp, dynamic=dynamic, fullgraph=True), comp
+
+
+def test_config1_mlp(oracle):
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    m = MLP().eval()
+    (x,) = make_mlp_inputs()
+    with torch.no_grad():
+        want = m(x)
+        opt, comp = _compile(m)
+        got = opt(x.cuda())
+        again = opt(x.cuda())
+    assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "mlp vs torch eager")
+    np.testing.assert_array_equal(again.cpu().numpy(), got.cpu().numpy())
+    # the same network spelt with the C oracle's primitives
+    w1, b1, w2, b2 = (p.detach().numpy() for p in (m.fc1.weight, m.fc1.bias, m.fc2.weight, m.fc2.bias))
+    h = oracle.unary("relu", oracle.matmul(x.numpy(), np.ascontiguousarray(w1.T)) + b1)
+    ref = oracle.matmul(h, np.ascontiguousarray(w2.T)) + b2
+    assert_close(got.cpu().numpy(), ref, F32_RTOL, F32_ATOL, "mlp vs C oracle")
+    # everything was compiled: one engine, two contraction kernels with fused bias (+relu)
+    assert len(comp.engines) == 1
+    kinds = [s.kind for s in comp.engines[0].steps if s.kind != "view"]
+    assert kinds == ["matmul", "matmul"]
+
+
+@pytest.mark.parametrize("batch,size", [(2, 64), (16, 224)])
+def test_config3_resnet18(batch, size):
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval()
+    (x,) = make_resnet_inputs(batch, size)
+    with torch.no_grad():
+        want = m(x)
+        opt, comp = _compile(m)
+        got = opt(x.cuda())
+    assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "resnet18 %dx%d" % (batch, size))
+    kinds = [s.kind for s in comp.engines[0].steps if s.kind != "view"]
+    # 20 convolutions with bias / relu / residual fused, one max-pool, one average pool, the FC matmul
+    assert kinds.count("conv") == 20 and kinds.count("ew") == 0 and kinds[-2:] == ["avg_pool", "matmul"]
+
+
+def test_config4_encoder_block_bf16_symbolic_batch():
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    enc = EncoderBlock().eval().to(torch.bfloat16)
+    ref = copy.deepcopy(enc).float()  # the bf16-rounded weights, fp32 arithmetic
+    (x8,) = make_encoder_inputs(8, 512, dtype=torch.bfloat16)
+    cm = compile_module(copy.deepcopy(enc).cuda(), (x8.cuda(),), dynamic_shapes=({0: torch.export.Dim("batch")},))
+    with torch.no_grad():
+        for B in (8, 1, 32):
+            (x,) = make_encoder_inputs(B, 512, seed=B, dtype=torch.bfloat16)
+            got = cm(x.cuda())
+            assert got.dtype == torch.bfloat16 and got.shape == (B, 512, 768)
+            assert_close(got.float().cpu().numpy(), ref(x.float()).numpy(), BF16_RTOL, 2e-2, "encoder block bf16 B=%d" % B)
+    # one plan, one instance per batch size
+    assert len(cm.engine.instances) == 3
+
+
+def test_config5_bert_f32_symbolic_seq():
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import BertEncoder, make_bert_inputs
+    bert = BertEncoder().eval()
+    ex = tuple(t.cuda() for t in make_bert_inputs(8, 128))
+    seq = torch.export.Dim("seq")
+    cm = compile_module(copy.deepcopy(bert).cuda(), ex, dynamic_shapes=({1: seq}, {3: seq}))
+    with torch.no_grad():
+        for S in (128, 256, 512):
+            x, mask = make_bert_inputs(8, S, seed=S)
+            got = cm(x.cuda(), mask.cuda())
+            assert_close(got.cpu().numpy(), bert(x, mask).numpy(), F32_RTOL, F32_ATOL, "bert f32 S=%d" % S)
+    assert len(cm.engine.instances) == 3
+
+
+def test_dynamic_torch_compile_reuses_one_engine():
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()
+    with torch.no_grad():
+        opt, comp = _compile(enc, dynamic=True)
+        for B, S in [(2, 8), (3, 16), (5, 24)]:
+            (x,) = make_encoder_inputs(B, S, 64, seed=B)
+            assert_close(opt(x.cuda()).cpu().numpy(), enc(x).numpy(), F32_RTOL, F32_ATOL, "dynamic %dx%d" % (B, S))
+    assert len(comp.engines) <= 2  # dynamo may compile a static graph first, then one dynamic graph
+
+
+OP_MODELS = ["Add", "Sub", "Mul", "Div", "Abs", "Relu", "ElewiseFusion1", "ReduceFusion1", "Transpose", "Slice", "Extract",
+             "Softmax", "Gelu", "LayerNorm", "BatchNorm2D_Inference", "Conv2D_NCHW_FCHW", "MaxPool2D"]
+
+
+@pytest.mark.parametrize("name", OP_MODELS)
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_op_models_static_and_dynamic(name, dynamic):
+    """The reference's per-op python tests: a tiny module, eager vs compiled, static and dynamic
+    (test/python/ops/*.py via check_model, utility.py:79-138); inference mode."""
+    import llcompiler_amd.test_models as tm
+    gen = torch.Generator().manual_seed(7)
+    shapes = {"LayerNorm": (3, 7, 96), "BatchNorm2D_Inference": (3, 3, 24, 24), "Conv2D_NCHW_FCHW": (3, 3, 24, 24),
+              "MaxPool2D": (3, 3, 24, 24), "Slice": (4, 5, 9), "Extract": (4, 6, 5), "Transpose": (2, 6, 5, 8)}
+    x = torch.randn(shapes.get(name, (3, 3, 24, 24)), generator=gen)
+    m = getattr(tm, name)().eval()
+    with torch.no_grad():
+        want = m(x)
+        opt, comp = _compile(m, dynamic=dynamic)
+        got = opt(x.cuda())
+    assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, name)
+    assert comp.engines, "nothing was compiled for %s" % name
+
+
+def test_two_input_op_models():
+    import llcompiler_amd.test_models as tm
+    gen = torch.Generator().manual_seed(8)
+    with torch.no_grad():
+        a, b = torch.randn(3, 3, generator=gen), torch.randn(3, 3, generator=gen)
+        opt, _ = _compile(tm.Matmul())
+        assert_close(opt(a.cuda(), b.cuda()).cpu().numpy(), (a @ b).numpy(), F32_RTOL, F32_ATOL, "matmul 3x3")
+        x, y = torch.randn(3, 224, 112, generator=gen), torch.randn(3, 224, 112, generator=gen)
+        opt, _ = _compile(tm.BatchMatmul())
+        assert_close(opt(x.cuda(), y.cuda()).cpu().numpy(), torch.bmm(x, y.transpose(-1, -2)).numpy(), F32_RTOL, 2e-5, "bmm")
+        p, q = torch.randn(1000, 224, generator=gen), torch.randn(1000, 224, generator=gen)
+        opt, _ = _compile(tm.Where())
+        assert_close(opt(p.cuda(), q.cuda()).cpu().numpy(), torch.where(p > q, p, q * 2).numpy(), 0, 0, "where")
+        lin = tm.Linear(1000).eval()
+        z = torch.randn(10, 1000, generator=gen)
+        opt, _ = _compile(lin)
+        assert_close(opt(z.cuda()).cpu().numpy(), lin(z).numpy(), F32_RTOL, F32_ATOL, "linear")
+        emb = tm.Embedding().eval()
+        idx = torch.randint(0, 50, (4, 9), generator=gen)
+        opt, _ = _compile(emb)
+        assert_close(opt(idx.cuda()).cpu().numpy(), emb(idx).numpy(), 0, 0, "embedding")
+
+
+def test_unsupported_nodes_fall_back_to_eager():
+    """The reference's rule: what the partitioner does not claim runs in torch eager
+    (llcompiler/compiler/torch_compile_config.py:94-98)."""
+    class M(torch.nn.Module):
+        def forward(self, x):
+            return torch.cumsum(torch.relu(x) + 1, dim=-1) * 2
+
+    x = torch.randn(5, 33, generator=torch.Generator().manual_seed(9))
+    with torch.no_grad():
+        opt, comp = _compile(M())
+        got = opt(x.cuda())
+    assert_close(got.cpu().numpy(), (torch.cumsum(torch.relu(x) + 1, -1) * 2).numpy(), F32_RTOL, F32_ATOL, "fallback")
+    assert len(comp.engines) == 2  # relu+1 before the cumsum, *2 after it
