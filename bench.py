@@ -48,35 +48,47 @@ class Case:
         self.calls[i % self.sets].launch()
 
 
-def build_cases(ops, device):
+class _Cases(list):
+    """Collects the suite; with a filter only the named cases are built (their operands allocated)."""
+
+    def __init__(self, only):
+        super().__init__()
+        self.only = only
+
+    def add(self, name, dtype_name, *rest):
+        if not self.only or ("%s_%s" % (name, dtype_name)) in self.only:
+            self.append(Case(name, dtype_name, *rest))
+
+
+def build_cases(ops, device, only=()):
     gen = torch.Generator().manual_seed(0)
-    cases = []
+    cases = _Cases(list(only))
     for dt_name, dt, es in (("f32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
         M = N = K = 2048
-        cases.append(Case("matmul", dt_name, "mfma", 2.0 * M * N * K, (M * K + K * N + M * N) * es,
+        cases.add("matmul", dt_name, "mfma", 2.0 * M * N * K, (M * K + K * N + M * N) * es,
                           lambda: (_uniform((M, K), dt, gen, device), _uniform((K, N), dt, gen, device),
                                    torch.empty((M, N), dtype=dt, device=device)),
-                          lambda a, b, o: ops.matmul(a, b, out=o, defer=True), 1))
+                          lambda a, b, o: ops.matmul(a, b, out=o, defer=True), 1)
         B, m, k, n = 32, 512, 64, 512
         nbytes = (B * m * k + B * k * n + B * m * n) * es
-        cases.append(Case("batch_matmul", dt_name, "hbm", 2.0 * B * m * n * k, nbytes,
+        cases.add("batch_matmul", dt_name, "hbm", 2.0 * B * m * n * k, nbytes,
                           lambda: (_uniform((B, m, k), dt, gen, device), _uniform((B, k, n), dt, gen, device),
                                    torch.empty((B, m, n), dtype=dt, device=device)),
-                          lambda a, b, o: ops.batch_matmul(a, b, out=o, defer=True), max(1, int(1.2e9 // nbytes))))
+                          lambda a, b, o: ops.batch_matmul(a, b, out=o, defer=True), max(1, int(1.2e9 // nbytes)))
         shape = (64, 1024, 1024)
         numel = 64 * 1024 * 1024
         prog = ops.make_program([("add", "r0", "in0", "in1"), ("relu", "r0", "r0")], "r0")
-        cases.append(Case("add_relu", dt_name, "hbm", 0.0, 3 * numel * es,
+        cases.add("add_relu", dt_name, "hbm", 0.0, 3 * numel * es,
                           lambda: (_uniform(shape, dt, gen, device), _uniform(shape, dt, gen, device),
                                    torch.empty(shape, dtype=dt, device=device)),
-                          lambda a, b, o, prog=prog, shape=shape, dt=dt: ops.elementwise(prog, [a, b], shape, dt, out=o, defer=True), 2))
-        cases.append(Case("softmax", dt_name, "hbm", 0.0, 2 * 4096 * 4096 * es,
+                          lambda a, b, o, prog=prog, shape=shape, dt=dt: ops.elementwise(prog, [a, b], shape, dt, out=o, defer=True), 2)
+        cases.add("softmax", dt_name, "hbm", 0.0, 2 * 4096 * 4096 * es,
                           lambda: (_uniform((4096, 4096), dt, gen, device), torch.empty((4096, 4096), dtype=dt, device=device)),
-                          lambda x, o: ops.softmax(x, out=o, defer=True), 8))
-        cases.append(Case("layernorm", dt_name, "hbm", 0.0, (2 * 8192 * 1024 + 2 * 1024) * es,
+                          lambda x, o: ops.softmax(x, out=o, defer=True), 8)
+        cases.add("layernorm", dt_name, "hbm", 0.0, (2 * 8192 * 1024 + 2 * 1024) * es,
                           lambda: (_uniform((8192, 1024), dt, gen, device), torch.ones(1024, dtype=dt, device=device),
                                    torch.zeros(1024, dtype=dt, device=device), torch.empty((8192, 1024), dtype=dt, device=device)),
-                          lambda x, g, b, o: ops.layer_norm(x, g, b, 1e-5, out=o, defer=True), 16))
+                          lambda x, g, b, o: ops.layer_norm(x, g, b, 1e-5, out=o, defer=True), 16)
     return cases
 
 
@@ -147,6 +159,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
+                    "these cases, for profiling one kernel at a time; the JSON line then describes that subset")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -154,7 +168,8 @@ def main():
         sys.exit("bench.py needs a GPU; there is no CPU fallback")
     from llcompiler_amd import ops
     device = torch.device("cuda", 0)
-    cases = build_cases(ops, device)
+    only = [n for n in args.only.split(",") if n]
+    cases = build_cases(ops, device, only)
 
     def step(i):
         for c in cases:

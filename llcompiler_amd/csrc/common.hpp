@@ -70,12 +70,10 @@ int check_launch(const char* kernel);
 
 // ---- device helpers ----
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
-// round to nearest even; NaN stays a quiet NaN
+// round to nearest even, NaN stays NaN: gfx950 converts in hardware (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const __bf16 b = static_cast<__bf16>(f);
+  return __builtin_bit_cast(uint16_t, b);
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }

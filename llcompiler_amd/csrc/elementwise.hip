@@ -1,15 +1,20 @@
 // Fused elementwise chains: one launch evaluates a whole chain of LLH elementwise ops.
 //
-// The chain arrives as a tiny register program (llc_ew_program).  Every lane owns E = VEC*U
-// consecutive-in-VEC output elements, loads all chain inputs first (16-byte vector loads, U of
-// them in flight per input), then runs the program on registers and stores once.  Program control
-// flow is uniform across the wave, so instruction decode runs on the scalar unit; the kernel is
-// bound by HBM traffic: bytes moved = each distinct input once + the output once.
+// The chain arrives as a tiny register program (llc_ew_program).  Every lane owns ONE vector of VEC
+// consecutive output elements (16 bytes of the output type), loads that vector of every chain input
+// first, runs the program on registers and stores once.  The grid covers the output exactly (one
+// vector per lane, no grid-stride loop): on this part many small waves keep more memory requests
+// in flight than few looping ones.  Large streams use non-temporal loads and stores, which is worth
+// ~10% of HBM bandwidth for data that is touched once.  Program control flow is uniform across the
+// wave, so instruction decode runs on the scalar unit; the kernel is bound by HBM traffic: bytes
+// moved = each distinct input once + the output once.
 //
 // Broadcast operands (llh.broadcast_to folded into the consumer) are read with stride 0; the host
 // collapses the iteration space to at most four dims so that the common cases (same shape, bias
 // over the last dim, per-channel NCHW, attention mask) need at most three integer divisions per
 // vector.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace llc {
@@ -17,22 +22,105 @@ namespace {
 
 constexpr int kMaxDims = 4;
 
-struct EwKernelParams {
-  llc_ew_program prog;
-  const char* in[LLC_EW_MAX_INPUTS];
-  int32_t in_dtype[LLC_EW_MAX_INPUTS];
-  int32_t in_stride[LLC_EW_MAX_INPUTS][kMaxDims];  // elements; innermost is 0 or 1
-  char* out;
-  int32_t out_dtype;
-  int32_t n_inputs;
-  uint32_t dims[kMaxDims];  // collapsed output extents, dims[3] innermost
-  int32_t flat;             // 1: every input is either same-shape contiguous or a scalar
+// Everything a wave needs before it can issue its first global load sits in one contiguous block,
+// so that it arrives with one wide scalar load instead of a chain of dependent ones.
+struct EwHot {
   uint32_t n_vec;           // number of VEC-wide vectors in the output
+  int32_t flat;             // 1: every input is either same-shape contiguous or a scalar
+  int32_t streaming;        // 1: non-temporal accesses for the full-size operands
+  int32_t n_inputs;
+  int32_t out_dtype;
+  int32_t n_insts;
+  int32_t result;
+  int32_t integer;
+  uint32_t dims[kMaxDims];  // collapsed output extents, dims[3] innermost
+  int32_t in_dtype[LLC_EW_MAX_INPUTS];
+  int32_t in_inner[LLC_EW_MAX_INPUTS];  // innermost stride: 0 or 1 when VEC > 1
 };
+
+struct EwKernelParams {
+  EwHot hot;
+  char* out;
+  const char* in[LLC_EW_MAX_INPUTS];
+  int32_t in_stride[LLC_EW_MAX_INPUTS][kMaxDims];  // elements
+  llc_ew_inst insts[LLC_EW_MAX_INSTS];
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// N bytes, naturally aligned, optionally with the non-temporal hint
+template <int N>
+struct Bytes {
+  alignas(N >= 16 ? 16 : N) unsigned char b[N];
+};
+template <int N>
+__device__ __forceinline__ Bytes<N> ld_bytes(const char* p, bool nt) {
+  Bytes<N> r;
+  if constexpr (N >= 16) {
+#pragma unroll
+    for (int i = 0; i < N / 16; ++i) {
+      u32x4 v = nt ? __builtin_nontemporal_load((const u32x4*)p + i) : ((const u32x4*)p)[i];
+      __builtin_memcpy(r.b + 16 * i, &v, 16);
+    }
+  } else if constexpr (N == 8) {
+    u32x2 v = nt ? __builtin_nontemporal_load((const u32x2*)p) : *(const u32x2*)p;
+    __builtin_memcpy(r.b, &v, 8);
+  } else if constexpr (N == 4) {
+    uint32_t v = nt ? __builtin_nontemporal_load((const uint32_t*)p) : *(const uint32_t*)p;
+    __builtin_memcpy(r.b, &v, 4);
+  } else if constexpr (N == 2) {
+    uint16_t v = *(const uint16_t*)p;
+    __builtin_memcpy(r.b, &v, 2);
+  } else {
+    r.b[0] = *(const unsigned char*)p;
+  }
+  return r;
+}
+template <int N>
+__device__ __forceinline__ void st_bytes(char* p, const Bytes<N>& r, bool nt) {
+  if constexpr (N >= 16) {
+#pragma unroll
+    for (int i = 0; i < N / 16; ++i) {
+      u32x4 v;
+      __builtin_memcpy(&v, r.b + 16 * i, 16);
+      if (nt) __builtin_nontemporal_store(v, (u32x4*)p + i);
+      else ((u32x4*)p)[i] = v;
+    }
+  } else if constexpr (N == 8) {
+    u32x2 v;
+    __builtin_memcpy(&v, r.b, 8);
+    if (nt) __builtin_nontemporal_store(v, (u32x2*)p);
+    else *(u32x2*)p = v;
+  } else if constexpr (N == 4) {
+    uint32_t v;
+    __builtin_memcpy(&v, r.b, 4);
+    if (nt) __builtin_nontemporal_store(v, (uint32_t*)p);
+    else *(uint32_t*)p = v;
+  } else if constexpr (N == 2) {
+    uint16_t v;
+    __builtin_memcpy(&v, r.b, 2);
+    *(uint16_t*)p = v;
+  } else {
+    *(unsigned char*)p = r.b[0];
+  }
+}
+
+template <typename S, int VEC>
+__device__ __forceinline__ void ld_elems(const char* base, uint32_t off, bool nt, S* dst) {
+  Bytes<(int)sizeof(S) * VEC> r = ld_bytes<(int)sizeof(S) * VEC>(base + (size_t)off * sizeof(S), nt);
+  __builtin_memcpy(dst, r.b, sizeof(S) * VEC);
+}
+template <typename S, int VEC>
+__device__ __forceinline__ void st_elems(char* base, uint32_t off, bool nt, const S* src) {
+  Bytes<(int)sizeof(S) * VEC> r;
+  __builtin_memcpy(r.b, src, sizeof(S) * VEC);
+  st_bytes<(int)sizeof(S) * VEC>(base + (size_t)off * sizeof(S), r, nt);
+}
 
 // ---- typed loads: VEC consecutive elements (inner stride 1) or one element repeated (stride 0) ----
 template <int VEC, typename CT>
-__device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t off, int inner_stride, CT* dst) {
+__device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t off, int inner_stride, bool nt, CT* dst) {
   if (inner_stride == 0) {
     CT v;
     switch (dtype) {
@@ -49,88 +137,88 @@ __device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t o
   }
   switch (dtype) {
     case LLC_FLOAT32: {
-      struct alignas(4 * VEC) P { float v[VEC]; };
-      P p = *(const P*)(base + (size_t)off * 4);
+      float t[VEC];
+      ld_elems<float, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)p.v[j];
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     case LLC_BFLOAT16: {
-      struct alignas(2 * VEC) P { uint16_t v[VEC]; };
-      P p = *(const P*)(base + (size_t)off * 2);
+      uint16_t t[VEC];
+      ld_elems<uint16_t, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)bf16_bits_to_f32(p.v[j]);
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)bf16_bits_to_f32(t[j]);
     } break;
     case LLC_FLOAT16: {
-      struct alignas(2 * VEC) P { uint16_t v[VEC]; };
-      P p = *(const P*)(base + (size_t)off * 2);
+      uint16_t t[VEC];
+      ld_elems<uint16_t, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)f16_bits_to_f32(p.v[j]);
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)f16_bits_to_f32(t[j]);
     } break;
     case LLC_INT64: {
-      struct alignas(VEC >= 2 ? 16 : 8) P { int64_t v[VEC]; };
-      P p = *(const P*)(base + (size_t)off * 8);
+      int64_t t[VEC];
+      ld_elems<int64_t, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)p.v[j];
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     case LLC_INT32: {
-      struct alignas(4 * VEC) P { int32_t v[VEC]; };
-      P p = *(const P*)(base + (size_t)off * 4);
+      int32_t t[VEC];
+      ld_elems<int32_t, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)p.v[j];
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     default: {
-      struct alignas(VEC) P { uint8_t v[VEC]; };
-      P p = *(const P*)(base + (size_t)off);
+      uint8_t t[VEC];
+      ld_elems<uint8_t, VEC>(base, off, nt, t);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = (CT)p.v[j];
+      for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
   }
 }
 
 template <int VEC, typename CT>
-__device__ __forceinline__ void store_vec(char* base, int dtype, uint32_t off, const CT* src) {
+__device__ __forceinline__ void store_vec(char* base, int dtype, uint32_t off, bool nt, const CT* src) {
   switch (dtype) {
     case LLC_FLOAT32: {
-      struct alignas(4 * VEC) P { float v[VEC]; } p;
+      float t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = (float)src[j];
-      *(P*)(base + (size_t)off * 4) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = (float)src[j];
+      st_elems<float, VEC>(base, off, nt, t);
     } break;
     case LLC_BFLOAT16: {
-      struct alignas(2 * VEC) P { uint16_t v[VEC]; } p;
+      uint16_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_bf16_bits((float)src[j]);
-      *(P*)(base + (size_t)off * 2) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = f32_to_bf16_bits((float)src[j]);
+      st_elems<uint16_t, VEC>(base, off, nt, t);
     } break;
     case LLC_FLOAT16: {
-      struct alignas(2 * VEC) P { uint16_t v[VEC]; } p;
+      uint16_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_f16_bits((float)src[j]);
-      *(P*)(base + (size_t)off * 2) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = f32_to_f16_bits((float)src[j]);
+      st_elems<uint16_t, VEC>(base, off, nt, t);
     } break;
     case LLC_INT64: {
-      struct alignas(VEC >= 2 ? 16 : 8) P { int64_t v[VEC]; } p;
+      int64_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = (int64_t)src[j];
-      *(P*)(base + (size_t)off * 8) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = (int64_t)src[j];
+      st_elems<int64_t, VEC>(base, off, nt, t);
     } break;
     case LLC_INT32: {
-      struct alignas(4 * VEC) P { int32_t v[VEC]; } p;
+      int32_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = (int32_t)src[j];
-      *(P*)(base + (size_t)off * 4) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = (int32_t)src[j];
+      st_elems<int32_t, VEC>(base, off, nt, t);
     } break;
     case LLC_INT1: {
-      struct alignas(VEC) P { uint8_t v[VEC]; } p;
+      uint8_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = src[j] != (CT)0 ? 1 : 0;
-      *(P*)(base + (size_t)off) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = src[j] != (CT)0 ? 1 : 0;
+      st_elems<uint8_t, VEC>(base, off, nt, t);
     } break;
     default: {
-      struct alignas(VEC) P { int8_t v[VEC]; } p;
+      uint8_t t[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = (int8_t)src[j];
-      *(P*)(base + (size_t)off) = p;
+      for (int j = 0; j < VEC; ++j) t[j] = (uint8_t)(int8_t)src[j];
+      st_elems<uint8_t, VEC>(base, off, nt, t);
     } break;
   }
 }
@@ -158,7 +246,7 @@ __device__ __forceinline__ void apply_all(int op, const float* av, const float* 
     LLC_EW_CASE(LLC_EW_ABS, fabsf(a))
     LLC_EW_CASE(LLC_EW_SQRT, sqrtf(a))
     LLC_EW_CASE(LLC_EW_EXP, expf(a))
-    LLC_EW_CASE(LLC_EW_RELU, nanmax(a, 0.0f))
+    LLC_EW_CASE(LLC_EW_RELU, a < 0.0f ? 0.0f : a)  // NaN passes through, like torch.relu
     LLC_EW_CASE(LLC_EW_RSQRT, 1.0f / sqrtf(a))
     LLC_EW_CASE(LLC_EW_NEG, -a)
     LLC_EW_CASE(LLC_EW_GELU, gelu_exact(a))
@@ -258,66 +346,67 @@ __device__ __forceinline__ void fetch(const RegFile<E, CT>& f, int sel, CT imm, 
 template <int VEC, int U, int MAXIN, typename CT>
 __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
   constexpr int E = VEC * U;
-  const uint32_t nthreads = gridDim.x * blockDim.x;
-  for (uint32_t v0 = blockIdx.x * blockDim.x + threadIdx.x; v0 < p.n_vec; v0 += nthreads * U) {
-    RegFile<E, CT> f;
-    // ---- phase 1: issue every load ----
+  const EwHot h = p.hot;
+  // block b owns vectors [b*256*U, (b+1)*256*U); slot u of a lane is vector b*256*U + u*256 + lane
+  const uint32_t v0 = blockIdx.x * (256u * U) + threadIdx.x;
+  if (v0 >= h.n_vec) return;
+  RegFile<E, CT> f;
+  const bool nt = h.streaming != 0;
+  // ---- phase 1: issue every load ----
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t v = v0 + u * nthreads;
-      if (v < p.n_vec) {
-        const uint32_t e = v * VEC;
-        uint32_t idx0 = 0, idx1 = 0, idx2 = 0, idx3 = e;
-        if (!p.flat) {
-          uint32_t t = e;
-          idx3 = t % p.dims[3];
-          t /= p.dims[3];
-          idx2 = t % p.dims[2];
-          t /= p.dims[2];
-          idx1 = t % p.dims[1];
-          idx0 = t / p.dims[1];
-        }
+  for (int u = 0; u < U; ++u) {
+    const uint32_t v = v0 + u * 256u;
+    if (U > 1 && v >= h.n_vec) break;
+    const uint32_t e = v * VEC;
+    uint32_t idx0 = 0, idx1 = 0, idx2 = 0, idx3 = e;
+    if (!h.flat) {
+      uint32_t t = e;
+      idx3 = t % h.dims[3];
+      t /= h.dims[3];
+      idx2 = t % h.dims[2];
+      t /= h.dims[2];
+      idx1 = t % h.dims[1];
+      idx0 = t / h.dims[1];
+    }
 #define LLC_LOAD_INPUT(K, ARR)                                                                          \
-  if (K < MAXIN && K < p.n_inputs) {                                                                    \
-    uint32_t off = idx3 * (uint32_t)p.in_stride[K][3];                                                  \
-    if (!p.flat)                                                                                        \
+  if (K < MAXIN && K < h.n_inputs) {                                                                    \
+    uint32_t off = idx3 * (uint32_t)h.in_inner[K];                                                      \
+    if (!h.flat)                                                                                        \
       off += idx0 * (uint32_t)p.in_stride[K][0] + idx1 * (uint32_t)p.in_stride[K][1] +                  \
              idx2 * (uint32_t)p.in_stride[K][2];                                                        \
-    load_vec<VEC, CT>(p.in[K], p.in_dtype[K], off, p.in_stride[K][3], &ARR[u * VEC]);                   \
+    load_vec<VEC, CT>(p.in[K], h.in_dtype[K], off, h.in_inner[K], nt, &ARR[u * VEC]);                   \
   }
-        LLC_LOAD_INPUT(0, f.i0)
-        LLC_LOAD_INPUT(1, f.i1)
-        LLC_LOAD_INPUT(2, f.i2)
-        LLC_LOAD_INPUT(3, f.i3)
-        LLC_LOAD_INPUT(4, f.i4)
-        LLC_LOAD_INPUT(5, f.i5)
+    LLC_LOAD_INPUT(0, f.i0)
+    LLC_LOAD_INPUT(1, f.i1)
+    LLC_LOAD_INPUT(2, f.i2)
+    LLC_LOAD_INPUT(3, f.i3)
+    LLC_LOAD_INPUT(4, f.i4)
+    LLC_LOAD_INPUT(5, f.i5)
 #undef LLC_LOAD_INPUT
-      }
+  }
+  // ---- phase 2: run the chain on registers ----
+  for (int i = 0; i < h.n_insts; ++i) {
+    const llc_ew_inst inst = p.insts[i];
+    CT a[E], b[E], c[E], d[E];
+    const CT imm = (CT)inst.imm;
+    fetch<E, MAXIN, CT>(f, inst.a, imm, a);
+    if (inst.op >= LLC_EW_ADD) fetch<E, MAXIN, CT>(f, inst.b, imm, b);
+    if (inst.op == LLC_EW_WHERE) fetch<E, MAXIN, CT>(f, inst.c, imm, c);
+    apply_all<E>(inst.op, a, b, c, d);
+    switch (inst.dst) {
+      case 0: LLC_COPY(f.r0, d); break;
+      case 1: LLC_COPY(f.r1, d); break;
+      case 2: LLC_COPY(f.r2, d); break;
+      default: LLC_COPY(f.r3, d); break;
     }
-    // ---- phase 2: run the chain on registers ----
-    for (int i = 0; i < p.prog.n_insts; ++i) {
-      const llc_ew_inst inst = p.prog.insts[i];
-      CT a[E], b[E], c[E], d[E];
-      const CT imm = (CT)inst.imm;
-      fetch<E, MAXIN, CT>(f, inst.a, imm, a);
-      if (inst.op >= LLC_EW_ADD) fetch<E, MAXIN, CT>(f, inst.b, imm, b);
-      if (inst.op == LLC_EW_WHERE) fetch<E, MAXIN, CT>(f, inst.c, imm, c);
-      apply_all<E>(inst.op, a, b, c, d);
-      switch (inst.dst) {
-        case 0: LLC_COPY(f.r0, d); break;
-        case 1: LLC_COPY(f.r1, d); break;
-        case 2: LLC_COPY(f.r2, d); break;
-        default: LLC_COPY(f.r3, d); break;
-      }
-    }
-    // ---- phase 3: store ----
-    CT res[E];
-    fetch<E, MAXIN, CT>(f, p.prog.result, (CT)0, res);
+  }
+  // ---- phase 3: store ----
+  CT res[E];
+  fetch<E, MAXIN, CT>(f, h.result, (CT)0, res);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t v = v0 + u * nthreads;
-      if (v < p.n_vec) store_vec<VEC, CT>(p.out, p.out_dtype, v * VEC, res + u * VEC);
-    }
+  for (int u = 0; u < U; ++u) {
+    const uint32_t v = v0 + u * 256u;
+    if (v < h.n_vec) store_vec<VEC, CT>(p.out, h.out_dtype, v * VEC, nt, res + u * VEC);
   }
 }
 #undef LLC_COPY
@@ -355,8 +444,10 @@ int validate_program(const llc_ew_program* prog, size_t n_inputs) {
 }
 
 template <int VEC, int U, typename CT>
-void launch_vec(const EwKernelParams& p, uint32_t blocks, hipStream_t stream) {
-  if (p.n_inputs <= 2)
+void launch_vec(const EwKernelParams& p, hipStream_t stream) {
+  const uint32_t per_block = 256u * U;
+  const uint32_t blocks = (p.hot.n_vec + per_block - 1) / per_block;  // exact cover, no grid-stride loop
+  if (p.hot.n_inputs <= 2)
     hipLaunchKernelGGL((ew_kernel<VEC, U, 2, CT>), dim3(blocks), dim3(256), 0, stream, p);
   else
     hipLaunchKernelGGL((ew_kernel<VEC, U, LLC_EW_MAX_INPUTS, CT>), dim3(blocks), dim3(256), 0, stream, p);
@@ -364,21 +455,17 @@ void launch_vec(const EwKernelParams& p, uint32_t blocks, hipStream_t stream) {
 
 template <typename CT>
 int launch(const EwKernelParams& p, int vec, hipStream_t stream) {
-  // lanes own 8 elements (4 for int64): two 16-byte loads per fp32 input, one per bf16/f16 input
-  const int u = vec == 8 ? 1 : 2;
-  // enough blocks to fill 256 CUs several times over, capped so each thread still loops a little
-  uint64_t want = ((uint64_t)p.n_vec + (uint64_t)256 * u - 1) / ((uint64_t)256 * u);
-  uint32_t blocks = (uint32_t)(want < 1 ? 1 : (want > 256u * 32u ? 256u * 32u : want));
+  static const int u_env = getenv("LLC_EW_U") ? atoi(getenv("LLC_EW_U")) : 1;  // experiment hook; one vector per lane measured best
   if constexpr (sizeof(CT) == 4) {
     switch (vec) {
-      case 8: launch_vec<8, 1, CT>(p, blocks, stream); break;
-      case 4: launch_vec<4, 2, CT>(p, blocks, stream); break;
-      case 2: launch_vec<2, 2, CT>(p, blocks, stream); break;
-      default: launch_vec<1, 2, CT>(p, blocks, stream); break;
+      case 8: if (u_env == 2) launch_vec<8, 2, CT>(p, stream); else launch_vec<8, 1, CT>(p, stream); break;
+      case 4: if (u_env == 1) launch_vec<4, 1, CT>(p, stream); else if (u_env == 4) launch_vec<4, 4, CT>(p, stream); else launch_vec<4, 2, CT>(p, stream); break;
+      case 2: launch_vec<2, 2, CT>(p, stream); break;
+      default: launch_vec<1, 2, CT>(p, stream); break;
     }
   } else {
-    if (vec >= 2) launch_vec<2, 2, CT>(p, blocks, stream);
-    else launch_vec<1, 2, CT>(p, blocks, stream);
+    if (vec >= 2) launch_vec<2, 2, CT>(p, stream);
+    else launch_vec<1, 2, CT>(p, stream);
   }
   return check_launch("ew_kernel");
 }
@@ -444,20 +531,24 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
   if (nc > kMaxDims)
     return set_error(LLC_ERR_LAYOUT, "elementwise: broadcast pattern needs %d index dims (max %d)", nc, kMaxDims);
 
-  EwKernelParams p;
-  p.prog = *prog;
-  p.n_inputs = (int)n_inputs;
+  EwKernelParams p{};
+  for (int i = 0; i < prog->n_insts; ++i) p.insts[i] = prog->insts[i];
+  p.hot.n_insts = prog->n_insts;
+  p.hot.result = prog->result;
+  p.hot.integer = prog->integer;
+  p.hot.n_inputs = (int)n_inputs;
   p.out = o.ptr;
-  p.out_dtype = o.dtype;
-  for (int d = 0; d < kMaxDims; ++d) p.dims[d] = 1;
-  for (int d = 0; d < nc; ++d) p.dims[kMaxDims - nc + d] = (uint32_t)cdim[d];
+  p.hot.out_dtype = o.dtype;
+  for (int d = 0; d < kMaxDims; ++d) p.hot.dims[d] = 1;
+  for (int d = 0; d < nc; ++d) p.hot.dims[kMaxDims - nc + d] = (uint32_t)cdim[d];
   bool flat = nc == 1;
   // widest vector: 16 bytes of the output type, shrunk until every access stays aligned and inside a row
   int vec = prog->integer ? 2 : (o.esize() <= 2 ? 8 : 4);
+  if (getenv("LLC_EW_VEC16") && o.esize() <= 2) vec = atoi(getenv("LLC_EW_VEC16"));  // experiment hook
   auto aligned = [](const void* ptr, size_t bytes) { return ((uintptr_t)ptr % bytes) == 0; };
   for (size_t k = 0; k < n_inputs; ++k) {
     p.in[k] = in[k].ptr;
-    p.in_dtype[k] = in[k].dtype;
+    p.hot.in_dtype[k] = in[k].dtype;
     for (int d = 0; d < kMaxDims; ++d) p.in_stride[k][d] = 0;
     for (int d = 0; d < nc; ++d) {
       if (cst[k][d] >= (int64_t)1 << 31 || cst[k][d] < 0)
@@ -468,7 +559,7 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
     if (inner != 0 && inner != 1) vec = 1;  // strided innermost access: one element per load, index scaled by the stride
   }
   while (vec > 1) {
-    bool ok = (p.dims[kMaxDims - 1] % vec) == 0 && aligned(o.ptr, vec * o.esize());
+    bool ok = (p.hot.dims[kMaxDims - 1] % vec) == 0 && aligned(o.ptr, vec * o.esize());
     for (size_t k = 0; ok && k < n_inputs; ++k) {
       if (p.in_stride[k][kMaxDims - 1] == 0) continue;
       ok = aligned(in[k].ptr, vec * in[k].esize());
@@ -477,7 +568,10 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
     if (ok) break;
     vec >>= 1;
   }
-  p.flat = flat ? 1 : 0;
-  p.n_vec = (uint32_t)(total / vec);
+  for (size_t k = 0; k < n_inputs; ++k) p.hot.in_inner[k] = p.in_stride[k][kMaxDims - 1];
+  p.hot.flat = flat ? 1 : 0;
+  p.hot.n_vec = (uint32_t)(total / vec);
+  // streams far larger than the L2 are touched once: non-temporal accesses keep them out of the caches
+  p.hot.streaming = (int64_t)total * (int64_t)o.esize() >= ((int64_t)32 << 20) ? 1 : 0;
   return prog->integer ? launch<int64_t>(p, vec, as_stream(stream)) : launch<float>(p, vec, as_stream(stream));
 }

@@ -5,6 +5,8 @@
 // when a row spans several waves), and the result is written once.  Statistics are always fp32.
 // Algorithmic traffic is therefore read + write of the tensor, which is what these kernels are
 // measured against.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace llc {
@@ -23,44 +25,98 @@ struct RowParams {
   int32_t cols;
   float eps;
   float scale;  // kReduce: result multiplied by this (1/HW for average pooling)
+  int32_t streaming;  // non-temporal accesses: the tensor is far larger than the caches and touched once
 };
 
-template <int VEC>
-__device__ __forceinline__ void load_row_vec(const char* base, int dtype, int64_t off, float* dst) {
-  if (dtype == LLC_FLOAT32) {
-    struct alignas(4 * VEC) P { float v[VEC]; };
-    P p = *(const P*)(base + off * 4);
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) dst[j] = p.v[j];
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// VEC elements of the storage type as raw bytes (16 bytes when VEC > 1), optionally non-temporal
+template <int VEC, int ES>
+struct RowPack {
+  alignas(VEC * ES) unsigned char b[VEC * ES];
+};
+template <int VEC, int ES>
+__device__ __forceinline__ RowPack<VEC, ES> ld_pack(const char* p, bool nt) {
+  RowPack<VEC, ES> r;
+  if constexpr (VEC * ES == 16) {
+    u32x4 v = nt ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+    __builtin_memcpy(r.b, &v, 16);
+  } else if constexpr (VEC * ES == 4) {
+    uint32_t v = *(const uint32_t*)p;
+    __builtin_memcpy(r.b, &v, 4);
   } else {
-    struct alignas(2 * VEC) P { uint16_t v[VEC]; };
-    P p = *(const P*)(base + off * 2);
+    uint16_t v = *(const uint16_t*)p;
+    __builtin_memcpy(r.b, &v, 2);
+  }
+  return r;
+}
+template <int VEC, int ES>
+__device__ __forceinline__ void st_pack(char* p, const RowPack<VEC, ES>& r, bool nt) {
+  if constexpr (VEC * ES == 16) {
+    u32x4 v;
+    __builtin_memcpy(&v, r.b, 16);
+    if (nt) __builtin_nontemporal_store(v, (u32x4*)p);
+    else *(u32x4*)p = v;
+  } else if constexpr (VEC * ES == 4) {
+    uint32_t v;
+    __builtin_memcpy(&v, r.b, 4);
+    *(uint32_t*)p = v;
+  } else {
+    uint16_t v;
+    __builtin_memcpy(&v, r.b, 2);
+    *(uint16_t*)p = v;
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_row_vec(const char* base, int dtype, int64_t off, float* dst, bool nt = false) {
+  if (dtype == LLC_FLOAT32) {
+    // rows are read 4 wide (fp32) or 8 wide (16-bit types), i.e. 16 bytes, or element-wise; the width
+    // that does not belong to a storage type is never launched for it and is only remapped so that the
+    // run-time dtype switch compiles
+    constexpr int V = VEC == 8 ? 4 : VEC;
+    RowPack<V, 4> p = ld_pack<V, 4>(base + off * 4, nt);
+    float t[V];
+    __builtin_memcpy(t, p.b, sizeof(t));
+#pragma unroll
+    for (int j = 0; j < V; ++j) dst[j] = t[j];
+  } else {
+    constexpr int V = VEC == 4 ? 8 : VEC;  // 16-bit rows are never read 4 wide
+    RowPack<V, 2> p = ld_pack<V, 2>(base + off * 2, nt);
+    uint16_t t[V];
+    __builtin_memcpy(t, p.b, sizeof(t));
     if (dtype == LLC_BFLOAT16) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = bf16_bits_to_f32(p.v[j]);
+      for (int j = 0; j < (V < VEC ? V : VEC); ++j) dst[j] = bf16_bits_to_f32(t[j]);
     } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) dst[j] = f16_bits_to_f32(p.v[j]);
+      for (int j = 0; j < (V < VEC ? V : VEC); ++j) dst[j] = f16_bits_to_f32(t[j]);
     }
   }
 }
 template <int VEC>
-__device__ __forceinline__ void store_row_vec(char* base, int dtype, int64_t off, const float* src) {
+__device__ __forceinline__ void store_row_vec(char* base, int dtype, int64_t off, const float* src, bool nt = false) {
   if (dtype == LLC_FLOAT32) {
-    struct alignas(4 * VEC) P { float v[VEC]; } p;
+    constexpr int V = VEC == 8 ? 4 : VEC;
+    float t[V];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) p.v[j] = src[j];
-    *(P*)(base + off * 4) = p;
+    for (int j = 0; j < V; ++j) t[j] = src[j];
+    RowPack<V, 4> p;
+    __builtin_memcpy(p.b, t, sizeof(t));
+    st_pack<V, 4>(base + off * 4, p, nt);
   } else {
-    struct alignas(2 * VEC) P { uint16_t v[VEC]; } p;
+    constexpr int V = VEC == 4 ? 8 : VEC;
+    uint16_t t[V];
     if (dtype == LLC_BFLOAT16) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_bf16_bits(src[j]);
+      for (int j = 0; j < V; ++j) t[j] = f32_to_bf16_bits(src[j < VEC ? j : 0]);
     } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) p.v[j] = f32_to_f16_bits(src[j]);
+      for (int j = 0; j < V; ++j) t[j] = f32_to_f16_bits(src[j < VEC ? j : 0]);
     }
-    *(P*)(base + off * 2) = p;
+    RowPack<V, 2> p;
+    __builtin_memcpy(p.b, t, sizeof(t));
+    st_pack<V, 2>(base + off * 2, p, nt);
   }
 }
 
@@ -112,7 +168,7 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
   for (int it = 0; it < ITEMS; ++it) {
     const int col = (it * TPR + lane) * VEC;
     ok[it] = row_ok && col < p.cols;
-    if (ok[it]) load_row_vec<VEC>(p.x, p.dtype, base + col, v[it]);
+    if (ok[it]) load_row_vec<VEC>(p.x, p.dtype, base + col, v[it], p.streaming != 0);
     else {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[it][j] = fill;
@@ -143,7 +199,7 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
       if (ok[it]) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[it][j] *= inv;
-        store_row_vec<VEC>(p.y, p.dtype, base + (it * TPR + lane) * VEC, v[it]);
+        store_row_vec<VEC>(p.y, p.dtype, base + (it * TPR + lane) * VEC, v[it], p.streaming != 0);
       }
     }
   } else if constexpr (OP == kLayerNorm) {
@@ -179,7 +235,7 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
           if (p.beta) t += b[j];
           v[it][j] = t;
         }
-        store_row_vec<VEC>(p.y, p.dtype, base + col, v[it]);
+        store_row_vec<VEC>(p.y, p.dtype, base + col, v[it], p.streaming != 0);
       }
     }
   } else {
@@ -306,7 +362,8 @@ void launch_items(const RowParams& p, int items, hipStream_t s) {
     case 1: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 1>), dim3(blocks), dim3(256), 0, s, p); break;
     case 2: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 2>), dim3(blocks), dim3(256), 0, s, p); break;
     case 4: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 4>), dim3(blocks), dim3(256), 0, s, p); break;
-    default: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 8>), dim3(blocks), dim3(256), 0, s, p); break;
+    case 8: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 8>), dim3(blocks), dim3(256), 0, s, p); break;
+    default: hipLaunchKernelGGL((row_kernel<OP, VEC, TPR, 16>), dim3(blocks), dim3(256), 0, s, p); break;
   }
 }
 
@@ -328,6 +385,11 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
       }
     }
   if (best_cap < 0) return false;
+  if (const char* ft = getenv("LLC_ROW_TPR")) {  // experiment hook
+    int t = atoi(ft);
+    for (int i : {1, 2, 4, 8, 16})
+      if ((int64_t)t * i * VEC >= p.cols) { best_t = t; best_i = i; break; }
+  }
   if (best_t == 16) launch_items<OP, VEC, 16>(p, best_i, s);
   else if (best_t == 64) launch_items<OP, VEC, 64>(p, best_i, s);
   else launch_items<OP, VEC, 256>(p, best_i, s);
@@ -335,8 +397,10 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
 }
 
 template <int OP>
-int launch_rows(const RowParams& p, hipStream_t s) {
+int launch_rows(const RowParams& p0, hipStream_t s) {
+  RowParams p = p0;
   if (p.rows == 0 || p.cols == 0) return LLC_OK;
+  p.streaming = p.rows * (int64_t)p.cols * (p.dtype == LLC_FLOAT32 ? 4 : 2) >= ((int64_t)32 << 20) ? 1 : 0;
   if (p.rows > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "row kernel: %lld rows", (long long)p.rows);
   const int es = p.dtype == LLC_FLOAT32 ? 4 : 2;
   const int wide = 16 / es;
