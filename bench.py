@@ -89,6 +89,13 @@ def build_cases(ops, device, only=()):
                           lambda: (_uniform((8192, 1024), dt, gen, device), torch.ones(1024, dtype=dt, device=device),
                                    torch.zeros(1024, dtype=dt, device=device), torch.empty((8192, 1024), dtype=dt, device=device)),
                           lambda x, g, b, o: ops.layer_norm(x, g, b, 1e-5, out=o, defer=True), 16)
+    # not part of the suite: a plain device copy of known size, used to calibrate the profiler's
+    # FETCH_SIZE / WRITE_SIZE counters (bench.py --only copy_f32)
+    if "copy_f32" in cases.only:
+        n = 64 * 1024 * 1024
+        cases.add("copy", "f32", "hbm", 0.0, 2 * n * 4,
+                  lambda: (_uniform((n,), torch.float32, gen, device), torch.empty(n, dtype=torch.float32, device=device)),
+                  lambda x, o: ops.copy(x, out=o, defer=True), 2)
     return cases
 
 
