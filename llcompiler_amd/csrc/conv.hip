@@ -11,7 +11,7 @@
 // The im2col matrix is never materialised.  Each lane owns one pixel column of the tile and a run
 // of consecutive k; it walks (c, kh, kw) incrementally, gathers X with bounds checks (lanes of a
 // wave read consecutive pixels, so loads coalesce for stride 1) and writes its run k-contiguous
-// into the same padded LDS tile layout the matmul kernel uses.  Weights go through the shared
+// into the same swizzled LDS tile layout the matmul kernel uses.  Weights go through the shared
 // vector loader.  fp32 tensors use the fp32 MFMA, bf16/f16 the 16-bit MFMA; accumulation is fp32.
 #include "gemm_core.hpp"
 
@@ -88,14 +88,13 @@ struct Im2colLoader {
 
   __device__ __forceinline__ void store(char* lds) const {
     const int j = threadIdx.x % BN, kpart = threadIdx.x / BN;
-    char* dst = lds + j * kRowStride + kpart * KPT * (int)sizeof(T);
     constexpr int EPV = 16 / sizeof(T);
 #pragma unroll
     for (int q = 0; q < KPT / EPV; ++q) {
       struct alignas(16) Pack { T e[EPV]; } pk;
 #pragma unroll
       for (int e = 0; e < EPV; ++e) pk.e[e] = v[q * EPV + e];
-      *(Pack*)(dst + q * 16) = pk;
+      *(Pack*)(lds + lds_off(j, kpart * KPT * (int)sizeof(T) + q * 16)) = pk;
     }
   }
 };
@@ -143,9 +142,7 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
       la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
       lb.load(p, (kt + 1) * BK);
     }
-    const char* sa = smem + cur * kBufBytes + (wm * WTM + li) * kRowStride + lh * 16;
-    const char* sb = smem + cur * kBufBytes + kABytes + (wn * WTN + li) * kRowStride + lh * 16;
-    mma_tile<T, TM, TN>(sa, sb, acc);
+    mma_tile<T, TM, TN>(smem + cur * kBufBytes, wm * WTM + li, smem + cur * kBufBytes + kABytes, wn * WTN + li, lh, acc);
     if (kt + 1 < nk) {
       la.store(smem + (cur ^ 1) * kBufBytes);
       lb.store(smem + (cur ^ 1) * kBufBytes + kABytes);

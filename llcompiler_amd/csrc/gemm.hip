@@ -7,10 +7,11 @@
 // Accumulation is always fp32.
 //
 // Data path per workgroup (256 lanes = 4 waves in a 2x2 grid, macro tile BM x BN):
-//   HBM/L2 --16-byte global loads--> registers --> LDS tile [row][128 bytes of k], rows padded to
-//   144 bytes so that the 16-byte fragment reads of 16 consecutive rows land in distinct banks
-//   --> ds_read_b128 fragments --> MFMA.  Two LDS buffers: global loads for k-tile t+1 are issued
-//   before the MFMAs of tile t and written to the other buffer after them, one barrier per tile.
+//   HBM/L2 --16-byte global loads--> registers --> LDS tile [row][128 bytes of k] whose 16-byte
+//   chunks are XOR-swizzled by the row (no padding; fragment reads, row copies and transposing
+//   stores all spread over the banks) --> ds_read_b128 fragments --> MFMA.  Two LDS buffers and two
+//   register stages: global loads for k-tile t+2 are issued before the MFMAs of tile t, tile t+1 is
+//   written to the other buffer after them, one barrier per tile.
 // A fragment is "8 consecutive k of one row" for both operands.  Operands whose unit-stride dim is
 // k (row-major A; B given as [N,K], i.e. a transposed weight view) are copied as they are; a
 // row-major B (unit stride along n) is transposed in registers on its way to LDS.  Anything else
@@ -41,7 +42,7 @@ struct GemmParams {
   int32_t tiles_m, tiles_n;
 };
 
-template <typename T, int BM, int BN, int LA, int LB>
+template <typename T, int BM, int BN, int LA, int LB, bool FULL>
 __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   constexpr int BK = kRowBytes / sizeof(T);
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
@@ -69,30 +70,49 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  TileLoader<T, BM, LA> la;
-  TileLoader<T, BN, LB> lb;
+  // Two register stages: the global loads of k-tile t+2 are issued before the MFMAs of tile t, tile t+1
+  // (issued one iteration earlier) is written to the other LDS buffer after them.  The loop is unrolled
+  // by two so that the stage index is a compile-time constant (register arrays, not scratch).
+  TileLoader<T, BM, LA> la0, la1;
+  TileLoader<T, BN, LB> lb0, lb1;
   const int nk = (p.K + BK - 1) / BK;
-  la.load(A, m0, p.M, 0, p.K, p.a_sm, p.a_sk);
-  lb.load(B, n0, p.N, 0, p.K, p.b_sn, p.b_sk);
-  la.store(smem);
-  lb.store(smem + kABytes);
+  la0.template load<FULL>(A, m0, p.M, 0, p.K, p.a_sm, p.a_sk);
+  lb0.template load<FULL>(B, n0, p.N, 0, p.K, p.b_sn, p.b_sk);
+  if (nk > 1) {
+    la1.template load<FULL>(A, m0, p.M, BK, p.K, p.a_sm, p.a_sk);
+    lb1.template load<FULL>(B, n0, p.N, BK, p.K, p.b_sn, p.b_sk);
+  }
+  la0.store(smem);
+  lb0.store(smem + kABytes);
   __syncthreads();
 
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      la.load(A, m0, p.M, (kt + 1) * BK, p.K, p.a_sm, p.a_sk);
-      lb.load(B, n0, p.N, (kt + 1) * BK, p.K, p.b_sn, p.b_sk);
-    }
-    const char* sa = smem + cur * kBufBytes + (wm * WTM + li) * kRowStride + lh * 16;
-    const char* sb = smem + cur * kBufBytes + kABytes + (wn * WTN + li) * kRowStride + lh * 16;
-    mma_tile<T, TM, TN>(sa, sb, acc);
-    if (kt + 1 < nk) {
-      la.store(smem + (cur ^ 1) * kBufBytes);
-      lb.store(smem + (cur ^ 1) * kBufBytes + kABytes);
-    }
-    __syncthreads();
+#define LLC_GEMM_STEP(KT, CUR, LA2, LB2, LA1, LB1, GUARDED)                                                     \
+  {                                                                                                             \
+    /* LA2/LB2: stage that held tile KT (now in LDS) and receives tile KT+2; LA1/LB1 hold tile KT+1 */          \
+    if (!(GUARDED) || (KT) + 2 < nk) {                                                                          \
+      LA2.template load<FULL>(A, m0, p.M, ((KT) + 2) * BK, p.K, p.a_sm, p.a_sk);                                \
+      LB2.template load<FULL>(B, n0, p.N, ((KT) + 2) * BK, p.K, p.b_sn, p.b_sk);                                \
+    }                                                                                                           \
+    mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,            \
+                        wn * WTN + li, lh, acc);                                                                \
+    if (!(GUARDED) || (KT) + 1 < nk) {                                                                          \
+      LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
+      LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
+    }                                                                                                           \
+    __syncthreads();                                                                                            \
   }
+  // steady state: no control flow inside the body (every load and store is known to be needed), so the
+  // accumulators stay where the MFMAs leave them; the last up to three tiles run the guarded form
+  int kt = 0;
+  for (; kt + 3 < nk; kt += 2) {
+    LLC_GEMM_STEP(kt, 0, la0, lb0, la1, lb1, false)
+    LLC_GEMM_STEP(kt + 1, 1, la1, lb1, la0, lb0, false)
+  }
+  for (; kt < nk; kt += 2) {
+    LLC_GEMM_STEP(kt, 0, la0, lb0, la1, lb1, true)
+    if (kt + 1 < nk) LLC_GEMM_STEP(kt + 1, 1, la1, lb1, la0, lb0, true)
+  }
+#undef LLC_GEMM_STEP
 
   // ---- epilogue.  32x32 accumulator layout: register r of lane (li, lh) is row 8*(r/4) + 4*lh + r%4,
   //      column li: for fixed r, 32 lanes store 32 consecutive columns of one row. ----
@@ -101,14 +121,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
-    if (col >= p.N) continue;
+    if (!FULL && col >= p.N) continue;
     const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, col) : 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        if (row >= p.M) continue;
+        if (!FULL && row >= p.M) continue;
         epilogue_store<T>(C, (int64_t)row * p.N + col, acc[i][j][r], p.alpha, bv, res, p.act);
       }
     }
@@ -121,11 +141,13 @@ int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
-  static bool attr_set = false;  // per instantiation
-  auto kern = gemm_kernel<T, BM, BN, LA, LB>;
-  if (!attr_set) {
+  static bool attr_set[2] = {false, false};  // per instantiation
+  // every tile complete: the unguarded instantiation (no per-access branches in the main loop)
+  const bool full = p.M % BM == 0 && p.N % BN == 0 && p.K % (kRowBytes / (int)sizeof(T)) == 0;
+  auto kern = full ? gemm_kernel<T, BM, BN, LA, LB, true> : gemm_kernel<T, BM, BN, LA, LB, false>;
+  if (!attr_set[full]) {
     LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
+    attr_set[full] = true;
   }
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffff || batch > 65535) return set_error(LLC_ERR_TOO_LARGE, "matmul: grid too large");

@@ -13,10 +13,19 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 namespace gemm {
 
 constexpr int kRowBytes = 128;   // bytes of k per LDS tile row
-constexpr int kRowStride = 144;  // padded row pitch in LDS
+constexpr int kRowStride = 128;  // row pitch in LDS: unpadded, 16-byte chunks XOR-swizzled by the row
 constexpr int kXcds = 8;
 
 enum Loader { kLoadKVec = 0, kLoadRVec = 1, kLoadGeneric = 2 };
+
+// LDS tile layout: row r holds 128 bytes of k; its eight 16-byte chunks are stored at chunk index
+// c ^ swz(r), swz(r) = (r ^ (r >> 3)) & 7.  Fragment reads (lanes = consecutive rows, one chunk each),
+// the k-contiguous copy (8 lanes = one row) and the transposing store (lanes = rows 8 apart) all
+// spread over the banks, with no padding bytes.
+__device__ __forceinline__ int lds_swz(int r) { return (r ^ (r >> 3)) & 7; }
+__device__ __forceinline__ int lds_off(int r, int kbyte) {
+  return r * kRowStride + ((((kbyte >> 4) ^ lds_swz(r)) & 7) << 4) + (kbyte & 15);
+}
 
 template <typename T> struct Elem;
 template <> struct Elem<float> { static constexpr int kDtype = LLC_FLOAT32; };
@@ -60,7 +69,9 @@ struct TileLoader {
   u32x4_t v[MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * 4 : 1)];
   T g[MODE == kLoadGeneric ? kGenElems : 1];
 
-  // rows: valid row count of the operand; row0/k0: tile origin; s_r / s_k: element strides
+  // rows: valid row count of the operand; row0/k0: tile origin; s_r / s_k: element strides.
+  // FULL: the tile lies entirely inside the operand, so no access is guarded.
+  template <bool FULL = false>
   __device__ __forceinline__ void load(const T* base, int row0, int rows, int k0, int K, int64_t s_r, int64_t s_k) {
     const int tid = threadIdx.x;
     if constexpr (MODE == kLoadKVec) {
@@ -70,7 +81,7 @@ struct TileLoader {
         const int r = vid >> 3, kv = vid & 7;
         const int gr = row0 + r, gk = k0 + kv * EPV;
         u32x4_t z = {0, 0, 0, 0};
-        if ((kVecs % 256 == 0 || vid < kVecs) && gr < rows && gk < K) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
+        if ((kVecs % 256 == 0 || vid < kVecs) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
         v[i] = z;
       }
     } else if constexpr (MODE == kLoadRVec) {
@@ -83,7 +94,7 @@ struct TileLoader {
         for (int kk = 0; kk < 4; ++kk) {
           const int gk = k0 + kb * 4 + kk;
           u32x4_t z = {0, 0, 0, 0};
-          if ((kRBlocks % 256 == 0 || bid < kRBlocks) && gr < rows && gk < K) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
+          if ((kRBlocks % 256 == 0 || bid < kRBlocks) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
           v[i * 4 + kk] = z;
         }
       }
@@ -94,7 +105,7 @@ struct TileLoader {
         const int r = e / BK, k = e % BK;
         const int gr = row0 + r, gk = k0 + k;
         T z = static_cast<T>(0.0f);
-        if (gr < rows && gk < K) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
+        if (FULL || (gr < rows && gk < K)) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
         g[i] = z;
       }
     }
@@ -106,7 +117,7 @@ struct TileLoader {
 #pragma unroll
       for (int i = 0; i < kIters; ++i) {
         const int vid = i * 256 + tid;
-        if (kVecs % 256 == 0 || vid < kVecs) *(u32x4_t*)(lds + (vid >> 3) * kRowStride + (vid & 7) * 16) = v[i];
+        if (kVecs % 256 == 0 || vid < kVecs) *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = v[i];
       }
     } else if constexpr (MODE == kLoadRVec) {
 #pragma unroll
@@ -114,13 +125,13 @@ struct TileLoader {
         const int bid = i * 256 + tid;
         if (!(kRBlocks % 256 == 0 || bid < kRBlocks)) continue;
         const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
-        char* dst = lds + (rb * EPV) * kRowStride + kb * 4 * (int)sizeof(T);
+        const int row0 = rb * EPV, kbyte = kb * 4 * (int)sizeof(T);
         const u32x4_t r0 = v[i * 4 + 0], r1 = v[i * 4 + 1], r2 = v[i * 4 + 2], r3 = v[i * 4 + 3];
         if constexpr (sizeof(T) == 4) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             u32x4_t o = {r0[j], r1[j], r2[j], r3[j]};
-            *(u32x4_t*)(dst + j * kRowStride) = o;
+            *(u32x4_t*)(lds + lds_off(row0 + j, kbyte)) = o;
           }
         } else {
 #pragma unroll
@@ -130,7 +141,7 @@ struct TileLoader {
             uint2 o;
             o.x = __builtin_amdgcn_perm(r1[j >> 1], r0[j >> 1], sel);
             o.y = __builtin_amdgcn_perm(r3[j >> 1], r2[j >> 1], sel);
-            *(uint2*)(dst + j * kRowStride) = o;
+            *(uint2*)(lds + lds_off(row0 + j, kbyte)) = o;
           }
         }
       }
@@ -138,7 +149,7 @@ struct TileLoader {
 #pragma unroll
       for (int i = 0; i < kGenElems; ++i) {
         const int e = i * 256 + tid;
-        *(T*)(lds + (e / BK) * kRowStride + (e % BK) * (int)sizeof(T)) = g[i];
+        *(T*)(lds + lds_off(e / BK, (e % BK) * (int)sizeof(T))) = g[i];
       }
     }
   }
@@ -169,17 +180,30 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm,
   tn = in_group / gsize;
 }
 
-// MFMAs of one LDS tile pair for one wave: TM x TN fragments of 32x32, four 16-byte k-chunks pairs.
-// sa / sb point at this lane's first fragment row (+ lane-half chunk offset) inside the A / B tile.
+// MFMAs of one LDS tile pair for one wave: TM x TN fragments of 32x32, four steps of two 16-byte
+// k-chunks (lane half lh takes chunk 2s+lh).  ta / tb are the A / B tiles; arow / brow are this lane's
+// first fragment row in each (fragment i covers rows arow + 32 i).
 template <typename T, int TM, int TN>
-__device__ __forceinline__ void mma_tile(const char* sa, const char* sb, f32x16_t (&acc)[TM][TN]) {
+__device__ __forceinline__ void mma_tile(const char* ta, int arow, const char* tb, int brow, int lh,
+                                         f32x16_t (&acc)[TM][TN]) {
+  int abase[TM], aswz[TM], bbase[TN], bswz[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    abase[i] = (arow + i * 32) * kRowStride;
+    aswz[i] = lds_swz(arow + i * 32);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    bbase[j] = (brow + j * 32) * kRowStride;
+    bswz[j] = lds_swz(brow + j * 32);
+  }
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     u32x4_t fa[TM], fb[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[i] = *(const u32x4_t*)(sa + i * 32 * kRowStride + s * 32);
+    for (int i = 0; i < TM; ++i) fa[i] = *(const u32x4_t*)(ta + abase[i] + (((2 * s + lh) ^ aswz[i]) << 4));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[j] = *(const u32x4_t*)(sb + j * 32 * kRowStride + s * 32);
+    for (int j = 0; j < TN; ++j) fb[j] = *(const u32x4_t*)(tb + bbase[j] + (((2 * s + lh) ^ bswz[j]) << 4));
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
