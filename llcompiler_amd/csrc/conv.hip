@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  TileLoader<T, BM, LA> la;
+  TileLoader<T, BM, LA, 256> la;
   Im2colLoader<T, BN> lb;
   lb.init(p, g, n0);
   const int nk = (p.Kdim + BK - 1) / BK;

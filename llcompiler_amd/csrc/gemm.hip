@@ -21,7 +21,29 @@
 // XCDs by the hardware, so ids are first regrouped per XCD and then walked in column-grouped order,
 // which gives each XCD's L2 a compact patch of the output (few distinct A row-panels / B
 // column-panels).
+#include <cstdlib>
+
 #include "gemm_core.hpp"
+
+// experiment switches: drop one phase of the main loop to see what the others cost (results are then wrong)
+#ifndef LLC_DBG_LOAD
+#define LLC_DBG_LOAD 1
+#endif
+#ifndef LLC_DBG_MMA
+#define LLC_DBG_MMA 1
+#endif
+#ifndef LLC_DBG_STORE
+#define LLC_DBG_STORE 1
+#endif
+#ifndef LLC_DBG_DMA
+#define LLC_DBG_DMA 1
+#endif
+#ifndef LLC_DBG_READ
+#define LLC_DBG_READ 1
+#endif
+#ifndef LLC_DBG_EPI
+#define LLC_DBG_EPI 1
+#endif
 
 namespace llc {
 using namespace gemm;
@@ -42,10 +64,11 @@ struct GemmParams {
   int32_t tiles_m, tiles_n;
 };
 
-template <typename T, int BM, int BN, int LA, int LB, bool FULL>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
+template <typename T, int BM, int BN, int WM, int WN, int LA, int LB, bool FULL>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) {
+  constexpr int NT = 64 * WM * WN;
   constexpr int BK = kRowBytes / sizeof(T);
-  constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+  constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int kABytes = BM * kRowStride, kBBytes = BN * kRowStride;
   constexpr int kBufBytes = kABytes + kBBytes;  // buffer b: A tile at b*kBufBytes, B tile right after it
@@ -59,7 +82,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int wm = wave / 2, wn = wave % 2;
+  const int wm = wave / WN, wn = wave % WN;
   const int li = lane % 32, lh = lane / 32;
 
   f32x16_t acc[TM][TN];
@@ -73,8 +96,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   // Two register stages: the global loads of k-tile t+2 are issued before the MFMAs of tile t, tile t+1
   // (issued one iteration earlier) is written to the other LDS buffer after them.  The loop is unrolled
   // by two so that the stage index is a compile-time constant (register arrays, not scratch).
-  TileLoader<T, BM, LA> la0, la1;
-  TileLoader<T, BN, LB> lb0, lb1;
+  TileLoader<T, BM, LA, NT> la0, la1;
+  TileLoader<T, BN, LB, NT> lb0, lb1;
   const int nk = (p.K + BK - 1) / BK;
   la0.template load<FULL>(A, m0, p.M, 0, p.K, p.a_sm, p.a_sk);
   lb0.template load<FULL>(B, n0, p.N, 0, p.K, p.b_sn, p.b_sk);
@@ -89,13 +112,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
 #define LLC_GEMM_STEP(KT, CUR, LA2, LB2, LA1, LB1, GUARDED)                                                     \
   {                                                                                                             \
     /* LA2/LB2: stage that held tile KT (now in LDS) and receives tile KT+2; LA1/LB1 hold tile KT+1 */          \
-    if (!(GUARDED) || (KT) + 2 < nk) {                                                                          \
+    if (LLC_DBG_LOAD && (!(GUARDED) || (KT) + 2 < nk)) {                                                        \
       LA2.template load<FULL>(A, m0, p.M, ((KT) + 2) * BK, p.K, p.a_sm, p.a_sk);                                \
       LB2.template load<FULL>(B, n0, p.N, ((KT) + 2) * BK, p.K, p.b_sn, p.b_sk);                                \
     }                                                                                                           \
-    mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,            \
-                        wn * WTN + li, lh, acc);                                                                \
-    if (!(GUARDED) || (KT) + 1 < nk) {                                                                          \
+    /* keep the loads up here: they must be in flight for two tiles, the scheduler would sink them */         \
+    \
+    if (LLC_DBG_MMA)                                                                                            \
+      mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,          \
+                          wn * WTN + li, lh, acc);                                                              \
+    \
+    if (LLC_DBG_STORE && (!(GUARDED) || (KT) + 1 < nk)) {                                                       \
       LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
       LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
     }                                                                                                           \
@@ -135,33 +162,318 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   }
 }
 
-template <typename T, int BM, int BN, int LA, int LB>
+// ---------------------------------------------------------------------------------------------
+// 16-bit operands, complete 128x128x64 tiles, 16-byte aligned rows: operands go HBM/L2 -> LDS
+// directly (global_load_lds_dwordx4, no staging registers and no ds_write), NS LDS stages deep.
+//
+// 8 waves = 2 (m) x 2 (n) x 2 (k halves): each wave owns a 64x64 accumulator tile over one half of
+// every k-tile, which halves the LDS fragment traffic per MFMA against a 32x64 wave tile while
+// keeping two waves per SIMD (an LDS instruction stream is rate-limited per wave).  The two k halves
+// are summed through LDS in the epilogue, which also turns the accumulator layout into row-major
+// 16-byte stores.
+//
+// LDS stage: A tile [128 m][128 B of k] with the row-XOR chunk swizzle of lds_off(); B tile either
+// the same [128 n][128 B of k] (B unit-stride along k) or, for a row-major B, the tile as it lies in
+// memory, [64 k][256 B of n], read back with ds_read_b64_tr_b16 (each 16-lane group reads a 4(k) x
+// 16(n) patch and receives, per lane, the four k of one n).  The swizzle is applied on the global
+// side: lane L of a load lands at LDS byte 16 L of its 1 KB slice, so it fetches the chunk that
+// belongs there.
+//
+// Frag registers are double-buffered across k-tiles: the ds_reads of tile t+1 are issued before the
+// MFMAs of tile t, one barrier per tile.  Load completion is tracked by hand (s_waitcnt vmcnt): every
+// wave issues exactly four loads per tile and nothing else in the loop uses that counter.
+enum { kBKMajor = 0, kBNMajor = 1 };
+
+// ds_read_b64_tr_b16: the 16 lanes of a group each address 8 bytes (four 16-bit values); lane i of the group
+// receives value i % 4 of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4.
+__device__ __forceinline__ uint2 lds_read_tr16(uint32_t addr) {
+  uint2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr));
+  return v;
+}
+#define LLC_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LLC_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+// s_waitcnt immediate (gfx9 encoding): vmcnt <= VM and lgkmcnt <= 0, expcnt untouched
+#define LLC_WAIT_VM_LGKM0(VM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (7 << 4) | (0 << 8) | (((VM) >> 4) << 14))
+
+constexpr int kDmaStage = 32768;       // bytes of one LDS stage: A tile, then B tile
+constexpr int kDmaBOff = 16384;
+constexpr int kStagePitch = 136;       // floats per row of the epilogue staging tile (bank spread)
+constexpr int kStageHalf = 128 * kStagePitch * 4;
+
+template <typename T, int BMODE, int NS>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
+  static_assert(sizeof(T) == 2, "16-bit operands");
+  extern __shared__ __align__(16) char smem[];
+  int tile_m, tile_n;
+  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * 128, n0 = tile_n * 128;
+  const int z = blockIdx.z;
+  const T* A = (const T*)p.A + (int64_t)z * p.a_sb;
+  const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+  const int li = lane % 32, lh = lane / 32;
+
+  // ---- global sources / LDS destinations of this wave's four loads per tile ----
+  const char* ga[2];
+  const char* gb[2];
+  int la[2], lb[2];
+  int64_t b_step;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int r0 = (wave * 2 + j) * 8, row = r0 + lane / 8;
+    ga[j] = (const char*)(A + (int64_t)(m0 + row) * p.a_sm + (((lane % 8) ^ lds_swz(row)) << 3));
+    la[j] = r0 * kRowStride;
+    if constexpr (BMODE == kBKMajor) {
+      gb[j] = (const char*)(B + (int64_t)(n0 + row) * p.b_sn + (((lane % 8) ^ lds_swz(row)) << 3));
+      lb[j] = kDmaBOff + r0 * kRowStride;
+    } else {
+      const int k0 = (wave * 2 + j) * 4, krow = k0 + lane / 16;
+      gb[j] = (const char*)(B + (int64_t)krow * p.b_sk + n0 + (((lane % 16) ^ ((krow & 3) << 2)) << 3));
+      lb[j] = kDmaBOff + k0 * 256;
+    }
+  }
+  if constexpr (BMODE == kBKMajor) b_step = 128;
+  else b_step = 64 * p.b_sk * 2;
+
+  // ---- fragment offsets inside a stage (fixed for the whole loop) ----
+  int oa[2][2], ob[2][2][BMODE == kBKMajor ? 1 : 2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int chunk = ks * 4 + s * 2 + lh;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ra = wm * 64 + i * 32 + li;
+      oa[s][i] = ra * kRowStride + ((chunk ^ lds_swz(ra)) << 4);
+      if constexpr (BMODE == kBKMajor) {
+        const int rb = wn * 64 + i * 32 + li;
+        ob[s][i][0] = kDmaBOff + rb * kRowStride + ((chunk ^ lds_swz(rb)) << 4);
+      } else {
+        // lane = 16 g + 4 jj + q reads 8 bytes: k row jj of the patch, n = 16 (g & 1) + 4 q .. + 3
+        const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
+        const int nchunk = (wn * 64 + i * 32) / 8 + 2 * (g & 1) + (q >> 1);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int krow = ks * 32 + s * 16 + 8 * (g >> 1) + 4 * u + jj;
+          ob[s][i][u] = kDmaBOff + krow * 256 + ((nchunk ^ (jj << 2)) << 4) + (q & 1) * 8;
+        }
+      }
+    }
+  }
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  u32x4_t fa[2][2][2], fb[2][2][2];  // [set][k step][fragment]
+  uint2 tb[2][2][2][2];              // row-major B: the two transposing reads of each B fragment
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the first stage
+
+  auto issue = [&](int stage) {
+    if (!LLC_DBG_DMA) return;
+    char* base = smem + stage * kDmaStage;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(ga[j]), LLC_LPTR(base + la[j]), 16, 0, 0);
+      ga[j] += 128;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(gb[j]), LLC_LPTR(base + lb[j]), 16, 0, 0);
+      gb[j] += b_step;
+    }
+  };
+#define LLC_DMA_READ(SET, STAGE)                                                                              \
+  if (LLC_DBG_READ) {                                                                                         \
+    const char* base = smem + (STAGE) * kDmaStage;                                                            \
+    _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i) {             \
+      fa[SET][s][i] = *(const u32x4_t*)(base + oa[s][i]);                                                     \
+      if constexpr (BMODE == kBKMajor) {                                                                      \
+        fb[SET][s][i] = *(const u32x4_t*)(base + ob[s][i][0]);                                                \
+      } else {                                                                                                \
+        _Pragma("unroll") for (int u = 0; u < 2; ++u)                                                         \
+            tb[SET][s][i][u] = lds_read_tr16(lds0 + (STAGE) * kDmaStage + ob[s][i][BMODE == kBKMajor ? 0 : u]); \
+      }                                                                                                       \
+    }                                                                                                         \
+  }
+// The transposing reads are issued from inline asm, which the compiler does not track: their results may be
+// used only after an s_waitcnt lgkmcnt(0).  LLC_DMA_TIE, placed right after that wait, makes every use
+// depend on it.
+#define LLC_DMA_TIE(SET)                                                                                      \
+  if constexpr (BMODE != kBKMajor) {                                                                          \
+    asm volatile("" : "+v"(tb[SET][0][0][0]), "+v"(tb[SET][0][0][1]), "+v"(tb[SET][0][1][0]), "+v"(tb[SET][0][1][1]), \
+                      "+v"(tb[SET][1][0][0]), "+v"(tb[SET][1][0][1]), "+v"(tb[SET][1][1][0]), "+v"(tb[SET][1][1][1])); \
+    _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i)               \
+        fb[SET][s][i] = u32x4_t{tb[SET][s][i][0].x, tb[SET][s][i][0].y, tb[SET][s][i][1].x, tb[SET][s][i][1].y}; \
+  }
+#define LLC_DMA_MMA(SET)                                                                                      \
+  if (LLC_DBG_MMA) _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i)                 \
+      _Pragma("unroll") for (int j = 0; j < 2; ++j) mfma_step<T>(fa[SET][s][i], fb[SET][s][j], acc[i][j]);
+
+  const int nk = p.K / 64;
+#pragma unroll
+  for (int x = 0; x < NS; ++x)
+    if (x < nk) issue(x);
+  if (nk >= NS) LLC_WAIT_VM_LGKM0(4 * (NS - 1));
+  else LLC_WAIT_VM_LGKM0(0);
+  __builtin_amdgcn_s_barrier();
+  LLC_DMA_READ(0, 0)
+
+  // Iteration t: tile t's fragments are in registers (set t & 1).  After the barrier tile t+1 is complete
+  // in LDS and stage t % NS is free again: it receives tile t + NS.
+  int t = 0, st = 0;  // st = t % NS
+#define LLC_DMA_NEXT(ST) ((ST) + 1 == NS ? 0 : (ST) + 1)
+#define LLC_DMA_STEADY(SET)                                                                                   \
+  {                                                                                                           \
+    LLC_WAIT_VM_LGKM0(4 * (NS - 2));                                                                          \
+    LLC_DMA_TIE(SET)                                                                                          \
+    __builtin_amdgcn_s_barrier();                                                                             \
+    issue(st);                                                                                                \
+    st = LLC_DMA_NEXT(st);                                                                                    \
+    LLC_DMA_READ((SET) ^ 1, st)                                                                               \
+    LLC_DMA_MMA(SET)                                                                                          \
+  }
+  for (; t + 1 + NS < nk; t += 2) {
+    LLC_DMA_STEADY(0)
+    LLC_DMA_STEADY(1)
+  }
+  // tail: whatever is still to be loaded is loaded, every wait is a full one
+#define LLC_DMA_TAIL(TT, SET)                                                                                 \
+  {                                                                                                           \
+    LLC_WAIT_VM_LGKM0(0);                                                                                     \
+    LLC_DMA_TIE(SET)                                                                                          \
+    __builtin_amdgcn_s_barrier();                                                                             \
+    if ((TT) + NS < nk) issue(st);                                                                            \
+    st = LLC_DMA_NEXT(st);                                                                                    \
+    if ((TT) + 1 < nk) LLC_DMA_READ((SET) ^ 1, st)                                                            \
+    LLC_DMA_MMA(SET)                                                                                          \
+  }
+  for (; t < nk; t += 2) {
+    LLC_DMA_TAIL(t, 0)
+    if (t + 1 < nk) LLC_DMA_TAIL(t + 1, 1)
+  }
+#undef LLC_DMA_READ
+#undef LLC_DMA_TIE
+#undef LLC_DMA_MMA
+#undef LLC_DMA_STEADY
+#undef LLC_DMA_TAIL
+#undef LLC_DMA_NEXT
+
+  // ---- epilogue: both k halves to LDS as fp32 [half][128][kStagePitch], then row-major 16-byte stores.
+  //      No wave reads operand tiles any more (the last fragments were in registers before the last
+  //      barrier) and no load is in flight. ----
+  if (!LLC_DBG_EPI && p.alpha != 123.0f) return;
+  float* stage = (float*)(smem + ks * kStageHalf);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * 64 + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+        stage[row * kStagePitch + wn * 64 + j * 32 + li] = acc[i][j][r];
+      }
+  __syncthreads();
+  T* C = (T*)p.C + (int64_t)z * p.c_sb;
+  const T* res = p.residual ? (const T*)p.residual + (int64_t)z * p.c_sb : nullptr;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int vid = it * 512 + threadIdx.x;
+    const int row = vid / 16, c0 = (vid % 16) * 8;
+    const float* s0 = (const float*)smem + row * kStagePitch + c0;
+    const float* s1 = (const float*)(smem + kStageHalf) + row * kStagePitch + c0;
+    float v[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float4 x = *(const float4*)(s0 + 4 * h), y = *(const float4*)(s1 + 4 * h);
+      v[4 * h + 0] = x.x + y.x;
+      v[4 * h + 1] = x.y + y.y;
+      v[4 * h + 2] = x.z + y.z;
+      v[4 * h + 3] = x.w + y.w;
+    }
+    const int64_t o = (int64_t)(m0 + row) * p.N + n0 + c0;
+    u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
+    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
+    if (res) rq = *(const u32x4_t*)(res + o);
+    u32x4_t outv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint16_t bb = (uint16_t)(bq[e / 2] >> (16 * (e & 1))), rb = (uint16_t)(rq[e / 2] >> (16 * (e & 1)));
+      float x = v[e] * p.alpha;
+      if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) x += bf16_bits_to_f32(bb);
+      else x += f16_bits_to_f32(bb);
+      if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
+      if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
+      else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
+      const uint32_t bits = (Elem<T>::kDtype == LLC_BFLOAT16) ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
+      if (e & 1) outv[e / 2] |= bits << 16;
+      else outv[e / 2] = bits;
+    }
+    *(u32x4_t*)(C + o) = outv;
+  }
+}
+
+template <typename T, int BMODE>
+int launch_dma(const GemmParams& p0, int batch, hipStream_t s) {
+#ifndef LLC_DMA_NS
+#define LLC_DMA_NS 4
+#endif
+  constexpr int NS = LLC_DMA_NS;
+  GemmParams p = p0;
+  p.tiles_m = p.M / 128;
+  p.tiles_n = p.N / 128;
+  const size_t lds = NS * kDmaStage > 2 * kStageHalf ? NS * kDmaStage : 2 * kStageHalf;
+  auto kern = gemm_dma_kernel<T, BMODE, NS>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(512), lds, s, p);
+  return check_launch("gemm_dma_kernel");
+}
+
+template <typename T, int BM, int BN, int WM, int WN, int LA, int LB>
 int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
   GemmParams p = p0;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
-  static bool attr_set[2] = {false, false};  // per instantiation
   // every tile complete: the unguarded instantiation (no per-access branches in the main loop)
   const bool full = p.M % BM == 0 && p.N % BN == 0 && p.K % (kRowBytes / (int)sizeof(T)) == 0;
-  auto kern = full ? gemm_kernel<T, BM, BN, LA, LB, true> : gemm_kernel<T, BM, BN, LA, LB, false>;
+  auto kern = full ? gemm_kernel<T, BM, BN, WM, WN, LA, LB, true> : gemm_kernel<T, BM, BN, WM, WN, LA, LB, false>;
+  static bool attr_set[2] = {false, false};  // per instantiation
   if (!attr_set[full]) {
     LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set[full] = true;
   }
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffff || batch > 65535) return set_error(LLC_ERR_TOO_LARGE, "matmul: grid too large");
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1, (unsigned)batch), dim3(256), lds, s, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1, (unsigned)batch), dim3(64 * WM * WN), lds, s, p);
   return check_launch("gemm_kernel");
 }
 
 template <typename T, int LA, int LB>
 int launch_tiles(const GemmParams& p, int batch, hipStream_t s) {
-  // 128x128 while it still yields enough workgroups for 256 CUs, smaller tiles for skinny outputs
+  // LDS instructions are rate-limited per wave (a wave gets one ds_read_b128 through every ~37 cycles
+  // whatever the other waves do), so the deep-K shapes run 8 waves on a 128x128 tile (two per SIMD,
+  // wave tile 32x64) to keep the LDS pipe and the matrix cores busy at once.  Short-K or skinny
+  // shapes keep 4 waves and rely on several workgroups per CU.
   const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch;
-  if (p.N > 64 && p.M > 64 && t128 >= 128) return launch_cfg<T, 128, 128, LA, LB>(p, batch, s);
-  if (p.N <= 64 && p.M > 64) return launch_cfg<T, 128, 64, LA, LB>(p, batch, s);
-  return launch_cfg<T, 64, 64, LA, LB>(p, batch, s);
+  static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
+  const bool deep = p.K >= 512;
+  if (p.N > 64 && p.M > 64 && t128 >= 128) {
+    if constexpr (LA != kLoadGeneric) {  // the element-wise loader needs too many registers for 8 waves
+      if ((deep && cfg_env != 4) || cfg_env == 8) return launch_cfg<T, 128, 128, 4, 2, LA, LB>(p, batch, s);
+    }
+    return launch_cfg<T, 128, 128, 2, 2, LA, LB>(p, batch, s);
+  }
+  if (p.N <= 64 && p.M > 64) return launch_cfg<T, 128, 64, 2, 2, LA, LB>(p, batch, s);
+  return launch_cfg<T, 64, 64, 2, 2, LA, LB>(p, batch, s);
 }
 
 template <typename T>
@@ -171,6 +483,14 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   const bool a_kvec = p.a_sk == 1 && p.a_sm % EPV == 0 && p.a_sb % EPV == 0 && p.K % EPV == 0 && al16(p.A);
   const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.K % EPV == 0 && al16(p.B);
   const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.N % EPV == 0 && al16(p.B);
+  if constexpr (sizeof(T) == 2) {
+    static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
+    const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
+    if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && p.K >= 256 &&
+        tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && (!p.bias || al16(p.bias)) &&
+        (!p.residual || al16(p.residual)))
+      return b_kvec ? launch_dma<T, kBKMajor>(p, batch, s) : launch_dma<T, kBNMajor>(p, batch, s);
+  }
   if (a_kvec && b_kvec) return launch_tiles<T, kLoadKVec, kLoadKVec>(p, batch, s);
   if (a_kvec && b_rvec) return launch_tiles<T, kLoadKVec, kLoadRVec>(p, batch, s);
   return launch_tiles<T, kLoadGeneric, kLoadGeneric>(p, batch, s);

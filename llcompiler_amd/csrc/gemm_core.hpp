@@ -49,24 +49,25 @@ __device__ __forceinline__ void mfma_step(const u32x4_t& a, const u32x4_t& b, f3
   }
 }
 
-// ---- global -> register staging of one operand tile: ROWS rows x 128 bytes of k ----
+// ---- global -> register staging of one operand tile: ROWS rows x 128 bytes of k, by NT lanes ----
 // kLoadKVec : unit stride along k.  Each lane moves 16-byte vectors (one row, 8 or 4 consecutive k).
-// kLoadRVec : unit stride along the row index.  Each lane owns a 4(k) x EPV(rows) block, transposed
-//             in registers before it is written to LDS.
+// kLoadRVec : unit stride along the row index.  Each lane owns a KB(k) x EPV(rows) block (KB = 4, or 2
+//             when that is what it takes to give every lane a block), transposed in registers before
+//             it is written to LDS.
 // kLoadGeneric : element-wise with arbitrary strides.
-template <typename T, int ROWS, int MODE>
+template <typename T, int ROWS, int MODE, int NT>
 struct TileLoader {
   static constexpr int EPV = 16 / sizeof(T);       // elements per 16 bytes
   static constexpr int BK = kRowBytes / sizeof(T);  // k extent of a tile
   static constexpr int kVecs = ROWS * 8;            // 16-byte vectors per tile
-  static constexpr int kIters = (kVecs + 255) / 256;
-  // kLoadRVec: blocks of 4 k x EPV rows
+  static constexpr int kIters = (kVecs + NT - 1) / NT;
   static constexpr int kRBlocksPerK = ROWS / EPV;
-  static constexpr int kRBlocks = (BK / 4) * kRBlocksPerK;
-  static constexpr int kRIters = (kRBlocks + 255) / 256;
-  static constexpr int kGenElems = ROWS * BK / 256;
+  static constexpr int KB = ((BK / 4) * kRBlocksPerK >= NT) ? 4 : 2;
+  static constexpr int kRBlocks = (BK / KB) * kRBlocksPerK;
+  static constexpr int kRIters = (kRBlocks + NT - 1) / NT;
+  static constexpr int kGenElems = (ROWS * BK + NT - 1) / NT;
 
-  u32x4_t v[MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * 4 : 1)];
+  u32x4_t v[MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * KB : 1)];
   T g[MODE == kLoadGeneric ? kGenElems : 1];
 
   // rows: valid row count of the operand; row0/k0: tile origin; s_r / s_k: element strides.
@@ -77,35 +78,35 @@ struct TileLoader {
     if constexpr (MODE == kLoadKVec) {
 #pragma unroll
       for (int i = 0; i < kIters; ++i) {
-        const int vid = i * 256 + tid;
+        const int vid = i * NT + tid;
         const int r = vid >> 3, kv = vid & 7;
         const int gr = row0 + r, gk = k0 + kv * EPV;
         u32x4_t z = {0, 0, 0, 0};
-        if ((kVecs % 256 == 0 || vid < kVecs) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
+        if ((kVecs % NT == 0 || vid < kVecs) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
         v[i] = z;
       }
     } else if constexpr (MODE == kLoadRVec) {
 #pragma unroll
       for (int i = 0; i < kRIters; ++i) {
-        const int bid = i * 256 + tid;
+        const int bid = i * NT + tid;
         const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
         const int gr = row0 + rb * EPV;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const int gk = k0 + kb * 4 + kk;
+        for (int kk = 0; kk < KB; ++kk) {
+          const int gk = k0 + kb * KB + kk;
           u32x4_t z = {0, 0, 0, 0};
-          if ((kRBlocks % 256 == 0 || bid < kRBlocks) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
-          v[i * 4 + kk] = z;
+          if ((kRBlocks % NT == 0 || bid < kRBlocks) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
+          v[i * KB + kk] = z;
         }
       }
     } else {
 #pragma unroll
       for (int i = 0; i < kGenElems; ++i) {
-        const int e = i * 256 + tid;
+        const int e = i * NT + tid;
         const int r = e / BK, k = e % BK;
         const int gr = row0 + r, gk = k0 + k;
         T z = static_cast<T>(0.0f);
-        if (FULL || (gr < rows && gk < K)) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
+        if (e < ROWS * BK && (FULL || (gr < rows && gk < K))) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
         g[i] = z;
       }
     }
@@ -116,24 +117,34 @@ struct TileLoader {
     if constexpr (MODE == kLoadKVec) {
 #pragma unroll
       for (int i = 0; i < kIters; ++i) {
-        const int vid = i * 256 + tid;
-        if (kVecs % 256 == 0 || vid < kVecs) *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = v[i];
+        const int vid = i * NT + tid;
+        if (kVecs % NT == 0 || vid < kVecs) *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = v[i];
       }
     } else if constexpr (MODE == kLoadRVec) {
 #pragma unroll
       for (int i = 0; i < kRIters; ++i) {
-        const int bid = i * 256 + tid;
-        if (!(kRBlocks % 256 == 0 || bid < kRBlocks)) continue;
+        const int bid = i * NT + tid;
+        if (!(kRBlocks % NT == 0 || bid < kRBlocks)) continue;
         const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
-        const int row0 = rb * EPV, kbyte = kb * 4 * (int)sizeof(T);
-        const u32x4_t r0 = v[i * 4 + 0], r1 = v[i * 4 + 1], r2 = v[i * 4 + 2], r3 = v[i * 4 + 3];
-        if constexpr (sizeof(T) == 4) {
+        const int row0 = rb * EPV, kbyte = kb * KB * (int)sizeof(T);
+        const u32x4_t r0 = v[i * KB + 0], r1 = v[i * KB + 1];
+        if constexpr (sizeof(T) == 4 && KB == 4) {
+          const u32x4_t r2 = v[i * KB + 2], r3 = v[i * KB + 3];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             u32x4_t o = {r0[j], r1[j], r2[j], r3[j]};
             *(u32x4_t*)(lds + lds_off(row0 + j, kbyte)) = o;
           }
-        } else {
+        } else if constexpr (sizeof(T) == 4) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            uint2 o;
+            o.x = r0[j];
+            o.y = r1[j];
+            *(uint2*)(lds + lds_off(row0 + j, kbyte)) = o;
+          }
+        } else if constexpr (KB == 4) {
+          const u32x4_t r2 = v[i * KB + 2], r3 = v[i * KB + 3];
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             // 16-bit element j of each k-row: low halves for even j, high halves for odd j
@@ -143,18 +154,23 @@ struct TileLoader {
             o.y = __builtin_amdgcn_perm(r3[j >> 1], r2[j >> 1], sel);
             *(uint2*)(lds + lds_off(row0 + j, kbyte)) = o;
           }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            *(uint32_t*)(lds + lds_off(row0 + j, kbyte)) = __builtin_amdgcn_perm(r1[j >> 1], r0[j >> 1], sel);
+          }
         }
       }
     } else {
 #pragma unroll
       for (int i = 0; i < kGenElems; ++i) {
-        const int e = i * 256 + tid;
-        *(T*)(lds + lds_off(e / BK, (e % BK) * (int)sizeof(T))) = g[i];
+        const int e = i * NT + tid;
+        if (e < ROWS * BK) *(T*)(lds + lds_off(e / BK, (e % BK) * (int)sizeof(T))) = g[i];
       }
     }
   }
 };
-
 
 __device__ __forceinline__ float load_as_f32(const char* p, int dtype, int64_t i) {
   if (dtype == LLC_FLOAT32) return ((const float*)p)[i];
@@ -183,7 +199,7 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm,
 // MFMAs of one LDS tile pair for one wave: TM x TN fragments of 32x32, four steps of two 16-byte
 // k-chunks (lane half lh takes chunk 2s+lh).  ta / tb are the A / B tiles; arow / brow are this lane's
 // first fragment row in each (fragment i covers rows arow + 32 i).
-template <typename T, int TM, int TN>
+template <typename T, int TM, int TN, int S0 = 0, int S1 = 4>
 __device__ __forceinline__ void mma_tile(const char* ta, int arow, const char* tb, int brow, int lh,
                                          f32x16_t (&acc)[TM][TN]) {
   int abase[TM], aswz[TM], bbase[TN], bswz[TN];
@@ -198,7 +214,7 @@ __device__ __forceinline__ void mma_tile(const char* ta, int arow, const char* t
     bswz[j] = lds_swz(brow + j * 32);
   }
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
+  for (int s = S0; s < S1; ++s) {
     u32x4_t fa[TM], fb[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[i] = *(const u32x4_t*)(ta + abase[i] + (((2 * s + lh) ^ aswz[i]) << 4));

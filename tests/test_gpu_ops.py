@@ -276,6 +276,43 @@ def test_matmul_bf16(ops, oracle, M, N, K):
     assert_close_bf16(host(goth), oracle.matmul(a, b, "mkn"), "NN f16 %s" % ((M, N, K),))
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 2048, 256), (1536, 1408, 448)])
+def test_matmul_16bit_complete_tiles(ops, oracle, M, N, K):
+    """Shapes that take the direct-to-LDS kernel (complete 128x128x64 tiles, >= 128 of them): row-major and
+    transposed-view rhs, bf16 and f16, with and without the fused epilogue."""
+    r = rng(M + N + K)
+    a = bf16_round(r.uniform(-1, 1, (M, K)))
+    b = bf16_round(r.uniform(-1, 1, (K, N)))
+    base = oracle.matmul(a, b, "mkn")
+    want = bf16_round(base)
+    da = dev(a, torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(da, dev(b, torch.bfloat16))), want, "NN bf16")
+    bt = dev(np.ascontiguousarray(b.T), torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(da, bt.t())), want, "NT bf16")
+    assert_close_bf16(host(ops.matmul(dev(a, torch.float16), dev(b, torch.float16))), base, "NN f16")
+    bth = dev(np.ascontiguousarray(b.T), torch.float16)
+    assert_close_bf16(host(ops.matmul(dev(a, torch.float16), bth.t())), base, "NT f16")
+    bias = bf16_round(r.standard_normal(N))
+    res = bf16_round(r.standard_normal((M, N)))
+    for act, alpha in [("none", 1.0), ("relu", 0.5), ("gelu", 0.125)]:
+        w = base * np.float32(alpha) + bias[None, :] + res
+        if act != "none":
+            w = oracle.unary(act, w)
+        epi = ops.Epilogue(alpha=alpha, bias=dev(bias, torch.bfloat16), residual=dev(res, torch.bfloat16), act=act)
+        assert_close_bf16(host(ops.matmul(da, dev(b, torch.bfloat16), epi)), bf16_round(w), "NN epilogue " + act)
+        assert_close_bf16(host(ops.matmul(da, bt.t(), epi)), bf16_round(w), "NT epilogue " + act)
+
+
+def test_batch_matmul_16bit_complete_tiles(ops, oracle):
+    r = rng(77)
+    a = bf16_round(r.uniform(-1, 1, (8, 512, 256)))
+    b = bf16_round(r.uniform(-1, 1, (8, 256, 512)))
+    want = bf16_round(oracle.batch_matmul(a, b, "mkn"))
+    assert_close_bf16(host(ops.batch_matmul(dev(a, torch.bfloat16), dev(b, torch.bfloat16))), want, "bmm bf16")
+    bt = dev(np.ascontiguousarray(b.transpose(0, 2, 1)), torch.bfloat16)
+    assert_close_bf16(host(ops.batch_matmul(dev(a, torch.bfloat16), bt.transpose(1, 2))), want, "bmm bf16 NT")
+
+
 def test_matmul_epilogue(ops, oracle):
     r = rng(21)
     M, N, K = 70, 136, 200
