@@ -411,6 +411,205 @@ __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
 }
 #undef LLC_COPY
 
+// ---------------------------------------------------------------------------------------------
+// Linear chains.  Most fused groups are a straight line: a running value that each op combines with
+// an input, an immediate or itself (add+relu, bias+gelu, scale+mask, ...).  For those the host
+// rewrites the program into accumulator form, "acc = op(acc, x)", with the input that seeds acc moved
+// to slot 0, and this kernel runs it without a register file: acc and up to three other inputs live
+// in named registers, an immediate is used as a scalar operand, and no operand is copied.  That
+// cuts the vector instructions per element severalfold, which is what bounds a 16-bit stream.
+enum { kKindNone = 0, kKindImm = 1, kKindAcc = 2, kKindIn1 = 3 };  // kKindIn1 + k: input slot 1 + k
+enum { kOpRSub = 23, kOpRDiv = 24, kOpRPow = 25 };                 // operand order swapped: x op acc
+
+#define LLC_CH_CASE(OP, EXPR)                         \
+  case OP:                                            \
+    _Pragma("unroll") for (int j = 0; j < E; ++j) {   \
+      const float a = acc[j], b = LLC_CH_B;           \
+      (void)b;                                        \
+      acc[j] = (EXPR);                                \
+    }                                                 \
+    break;
+template <int E>
+__device__ __forceinline__ void chain_unary(int op, float* acc) {
+#define LLC_CH_B 0.0f
+  switch (op) {
+    LLC_CH_CASE(LLC_EW_ABS, fabsf(a))
+    LLC_CH_CASE(LLC_EW_SQRT, sqrtf(a))
+    LLC_CH_CASE(LLC_EW_EXP, expf(a))
+    LLC_CH_CASE(LLC_EW_RELU, a < 0.0f ? 0.0f : a)
+    LLC_CH_CASE(LLC_EW_RSQRT, 1.0f / sqrtf(a))
+    LLC_CH_CASE(LLC_EW_NEG, -a)
+    LLC_CH_CASE(LLC_EW_GELU, gelu_exact(a))
+    LLC_CH_CASE(LLC_EW_TANH, tanhf(a))
+    LLC_CH_CASE(LLC_EW_ERF, erff(a))
+    LLC_CH_CASE(LLC_EW_SIGMOID, 1.0f / (1.0f + expf(-a)))
+    LLC_CH_CASE(LLC_EW_LOG, logf(a))
+    LLC_CH_CASE(LLC_EW_RECIP, 1.0f / a)
+    default: break;  // LLC_EW_MOV
+  }
+#undef LLC_CH_B
+}
+#define LLC_CH_BINARY_CASES                                   \
+    LLC_CH_CASE(LLC_EW_ADD, a + b)                            \
+    LLC_CH_CASE(LLC_EW_SUB, a - b)                            \
+    LLC_CH_CASE(kOpRSub, b - a)                               \
+    LLC_CH_CASE(LLC_EW_MUL, a * b)                            \
+    LLC_CH_CASE(LLC_EW_DIV, a / b)                            \
+    LLC_CH_CASE(kOpRDiv, b / a)                               \
+    LLC_CH_CASE(LLC_EW_MAX, nanmax(a, b))                     \
+    LLC_CH_CASE(LLC_EW_MIN, nanmin(a, b))                     \
+    LLC_CH_CASE(LLC_EW_POW, powf(a, b))                       \
+    LLC_CH_CASE(kOpRPow, powf(b, a))                          \
+    LLC_CH_CASE(LLC_EW_CMP_EQ, a == b ? 1.0f : 0.0f)          \
+    LLC_CH_CASE(LLC_EW_CMP_NE, a != b ? 1.0f : 0.0f)          \
+    LLC_CH_CASE(LLC_EW_CMP_GE, a >= b ? 1.0f : 0.0f)          \
+    LLC_CH_CASE(LLC_EW_CMP_GT, a > b ? 1.0f : 0.0f)           \
+    LLC_CH_CASE(LLC_EW_CMP_LE, a <= b ? 1.0f : 0.0f)          \
+    LLC_CH_CASE(LLC_EW_CMP_LT, a < b ? 1.0f : 0.0f)
+template <int E>
+__device__ __forceinline__ void chain_binary(int op, float* acc, const float* x) {
+#define LLC_CH_B x[j]
+  switch (op) {
+    LLC_CH_BINARY_CASES
+    default: break;
+  }
+#undef LLC_CH_B
+}
+template <int E>
+__device__ __forceinline__ void chain_binary_imm(int op, float* acc, float imm) {
+#define LLC_CH_B imm
+  switch (op) {
+    LLC_CH_BINARY_CASES
+    default: break;
+  }
+#undef LLC_CH_B
+}
+#undef LLC_CH_CASE
+#undef LLC_CH_BINARY_CASES
+
+// insts[i]: op (with the swapped forms above), b = operand kind, imm
+template <int VEC, int NIN>
+__global__ __launch_bounds__(256) void ew_chain_kernel(const EwKernelParams p) {
+  constexpr int E = VEC;
+  const EwHot h = p.hot;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= h.n_vec) return;
+  const bool nt = h.streaming != 0;
+  const uint32_t e = v * VEC;
+  uint32_t idx0 = 0, idx1 = 0, idx2 = 0, idx3 = e;
+  if (!h.flat) {
+    uint32_t t = e;
+    idx3 = t % h.dims[3];
+    t /= h.dims[3];
+    idx2 = t % h.dims[2];
+    t /= h.dims[2];
+    idx1 = t % h.dims[1];
+    idx0 = t / h.dims[1];
+  }
+  float acc[E], x1[E], x2[E], x3[E];
+#define LLC_LOAD_INPUT(K, ARR)                                                                          \
+  if (K < NIN && K < h.n_inputs) {                                                                      \
+    uint32_t off = idx3 * (uint32_t)h.in_inner[K];                                                      \
+    if (!h.flat)                                                                                        \
+      off += idx0 * (uint32_t)p.in_stride[K][0] + idx1 * (uint32_t)p.in_stride[K][1] +                  \
+             idx2 * (uint32_t)p.in_stride[K][2];                                                        \
+    load_vec<VEC, float>(p.in[K], h.in_dtype[K], off, h.in_inner[K], nt, ARR);                          \
+  }
+  LLC_LOAD_INPUT(0, acc)
+  LLC_LOAD_INPUT(1, x1)
+  LLC_LOAD_INPUT(2, x2)
+  LLC_LOAD_INPUT(3, x3)
+#undef LLC_LOAD_INPUT
+  for (int i = 0; i < h.n_insts; ++i) {
+    const int op = p.insts[i].op, kind = p.insts[i].b;
+    switch (kind) {
+      case kKindNone: chain_unary<E>(op, acc); break;
+      case kKindImm: chain_binary_imm<E>(op, acc, p.insts[i].imm); break;
+      case kKindAcc: chain_binary<E>(op, acc, acc); break;
+      case kKindIn1: if constexpr (NIN > 1) chain_binary<E>(op, acc, x1); break;
+      case kKindIn1 + 1: if constexpr (NIN > 2) chain_binary<E>(op, acc, x2); break;
+      default: if constexpr (NIN > 2) chain_binary<E>(op, acc, x3); break;
+    }
+  }
+  store_vec<VEC, float>(p.out, h.out_dtype, e, nt, acc);
+}
+
+// Rewrites a program into accumulator form if it is a straight line.  On success fills chain[] (op, b = kind,
+// imm), slot[] (original input index held by each slot) and the counts.
+bool linearize(const llc_ew_program* prog, size_t n_inputs, llc_ew_inst* chain, int* n_chain, int* slot, int* n_slots) {
+  if (prog->integer || prog->n_insts == 0) return false;
+  auto is_in = [&](int s) { return s >= LLC_EW_IN0 && s < LLC_EW_IN0 + (int)n_inputs; };
+  auto swapped = [](int op) {
+    switch (op) {
+      case LLC_EW_SUB: return (int)kOpRSub;
+      case LLC_EW_DIV: return (int)kOpRDiv;
+      case LLC_EW_POW: return (int)kOpRPow;
+      case LLC_EW_CMP_GE: return (int)LLC_EW_CMP_LE;
+      case LLC_EW_CMP_LE: return (int)LLC_EW_CMP_GE;
+      case LLC_EW_CMP_GT: return (int)LLC_EW_CMP_LT;
+      case LLC_EW_CMP_LT: return (int)LLC_EW_CMP_GT;
+      default: return op;  // commutative
+    }
+  };
+  *n_slots = 1;
+  slot[0] = -1;
+  auto slot_of = [&](int input) {  // slots 1.. hold the operands; the seed of acc always has slot 0 to itself
+    for (int k = 1; k < *n_slots; ++k)
+      if (slot[k] == input) return k;
+    if (*n_slots >= 4) return -1;
+    slot[*n_slots] = input;
+    return (*n_slots)++;
+  };
+  int cur = -1;  // register that holds acc
+  for (int i = 0; i < prog->n_insts; ++i) {
+    const llc_ew_inst& in = prog->insts[i];
+    llc_ew_inst& o = chain[i];
+    o = in;
+    if (in.op == LLC_EW_WHERE) return false;
+    const bool binary = in.op >= LLC_EW_ADD;
+    int a = in.a, b = binary ? in.b : -1;
+    auto is_acc = [&](int s) { return i == 0 ? false : s == cur; };
+    if (i == 0) {
+      // seed: an input operand becomes acc
+      if (!is_in(a)) {
+        if (!binary || !is_in(b)) return false;
+        const int t = a;
+        a = b;
+        b = t;
+        o.op = swapped(in.op);
+      }
+      slot[0] = a - LLC_EW_IN0;
+      if (binary && b == a) b = -2;  // both operands are the seed
+    } else {
+      if (!is_acc(a)) {
+        if (!binary || !is_acc(b)) return false;
+        const int t = a;
+        a = b;
+        b = t;
+        o.op = swapped(in.op);
+      }
+      if (binary && is_acc(b)) b = -2;
+    }
+    if (!binary) {
+      o.b = kKindNone;
+    } else if (b == -2) {
+      o.b = kKindAcc;
+    } else if (b == LLC_EW_IMM) {
+      o.b = kKindImm;
+    } else if (is_in(b)) {
+      const int k = slot_of(b - LLC_EW_IN0);
+      if (k < 0) return false;
+      o.b = kKindIn1 + (k - 1);
+    } else {
+      return false;  // an older register: not a straight line
+    }
+    cur = in.dst;
+  }
+  if (prog->result != cur) return false;
+  *n_chain = prog->n_insts;
+  return true;
+}
+
 bool float_compute_dtype(int t) {
   return t == LLC_FLOAT32 || t == LLC_BFLOAT16 || t == LLC_FLOAT16 || t == LLC_INT64 || t == LLC_INT32 ||
          t == LLC_INT1 || t == LLC_INT8;
@@ -470,6 +669,24 @@ int launch(const EwKernelParams& p, int vec, hipStream_t stream) {
   return check_launch("ew_kernel");
 }
 
+template <int VEC>
+void launch_chain_vec(const EwKernelParams& p, hipStream_t stream) {
+  const uint32_t blocks = (p.hot.n_vec + 255u) / 256u;  // exact cover: one vector per lane
+  if (p.hot.n_inputs <= 1) hipLaunchKernelGGL((ew_chain_kernel<VEC, 1>), dim3(blocks), dim3(256), 0, stream, p);
+  else if (p.hot.n_inputs == 2) hipLaunchKernelGGL((ew_chain_kernel<VEC, 2>), dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((ew_chain_kernel<VEC, 4>), dim3(blocks), dim3(256), 0, stream, p);
+}
+
+int launch_chain(const EwKernelParams& p, int vec, hipStream_t stream) {
+  switch (vec) {
+    case 8: launch_chain_vec<8>(p, stream); break;
+    case 4: launch_chain_vec<4>(p, stream); break;
+    case 2: launch_chain_vec<2>(p, stream); break;
+    default: launch_chain_vec<1>(p, stream); break;
+  }
+  return check_launch("ew_chain_kernel");
+}
+
 }  // namespace
 }  // namespace llc
 
@@ -501,10 +718,18 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
   if (total == 0) return LLC_OK;
   if (total >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "elementwise: %lld elements (max 2^31-1)", (long long)total);
 
+  // a straight-line program runs in accumulator form on the inputs it names, seed first
+  llc_ew_inst chain[LLC_EW_MAX_INSTS];
+  int n_chain = 0, slot[4], n_slots = 0;
+  const bool linear = linearize(prog, n_inputs, chain, &n_chain, slot, &n_slots);
+  View ine[LLC_EW_MAX_INPUTS];
+  size_t ne = linear ? (size_t)n_slots : n_inputs;
+  for (size_t k = 0; k < ne; ++k) ine[k] = linear ? in[slot[k]] : in[k];
+
   // effective strides (0 on broadcast dims), then collapse adjacent dims that stay affine for all inputs
   int64_t est[LLC_EW_MAX_INPUTS][LLC_MAX_RANK];
-  for (size_t k = 0; k < n_inputs; ++k)
-    for (int d = 0; d < o.rank; ++d) est[k][d] = (in[k].size[d] == 1 && o.size[d] != 1) ? 0 : (in[k].size[d] == 1 ? 0 : in[k].stride[d]);
+  for (size_t k = 0; k < ne; ++k)
+    for (int d = 0; d < o.rank; ++d) est[k][d] = (ine[k].size[d] == 1 && o.size[d] != 1) ? 0 : (ine[k].size[d] == 1 ? 0 : ine[k].stride[d]);
   int64_t cdim[LLC_MAX_RANK];
   int64_t cst[LLC_EW_MAX_INPUTS][LLC_MAX_RANK];
   int nc = 0;
@@ -512,31 +737,31 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
     if (o.size[d] == 1) continue;
     bool merge = nc > 0;
     if (merge)
-      for (size_t k = 0; k < n_inputs; ++k)
+      for (size_t k = 0; k < ne; ++k)
         if (cst[k][nc - 1] != est[k][d] * o.size[d]) { merge = false; break; }
     if (merge) {
       cdim[nc - 1] *= o.size[d];
-      for (size_t k = 0; k < n_inputs; ++k) cst[k][nc - 1] = est[k][d];
+      for (size_t k = 0; k < ne; ++k) cst[k][nc - 1] = est[k][d];
     } else {
       cdim[nc] = o.size[d];
-      for (size_t k = 0; k < n_inputs; ++k) cst[k][nc] = est[k][d];
+      for (size_t k = 0; k < ne; ++k) cst[k][nc] = est[k][d];
       ++nc;
     }
   }
   if (nc == 0) {
     cdim[0] = 1;
-    for (size_t k = 0; k < n_inputs; ++k) cst[k][0] = 0;
+    for (size_t k = 0; k < ne; ++k) cst[k][0] = 0;
     nc = 1;
   }
   if (nc > kMaxDims)
     return set_error(LLC_ERR_LAYOUT, "elementwise: broadcast pattern needs %d index dims (max %d)", nc, kMaxDims);
 
   EwKernelParams p{};
-  for (int i = 0; i < prog->n_insts; ++i) p.insts[i] = prog->insts[i];
+  for (int i = 0; i < prog->n_insts; ++i) p.insts[i] = linear ? chain[i] : prog->insts[i];
   p.hot.n_insts = prog->n_insts;
   p.hot.result = prog->result;
   p.hot.integer = prog->integer;
-  p.hot.n_inputs = (int)n_inputs;
+  p.hot.n_inputs = (int)ne;
   p.out = o.ptr;
   p.hot.out_dtype = o.dtype;
   for (int d = 0; d < kMaxDims; ++d) p.hot.dims[d] = 1;
@@ -546,9 +771,9 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
   int vec = prog->integer ? 2 : (o.esize() <= 2 ? 8 : 4);
   if (getenv("LLC_EW_VEC16") && o.esize() <= 2) vec = atoi(getenv("LLC_EW_VEC16"));  // experiment hook
   auto aligned = [](const void* ptr, size_t bytes) { return ((uintptr_t)ptr % bytes) == 0; };
-  for (size_t k = 0; k < n_inputs; ++k) {
-    p.in[k] = in[k].ptr;
-    p.hot.in_dtype[k] = in[k].dtype;
+  for (size_t k = 0; k < ne; ++k) {
+    p.in[k] = ine[k].ptr;
+    p.hot.in_dtype[k] = ine[k].dtype;
     for (int d = 0; d < kMaxDims; ++d) p.in_stride[k][d] = 0;
     for (int d = 0; d < nc; ++d) {
       if (cst[k][d] >= (int64_t)1 << 31 || cst[k][d] < 0)
@@ -560,18 +785,19 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
   }
   while (vec > 1) {
     bool ok = (p.hot.dims[kMaxDims - 1] % vec) == 0 && aligned(o.ptr, vec * o.esize());
-    for (size_t k = 0; ok && k < n_inputs; ++k) {
+    for (size_t k = 0; ok && k < ne; ++k) {
       if (p.in_stride[k][kMaxDims - 1] == 0) continue;
-      ok = aligned(in[k].ptr, vec * in[k].esize());
+      ok = aligned(ine[k].ptr, vec * ine[k].esize());
       for (int d = 0; ok && d < kMaxDims - 1; ++d) ok = (p.in_stride[k][d] % vec) == 0;
     }
     if (ok) break;
     vec >>= 1;
   }
-  for (size_t k = 0; k < n_inputs; ++k) p.hot.in_inner[k] = p.in_stride[k][kMaxDims - 1];
+  for (size_t k = 0; k < ne; ++k) p.hot.in_inner[k] = p.in_stride[k][kMaxDims - 1];
   p.hot.flat = flat ? 1 : 0;
   p.hot.n_vec = (uint32_t)(total / vec);
   // streams far larger than the L2 are touched once: non-temporal accesses keep them out of the caches
   p.hot.streaming = (int64_t)total * (int64_t)o.esize() >= ((int64_t)32 << 20) ? 1 : 0;
+  if (linear) return launch_chain(p, vec, as_stream(stream));
   return prog->integer ? launch<int64_t>(p, vec, as_stream(stream)) : launch<float>(p, vec, as_stream(stream));
 }

@@ -51,6 +51,40 @@ def test_fused_chain_with_immediates(ops, oracle):
     np.testing.assert_array_equal(host(got), want)
 
 
+def test_straight_line_and_dag_programs(ops, oracle):
+    """Straight-line chains are rewritten to accumulator form by the library (operands swapped, seed input moved
+    first); a program that keeps two values alive runs on the register-file interpreter.  Same results either way."""
+    r = rng(31)
+    shape = (5, 130)
+    x = r.uniform(0.5, 1.5, shape).astype(np.float32)
+    y = r.uniform(0.5, 1.5, shape).astype(np.float32)
+    z = r.standard_normal(shape).astype(np.float32)
+    B, U, F = oracle.binary, oracle.unary, np.full_like
+    cases = [
+        # immediate or input on the left of a non-commutative op
+        ([("sub", "r0", 2.0, "in0"), ("div", "r0", "in1", "r0"), ("pow", "r0", 1.5, "r0")], "r0", [x, y],
+         lambda: B("pow", F(x, 1.5), B("div", y, B("sub", F(x, 2.0), x)))),
+        # the running value on the right of a compare
+        ([("mul", "r1", "in0", 0.5), ("gt", "r1", "in1", "r1")], "r1", [x, y],
+         lambda: oracle.compare("GT", y, B("mul", x, F(x, 0.5))).astype(np.float32)),
+        # seed input used again later, three other inputs, input order unlike slot order
+        ([("add", "r0", "in2", "in0"), ("mul", "r0", "r0", "in2"), ("sub", "r0", "r0", "in1"), ("max", "r0", "in3", "r0")],
+         "r0", [x, y, z, x * 0.25], lambda: B("max", x * np.float32(0.25), B("sub", B("mul", B("add", z, x), z), y))),
+        # x op x on the seed and on the running value
+        ([("mul", "r0", "in0", "in0"), ("add", "r0", "r0", "r0"), ("sqrt", "r0", "r0")], "r0", [x],
+         lambda: U("sqrt", B("add", B("mul", x, x), B("mul", x, x)))),
+        # two live values: not a straight line
+        ([("add", "r0", "in0", "in1"), ("mul", "r1", "in0", "in1"), ("sub", "r2", "r0", "r1")], "r2", [x, y],
+         lambda: B("sub", B("add", x, y), B("mul", x, y))),
+        # result is not the last value written
+        ([("add", "r0", "in0", "in1"), ("neg", "r1", "r0")], "r0", [x, y], lambda: B("add", x, y)),
+    ]
+    for insts, result, inputs, want in cases:
+        prog = ops.make_program(insts, result)
+        got = ops.elementwise(prog, [dev(t) for t in inputs], shape, torch.float32)
+        assert_close_f32(host(got), want(), str(insts))
+
+
 @pytest.mark.parametrize("name", ["abs", "sqrt", "exp", "relu", "rsqrt", "neg", "gelu", "tanh", "erf", "sigmoid", "log", "recip"])
 def test_unary_ops(ops, oracle, name):
     r = rng(3)
