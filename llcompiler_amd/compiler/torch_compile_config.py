@@ -1,8 +1,11 @@
 """Decomposition set and operator support used when an FX graph is partitioned for compilation.
 
 Counterpart of llcompiler/compiler/torch_compile_config.py.  LLC_DECOMPOSITIONS is the reference's
-set (:12-28) without aten._softmax: softmax has a kernel of its own here, so the op is kept whole
-(a graph that arrives already decomposed is re-fused by llh.passes.fuse_softmax).  Operator support
+set (:12-28) without aten._softmax and aten.addmm: softmax has a kernel of its own here, so the op is
+kept whole (a graph that arrives already decomposed is re-fused by llh.passes.fuse_softmax); addmm is
+translated directly to matmul + add, and aten.add / sub / mul / div are translated as they are,
+because their decompositions wrap every 16-bit op in converts to and from fp32 (the kernels compute in
+fp32 and round once anyway), which also hides bias, residual and scale from the epilogue fusion.  Operator support
 is "the importer has a translator and the node's attributes are ones the kernels implement";
 everything else stays in torch eager, the reference's fallback rule (:94-98).
 """
@@ -17,14 +20,9 @@ aten = torch.ops.aten
 prims = torch.ops.prims
 
 LLC_DECOMPOSITIONS = {
-    aten.addmm,
     aten.expand,
     aten._unsafe_view,
     aten.transpose,
-    aten.add,
-    aten.mul,
-    aten.sub,
-    aten.div,
     aten.threshold_backward,
     aten.native_batch_norm_backward,
     aten.masked_fill,

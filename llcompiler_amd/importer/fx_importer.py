@@ -90,6 +90,21 @@ def _mm(ctx, node):
     return ctx.g.add_op("matmul", [ctx.val(node.args[0]), ctx.val(node.args[1])])
 
 
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.addmm.default)
+def _addmm(ctx, node):
+    """beta * bias + alpha * (a @ b), kept whole: torch's own decomposition of addmm computes 16-bit operands in
+    fp32 (a convert before and after every matmul), while the kernel takes them as they are and accumulates
+    in fp32.  The add folds into the matmul's epilogue."""
+    bias, a, b = (ctx.val(x) for x in node.args[:3])
+    beta, alpha = node.kwargs.get("beta", 1), node.kwargs.get("alpha", 1)
+    out = ctx.g.add_op("matmul", [a, b])
+    if alpha != 1:
+        out = ctx.g.add_op("mul", [out, ctx.g.constant(alpha, out.dtype)])
+    if beta != 1:
+        bias = ctx.g.add_op("mul", [bias, ctx.g.constant(beta, bias.dtype)])
+    return ctx.g.add_op("add", [out, bias])
+
+
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.bmm.default)
 def _bmm(ctx, node):
     return ctx.g.add_op("batch_matmul", [ctx.val(node.args[0]), ctx.val(node.args[1])])
