@@ -56,6 +56,12 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 
 int check_launch(const char* kernel);
 
+// Scratch device memory for kernels that keep partial results (split-k).  One buffer per device, grown on
+// demand (the device is drained before the old buffer is released) and kept until the process ends.
+// Kernels of one stream run in order, so successive calls on a stream can share it; calls that overlap
+// on different streams of one device must not both use kernels that need it.
+int get_workspace(size_t bytes, void** out);
+
 #define LLC_TRY(expr)              \
   do {                             \
     int _st = (expr);              \

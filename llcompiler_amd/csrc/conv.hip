@@ -13,8 +13,16 @@
 // wave read consecutive pixels, so loads coalesce for stride 1) and writes its run k-contiguous
 // into the same swizzled LDS tile layout the matmul kernel uses.  Weights go through the shared
 // vector loader.  fp32 tensors use the fp32 MFMA, bf16/f16 the 16-bit MFMA; accumulation is fp32.
+#include <cstdlib>
+
 #include "gemm_core.hpp"
 
+#ifndef LLC_DBG_CONV_GATHER
+#define LLC_DBG_CONV_GATHER 1
+#endif
+#ifndef LLC_DBG_CONV_MMA
+#define LLC_DBG_CONV_MMA 1
+#endif
 namespace llc {
 using namespace gemm;
 namespace {
@@ -33,6 +41,8 @@ struct ConvParams {
   float alpha;
   int32_t act;
   int32_t tiles_m, tiles_n;
+  int32_t splits;  // split-k factor (fp32 kernel)
+  char* partial;   // [splits][F][ncols] fp32 partial sums when splits > 1
 };
 
 // Gathers this lane's run of k for one pixel column of the im2col matrix.
@@ -140,9 +150,9 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
       la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
-      lb.load(p, (kt + 1) * BK);
+      if (LLC_DBG_CONV_GATHER) lb.load(p, (kt + 1) * BK);
     }
-    mma_tile<T, TM, TN>(smem + cur * kBufBytes, wm * WTM + li, smem + cur * kBufBytes + kABytes, wn * WTN + li, lh, acc);
+    if (LLC_DBG_CONV_MMA) mma_tile<T, TM, TN>(smem + cur * kBufBytes, wm * WTM + li, smem + cur * kBufBytes + kABytes, wn * WTN + li, lh, acc);
     if (kt + 1 < nk) {
       la.store(smem + (cur ^ 1) * kBufBytes);
       lb.store(smem + (cur ^ 1) * kBufBytes + kABytes);
@@ -170,6 +180,306 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 convolutions with Kdim % 4 == 0 (every layer but an RGB stem).
+//
+// The pixel operand is staged the way it lies in memory: LDS tile [32 k][BN pixels], pixels
+// contiguous.  For a fixed (c, kh, kw) consecutive output pixels of a stride-1 convolution read
+// consecutive input elements, so a lane gathers four pixels with one (4-byte aligned) 16-byte load;
+// window borders, image-row ends and strided convolutions take the element path.  The fp32 MFMA
+// (32x32x2) takes one k per lane and instruction, which fits that layout: lane (li, lh) reads NJ
+// consecutive pixels of row k = k0 + 4 lh + s with one ds_read and uses them as the B operands of NJ
+// interleaved column sets (column set j of a wave holds pixels NJ li + j), while one 16-byte read of
+// the k-contiguous weight tile gives the A operands of four k.  One A read and four B reads feed
+// 4 NJ MFMAs, and because a lane's NJ accumulators are consecutive pixels of one filter plane the
+// epilogue stores 4 NJ bytes per lane straight into NCHW, with no staging.
+//
+// Layers with few output pixels (late ResNet stages) do not have enough tiles for 256 CUs: their
+// reduction is split over blockIdx.y, partial sums go to the scratch buffer in a fixed layout
+// [split][F][pixels], and a second kernel adds them in split order (deterministic) and applies the
+// epilogue.
+typedef float f32x4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+template <int WM, int WN, int NJ>
+__global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
+  constexpr int BM = 32 * WM, BN = 32 * NJ * WN, BK = 32;
+  constexpr int kABytes = BM * kRowStride;
+  constexpr int kBPitch = BN * 4;
+  constexpr int kBuf = kABytes + BK * kBPitch;
+  constexpr int VC = BN / 4;    // 4-pixel columns of the tile
+  constexpr int KG = 256 / VC;  // lanes sharing one of them
+  constexpr int KPT = BK / KG;  // consecutive k per lane
+  static_assert(WM * WN == 4 && KPT >= 1, "4 waves");
+  extern __shared__ __align__(16) char smem[];
+
+  int tile_m, tile_n;
+  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int g = blockIdx.z, split = blockIdx.y;
+  const float* X = (const float*)p.X;
+  const float* Wg = (const float*)p.W + (int64_t)g * p.Fg * p.Kdim;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int wm = wave / WN, wn = wave % WN;
+  const int li = lane % 32, lh = lane / 32;
+  const int ohw = p.OH * p.OW, khw = p.KH * p.KW;
+
+  // ---- this lane's four pixels ----
+  const int vc = threadIdx.x % VC, kg = threadIdx.x / VC;
+  int pbase[4], pih[4], piw[4];
+  bool pvalid[4];
+  bool vec_ok;
+  {
+    const int col0 = n0 + 4 * vc;
+    const int nn = col0 < p.ncols ? col0 / ohw : 0;
+    const int pix = col0 < p.ncols ? col0 - nn * ohw : 0;
+    const int oh = pix / p.OW, ow = pix - oh * p.OW;
+    const bool one_row = col0 + 3 < p.ncols && ow + 3 < p.OW;
+    vec_ok = one_row && p.sw == 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (one_row) {
+        pvalid[j] = true;
+        pbase[j] = (nn * p.C + g * p.Cg) * p.H * p.Wd;
+        pih[j] = oh * p.sh - p.ph;
+        piw[j] = (ow + j) * p.sw - p.pw;
+      } else {
+        const int col = col0 + j;
+        pvalid[j] = col < p.ncols;
+        const int n2 = pvalid[j] ? col / ohw : 0;
+        const int px = pvalid[j] ? col - n2 * ohw : 0;
+        const int oh2 = px / p.OW, ow2 = px - oh2 * p.OW;
+        pbase[j] = (n2 * p.C + g * p.Cg) * p.H * p.Wd;
+        pih[j] = oh2 * p.sh - p.ph;
+        piw[j] = ow2 * p.sw - p.pw;
+      }
+    }
+  }
+
+  TileLoader<float, BM, kLoadKVec, 256> la;
+  f32x4_t bv[KPT];
+  auto gather = [&](int kt) {
+    int k = kt * BK + kg * KPT;
+    int c = k / khw;
+    int r = k - c * khw;
+    int kh = r / p.KW;
+    int kw = r - kh * p.KW;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (k < p.Kdim) {
+        const int dh = kh * p.dh, dw = kw * p.dw;
+        if (vec_ok) {
+          const int ih = pih[0] + dh, iw = piw[0] + dw;
+          if (ih >= 0 && ih < p.H) {
+            const float* src = X + pbase[0] + (c * p.H + ih) * p.Wd + iw;
+            if (iw >= 0 && iw + 3 < p.Wd) {
+              v = *(const f32x4u_t*)src;
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (iw + j >= 0 && iw + j < p.Wd) v[j] = src[j];
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int ih = pih[j] + dh, iw = piw[j] + dw;
+            if (pvalid[j] && ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd) v[j] = X[pbase[j] + (c * p.H + ih) * p.Wd + iw];
+          }
+        }
+      }
+      bv[i] = v;
+      ++k;
+      if (++kw == p.KW) {
+        kw = 0;
+        if (++kh == p.KH) {
+          kh = 0;
+          ++c;
+        }
+      }
+    }
+  };
+  auto store_b = [&](char* tb) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) *(f32x4_t*)(tb + (kg * KPT + i) * kBPitch + vc * 16) = bv[i];
+  };
+
+  f32x16_t acc[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+  const int arow = wm * 32 + li;
+  const int abase = arow * kRowStride, aswz = lds_swz(arow);
+  auto mma = [&](const char* ta, const char* tb) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const u32x4_t a = *(const u32x4_t*)(ta + abase + (((2 * ks + lh) ^ aswz) << 4));
+#pragma unroll
+      for (int s2 = 0; s2 < 4; ++s2) {
+        const float* bp = (const float*)(tb + (ks * 8 + 4 * lh + s2) * kBPitch) + wn * 32 * NJ + NJ * li;
+        float b[NJ];
+        if constexpr (NJ == 4) {
+          const f32x4_t q = *(const f32x4_t*)bp;
+          b[0] = q[0]; b[1] = q[1]; b[2] = q[2]; b[3] = q[3];
+        } else {
+          const f32x2_t q = *(const f32x2_t*)bp;
+          b[0] = q[0]; b[1] = q[1];
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[s2]), b[j], acc[j], 0, 0, 0);
+      }
+    }
+  };
+
+  // k-tiles of this split
+  const int nk = (p.Kdim + BK - 1) / BK;
+  const int kt0 = (int)((int64_t)split * nk / p.splits), kt1 = (int)((int64_t)(split + 1) * nk / p.splits);
+  la.load(Wg, m0, p.Fg, kt0 * BK, p.Kdim, p.Kdim, 1);
+  gather(kt0);
+  la.store(smem);
+  store_b(smem + kABytes);
+  __syncthreads();
+  int cur = 0;
+  for (int kt = kt0; kt + 1 < kt1; ++kt) {
+    la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
+    gather(kt + 1);
+    mma(smem + cur * kBuf, smem + cur * kBuf + kABytes);
+    la.store(smem + (cur ^ 1) * kBuf);
+    store_b(smem + (cur ^ 1) * kBuf + kABytes);
+    __syncthreads();
+    cur ^= 1;
+  }
+  mma(smem + cur * kBuf, smem + cur * kBuf + kABytes);
+
+  // ---- epilogue: lane holds NJ consecutive pixels (columns) of 16 filter rows ----
+  const int col = n0 + wn * 32 * NJ + NJ * li;
+  if (col >= p.ncols) return;
+  if (p.splits > 1) {
+    float* part = (float*)p.partial;
+    const bool vec = p.ncols % NJ == 0;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = m0 + wm * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+      if (row >= p.Fg) continue;
+      float* dst = part + ((int64_t)split * p.F + g * p.Fg + row) * p.ncols + col;
+      if (vec) {
+        if constexpr (NJ == 4) *(f32x4_t*)dst = f32x4_t{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        else *(f32x2_t*)dst = f32x2_t{acc[0][r], acc[1][r]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+          if (col + j < p.ncols) dst[j] = acc[j][r];
+      }
+    }
+    return;
+  }
+  float* Y = (float*)p.Y;
+  const float* res = (const float*)p.residual;
+  const bool vec = ohw % NJ == 0;  // then the NJ pixels share an image and are contiguous and aligned
+  const int nn = col / ohw, pix = col - nn * ohw;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = m0 + wm * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+    if (row >= p.Fg) continue;
+    const int f = g * p.Fg + row;
+    const float bvv = p.bias ? ((const float*)p.bias)[f] : 0.0f;
+    float o[NJ];
+    int64_t idx[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (vec) idx[j] = ((int64_t)nn * p.F + f) * ohw + pix + j;
+      else {
+        const int cj = col + j < p.ncols ? col + j : col;
+        const int n2 = cj / ohw;
+        idx[j] = ((int64_t)n2 * p.F + f) * ohw + (cj - n2 * ohw);
+      }
+    }
+    float rr[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) rr[j] = 0.0f;
+    if (res) {
+      if (vec) {
+        if constexpr (NJ == 4) { const f32x4_t q = *(const f32x4_t*)(res + idx[0]); rr[0] = q[0]; rr[1] = q[1]; rr[2] = q[2]; rr[3] = q[3]; }
+        else { const f32x2_t q = *(const f32x2_t*)(res + idx[0]); rr[0] = q[0]; rr[1] = q[1]; }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) rr[j] = res[idx[j]];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      float v = acc[j][r] * p.alpha + bvv;
+      if (res) v += rr[j];
+      if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
+      else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
+      o[j] = v;
+    }
+    if (vec) {
+      if constexpr (NJ == 4) *(f32x4_t*)(Y + idx[0]) = f32x4_t{o[0], o[1], o[2], o[3]};
+      else *(f32x2_t*)(Y + idx[0]) = f32x2_t{o[0], o[1]};
+    } else {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+        if (col + j < p.ncols) Y[idx[j]] = o[j];
+    }
+  }
+}
+
+// Sums the split partials [splits][F][ncols] in split order and applies the epilogue.
+__global__ __launch_bounds__(256) void conv_split_reduce_kernel(const ConvParams p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)p.F * p.ncols;
+  if (i >= total) return;
+  const int f = (int)(i / p.ncols), col = (int)(i - (int64_t)f * p.ncols);
+  const float* part = (const float*)p.partial;
+  float s = 0.0f;
+  for (int k = 0; k < p.splits; ++k) s += part[(int64_t)k * total + i];
+  const int ohw = p.OH * p.OW;
+  const int nn = col / ohw, pix = col - nn * ohw;
+  const int64_t o = ((int64_t)nn * p.F + f) * ohw + pix;
+  float v = s * p.alpha + (p.bias ? ((const float*)p.bias)[f] : 0.0f);
+  if (p.residual) v += ((const float*)p.residual)[o];
+  if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
+  else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
+  ((float*)p.Y)[o] = v;
+}
+
+int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
+  constexpr int BM = 64, BN = 128;
+  ConvParams p = p0;
+  p.tiles_m = (p.Fg + BM - 1) / BM;
+  p.tiles_n = (p.ncols + BN - 1) / BN;
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles > 0x7fffffff || groups > 65535) return set_error(LLC_ERR_TOO_LARGE, "conv: grid too large");
+  const int nk = (p.Kdim + 31) / 32;
+  // enough workgroups for two per CU, at least eight k-tiles per split
+  int splits = 1;
+  if (tiles * groups < 384) {
+    splits = (int)((512 + tiles * groups - 1) / (tiles * groups));
+    if (splits > nk / 8) splits = nk / 8;
+    if (splits < 1) splits = 1;
+  }
+  p.splits = splits;
+  if (splits > 1) {
+    void* ws = nullptr;
+    LLC_TRY(get_workspace((size_t)splits * p.F * p.ncols * sizeof(float), &ws));
+    p.partial = (char*)ws;
+  }
+  const size_t lds = 2 * (size_t)(BM * kRowStride + 32 * BN * 4);
+  hipLaunchKernelGGL((conv_f32_kernel<2, 2, 2>), dim3((unsigned)tiles, (unsigned)splits, (unsigned)groups), dim3(256), lds, s, p);
+  LLC_TRY(check_launch("conv_f32_kernel"));
+  if (splits > 1) {
+    const int64_t total = (int64_t)p.F * p.ncols;
+    hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
+    LLC_TRY(check_launch("conv_split_reduce_kernel"));
+  }
+  return LLC_OK;
 }
 
 template <typename T, int BM, int BN, int LA>
@@ -203,6 +513,12 @@ template <typename T>
 int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
   const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
+  if constexpr (sizeof(T) == 4) {
+    static const bool old_env = getenv("LLC_CONV_OLD") != nullptr;  // experiment hook
+    if (w_vec && !old_env && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
+        ((uintptr_t)p.X % 4) == 0)
+      return launch_f32(p, groups, s);
+  }
   if (w_vec) return launch_tiles<T, kLoadKVec>(p, groups, s);
   return launch_tiles<T, kLoadGeneric>(p, groups, s);
 }

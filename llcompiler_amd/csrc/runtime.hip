@@ -42,6 +42,31 @@ int check_launch(const char* kernel) {
   return LLC_OK;
 }
 
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_ws[kMaxDevices];
+size_t g_ws_cap[kMaxDevices];
+}  // namespace
+
+int get_workspace(size_t bytes, void** out) {
+  int dev = 0;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "workspace: device %d", dev);
+  if (bytes > g_ws_cap[dev]) {
+    if (g_ws[dev]) {
+      LLC_HIP_TRY(hipDeviceSynchronize());
+      LLC_HIP_TRY(hipFree(g_ws[dev]));
+      g_ws[dev] = nullptr;
+      g_ws_cap[dev] = 0;
+    }
+    const size_t cap = ((bytes + bytes / 2) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    LLC_HIP_TRY(hipMalloc(&g_ws[dev], cap));
+    g_ws_cap[dev] = cap;
+  }
+  *out = g_ws[dev];
+  return LLC_OK;
+}
+
 }  // namespace llc
 
 using namespace llc;

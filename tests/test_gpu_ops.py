@@ -397,6 +397,10 @@ CONV_CASES = [
     (3, 3, 12, 12, 2, 5, 5, (2, 2), (1, 1), (1, 1), 1),
     (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),   # basic-block conv
     (2, 128, 7, 7, 256, 3, 3, (1, 1), (2, 2), (1, 1), 1),
+    (2, 8, 15, 13, 72, 3, 3, (1, 1), (1, 1), (1, 1), 1),    # rows of 13 pixels: 4-pixel gathers straddle row ends
+    (1, 16, 20, 20, 32, 3, 3, (2, 2), (1, 1), (2, 2), 1),   # dilated, stride 1
+    (2, 8, 12, 16, 16, 3, 3, (1, 1), (1, 1), (1, 1), 2),    # groups, stride 1
+    (4, 256, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1),   # few pixels, deep reduction: split over k
 ]
 
 
