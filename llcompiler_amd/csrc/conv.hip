@@ -41,6 +41,7 @@ struct ConvParams {
   float alpha;
   int32_t act;
   int32_t tiles_m, tiles_n;
+  int32_t OWp;     // fp32 kernel: output row length padded to a multiple of 4 (ncols counts padded pixels)
   int32_t splits;  // split-k factor (fp32 kernel)
   char* partial;   // [splits][F][ncols] fp32 partial sums when splits > 1
 };
@@ -204,7 +205,7 @@ typedef float f32x4u_t __attribute__((ext_vector_type(4), aligned(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
-template <int WM, int WN, int NJ>
+template <int WM, int WN, int NJ, bool AFULL>
 __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   constexpr int BM = 32 * WM, BN = 32 * NJ * WN, BK = 32;
   constexpr int kABytes = BM * kRowStride;
@@ -225,43 +226,32 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int wm = wave / WN, wn = wave % WN;
   const int li = lane % 32, lh = lane / 32;
-  const int ohw = p.OH * p.OW, khw = p.KH * p.KW;
+  const int khw = p.KH * p.KW;
 
-  // ---- this lane's four pixels ----
+  // ---- this lane's four pixels: consecutive in one output row (rows are padded to OWp) ----
   const int vc = threadIdx.x % VC, kg = threadIdx.x / VC;
-  int pbase[4], pih[4], piw[4];
-  bool pvalid[4];
-  bool vec_ok;
+  int pbase, pih, piw0;
   {
     const int col0 = n0 + 4 * vc;
-    const int nn = col0 < p.ncols ? col0 / ohw : 0;
-    const int pix = col0 < p.ncols ? col0 - nn * ohw : 0;
-    const int oh = pix / p.OW, ow = pix - oh * p.OW;
-    const bool one_row = col0 + 3 < p.ncols && ow + 3 < p.OW;
-    vec_ok = one_row && p.sw == 1;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (one_row) {
-        pvalid[j] = true;
-        pbase[j] = (nn * p.C + g * p.Cg) * p.H * p.Wd;
-        pih[j] = oh * p.sh - p.ph;
-        piw[j] = (ow + j) * p.sw - p.pw;
-      } else {
-        const int col = col0 + j;
-        pvalid[j] = col < p.ncols;
-        const int n2 = pvalid[j] ? col / ohw : 0;
-        const int px = pvalid[j] ? col - n2 * ohw : 0;
-        const int oh2 = px / p.OW, ow2 = px - oh2 * p.OW;
-        pbase[j] = (n2 * p.C + g * p.Cg) * p.H * p.Wd;
-        pih[j] = oh2 * p.sh - p.ph;
-        piw[j] = ow2 * p.sw - p.pw;
-      }
-    }
+    const int in_range = col0 < p.ncols;
+    const int rowi = in_range ? col0 / p.OWp : 0;  // n * OH + oh
+    const int ow = in_range ? col0 - rowi * p.OWp : 0;
+    const int nn = rowi / p.OH, oh = rowi - nn * p.OH;
+    pbase = (nn * p.C + g * p.Cg) * p.H * p.Wd;
+    pih = oh * p.sh - p.ph;
+    piw0 = ow * p.sw - p.pw;
   }
+  const bool wide = p.sw == 1 && p.Wd >= 4;  // four pixels read four consecutive elements
 
+  // The gather is split in two: `gather_issue` computes addresses and issues every load of the next tile
+  // (before the MFMAs of the current one), `gather_finish` zeroes what lies outside the image and writes
+  // the tile to LDS (after them).  The loads are inline asm so that they stay where they are written and
+  // stay unconditional: written as guarded C++ loads they compile to a branch and a wait per element,
+  // which puts every memory round trip on the critical path.  Addresses are clamped into the tensor.
   TileLoader<float, BM, kLoadKVec, 256> la;
-  f32x4_t bv[KPT];
-  auto gather = [&](int kt) {
+  f32x4_t raw[KPT];
+  int gd[KPT];     // wide: 3 + offset of the wanted run inside the loaded window, 7 = all zero; else: valid bits
+  auto gather_issue = [&](int kt) {
     int k = kt * BK + kg * KPT;
     int c = k / khw;
     int r = k - c * khw;
@@ -269,30 +259,30 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
     int kw = r - kh * p.KW;
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (k < p.Kdim) {
-        const int dh = kh * p.dh, dw = kw * p.dw;
-        if (vec_ok) {
-          const int ih = pih[0] + dh, iw = piw[0] + dw;
-          if (ih >= 0 && ih < p.H) {
-            const float* src = X + pbase[0] + (c * p.H + ih) * p.Wd + iw;
-            if (iw >= 0 && iw + 3 < p.Wd) {
-              v = *(const f32x4u_t*)src;
-            } else {
+      const bool kin = k < p.Kdim;
+      const int ihr = pih + kh * p.dh, iw = piw0 + kw * p.dw;
+      const bool hok = kin && ihr >= 0 && ihr < p.H;
+      const int ih = ihr < 0 ? 0 : (ihr >= p.H ? p.H - 1 : ihr);
+      const float* rowp = X + pbase + ((kin ? c : 0) * p.H + ih) * p.Wd;
+      if (wide) {
+        // window of four elements clamped into the row
+        const int st = iw < 0 ? 0 : (iw > p.Wd - 4 ? p.Wd - 4 : iw);
+        const float* src = rowp + st;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(raw[i]) : "v"(src));
+        gd[i] = hok ? iw - st + 3 : 7;
+      } else {
+        int mask = 0;
 #pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if (iw + j >= 0 && iw + j < p.Wd) v[j] = src[j];
-            }
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int ih = pih[j] + dh, iw = piw[j] + dw;
-            if (pvalid[j] && ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd) v[j] = X[pbase[j] + (c * p.H + ih) * p.Wd + iw];
-          }
+        for (int j = 0; j < 4; ++j) {
+          const int x = iw + j * p.sw;
+          const float* src = rowp + (x < 0 ? 0 : (x >= p.Wd ? p.Wd - 1 : x));
+          float t;
+          asm volatile("global_load_dword %0, %1, off" : "=v"(t) : "v"(src));
+          raw[i][j] = t;
+          mask |= (hok && x >= 0 && x < p.Wd) ? (1 << j) : 0;
         }
+        gd[i] = mask;
       }
-      bv[i] = v;
       ++k;
       if (++kw == p.KW) {
         kw = 0;
@@ -303,9 +293,32 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
       }
     }
   };
-  auto store_b = [&](char* tb) {
+  auto gather_finish = [&](char* tb) {
+    static_assert(KPT == 4, "the wait below names four registers");
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) *(f32x4_t*)(tb + (kg * KPT + i) * kBPitch + vc * 16) = bv[i];
+    for (int i = 0; i < KPT; ++i) {
+      u32x4_t v;
+      const u32x4_t e = __builtin_bit_cast(u32x4_t, raw[i]);
+      if (wide) {
+        // out[j] = window[j + d], zero outside: a funnel shift by sh = d + 3 (0..6, 7 = all zero) over
+        // {0,0,0,e0,e1,e2,e3,0,0,0}, one bit of the shift per stage, each select a bit-field insert
+        const uint32_t sh = (uint32_t)gd[i];
+        const uint32_t m4 = 0u - ((sh >> 2) & 1u), m2 = 0u - ((sh >> 1) & 1u), m1 = 0u - (sh & 1u);
+        const uint32_t x0 = e[1] & m4, x1 = e[2] & m4, x2 = e[3] & m4;
+        const uint32_t x3 = e[0] & ~m4, x4 = e[1] & ~m4, x5 = e[2] & ~m4, x6 = e[3] & ~m4;
+        const uint32_t y0 = (x2 & m2) | (x0 & ~m2), y1 = (x3 & m2) | (x1 & ~m2), y2 = (x4 & m2) | (x2 & ~m2);
+        const uint32_t y3 = (x5 & m2) | (x3 & ~m2), y4 = (x6 & m2) | (x4 & ~m2);
+        v[0] = (y1 & m1) | (y0 & ~m1);
+        v[1] = (y2 & m1) | (y1 & ~m1);
+        v[2] = (y3 & m1) | (y2 & ~m1);
+        v[3] = (y4 & m1) | (y3 & ~m1);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = e[j] & (0u - (((uint32_t)gd[i] >> j) & 1u));
+      }
+      *(u32x4_t*)(tb + (kg * KPT + i) * kBPitch + vc * 16) = v;
+    }
   };
 
   f32x16_t acc[NJ];
@@ -340,18 +353,18 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   // k-tiles of this split
   const int nk = (p.Kdim + BK - 1) / BK;
   const int kt0 = (int)((int64_t)split * nk / p.splits), kt1 = (int)((int64_t)(split + 1) * nk / p.splits);
-  la.load(Wg, m0, p.Fg, kt0 * BK, p.Kdim, p.Kdim, 1);
-  gather(kt0);
+  la.template load<AFULL>(Wg, m0, p.Fg, kt0 * BK, p.Kdim, p.Kdim, 1);
+  gather_issue(kt0);
   la.store(smem);
-  store_b(smem + kABytes);
+  gather_finish(smem + kABytes);
   __syncthreads();
   int cur = 0;
   for (int kt = kt0; kt + 1 < kt1; ++kt) {
-    la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
-    gather(kt + 1);
+    la.template load<AFULL>(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
+    gather_issue(kt + 1);
     mma(smem + cur * kBuf, smem + cur * kBuf + kABytes);
     la.store(smem + (cur ^ 1) * kBuf);
-    store_b(smem + (cur ^ 1) * kBuf + kABytes);
+    gather_finish(smem + (cur ^ 1) * kBuf + kABytes);
     __syncthreads();
     cur ^= 1;
   }
@@ -361,55 +374,42 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   const int col = n0 + wn * 32 * NJ + NJ * li;
   if (col >= p.ncols) return;
   if (p.splits > 1) {
-    float* part = (float*)p.partial;
-    const bool vec = p.ncols % NJ == 0;
+    float* part = (float*)p.partial;  // [split][F][padded pixels]: NJ divides the padded row length
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = m0 + wm * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
       if (row >= p.Fg) continue;
       float* dst = part + ((int64_t)split * p.F + g * p.Fg + row) * p.ncols + col;
-      if (vec) {
-        if constexpr (NJ == 4) *(f32x4_t*)dst = f32x4_t{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-        else *(f32x2_t*)dst = f32x2_t{acc[0][r], acc[1][r]};
-      } else {
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-          if (col + j < p.ncols) dst[j] = acc[j][r];
-      }
+      if constexpr (NJ == 4) *(f32x4_t*)dst = f32x4_t{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      else *(f32x2_t*)dst = f32x2_t{acc[0][r], acc[1][r]};
     }
     return;
   }
   float* Y = (float*)p.Y;
   const float* res = (const float*)p.residual;
-  const bool vec = ohw % NJ == 0;  // then the NJ pixels share an image and are contiguous and aligned
-  const int nn = col / ohw, pix = col - nn * ohw;
+  const int rowi = col / p.OWp, ow = col - rowi * p.OWp;  // rowi = n * OH + oh
+  const int nn = rowi / p.OH, oh = rowi - nn * p.OH;
+  const int nv = p.OW - ow < NJ ? (p.OW - ow < 0 ? 0 : p.OW - ow) : NJ;  // pixels of this lane that exist
+  if (nv == 0) return;              // padding pixels
+  const bool vec = p.OW % NJ == 0;  // then all NJ exist and their address is NJ * 4 byte aligned
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int row = m0 + wm * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
     if (row >= p.Fg) continue;
     const int f = g * p.Fg + row;
     const float bvv = p.bias ? ((const float*)p.bias)[f] : 0.0f;
-    float o[NJ];
-    int64_t idx[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      if (vec) idx[j] = ((int64_t)nn * p.F + f) * ohw + pix + j;
-      else {
-        const int cj = col + j < p.ncols ? col + j : col;
-        const int n2 = cj / ohw;
-        idx[j] = ((int64_t)n2 * p.F + f) * ohw + (cj - n2 * ohw);
-      }
-    }
-    float rr[NJ];
+    const int64_t o0 = (((int64_t)nn * p.F + f) * p.OH + oh) * p.OW + ow;
+    float rr[NJ], o[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; ++j) rr[j] = 0.0f;
     if (res) {
       if (vec) {
-        if constexpr (NJ == 4) { const f32x4_t q = *(const f32x4_t*)(res + idx[0]); rr[0] = q[0]; rr[1] = q[1]; rr[2] = q[2]; rr[3] = q[3]; }
-        else { const f32x2_t q = *(const f32x2_t*)(res + idx[0]); rr[0] = q[0]; rr[1] = q[1]; }
+        if constexpr (NJ == 4) { const f32x4_t q = *(const f32x4_t*)(res + o0); rr[0] = q[0]; rr[1] = q[1]; rr[2] = q[2]; rr[3] = q[3]; }
+        else { const f32x2_t q = *(const f32x2_t*)(res + o0); rr[0] = q[0]; rr[1] = q[1]; }
       } else {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) rr[j] = res[idx[j]];
+        for (int j = 0; j < NJ; ++j)
+          if (j < nv) rr[j] = res[o0 + j];
       }
     }
 #pragma unroll
@@ -421,38 +421,47 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
       o[j] = v;
     }
     if (vec) {
-      if constexpr (NJ == 4) *(f32x4_t*)(Y + idx[0]) = f32x4_t{o[0], o[1], o[2], o[3]};
-      else *(f32x2_t*)(Y + idx[0]) = f32x2_t{o[0], o[1]};
+      if constexpr (NJ == 4) *(f32x4_t*)(Y + o0) = f32x4_t{o[0], o[1], o[2], o[3]};
+      else *(f32x2_t*)(Y + o0) = f32x2_t{o[0], o[1]};
     } else {
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
-        if (col + j < p.ncols) Y[idx[j]] = o[j];
+        if (j < nv) Y[o0 + j] = o[j];
     }
   }
 }
 
 // Sums the split partials [splits][F][ncols] in split order and applies the epilogue.
 __global__ __launch_bounds__(256) void conv_split_reduce_kernel(const ConvParams p) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t total = (int64_t)p.F * p.ncols;
-  if (i >= total) return;
-  const int f = (int)(i / p.ncols), col = (int)(i - (int64_t)f * p.ncols);
-  const float* part = (const float*)p.partial;
-  float s = 0.0f;
-  for (int k = 0; k < p.splits; ++k) s += part[(int64_t)k * total + i];
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into Y
   const int ohw = p.OH * p.OW;
-  const int nn = col / ohw, pix = col - nn * ohw;
-  const int64_t o = ((int64_t)nn * p.F + f) * ohw + pix;
+  const int64_t total = (int64_t)p.N * p.F * ohw;
+  if (i >= total) return;
+  const int ow = (int)(i % p.OW);
+  const int64_t t = i / p.OW;
+  const int oh = (int)(t % p.OH);
+  const int64_t t2 = t / p.OH;
+  const int f = (int)(t2 % p.F), nn = (int)(t2 / p.F);
+  const int col = (nn * p.OH + oh) * p.OWp + ow;
+  const float* part = (const float*)p.partial + (int64_t)f * p.ncols + col;
+  const int64_t stride = (int64_t)p.F * p.ncols;
+  float s = 0.0f;
+  for (int k = 0; k < p.splits; ++k) s += part[k * stride];
   float v = s * p.alpha + (p.bias ? ((const float*)p.bias)[f] : 0.0f);
-  if (p.residual) v += ((const float*)p.residual)[o];
+  if (p.residual) v += ((const float*)p.residual)[i];
   if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
   else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
-  ((float*)p.Y)[o] = v;
+  ((float*)p.Y)[i] = v;
 }
 
 int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
   constexpr int BM = 64, BN = 128;
   ConvParams p = p0;
+  // pixel columns: output rows padded to a multiple of 4, so that a lane's four pixels share a row
+  p.OWp = (p.OW + 3) / 4 * 4;
+  const int64_t ncols = (int64_t)p.N * p.OH * p.OWp;
+  if (ncols >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "conv: too many output pixels");
+  p.ncols = (int)ncols;
   p.tiles_m = (p.Fg + BM - 1) / BM;
   p.tiles_n = (p.ncols + BN - 1) / BN;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
@@ -460,9 +469,11 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
   const int nk = (p.Kdim + 31) / 32;
   // enough workgroups for two per CU, at least eight k-tiles per split
   int splits = 1;
-  if (tiles * groups < 384) {
-    splits = (int)((512 + tiles * groups - 1) / (tiles * groups));
-    if (splits > nk / 8) splits = nk / 8;
+  static const int target_env = getenv("LLC_CONV_BLOCKS") ? atoi(getenv("LLC_CONV_BLOCKS")) : 512;  // experiment hook
+  static const int mink_env = getenv("LLC_CONV_MINK") ? atoi(getenv("LLC_CONV_MINK")) : 8;          // experiment hook
+  if (tiles * groups < target_env * 3 / 4) {
+    splits = (int)((target_env + tiles * groups - 1) / (tiles * groups));
+    if (splits > nk / mink_env) splits = nk / mink_env;
     if (splits < 1) splits = 1;
   }
   p.splits = splits;
@@ -472,10 +483,13 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
     p.partial = (char*)ws;
   }
   const size_t lds = 2 * (size_t)(BM * kRowStride + 32 * BN * 4);
-  hipLaunchKernelGGL((conv_f32_kernel<2, 2, 2>), dim3((unsigned)tiles, (unsigned)splits, (unsigned)groups), dim3(256), lds, s, p);
+  // weight tiles complete in both dims: unguarded weight loads
+  const bool afull = p.Fg % BM == 0 && p.Kdim % 32 == 0;
+  auto kern = afull ? conv_f32_kernel<2, 2, 2, true> : conv_f32_kernel<2, 2, 2, false>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)splits, (unsigned)groups), dim3(256), lds, s, p);
   LLC_TRY(check_launch("conv_f32_kernel"));
   if (splits > 1) {
-    const int64_t total = (int64_t)p.F * p.ncols;
+    const int64_t total = (int64_t)p.N * p.F * p.OH * p.OW;
     hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     LLC_TRY(check_launch("conv_split_reduce_kernel"));
   }
