@@ -56,7 +56,7 @@ class _Cases(list):
         self.only = only
 
     def add(self, name, dtype_name, *rest):
-        if not self.only or ("%s_%s" % (name, dtype_name)) in self.only:
+        if not self.only or "all" in self.only or ("%s_%s" % (name, dtype_name)) in self.only:
             self.append(Case(name, dtype_name, *rest))
 
 
@@ -113,6 +113,17 @@ def time_gpu(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+# HBM bytes per launch (reads + writes) of each case's kernel, from two rocprofv3 counter runs over this
+# same workload (FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain copy of known
+# size gives): profiles/single_op_suite_hbm_counters.md holds the commands and the table.  Counters cannot
+# be read from inside a timed run, so these are carried as measured constants of the kernels as committed.
+MEASURED_TRAFFIC_BYTES = {
+    "matmul_f32": 117758192, "matmul_bf16": 59044501, "batch_matmul_f32": 59286732, "batch_matmul_bf16": 30304309,
+    "add_relu_f32": 805453727, "add_relu_bf16": 402808062, "softmax_f32": 134297839, "softmax_bf16": 67193794,
+    "layernorm_f32": 67269002, "layernorm_bf16": 33671537, "copy_f32": 536870912,
+}
+
+
 def roofline_of(case, ms):
     if case.bound == "mfma":
         achieved = case.flops / (ms * 1e-3) / 1e12
@@ -122,8 +133,9 @@ def roofline_of(case, ms):
         achieved = case.bytes / (ms * 1e-3) / 1e9
         peak = PEAK_HBM_GBS
         unit = "GB/s"
-    return {"kernel": "%s_%s" % (case.name, case.dtype_name), "bound": case.bound, "achieved": round(achieved, 2),
-            "peak": peak, "unit": unit, "frac": round(achieved / peak, 4), "traffic": None, "avg_ms": round(ms, 5)}
+    name = "%s_%s" % (case.name, case.dtype_name)
+    return {"kernel": name, "bound": case.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "avg_ms": round(ms, 5)}
 
 
 def cpu_baseline():
@@ -167,7 +179,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
-                    "these cases, for profiling one kernel at a time; the JSON line then describes that subset")
+                    "these cases, for profiling one kernel at a time (`all` = the whole suite, `copy_f32` adds the "
+                    "counter calibration copy); the JSON line then describes that subset")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
