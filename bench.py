@@ -2,12 +2,12 @@
 """Headline benchmark: the single-op suite (matmul, batch_matmul, fused add+relu, softmax,
 layernorm; fp32 and bf16) run through the C-ABI kernel library on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-models] [--only a,b]
 
 A step is one pass over all ten ops with their inputs already resident in HBM.  Prints ONE JSON
 line: whole-suite latency per pass, the roofline of the kernel that dominates the pass (and of
-every other kernel under "kernels"), and the CPU oracle timed on a bounded sample of the same
-workload on this host.
+every other kernel under "kernels"), the end-to-end latencies of the four model configurations
+("model_latency_ms"), and the CPU oracle timed on a bounded sample of the same workload on this host.
 """
 import argparse
 import json
@@ -172,12 +172,57 @@ def cpu_baseline():
             "per_op_ms": {k: round(v * 1e3, 1) for k, v in parts.items()}}
 
 
+def model_latencies():
+    """End-to-end latency per batch of the other four configurations (whole compiled graphs through the
+    executor, inputs resident on the GPU, synchronised wall clock over repeated calls): an MLP, ResNet-18
+    with folded batch norm, a bf16 encoder block compiled once with a symbolic batch, and a 12-layer BERT-base
+    shaped encoder compiled once with a symbolic sequence length.  Reported next to the suite, not part of
+    `value`."""
+    import copy
+    import warnings
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18Folded, make_bert_inputs,
+                                            make_encoder_inputs, make_mlp_inputs, make_resnet_inputs)
+    warnings.filterwarnings("ignore")
+
+    def timed(f, n, w):
+        for _ in range(w):
+            f()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            f()
+        torch.cuda.synchronize()
+        return round((time.perf_counter() - t0) * 1e3 / n, 4)
+
+    res = {}
+    with torch.no_grad():
+        x = make_mlp_inputs()[0].cuda()
+        cm = compile_module(MLP().cuda(), (x,))
+        res["mlp_f32_batch4_ms"] = timed(lambda: cm(x), 200, 20)
+        xs = make_resnet_inputs(16, 224)[0].cuda()
+        cr = compile_module(ResNet18Folded().cuda(), (xs,))
+        res["resnet18_f32_batch16_ms"] = timed(lambda: cr(xs), 20, 3)
+        xe = make_encoder_inputs(8, 512)[0].to(torch.bfloat16).cuda()
+        ce = compile_module(EncoderBlock().to(torch.bfloat16).cuda(), (xe,), dynamic_shapes=({0: torch.export.Dim("batch")},))
+        for b in (1, 8, 32):
+            xb = make_encoder_inputs(b, 512, seed=b)[0].to(torch.bfloat16).cuda()
+            res["encoder_block_bf16_seq512_batch%d_ms" % b] = timed(lambda: ce(xb), 50, 5)
+        cb = compile_module(BertEncoder().cuda(), tuple(t.cuda() for t in make_bert_inputs(8, 128)),
+                            dynamic_shapes=({1: torch.export.Dim("seq")}, {3: torch.export.Dim("seq")}))
+        for sl in (128, 256, 512):
+            xi, mi = (t.cuda() for t in make_bert_inputs(8, sl, seed=sl))
+            res["bert_base_f32_batch8_seq%d_ms" % sl] = timed(lambda: cb(xi, mi), 10, 2)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-models", action="store_true", help="skip the end-to-end latencies of the model configurations")
     ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
                     "these cases, for profiling one kernel at a time (`all` = the whole suite, `copy_f32` adds the "
                     "counter calibration copy); the JSON line then describes that subset")
@@ -209,6 +254,11 @@ def main():
         "dominant_kernel": dominant["kernel"],
         "kernels": kernels,
     }
+    if not args.no_models and not only:
+        try:
+            out["model_latency_ms"] = model_latencies()
+        except Exception as e:  # the suite's line is still worth printing
+            out["model_latency_ms"] = {"error": "%s: %s" % (type(e).__name__, e)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
