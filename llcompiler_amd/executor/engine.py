@@ -332,8 +332,9 @@ class Instance:
             p = (in_ptrs[idx] if kind == "in" else out_ptrs[idx]) + delta
             ref.desc.data = p
             ref.desc.base = p
+        stream = C.current_stream(self.device)
         for c in self.calls:
-            c.launch()
+            c.launch(stream)
         results = []
         for spec in self.output_plan:
             if spec[0] == "tensor":

@@ -27,8 +27,10 @@ class Call:
     def __init__(self, fn, args, keep, out, device):
         self.fn, self.args, self.keep, self.out, self.device = fn, args, keep, out, device
 
-    def launch(self):
-        st = self.fn(*self.args, C.current_stream(self.device))
+    def launch(self, stream=None):
+        """stream: a ctypes stream handle to launch on (C.current_stream(device) when None; callers that
+        launch many calls in a row look it up once)."""
+        st = self.fn(*self.args, C.current_stream(self.device) if stream is None else stream)
         if st != 0:
             C.check(st)
         return self.out
