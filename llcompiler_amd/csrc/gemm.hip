@@ -184,6 +184,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 // MFMAs of tile t, one barrier per tile.  Load completion is tracked by hand (s_waitcnt vmcnt): every
 // wave issues exactly four loads per tile and nothing else in the loop uses that counter.
 enum { kBKMajor = 0, kBNMajor = 1 };
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // ds_read_b64_tr_b16: the 16 lanes of a group each address 8 bytes (four 16-bit values); lane i of the group
 // receives value i % 4 of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4.
@@ -202,6 +203,76 @@ constexpr int kDmaBOff = 16384;
 constexpr int kStagePitch = 136;       // floats per row of the epilogue staging tile (bank spread)
 constexpr int kStageHalf = 128 * kStagePitch * 4;
 
+// Addresses of one wave's share of the direct-to-LDS loads and of its fragment reads (see the layout notes
+// above).  Wave = ks * 4 + wm * 2 + wn.
+template <typename T, int BMODE>
+struct DmaOperands {
+  const char* ga[2];
+  const char* gb[2];
+  int la[2], lb[2];
+  int64_t b_step;
+  int oa[2][2], ob[2][2][BMODE == kBKMajor ? 1 : 2];  // [k step][fragment]([transposing read])
+
+  __device__ __forceinline__ void init(const GemmParams& p, const T* A, const T* B, int m0, int n0, int wave, int lane) {
+    const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+    const int li = lane % 32, lh = lane / 32;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r0 = (wave * 2 + j) * 8, row = r0 + lane / 8;
+      ga[j] = (const char*)(A + (int64_t)(m0 + row) * p.a_sm + (((lane % 8) ^ lds_swz(row)) << 3));
+      la[j] = r0 * kRowStride;
+      if constexpr (BMODE == kBKMajor) {
+        gb[j] = (const char*)(B + (int64_t)(n0 + row) * p.b_sn + (((lane % 8) ^ lds_swz(row)) << 3));
+        lb[j] = kDmaBOff + r0 * kRowStride;
+      } else {
+        const int k0 = (wave * 2 + j) * 4, krow = k0 + lane / 16;
+        gb[j] = (const char*)(B + (int64_t)krow * p.b_sk + n0 + (((lane % 16) ^ ((krow & 3) << 2)) << 3));
+        lb[j] = kDmaBOff + k0 * 256;
+      }
+    }
+    if constexpr (BMODE == kBKMajor) b_step = 128;
+    else b_step = 64 * p.b_sk * 2;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int chunk = ks * 4 + s * 2 + lh;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int ra = wm * 64 + i * 32 + li;
+        oa[s][i] = ra * kRowStride + ((chunk ^ lds_swz(ra)) << 4);
+        if constexpr (BMODE == kBKMajor) {
+          const int rb = wn * 64 + i * 32 + li;
+          ob[s][i][0] = kDmaBOff + rb * kRowStride + ((chunk ^ lds_swz(rb)) << 4);
+        } else {
+          // lane = 16 g + 4 jj + q reads 8 bytes: k row jj of the patch, n = 16 (g & 1) + 4 q .. + 3
+          const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
+          const int nchunk = (wn * 64 + i * 32) / 8 + 2 * (g & 1) + (q >> 1);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int krow = ks * 32 + s * 16 + 8 * (g >> 1) + 4 * u + jj;
+            ob[s][i][u] = kDmaBOff + krow * 256 + ((nchunk ^ (jj << 2)) << 4) + (q & 1) * 8;
+          }
+        }
+      }
+    }
+  }
+
+  // next k-tile of both operands into `stage`
+  __device__ __forceinline__ void issue(char* smem, int stage) {
+    if (!LLC_DBG_DMA) return;
+    char* base = smem + stage * kDmaStage;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(ga[j]), LLC_LPTR(base + la[j]), 16, 0, 0);
+      ga[j] += 128;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(gb[j]), LLC_LPTR(base + lb[j]), 16, 0, 0);
+      gb[j] += b_step;
+    }
+  }
+};
+
 template <typename T, int BMODE, int NS>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   static_assert(sizeof(T) == 2, "16-bit operands");
@@ -216,52 +287,8 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
   const int li = lane % 32, lh = lane / 32;
 
-  // ---- global sources / LDS destinations of this wave's four loads per tile ----
-  const char* ga[2];
-  const char* gb[2];
-  int la[2], lb[2];
-  int64_t b_step;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int r0 = (wave * 2 + j) * 8, row = r0 + lane / 8;
-    ga[j] = (const char*)(A + (int64_t)(m0 + row) * p.a_sm + (((lane % 8) ^ lds_swz(row)) << 3));
-    la[j] = r0 * kRowStride;
-    if constexpr (BMODE == kBKMajor) {
-      gb[j] = (const char*)(B + (int64_t)(n0 + row) * p.b_sn + (((lane % 8) ^ lds_swz(row)) << 3));
-      lb[j] = kDmaBOff + r0 * kRowStride;
-    } else {
-      const int k0 = (wave * 2 + j) * 4, krow = k0 + lane / 16;
-      gb[j] = (const char*)(B + (int64_t)krow * p.b_sk + n0 + (((lane % 16) ^ ((krow & 3) << 2)) << 3));
-      lb[j] = kDmaBOff + k0 * 256;
-    }
-  }
-  if constexpr (BMODE == kBKMajor) b_step = 128;
-  else b_step = 64 * p.b_sk * 2;
-
-  // ---- fragment offsets inside a stage (fixed for the whole loop) ----
-  int oa[2][2], ob[2][2][BMODE == kBKMajor ? 1 : 2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int chunk = ks * 4 + s * 2 + lh;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int ra = wm * 64 + i * 32 + li;
-      oa[s][i] = ra * kRowStride + ((chunk ^ lds_swz(ra)) << 4);
-      if constexpr (BMODE == kBKMajor) {
-        const int rb = wn * 64 + i * 32 + li;
-        ob[s][i][0] = kDmaBOff + rb * kRowStride + ((chunk ^ lds_swz(rb)) << 4);
-      } else {
-        // lane = 16 g + 4 jj + q reads 8 bytes: k row jj of the patch, n = 16 (g & 1) + 4 q .. + 3
-        const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
-        const int nchunk = (wn * 64 + i * 32) / 8 + 2 * (g & 1) + (q >> 1);
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int krow = ks * 32 + s * 16 + 8 * (g >> 1) + 4 * u + jj;
-          ob[s][i][u] = kDmaBOff + krow * 256 + ((nchunk ^ (jj << 2)) << 4) + (q & 1) * 8;
-        }
-      }
-    }
-  }
+  DmaOperands<T, BMODE> op;
+  op.init(p, A, B, m0, n0, wave, lane);
 
   f32x16_t acc[2][2];
 #pragma unroll
@@ -274,30 +301,17 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   uint2 tb[2][2][2][2];              // row-major B: the two transposing reads of each B fragment
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the first stage
 
-  auto issue = [&](int stage) {
-    if (!LLC_DBG_DMA) return;
-    char* base = smem + stage * kDmaStage;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      __builtin_amdgcn_global_load_lds(LLC_GPTR(ga[j]), LLC_LPTR(base + la[j]), 16, 0, 0);
-      ga[j] += 128;
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      __builtin_amdgcn_global_load_lds(LLC_GPTR(gb[j]), LLC_LPTR(base + lb[j]), 16, 0, 0);
-      gb[j] += b_step;
-    }
-  };
+  auto issue = [&](int stage) { op.issue(smem, stage); };
 #define LLC_DMA_READ(SET, STAGE)                                                                              \
   if (LLC_DBG_READ) {                                                                                         \
     const char* base = smem + (STAGE) * kDmaStage;                                                            \
     _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i) {             \
-      fa[SET][s][i] = *(const u32x4_t*)(base + oa[s][i]);                                                     \
+      fa[SET][s][i] = *(const u32x4_t*)(base + op.oa[s][i]);                                                     \
       if constexpr (BMODE == kBKMajor) {                                                                      \
-        fb[SET][s][i] = *(const u32x4_t*)(base + ob[s][i][0]);                                                \
+        fb[SET][s][i] = *(const u32x4_t*)(base + op.ob[s][i][0]);                                                \
       } else {                                                                                                \
         _Pragma("unroll") for (int u = 0; u < 2; ++u)                                                         \
-            tb[SET][s][i][u] = lds_read_tr16(lds0 + (STAGE) * kDmaStage + ob[s][i][BMODE == kBKMajor ? 0 : u]); \
+            tb[SET][s][i][u] = lds_read_tr16(lds0 + (STAGE) * kDmaStage + op.ob[s][i][BMODE == kBKMajor ? 0 : u]); \
       }                                                                                                       \
     }                                                                                                         \
   }
@@ -438,6 +452,190 @@ int launch_dma(const GemmParams& p0, int batch, hipStream_t s) {
   return check_launch("gemm_dma_kernel");
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same tile and wave layout for short reductions (few k-tiles per output tile), where the pipeline
+// fill and the epilogue of a workgroup weigh as much as its main loop: two workgroups per CU, so that one
+// computes while the other fills or stores.  That halves what a workgroup may hold: two LDS stages (64 KB;
+// the epilogue staging fits in the same space), at most 128 registers per lane, hence fragments of one
+// k-tile at a time (the other workgroup's waves cover the LDS latency).  The load of tile t+1 is issued at
+// the start of iteration t, into the stage all waves left at the barrier.
+//
+// MFMA operands are swapped (C^T = B^T A^T per fragment pair), which leaves every lane with four
+// consecutive columns of one row per accumulator quad: all epilogue LDS traffic is 16-byte accesses.
+// The k halves meet through a lane-private layout (same lane, same register in both waves of a pair),
+// the sums go to a row-major fp32 tile, and all eight waves apply the epilogue and store 16 bytes per lane.
+constexpr int kStage2Pitch = 132;  // floats per row of the fp32 staging tile
+constexpr int kDma2Lds = 128 * kStage2Pitch * 4 > 2 * kDmaStage ? 128 * kStage2Pitch * 4 : 2 * kDmaStage;
+// s_waitcnt immediate: lgkmcnt <= 0, vmcnt and expcnt untouched
+#define LLC_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
+
+template <typename T, int BMODE>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_dma2_kernel(const GemmParams p) {
+  static_assert(sizeof(T) == 2, "16-bit operands");
+  extern __shared__ __align__(16) char smem[];
+  int tile_m, tile_n;
+  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * 128, n0 = tile_n * 128;
+  const int z = blockIdx.z;
+  const T* A = (const T*)p.A + (int64_t)z * p.a_sb;
+  const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+  const int li = lane % 32, lh = lane / 32;
+  DmaOperands<T, BMODE> op;
+  op.init(p, A, B, m0, n0, wave, lane);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+
+  f32x16_t acc[2][2];  // [A fragment][B fragment]; register r: row li of the A fragment, column 8 (r/4) + 4 lh + r%4
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int nk = p.K / 64;
+  op.issue(smem, 0);
+  if (nk > 1) op.issue(smem, 1);
+  for (int t = 0; t < nk; ++t) {
+    const int st = t & 1;
+    // tile t has landed (at t = 0 tile 1 may still be in flight); after the barrier nobody reads the other stage
+    if (t == 0 && nk > 1) LLC_WAIT_VM_LGKM0(4);
+    else LLC_WAIT_VM_LGKM0(0);
+    __builtin_amdgcn_s_barrier();
+    if (t >= 1 && t + 1 < nk) op.issue(smem, st ^ 1);
+    const char* base = smem + st * kDmaStage;
+    u32x4_t fa[2][2], fb[2][2];
+    if constexpr (BMODE == kBKMajor) {
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          fa[s2][i] = *(const u32x4_t*)(base + op.oa[s2][i]);
+          fb[s2][i] = *(const u32x4_t*)(base + op.ob[s2][i][0]);
+        }
+    } else {
+      uint2 tb[2][2][2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          fa[s2][i] = *(const u32x4_t*)(base + op.oa[s2][i]);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) tb[s2][i][u] = lds_read_tr16(lds0 + st * kDmaStage + op.ob[s2][i][BMODE == kBKMajor ? 0 : u]);
+        }
+      // the transposing reads are inline asm: wait for them by hand and make every use depend on the wait
+      LLC_WAIT_LGKM0();
+      asm volatile("" : "+v"(tb[0][0][0]), "+v"(tb[0][0][1]), "+v"(tb[0][1][0]), "+v"(tb[0][1][1]), "+v"(tb[1][0][0]),
+                        "+v"(tb[1][0][1]), "+v"(tb[1][1][0]), "+v"(tb[1][1][1]));
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fb[s2][i] = u32x4_t{tb[s2][i][0].x, tb[s2][i][0].y, tb[s2][i][1].x, tb[s2][i][1].y};
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) mfma_step<T>(fb[s2][j], fa[s2][i], acc[i][j]);  // swapped: lane = row, quad = 4 columns
+  }
+
+  // ---- epilogue ----
+  LLC_WAIT_LGKM0();
+  __builtin_amdgcn_s_barrier();  // every wave has read its last fragments: the stages are free
+  {
+    // k halves: same lane, same register in both waves of a pair
+    char* priv = smem + ((((wave & 3) * 16) * 64 + lane) << 4);
+    if (ks == 1) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *(f32x4_t*)(priv + (((i * 2 + j) * 4 + q) << 10)) = f32x4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    }
+    __syncthreads();
+    if (ks == 0) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4_t o = *(const f32x4_t*)(priv + (((i * 2 + j) * 4 + q) << 10));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += o[e];
+          }
+    }
+    __syncthreads();
+    if (ks == 0) {
+      float* tile = (float*)smem;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *(f32x4_t*)(tile + (wm * 64 + i * 32 + li) * kStage2Pitch + wn * 64 + j * 32 + 8 * q + 4 * lh) =
+                f32x4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    }
+    __syncthreads();
+  }
+  T* C = (T*)p.C + (int64_t)z * p.c_sb;
+  const T* res = p.residual ? (const T*)p.residual + (int64_t)z * p.c_sb : nullptr;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int vid = it * 512 + threadIdx.x;
+    const int row = vid / 16, c0 = (vid % 16) * 8;
+    const float* s0 = (const float*)smem + row * kStage2Pitch + c0;
+    float v[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const f32x4_t x = *(const f32x4_t*)(s0 + 4 * h);
+      v[4 * h + 0] = x[0];
+      v[4 * h + 1] = x[1];
+      v[4 * h + 2] = x[2];
+      v[4 * h + 3] = x[3];
+    }
+    const int64_t o = (int64_t)(m0 + row) * p.N + n0 + c0;
+    u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
+    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
+    if (res) rq = *(const u32x4_t*)(res + o);
+    u32x4_t outv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint16_t bb = (uint16_t)(bq[e / 2] >> (16 * (e & 1))), rb = (uint16_t)(rq[e / 2] >> (16 * (e & 1)));
+      float x = v[e] * p.alpha;
+      if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) x += bf16_bits_to_f32(bb);
+      else x += f16_bits_to_f32(bb);
+      if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
+      if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
+      else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
+      const uint32_t bits = (Elem<T>::kDtype == LLC_BFLOAT16) ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
+      if (e & 1) outv[e / 2] |= bits << 16;
+      else outv[e / 2] = bits;
+    }
+    *(u32x4_t*)(C + o) = outv;
+  }
+}
+
+template <typename T, int BMODE>
+int launch_dma2(const GemmParams& p0, int batch, hipStream_t s) {
+  GemmParams p = p0;
+  p.tiles_m = p.M / 128;
+  p.tiles_n = p.N / 128;
+  auto kern = gemm_dma2_kernel<T, BMODE>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kDma2Lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(512), kDma2Lds, s, p);
+  return check_launch("gemm_dma2_kernel");
+}
+
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB>
 int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
   GemmParams p = p0;
@@ -490,7 +688,13 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
     if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && p.K >= 256 &&
         tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && (!p.bias || al16(p.bias)) &&
         (!p.residual || al16(p.residual)))
+    {
+      // short reductions, or more tiles than one round of workgroups: two workgroups per CU
+      static const int two_env = getenv("LLC_GEMM_TWO") ? atoi(getenv("LLC_GEMM_TWO")) : -1;  // experiment hook
+      const bool two = two_env >= 0 ? two_env != 0 : (p.K <= 1536 && tiles >= 512);
+      if (two) return b_kvec ? launch_dma2<T, kBKMajor>(p, batch, s) : launch_dma2<T, kBNMajor>(p, batch, s);
       return b_kvec ? launch_dma<T, kBKMajor>(p, batch, s) : launch_dma<T, kBNMajor>(p, batch, s);
+    }
   }
   if (a_kvec && b_kvec) return launch_tiles<T, kLoadKVec, kLoadKVec>(p, batch, s);
   if (a_kvec && b_rvec) return launch_tiles<T, kLoadKVec, kLoadRVec>(p, batch, s);

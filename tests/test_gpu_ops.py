@@ -310,9 +310,10 @@ def test_matmul_bf16(ops, oracle, M, N, K):
     assert_close_bf16(host(goth), oracle.matmul(a, b, "mkn"), "NN f16 %s" % ((M, N, K),))
 
 
-@pytest.mark.parametrize("M,N,K", [(1024, 2048, 256), (1536, 1408, 448)])
+@pytest.mark.parametrize("M,N,K", [(1024, 2048, 256), (1536, 1408, 448), (4096, 2048, 256)])
 def test_matmul_16bit_complete_tiles(ops, oracle, M, N, K):
-    """Shapes that take the direct-to-LDS kernel (complete 128x128x64 tiles, >= 128 of them): row-major and
+    """Shapes that take the direct-to-LDS kernels (complete 128x128x64 tiles, >= 128 of them; the last shape
+    has enough tiles and a short enough reduction for the two-workgroups-per-CU form): row-major and
     transposed-view rhs, bf16 and f16, with and without the fused epilogue."""
     r = rng(M + N + K)
     a = bf16_round(r.uniform(-1, 1, (M, K)))
