@@ -685,7 +685,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
     static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
-    if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && p.K >= 256 &&
+    if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
         tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && (!p.bias || al16(p.bias)) &&
         (!p.residual || al16(p.residual)))
     {
