@@ -150,6 +150,30 @@ __device__ __forceinline__ float row_reduce(float v, float* smem) {
   return v;
 }
 
+// 16 bytes of a row as VEC floats (VEC = 4: fp32; VEC = 8: bf16 / f16).  The load itself does not depend on
+// the storage type; the conversion branches on it, uniformly, after every load of the lane has been issued.
+template <int VEC>
+__device__ __forceinline__ void unpack_row_vec(const u32x4& raw, int dtype, float* dst) {
+  if constexpr (VEC == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dst[j] = __uint_as_float(raw[j]);
+  } else {
+    if (dtype == LLC_BFLOAT16) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        dst[2 * j] = __uint_as_float(raw[j] << 16);
+        dst[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        dst[2 * j] = f16_bits_to_f32((uint16_t)(raw[j] & 0xffffu));
+        dst[2 * j + 1] = f16_bits_to_f32((uint16_t)(raw[j] >> 16));
+      }
+    }
+  }
+}
+
 template <int OP, int VEC, int TPR, int ITEMS>
 __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
   __shared__ float smem[4];
@@ -158,20 +182,66 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
   const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
   const bool row_ok = row < p.rows;
   const int64_t base = row * p.cols;
+  // full: every lane of the launch owns ITEMS complete vectors, nothing to mask
+  const bool full = p.cols == TPR * ITEMS * VEC && p.rows % RPB == 0;
 
   float v[ITEMS][VEC];
   bool ok[ITEMS];
+  u32x4 graw[OP == kLayerNorm && VEC > 1 ? ITEMS : 1], braw[OP == kLayerNorm && VEC > 1 ? ITEMS : 1];  // scale / bias
   const float fill = (OP == kSoftmax) ? -INFINITY
                      : (OP == kReduce) ? (p.kind == LLC_REDUCE_SUM ? 0.0f : (p.kind == LLC_REDUCE_MAX ? -INFINITY : INFINITY))
                                        : 0.0f;
+  if constexpr (VEC > 1) {
+    // Every load is issued before anything waits: unconditional, from an address clamped into the tensor
+    // (a guarded load compiles to a branch with a wait inside, which serialises the round trips).
+    const int es = p.dtype == LLC_FLOAT32 ? 4 : 2;
+    const int64_t crow = row_ok ? row : p.rows - 1;
+    u32x4 raw[ITEMS];
+    const u32x4* src[ITEMS];
+    int ccol[ITEMS];
 #pragma unroll
-  for (int it = 0; it < ITEMS; ++it) {
-    const int col = (it * TPR + lane) * VEC;
-    ok[it] = row_ok && col < p.cols;
-    if (ok[it]) load_row_vec<VEC>(p.x, p.dtype, base + col, v[it], p.streaming != 0);
-    else {
+    for (int it = 0; it < ITEMS; ++it) {
+      const int col = (it * TPR + lane) * VEC;
+      ok[it] = row_ok && col < p.cols;
+      ccol[it] = col < p.cols ? col : p.cols - VEC;
+      src[it] = (const u32x4*)(p.x + (crow * p.cols + ccol[it]) * es);
+    }
+    if (p.streaming) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) v[it][j] = fill;
+      for (int it = 0; it < ITEMS; ++it) raw[it] = __builtin_nontemporal_load(src[it]);
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) raw[it] = *src[it];
+    }
+    if constexpr (OP == kLayerNorm) {
+      // scale and bias do not depend on the statistics: their loads travel while the row is reduced
+      if (p.gamma) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) graw[it] = *(const u32x4*)(p.gamma + (int64_t)ccol[it] * es);
+      }
+      if (p.beta) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) braw[it] = *(const u32x4*)(p.beta + (int64_t)ccol[it] * es);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) unpack_row_vec<VEC>(raw[it], p.dtype, v[it]);
+    if (!full) {
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[it][j] = ok[it] ? v[it][j] : fill;
+    }
+  } else {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int col = (it * TPR + lane) * VEC;
+      ok[it] = row_ok && col < p.cols;
+      if (ok[it]) load_row_vec<VEC>(p.x, p.dtype, base + col, v[it], p.streaming != 0);
+      else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[it][j] = fill;
+      }
     }
   }
 
@@ -187,8 +257,10 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
     for (int it = 0; it < ITEMS; ++it)
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        // masked lanes hold -inf: exp(-inf - m) = 0 for finite m; keep them out when m is -inf too
-        float e = ok[it] ? expf(v[it][j] - m) : 0.0f;
+        // exp through the hardware exp2 (relative error below 1e-5 for arguments down to -88).  Masked
+        // lanes hold -inf: exp(-inf - m) = 0 for finite m; they are kept out when m is -inf too
+        float e = __builtin_amdgcn_exp2f((v[it][j] - m) * 1.4426950408889634f);
+        if (!full) e = ok[it] ? e : 0.0f;
         v[it][j] = e;
         s += e;
       }
@@ -215,7 +287,8 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
     for (int it = 0; it < ITEMS; ++it)
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        float d = ok[it] ? v[it][j] - mean : 0.0f;
+        float d = v[it][j] - mean;
+        if (!full) d = ok[it] ? d : 0.0f;
         v[it][j] = d;
         q += d * d;
       }
@@ -226,8 +299,13 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
       if (ok[it]) {
         const int col = (it * TPR + lane) * VEC;
         float g[VEC], b[VEC];
-        if (p.gamma) load_row_vec<VEC>(p.gamma, p.dtype, col, g);
-        if (p.beta) load_row_vec<VEC>(p.beta, p.dtype, col, b);
+        if constexpr (VEC > 1) {
+          if (p.gamma) unpack_row_vec<VEC>(graw[it], p.dtype, g);
+          if (p.beta) unpack_row_vec<VEC>(braw[it], p.dtype, b);
+        } else {
+          if (p.gamma) load_row_vec<VEC>(p.gamma, p.dtype, col, g);
+          if (p.beta) load_row_vec<VEC>(p.beta, p.dtype, col, b);
+        }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           float t = v[it][j] * rstd;
