@@ -53,7 +53,9 @@ struct Im2colLoader {
   static constexpr int KPT = BK * BN / 256;   // consecutive k per lane
   static constexpr int kParts = 256 / BN;     // lanes sharing one column
   static_assert(KPT * sizeof(T) % 16 == 0, "a lane's run must be whole 16-byte vectors");
+  static_assert(KPT <= 32, "one mask word");
   T v[KPT];
+  uint32_t okm;
   const T* plane0;  // X + (n*C + g*Cg)*H*W for this lane's pixel
   int ih0, iw0;
   bool valid;
@@ -71,6 +73,9 @@ struct Im2colLoader {
     plane0 = (const T*)p.X + ((int64_t)n * p.C + (int64_t)g * p.Cg) * p.H * p.Wd;
   }
 
+  // Every element is loaded unconditionally from an index clamped into the image; which ones lie outside
+  // (padding, k tail, columns past the batch) is kept as a bit mask and applied when the run is written to
+  // LDS.  Guarded loads would compile to a branch with a wait each: one memory round trip after the other.
   __device__ __forceinline__ void load(const ConvParams& p, int k0) {
     const int kpart = threadIdx.x / BN;
     int k = k0 + kpart * KPT;
@@ -79,13 +84,15 @@ struct Im2colLoader {
     int r = k - c * khw;
     int kh = r / p.KW;
     int kw = r - kh * p.KW;
+    okm = 0;
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      T z = static_cast<T>(0.0f);
       const int ih = ih0 + kh * p.dh, iw = iw0 + kw * p.dw;
-      if (valid && k < p.Kdim && ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd)
-        z = plane0[((int64_t)c * p.H + ih) * p.Wd + iw];
-      v[i] = z;
+      const bool ok = valid && k < p.Kdim && ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd;
+      const int cc = k < p.Kdim ? c : 0;
+      const int ch = ih < 0 ? 0 : (ih >= p.H ? p.H - 1 : ih), cw = iw < 0 ? 0 : (iw >= p.Wd ? p.Wd - 1 : iw);
+      v[i] = plane0[((int64_t)cc * p.H + ch) * p.Wd + cw];
+      okm |= ok ? (1u << i) : 0u;
       ++k;
       if (++kw == p.KW) {
         kw = 0;
@@ -104,7 +111,7 @@ struct Im2colLoader {
     for (int q = 0; q < KPT / EPV; ++q) {
       struct alignas(16) Pack { T e[EPV]; } pk;
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) pk.e[e] = v[q * EPV + e];
+      for (int e = 0; e < EPV; ++e) pk.e[e] = (okm >> (q * EPV + e)) & 1u ? v[q * EPV + e] : static_cast<T>(0.0f);
       *(Pack*)(lds + lds_off(j, kpart * KPT * (int)sizeof(T) + q * 16)) = pk;
     }
   }

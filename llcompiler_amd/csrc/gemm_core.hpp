@@ -69,21 +69,39 @@ struct TileLoader {
 
   u32x4_t v[MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * KB : 1)];
   T g[MODE == kLoadGeneric ? kGenElems : 1];
+  uint32_t okm = 0xffffffffu;  // bit per vector of v: inside the operand (partial tiles)
+  static_assert((MODE == kLoadKVec ? kIters : (MODE == kLoadRVec ? kRIters * KB : 1)) <= 32, "one mask word");
 
   // rows: valid row count of the operand; row0/k0: tile origin; s_r / s_k: element strides.
   // FULL: the tile lies entirely inside the operand, so no access is guarded.
   template <bool FULL = false>
   __device__ __forceinline__ void load(const T* base, int row0, int rows, int k0, int K, int64_t s_r, int64_t s_k) {
     const int tid = threadIdx.x;
+    // Partial tiles: every load is issued unconditionally from an index clamped into the operand; which
+    // vectors lie outside is kept as a bit mask and applied when the tile is written to LDS (a guarded load
+    // compiles to a branch with a wait inside: one memory round trip after the other, none of them in
+    // flight across the MFMAs).
     if constexpr (MODE == kLoadKVec) {
 #pragma unroll
       for (int i = 0; i < kIters; ++i) {
         const int vid = i * NT + tid;
         const int r = vid >> 3, kv = vid & 7;
         const int gr = row0 + r, gk = k0 + kv * EPV;
-        u32x4_t z = {0, 0, 0, 0};
-        if ((kVecs % NT == 0 || vid < kVecs) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
-        v[i] = z;
+        if constexpr (FULL) {
+          if (kVecs % NT == 0 || vid < kVecs) v[i] = *(const u32x4_t*)(base + (int64_t)gr * s_r + gk);
+        } else {
+          const int cr = gr < rows ? gr : rows - 1, ck = gk < K ? gk : K - EPV;
+          v[i] = *(const u32x4_t*)(base + (int64_t)cr * s_r + ck);
+        }
+      }
+      if constexpr (!FULL) {
+        okm = 0;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+          const int vid = i * NT + tid;
+          const bool ok = (kVecs % NT == 0 || vid < kVecs) && row0 + (vid >> 3) < rows && k0 + (vid & 7) * EPV < K;
+          okm |= ok ? (1u << i) : 0u;
+        }
       }
     } else if constexpr (MODE == kLoadRVec) {
 #pragma unroll
@@ -94,9 +112,25 @@ struct TileLoader {
 #pragma unroll
         for (int kk = 0; kk < KB; ++kk) {
           const int gk = k0 + kb * KB + kk;
-          u32x4_t z = {0, 0, 0, 0};
-          if ((kRBlocks % NT == 0 || bid < kRBlocks) && (FULL || (gr < rows && gk < K))) z = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
-          v[i * KB + kk] = z;
+          if constexpr (FULL) {
+            if (kRBlocks % NT == 0 || bid < kRBlocks) v[i * KB + kk] = *(const u32x4_t*)(base + (int64_t)gk * s_k + gr);
+          } else {
+            const int cr = gr < rows ? gr : rows - EPV, ck = gk < K ? gk : K - 1;
+            v[i * KB + kk] = *(const u32x4_t*)(base + (int64_t)ck * s_k + cr);
+          }
+        }
+      }
+      if constexpr (!FULL) {
+        okm = 0;
+#pragma unroll
+        for (int i = 0; i < kRIters; ++i) {
+          const int bid = i * NT + tid;
+          const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
+#pragma unroll
+          for (int kk = 0; kk < KB; ++kk) {
+            const bool ok = (kRBlocks % NT == 0 || bid < kRBlocks) && row0 + rb * EPV < rows && k0 + kb * KB + kk < K;
+            okm |= ok ? (1u << (i * KB + kk)) : 0u;
+          }
         }
       }
     } else {
@@ -105,11 +139,21 @@ struct TileLoader {
         const int e = i * NT + tid;
         const int r = e / BK, k = e % BK;
         const int gr = row0 + r, gk = k0 + k;
-        T z = static_cast<T>(0.0f);
-        if (e < ROWS * BK && (FULL || (gr < rows && gk < K))) z = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
-        g[i] = z;
+        if constexpr (FULL) {
+          if (e < ROWS * BK) g[i] = base[(int64_t)gr * s_r + (int64_t)gk * s_k];
+        } else {
+          const bool ok = e < ROWS * BK && gr < rows && gk < K;
+          const int cr = gr < rows ? gr : rows - 1, ck = gk < K ? gk : K - 1;
+          const T z = base[(int64_t)cr * s_r + (int64_t)ck * s_k];
+          g[i] = ok ? z : static_cast<T>(0.0f);
+        }
       }
     }
+  }
+
+  __device__ __forceinline__ u32x4_t masked(int i) const {
+    const uint32_t m = 0u - ((okm >> i) & 1u);
+    return u32x4_t{v[i][0] & m, v[i][1] & m, v[i][2] & m, v[i][3] & m};
   }
 
   __device__ __forceinline__ void store(char* lds) const {
@@ -118,7 +162,7 @@ struct TileLoader {
 #pragma unroll
       for (int i = 0; i < kIters; ++i) {
         const int vid = i * NT + tid;
-        if (kVecs % NT == 0 || vid < kVecs) *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = v[i];
+        if (kVecs % NT == 0 || vid < kVecs) *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = masked(i);
       }
     } else if constexpr (MODE == kLoadRVec) {
 #pragma unroll
@@ -127,9 +171,9 @@ struct TileLoader {
         if (!(kRBlocks % NT == 0 || bid < kRBlocks)) continue;
         const int rb = bid % kRBlocksPerK, kb = bid / kRBlocksPerK;
         const int row0 = rb * EPV, kbyte = kb * KB * (int)sizeof(T);
-        const u32x4_t r0 = v[i * KB + 0], r1 = v[i * KB + 1];
+        const u32x4_t r0 = masked(i * KB + 0), r1 = masked(i * KB + 1);
         if constexpr (sizeof(T) == 4 && KB == 4) {
-          const u32x4_t r2 = v[i * KB + 2], r3 = v[i * KB + 3];
+          const u32x4_t r2 = masked(i * KB + 2), r3 = masked(i * KB + 3);
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             u32x4_t o = {r0[j], r1[j], r2[j], r3[j]};
@@ -144,7 +188,7 @@ struct TileLoader {
             *(uint2*)(lds + lds_off(row0 + j, kbyte)) = o;
           }
         } else if constexpr (KB == 4) {
-          const u32x4_t r2 = v[i * KB + 2], r3 = v[i * KB + 3];
+          const u32x4_t r2 = masked(i * KB + 2), r3 = masked(i * KB + 3);
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             // 16-bit element j of each k-row: low halves for even j, high halves for odd j
