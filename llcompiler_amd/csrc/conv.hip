@@ -258,33 +258,41 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   TileLoader<float, BM, kLoadKVec, 256> la;
   f32x4_t raw[KPT];
   int gd[KPT];     // wide: 3 + offset of the wanted run inside the loaded window, 7 = all zero; else: valid bits
-  auto gather_issue = [&](int kt) {
-    int k = kt * BK + kg * KPT;
-    int c = k / khw;
-    int r = k - c * khw;
-    int kh = r / p.KW;
-    int kw = r - kh * p.KW;
+  // (c, kh, kw) of this lane's first k in the tile being gathered, kept across tiles: a tile advances k by 32,
+  // added in the mixed radix (c, kh, kw) with one carry per digit (two integer divisions per tile otherwise)
+  const int kstart = (int)((int64_t)blockIdx.y * ((p.Kdim + BK - 1) / BK) / p.splits) * BK + kg * KPT;
+  int gk = kstart;
+  int gc = kstart / khw;
+  int gkh = (kstart - gc * khw) / p.KW;
+  int gkw = kstart - gc * khw - gkh * p.KW;
+  const int step_c = BK / khw, step_kh = (BK - step_c * khw) / p.KW, step_kw = BK - step_c * khw - step_kh * p.KW;
+  const int hw = p.H * p.Wd;
+  // offset of the wanted run inside the clamped window: -pw .. OWp - W - pw + (KW-1) dw over all taps and
+  // pixel groups; within -1..1 for 3x3 pad 1 on rows that are a multiple of 4 wide
+  const bool small_shift = p.pw <= 1 && p.OWp - p.Wd - p.pw + (p.KW - 1) * p.dw <= 1;
+  auto gather_issue = [&]() {
+    int k = gk, c = gc, kh = gkh, kw = gkw;
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const bool kin = k < p.Kdim;
       const int ihr = pih + kh * p.dh, iw = piw0 + kw * p.dw;
       const bool hok = kin && ihr >= 0 && ihr < p.H;
       const int ih = ihr < 0 ? 0 : (ihr >= p.H ? p.H - 1 : ihr);
-      const float* rowp = X + pbase + ((kin ? c : 0) * p.H + ih) * p.Wd;
+      const int rowoff = pbase + (kin ? c : 0) * hw + ih * p.Wd;  // floats from X
       if (wide) {
         // window of four elements clamped into the row
         const int st = iw < 0 ? 0 : (iw > p.Wd - 4 ? p.Wd - 4 : iw);
-        const float* src = rowp + st;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(raw[i]) : "v"(src));
+        const uint32_t boff = (uint32_t)(rowoff + st) * 4u;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(raw[i]) : "v"(boff), "s"(X));
         gd[i] = hok ? iw - st + 3 : 7;
       } else {
         int mask = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int x = iw + j * p.sw;
-          const float* src = rowp + (x < 0 ? 0 : (x >= p.Wd ? p.Wd - 1 : x));
+          const uint32_t boff = (uint32_t)(rowoff + (x < 0 ? 0 : (x >= p.Wd ? p.Wd - 1 : x))) * 4u;
           float t;
-          asm volatile("global_load_dword %0, %1, off" : "=v"(t) : "v"(src));
+          asm volatile("global_load_dword %0, %1, %2" : "=v"(t) : "v"(boff), "s"(X));
           raw[i][j] = t;
           mask |= (hok && x >= 0 && x < p.Wd) ? (1 << j) : 0;
         }
@@ -299,6 +307,19 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
         }
       }
     }
+    // next tile
+    gk += BK;
+    gkw += step_kw;
+    if (gkw >= p.KW) {
+      gkw -= p.KW;
+      ++gkh;
+    }
+    gkh += step_kh;
+    if (gkh >= p.KH) {
+      gkh -= p.KH;
+      ++gc;
+    }
+    gc += step_c;
   };
   auto gather_finish = [&](char* tb) {
     static_assert(KPT == 4, "the wait below names four registers");
@@ -307,10 +328,17 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
     for (int i = 0; i < KPT; ++i) {
       u32x4_t v;
       const u32x4_t e = __builtin_bit_cast(u32x4_t, raw[i]);
-      if (wide) {
+      const uint32_t sh = (uint32_t)gd[i];
+      if (wide && small_shift) {
+        // sh = 3: the window is the run; 4: the run starts one element later; 2: one earlier; 7: all zero
+        const uint32_t m0 = sh == 3u ? 0xffffffffu : 0u, ml = sh == 2u ? 0xffffffffu : 0u, mr = sh == 4u ? 0xffffffffu : 0u;
+        v[0] = (e[0] & m0) | (e[1] & mr);
+        v[1] = (e[1] & m0) | (e[2] & mr) | (e[0] & ml);
+        v[2] = (e[2] & m0) | (e[3] & mr) | (e[1] & ml);
+        v[3] = (e[3] & m0) | (e[2] & ml);
+      } else if (wide) {
         // out[j] = window[j + d], zero outside: a funnel shift by sh = d + 3 (0..6, 7 = all zero) over
         // {0,0,0,e0,e1,e2,e3,0,0,0}, one bit of the shift per stage, each select a bit-field insert
-        const uint32_t sh = (uint32_t)gd[i];
         const uint32_t m4 = 0u - ((sh >> 2) & 1u), m2 = 0u - ((sh >> 1) & 1u), m1 = 0u - (sh & 1u);
         const uint32_t x0 = e[1] & m4, x1 = e[2] & m4, x2 = e[3] & m4;
         const uint32_t x3 = e[0] & ~m4, x4 = e[1] & ~m4, x5 = e[2] & ~m4, x6 = e[3] & ~m4;
@@ -322,7 +350,7 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
         v[3] = (y4 & m1) | (y3 & ~m1);
       } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = e[j] & (0u - (((uint32_t)gd[i] >> j) & 1u));
+        for (int j = 0; j < 4; ++j) v[j] = e[j] & (0u - ((sh >> j) & 1u));
       }
       *(u32x4_t*)(tb + (kg * KPT + i) * kBPitch + vc * 16) = v;
     }
@@ -361,14 +389,14 @@ __global__ __launch_bounds__(256) void conv_f32_kernel(const ConvParams p) {
   const int nk = (p.Kdim + BK - 1) / BK;
   const int kt0 = (int)((int64_t)split * nk / p.splits), kt1 = (int)((int64_t)(split + 1) * nk / p.splits);
   la.template load<AFULL>(Wg, m0, p.Fg, kt0 * BK, p.Kdim, p.Kdim, 1);
-  gather_issue(kt0);
+  gather_issue();
   la.store(smem);
   gather_finish(smem + kABytes);
   __syncthreads();
   int cur = 0;
   for (int kt = kt0; kt + 1 < kt1; ++kt) {
     la.template load<AFULL>(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
-    gather_issue(kt + 1);
+    gather_issue();
     mma(smem + cur * kBuf, smem + cur * kBuf + kABytes);
     la.store(smem + (cur ^ 1) * kBuf);
     gather_finish(smem + (cur ^ 1) * kBuf + kABytes);
@@ -537,7 +565,7 @@ int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   if constexpr (sizeof(T) == 4) {
     static const bool old_env = getenv("LLC_CONV_OLD") != nullptr;  // experiment hook
     if (w_vec && !old_env && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
-        ((uintptr_t)p.X % 4) == 0)
+        ((uintptr_t)p.X % 4) == 0 && (int64_t)p.N * p.C * p.H * p.Wd < ((int64_t)1 << 30))  // 32-bit byte offsets
       return launch_f32(p, groups, s);
   }
   if (w_vec) return launch_tiles<T, kLoadKVec>(p, groups, s);

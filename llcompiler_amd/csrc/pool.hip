@@ -17,7 +17,10 @@ struct PoolParams {
 };
 
 
-template <int DT>
+// K > 0: a K x K window known at compile time.  All K*K loads are issued unconditionally from indices
+// clamped into the plane, then combined (a load guarded by the window test compiles to a branch with a wait:
+// one memory round trip per tap).  K == 0: any window, tap by tap.
+template <int DT, int K>
 __global__ __launch_bounds__(256) void max_pool_kernel(const PoolParams p) {
   const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (o >= p.total) return;
@@ -27,6 +30,31 @@ __global__ __launch_bounds__(256) void max_pool_kernel(const PoolParams p) {
   const int64_t nc = t / p.OH;
   const int64_t plane = nc * p.H * p.W;
   float acc = p.init_zero ? 0.0f : -INFINITY;
+  if constexpr (K > 0) {
+    float tap[K * K];
+    bool ok[K * K];
+#pragma unroll
+    for (int kh = 0; kh < K; ++kh) {
+      const int ih = oh * p.sh - p.ph + kh * p.dh;
+      const int ch = ih < 0 ? 0 : (ih >= p.H ? p.H - 1 : ih);
+#pragma unroll
+      for (int kw = 0; kw < K; ++kw) {
+        const int iw = ow * p.sw - p.pw + kw * p.dw;
+        const int cw = iw < 0 ? 0 : (iw >= p.W ? p.W - 1 : iw);
+        ok[kh * K + kw] = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+        const int64_t i = plane + (int64_t)ch * p.W + cw;
+        if constexpr (DT == LLC_FLOAT32) tap[kh * K + kw] = ((const float*)p.x)[i];
+        else if constexpr (DT == LLC_BFLOAT16) tap[kh * K + kw] = bf16_bits_to_f32(((const uint16_t*)p.x)[i]);
+        else tap[kh * K + kw] = f16_bits_to_f32(((const uint16_t*)p.x)[i]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < K * K; ++j) {
+      const float v = tap[j];
+      const float m = (v > acc || v != v) ? v : acc;  // NaN propagates, like stablehlo.maximum / torch
+      acc = ok[j] ? m : acc;
+    }
+  } else
   for (int kh = 0; kh < p.KH; ++kh) {
     const int ih = oh * p.sh - p.ph + kh * p.dh;
     if (ih < 0 || ih >= p.H) continue;
@@ -93,8 +121,14 @@ extern "C" int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* at, l
   const int64_t blocks = (p.total + 255) / 256;
   if (blocks > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "max_pool: output too large");
   hipStream_t s = as_stream(stream);
-  if (a.dtype == LLC_FLOAT32) hipLaunchKernelGGL((max_pool_kernel<LLC_FLOAT32>), dim3((unsigned)blocks), dim3(256), 0, s, p);
-  else if (a.dtype == LLC_BFLOAT16) hipLaunchKernelGGL((max_pool_kernel<LLC_BFLOAT16>), dim3((unsigned)blocks), dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((max_pool_kernel<LLC_FLOAT16>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+  const bool k3 = p.KH == 3 && p.KW == 3, k2 = p.KH == 2 && p.KW == 2;
+#define LLC_POOL_LAUNCH(DT)                                                                                         \
+  if (k3) hipLaunchKernelGGL((max_pool_kernel<DT, 3>), dim3((unsigned)blocks), dim3(256), 0, s, p);                 \
+  else if (k2) hipLaunchKernelGGL((max_pool_kernel<DT, 2>), dim3((unsigned)blocks), dim3(256), 0, s, p);            \
+  else hipLaunchKernelGGL((max_pool_kernel<DT, 0>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+  if (a.dtype == LLC_FLOAT32) { LLC_POOL_LAUNCH(LLC_FLOAT32) }
+  else if (a.dtype == LLC_BFLOAT16) { LLC_POOL_LAUNCH(LLC_BFLOAT16) }
+  else { LLC_POOL_LAUNCH(LLC_FLOAT16) }
+#undef LLC_POOL_LAUNCH
   return check_launch("max_pool_kernel");
 }
