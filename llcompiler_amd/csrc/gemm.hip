@@ -665,6 +665,17 @@ int launch_tiles(const GemmParams& p, int batch, hipStream_t s) {
   const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch;
   static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
   const bool deep = p.K >= 512;
+  static const int tile_env = getenv("LLC_GEMM_TILE") ? atoi(getenv("LLC_GEMM_TILE")) : 0;  // experiment hook
+  if (tile_env == 64) return launch_cfg<T, 64, 64, 2, 2, LA, LB>(p, batch, s);
+  if (tile_env == 12864) return launch_cfg<T, 128, 64, 2, 2, LA, LB>(p, batch, s);
+  if constexpr (sizeof(T) == 4) {
+    // fp32 is bound by the (slow) fp32 MFMA, not by LDS or L2: what counts is how evenly the tiles fill the
+    // 256 CUs.  A last round that is mostly empty costs more than the ~7% a 64x64 tile loses to a 128x128 one.
+    auto fill = [](int64_t blocks) { return (double)blocks / (double)(((blocks + 255) / 256) * 256); };
+    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * batch;
+    if (p.N > 64 && p.M > 64 && fill(t128) < 0.8 && fill(t64) > fill(t128) + 0.1)
+      return launch_cfg<T, 64, 64, 2, 2, LA, LB>(p, batch, s);
+  }
   if (p.N > 64 && p.M > 64 && t128 >= 128) {
     if constexpr (LA != kLoadGeneric) {  // the element-wise loader needs too many registers for 8 waves
       if ((deep && cfg_env != 4) || cfg_env == 8) return launch_cfg<T, 128, 128, 4, 2, LA, LB>(p, batch, s);
