@@ -416,6 +416,7 @@ class ExecutionEngine:
         self.graph = graph
         self.steps = make_plan(graph)
         self.instances = {}
+        self._fast = {}
 
     def run(self, *args):
         raise NotImplementedError
@@ -456,6 +457,15 @@ class Torch_ExecutionEngine(ExecutionEngine):
         # ([inputs...]) case, as in the reference
         if len(args) == 1 and isinstance(args[0], (list, tuple)):
             args = tuple(args[0])
+        # a call whose arguments look exactly like an earlier, validated one (same ints, same tensor types,
+        # shapes, strides and devices) goes straight to that call's instance
+        fast_key = tuple(a if not isinstance(a, torch.Tensor) else (a.dtype, a.shape, a.stride(), a.device) for a in args)
+        hit = self._fast.get(fast_key)
+        if hit is not None:
+            results = hit.run([a for a in args if isinstance(a, torch.Tensor)])
+            if getattr(self.graph, "single_output", len(results) == 1) and len(results) == 1:
+                return results[0]
+            return results
         inputs = self.trans_to_tensor(*args)
         g = self.graph
         if len(inputs) != len(g.inputs):
@@ -478,6 +488,7 @@ class Torch_ExecutionEngine(ExecutionEngine):
             C.init(device.index or 0)
             inst = Instance(g, self.steps, env, inputs, device)
             self.instances[key] = inst
+        self._fast[fast_key] = inst
         results = inst.run(inputs)
         if getattr(g, "single_output", len(results) == 1) and len(results) == 1:
             return results[0]
