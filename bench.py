@@ -219,8 +219,8 @@ def model_latencies():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-models", action="store_true", help="skip the end-to-end latencies of the model configurations")
     ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
@@ -242,8 +242,10 @@ def main():
 
     torch.cuda.synchronize()
     ms_per_step = time_gpu(step, args.steps, args.warmup)
-    # per-kernel average durations, each in its own timed loop
-    kernels = [roofline_of(c, time_gpu(c.run, args.steps, args.warmup)) for c in cases]
+    # per-kernel average durations, each in its own timed loop of at least 100 launches after 20 untimed ones:
+    # a few milliseconds of work after an idle period run below the sustained clocks (the fp32 matmul reads 155 us
+    # over 20 launches and 134 us over 100)
+    kernels = [roofline_of(c, time_gpu(c.run, max(args.steps, 100), max(args.warmup, 20))) for c in cases]
     dominant = max(kernels, key=lambda k: k["avg_ms"])
     out = {
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,

@@ -264,10 +264,22 @@ __device__ __forceinline__ void mma_tile(const char* ta, int arow, const char* t
     for (int i = 0; i < TM; ++i) fa[i] = *(const u32x4_t*)(ta + abase[i] + (((2 * s + lh) ^ aswz[i]) << 4));
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[j] = *(const u32x4_t*)(tb + bbase[j] + (((2 * s + lh) ^ bswz[j]) << 4));
+    if constexpr (sizeof(T) == 4) {
+      // four fp32 MFMAs per fragment pair (one per k slot of the 16-byte chunk): walk the k slots outermost so
+      // that consecutive MFMAs write different accumulators instead of forming a dependent chain of four
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) mfma_step<T>(fa[i], fb[j], acc[i][j]);
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(fa[i][q]), __uint_as_float(fb[j][q]), acc[i][j], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mfma_step<T>(fa[i], fb[j], acc[i][j]);
+    }
   }
 }
 
