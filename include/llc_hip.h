@@ -100,7 +100,10 @@ int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilo
                    void* stream);
 
 /* llh.batch_matmul (LLHOps.td:446-452; LLHToHLO.cpp:363-382: batch dims {0}/{0}, contracting lhs
- * dim 2 with rhs dim 1): rank 3.  The two inner dims of each operand may be a transposed view. */
+ * dim 2 with rhs dim 1): rank 3.  The two inner dims of each operand may be a transposed view.
+ * Extension: either operand (and the contiguous output) may be rank 4, [B0, B1, rows, cols], with any
+ * strides on the two batch dims; batch b of the op is (b / B1, b % B1).  The head split of an attention
+ * layer, [B, S, H*D] viewed as [B, H, S, D], is then read in place instead of being copied first. */
 int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                          void* stream);
 

@@ -59,6 +59,10 @@ struct GemmParams {
   int64_t a_sm, a_sk, a_sb;  // element strides of A along m, k, batch
   int64_t b_sk, b_sn, b_sb;  // element strides of B along k, n, batch
   int64_t c_sb;              // batch stride of C (rows are contiguous, pitch N)
+  // Two-level batches ([B0, B1, M, K] operands: attention heads taken as a strided view of [B, S, H*D]):
+  // batch z = z0 * bdiv + z1 reads A + z0 * a_sb + z1 * a_sb1.  One-level batches have bdiv = 1.
+  int64_t a_sb1, b_sb1;
+  int32_t bdiv;
   float alpha;
   int32_t act;
   int32_t tiles_m, tiles_n;
@@ -78,8 +82,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int z = blockIdx.z;
-  const T* A = (const T*)p.A + (int64_t)z * p.a_sb;
-  const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
+  const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
+  const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
+  const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int wm = wave / WN, wn = wave % WN;
@@ -281,8 +286,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * 128, n0 = tile_n * 128;
   const int z = blockIdx.z;
-  const T* A = (const T*)p.A + (int64_t)z * p.a_sb;
-  const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
+  const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
+  const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
+  const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
   const int li = lane % 32, lh = lane / 32;
@@ -477,8 +483,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * 128, n0 = tile_n * 128;
   const int z = blockIdx.z;
-  const T* A = (const T*)p.A + (int64_t)z * p.a_sb;
-  const T* B = (const T*)p.B + (int64_t)z * p.b_sb;
+  const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
+  const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
+  const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int ks = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
   const int li = lane % 32, lh = lane / 32;
@@ -690,9 +697,9 @@ template <typename T>
 int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
   auto al16 = [](const void* q) { return ((uintptr_t)q % 16) == 0; };
-  const bool a_kvec = p.a_sk == 1 && p.a_sm % EPV == 0 && p.a_sb % EPV == 0 && p.K % EPV == 0 && al16(p.A);
-  const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.K % EPV == 0 && al16(p.B);
-  const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.N % EPV == 0 && al16(p.B);
+  const bool a_kvec = p.a_sk == 1 && p.a_sm % EPV == 0 && p.a_sb % EPV == 0 && p.a_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.A);
+  const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.B);
+  const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.N % EPV == 0 && al16(p.B);
   if constexpr (sizeof(T) == 2) {
     static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
@@ -780,6 +787,7 @@ extern "C" int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, cons
   p.a_sk = a.stride[1];
   p.b_sk = b.stride[0];
   p.b_sn = b.stride[1];
+  p.bdiv = 1;
   LLC_TRY(fill_epilogue(epi, o, p.N, &p));
   return gemm_dispatch(a.dtype, p, 1, as_stream(stream));
 }
@@ -790,37 +798,58 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
   LLC_TRY(make_view(lhs, "batch_matmul lhs", &a));
   LLC_TRY(make_view(rhs, "batch_matmul rhs", &b));
   LLC_TRY(make_view(out, "batch_matmul out", &o));
-  if (a.rank != 3 || b.rank != 3 || o.rank != 3) return set_error(LLC_ERR_SHAPE, "batch_matmul: rank-3 tensors expected (LLH_3DTensor)");
+  // LLH_3DTensor operands; as an extension an operand may be rank 4, [B0, B1, M, K]: the head split of an
+  // attention layer is then a strided view of the [B, S, H*D] activation instead of a copy.
+  if ((a.rank != 3 && a.rank != 4) || (b.rank != 3 && b.rank != 4) || (o.rank != 3 && o.rank != 4))
+    return set_error(LLC_ERR_SHAPE, "batch_matmul: rank-3 tensors expected (LLH_3DTensor), or rank 4 with two batch dims");
   if (a.dtype != b.dtype || a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "batch_matmul: operand types differ");
-  if (a.size[0] != b.size[0] || o.size[0] != a.size[0] || a.size[2] != b.size[1] || o.size[1] != a.size[1] || o.size[2] != b.size[2])
-    return set_error(LLC_ERR_SHAPE, "batch_matmul: [%lld,%lld,%lld] x [%lld,%lld,%lld] -> [%lld,%lld,%lld]", (long long)a.size[0],
-                     (long long)a.size[1], (long long)a.size[2], (long long)b.size[0], (long long)b.size[1], (long long)b.size[2],
-                     (long long)o.size[0], (long long)o.size[1], (long long)o.size[2]);
+  const int ra = a.rank - 2, rb = b.rank - 2, ro = o.rank - 2;  // number of batch dims
+  const int64_t nba = ra == 2 ? a.size[0] * a.size[1] : a.size[0], nbb = rb == 2 ? b.size[0] * b.size[1] : b.size[0];
+  const int64_t nbo = ro == 2 ? o.size[0] * o.size[1] : o.size[0];
+  int64_t bdiv = 1;
+  if (ra == 2) bdiv = a.size[1];
+  if (rb == 2) {
+    if (ra == 2 && b.size[1] != bdiv) return set_error(LLC_ERR_SHAPE, "batch_matmul: inner batch extents differ");
+    bdiv = b.size[1];
+  }
+  if (nba != nbb || nbo != nba || a.size[ra + 1] != b.size[rb] || o.size[ro] != a.size[ra] || o.size[ro + 1] != b.size[rb + 1] ||
+      (bdiv > 0 && nba % (bdiv ? bdiv : 1) != 0))
+    return set_error(LLC_ERR_SHAPE, "batch_matmul: [%lld x %lld,%lld] x [%lld x %lld,%lld] -> [%lld x %lld,%lld]", (long long)nba,
+                     (long long)a.size[ra], (long long)a.size[ra + 1], (long long)nbb, (long long)b.size[rb], (long long)b.size[rb + 1],
+                     (long long)nbo, (long long)o.size[ro], (long long)o.size[ro + 1]);
   if (!o.contiguous()) return set_error(LLC_ERR_LAYOUT, "batch_matmul: output must be contiguous");
-  if (a.size[1] > 0x7fffffff || a.size[2] > 0x7fffffff || b.size[2] > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "batch_matmul: extent too large");
+  if (a.size[ra] > 0x7fffffff || a.size[ra + 1] > 0x7fffffff || b.size[rb + 1] > 0x7fffffff || bdiv > 0x7fffffff)
+    return set_error(LLC_ERR_TOO_LARGE, "batch_matmul: extent too large");
   GemmParams p{};
   p.A = a.ptr;
   p.B = b.ptr;
   p.C = o.ptr;
-  p.M = (int)a.size[1];
-  p.K = (int)a.size[2];
-  p.N = (int)b.size[2];
-  p.a_sb = a.stride[0];
-  p.a_sm = a.stride[1];
-  p.a_sk = a.stride[2];
-  p.b_sb = b.stride[0];
-  p.b_sk = b.stride[1];
-  p.b_sn = b.stride[2];
+  p.M = (int)a.size[ra];
+  p.K = (int)a.size[ra + 1];
+  p.N = (int)b.size[rb + 1];
+  p.bdiv = (int)(bdiv > 0 ? bdiv : 1);
+  // batch z = z0 * bdiv + z1; a one-level operand with batch stride s is (bdiv * s, s)
+  if (ra == 2) { p.a_sb = a.stride[0]; p.a_sb1 = a.stride[1]; }
+  else { p.a_sb = a.stride[0] * p.bdiv; p.a_sb1 = a.stride[0]; }
+  p.a_sm = a.stride[ra];
+  p.a_sk = a.stride[ra + 1];
+  if (rb == 2) { p.b_sb = b.stride[0]; p.b_sb1 = b.stride[1]; }
+  else { p.b_sb = b.stride[0] * p.bdiv; p.b_sb1 = b.stride[0]; }
+  p.b_sk = b.stride[rb];
+  p.b_sn = b.stride[rb + 1];
   p.c_sb = (int64_t)p.M * p.N;
   LLC_TRY(fill_epilogue(epi, o, p.N, &p));
   // blockIdx.z carries the batch; larger batches are issued in slices
   hipStream_t s = as_stream(stream);
-  const int64_t nb = a.size[0];
-  for (int64_t z0 = 0; z0 < nb; z0 += 65535) {
+  const int64_t nb = nba;
+  // slices of whole outer batches, at most 65535 batches each
+  const int64_t per = p.bdiv > 65535 ? 0 : (65535 / p.bdiv) * p.bdiv;
+  if (per == 0) return set_error(LLC_ERR_TOO_LARGE, "batch_matmul: inner batch extent %d", p.bdiv);
+  for (int64_t z0 = 0; z0 < nb; z0 += per) {
     GemmParams q = p;
-    const int cnt = (int)((nb - z0) < 65535 ? (nb - z0) : 65535);
-    q.A = p.A + z0 * p.a_sb * (int64_t)a.esize();
-    q.B = p.B + z0 * p.b_sb * (int64_t)a.esize();
+    const int cnt = (int)((nb - z0) < per ? (nb - z0) : per);
+    q.A = p.A + (z0 / p.bdiv) * p.a_sb * (int64_t)a.esize();
+    q.B = p.B + (z0 / p.bdiv) * p.b_sb * (int64_t)a.esize();
     q.C = p.C + z0 * p.c_sb * (int64_t)a.esize();
     if (p.residual) q.residual = p.residual + z0 * p.c_sb * (int64_t)a.esize();
     LLC_TRY(gemm_dispatch(a.dtype, q, cnt, s));

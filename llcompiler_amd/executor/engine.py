@@ -63,6 +63,16 @@ class _Pool:
         self.free.setdefault(buf.numel(), []).append(buf)
 
 
+class _LazyReshape:
+    """A reshape that is not a view of its source (e.g. the head split [B,S,H,D] -> permute -> [B*H,S,D]): the
+    copy is made only if a consumer needs the reshaped tensor; batch_matmul reads the 4-D source in place."""
+
+    __slots__ = ("src", "shape", "done")
+
+    def __init__(self, src, shape):
+        self.src, self.shape, self.done = src, tuple(shape), None
+
+
 class Instance:
     """A plan specialised to concrete extents: a flat list of prepared kernel calls."""
 
@@ -167,9 +177,32 @@ class Instance:
                 self._launch_later(ops.copy(t, out=c, defer=True))
             return c
 
+        def materialise(x):
+            if isinstance(x, _LazyReshape):
+                if x.done is None:
+                    n = x.src.numel()
+                    buf = pool.take(n * x.src.dtype.itemsize)
+                    self.keep.append(buf)  # stays private to this instance
+                    c = buf[: n * x.src.dtype.itemsize].view(x.src.dtype).view(tuple(x.src.shape))
+                    if n:
+                        self._launch_later(ops.copy(x.src, out=c, defer=True))
+                    x.done = c.view(x.shape)
+                return x.done
+            return x
+
+        def batched_operand(x):
+            """A lazy [B0*B1, R, C] reshape of a 4-D tensor goes to batch_matmul as that 4-D tensor."""
+            if isinstance(x, _LazyReshape) and x.done is None and x.src.dim() == 4 and \
+                    x.shape == (x.src.shape[0] * x.src.shape[1], x.src.shape[2], x.src.shape[3]):
+                return x.src
+            return materialise(x)
+
         for si, st in enumerate(steps):
             k = st.kind
-            ins = [val[id(v)] for v in st.inputs]
+            if k == "batch_matmul":
+                ins = [batched_operand(val[id(v)]) for v in st.inputs]
+            else:
+                ins = [materialise(val[id(v)]) for v in st.inputs]
             if k == "view":
                 before = len(temps)
                 val[id(st.output)] = self._view(st, ins[0], contiguous)
@@ -191,8 +224,8 @@ class Instance:
                 e = st.attrs["epilogue"]
                 out = new_tensor(st.output)
                 natural = _concrete(st.attrs["natural_shape"], self.env)
-                bias = val[id(e["bias"])] if e["bias"] is not None else None
-                res = val[id(e["residual"])] if e["residual"] is not None else None
+                bias = materialise(val[id(e["bias"])]) if e["bias"] is not None else None
+                res = materialise(val[id(e["residual"])]) if e["residual"] is not None else None
                 if bias is not None:
                     bias = contiguous(bias.reshape(-1) if bias.is_contiguous() else bias).reshape(-1)
                 if res is not None:
@@ -259,7 +292,7 @@ class Instance:
         self.output_plan = []
         for o in g.outputs:
             if isinstance(o, Value):
-                t = val[id(o)]
+                t = materialise(val[id(o)])
                 root = self._roots.get(t.untyped_storage().data_ptr())
                 if root is None or root[0] != "out" or not t.is_contiguous():
                     # an output that aliases an input or an intermediate view: materialise it per call
@@ -294,7 +327,7 @@ class Instance:
             try:
                 return t.view(shape)
             except RuntimeError:
-                return contiguous(t).view(shape)
+                return _LazyReshape(t, shape)
         if op == "transpose":
             return t.permute(*a["perms"])
         if op == "broadcast_to":

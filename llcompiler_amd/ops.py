@@ -78,7 +78,10 @@ def matmul(a, b, epilogue=None, out=None, defer=False):
 def batch_matmul(a, b, epilogue=None, out=None, defer=False):
     dev = _dev(a)
     if out is None:
-        out = torch.empty((a.shape[0], a.shape[1], b.shape[2]), dtype=a.dtype, device=dev)
+        nb = 1
+        for d in a.shape[:-2]:
+            nb *= d
+        out = torch.empty((nb, a.shape[-2], b.shape[-1]), dtype=a.dtype, device=dev)
     ra, rb, ro = C.tensor_ref(a), C.tensor_ref(b), C.tensor_ref(out)
     return _launch(C.lib().llc_hip_batch_matmul, (ra.ptr, rb.ptr, _epi(epilogue), ro.ptr), (ra, rb, ro, epilogue), out,
                    dev, defer)

@@ -379,6 +379,33 @@ def test_batch_matmul(ops, oracle, B, M, N, K):
     assert_close_bf16(host(gotb), bf16_round(oracle.batch_matmul(ab, bb, "mkn")), "bmm bf16")
 
 
+def test_batch_matmul_two_level_batches(ops, oracle):
+    """Rank-4 operands [B0, B1, M, K]: the attention head split read in place from a [B, S, H*D] activation
+    (q and v as permuted views, k as the permuted and transposed view), against the oracle on materialised
+    copies.  fp32 (register-staged kernel) and bf16 (direct-to-LDS kernel for the scores shape)."""
+    r = rng(91)
+    B, S, H, D = 4, 256, 8, 64
+    q = r.uniform(-1, 1, (B, S, H * D)).astype(np.float32)
+    k = r.uniform(-1, 1, (B, S, H * D)).astype(np.float32)
+    v = r.uniform(-1, 1, (B, S, H * D)).astype(np.float32)
+    heads = lambda x: np.ascontiguousarray(x.reshape(B, S, H, D).transpose(0, 2, 1, 3)).reshape(B * H, S, D)
+    kt = np.ascontiguousarray(heads(k).transpose(0, 2, 1))
+    for dt, close, rnd in ((torch.float32, assert_close_f32, lambda x: x), (torch.bfloat16, assert_close_bf16, bf16_round)):
+        qd, kd, vd = (dev(rnd(x), dt) for x in (q, k, v))
+        q4 = qd.view(B, S, H, D).permute(0, 2, 1, 3)
+        k4 = kd.view(B, S, H, D).permute(0, 2, 3, 1)
+        v4 = vd.view(B, S, H, D).permute(0, 2, 1, 3)
+        scores = ops.batch_matmul(q4, k4, ops.Epilogue(alpha=0.125))
+        want = oracle.batch_matmul(heads(rnd(q)), np.ascontiguousarray(heads(rnd(k)).transpose(0, 2, 1)), "mkn") * np.float32(0.125)
+        assert tuple(scores.shape) == (B * H, S, S)
+        close(host(scores), rnd(want), "scores %s" % dt)
+        # one-level lhs with a two-level rhs
+        p = r.uniform(0, 1, (B * H, S, S)).astype(np.float32)
+        ctx = ops.batch_matmul(dev(rnd(p), dt), v4)
+        close(host(ctx), rnd(oracle.batch_matmul(rnd(p), heads(rnd(v)), "mkn")), "context %s" % dt)
+    del kt
+
+
 def test_matmul_shape_errors(ops):
     from llcompiler_amd._capi import LlcHipError
     with pytest.raises(LlcHipError, match="matmul"):
