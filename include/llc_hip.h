@@ -103,7 +103,9 @@ int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilo
  * dim 2 with rhs dim 1): rank 3.  The two inner dims of each operand may be a transposed view.
  * Extension: either operand (and the contiguous output) may be rank 4, [B0, B1, rows, cols], with any
  * strides on the two batch dims; batch b of the op is (b / B1, b % B1).  The head split of an attention
- * layer, [B, S, H*D] viewed as [B, H, S, D], is then read in place instead of being copied first. */
+ * layer, [B, S, H*D] viewed as [B, H, S, D], is then read in place instead of being copied first.  A rank-4
+ * output may also be strided (unit stride on its last dim; no residual then): the head merge back to
+ * [B, S, H*D] is written in place. */
 int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                          void* stream);
 

@@ -58,7 +58,8 @@ struct GemmParams {
   int32_t M, N, K;
   int64_t a_sm, a_sk, a_sb;  // element strides of A along m, k, batch
   int64_t b_sk, b_sn, b_sb;  // element strides of B along k, n, batch
-  int64_t c_sb;              // batch stride of C (rows are contiguous, pitch N)
+  int64_t c_sb;              // batch stride of C (outer batch stride when bdiv > 1)
+  int64_t c_sb1, c_sm;       // inner batch stride and row pitch of C (c_sm = N, c_sb1 = M N for a contiguous output)
   // Two-level batches ([B0, B1, M, K] operands: attention heads taken as a strided view of [B, S, H*D]):
   // batch z = z0 * bdiv + z1 reads A + z0 * a_sb + z1 * a_sb1.  One-level batches have bdiv = 1.
   int64_t a_sb1, b_sb1;
@@ -149,8 +150,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   // ---- epilogue.  32x32 accumulator layout: register r of lane (li, lh) is row 8*(r/4) + 4*lh + r%4,
   //      column li: for fixed r, 32 lanes store 32 consecutive columns of one row. ----
   if (!LLC_DBG_EPI && p.alpha != 123.0f) return;
-  T* C = (T*)p.C + (int64_t)z * p.c_sb;
-  const char* res = p.residual ? p.residual + (int64_t)z * p.c_sb * (int64_t)sizeof(T) : nullptr;
+  const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
+  T* C = (T*)p.C + c_off;
+  const char* res = p.residual ? p.residual + c_off * (int64_t)sizeof(T) : nullptr;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
         if (!FULL && row >= p.M) continue;
-        epilogue_store<T>(C, (int64_t)row * p.N + col, acc[i][j][r], p.alpha, bv, res, p.act);
+        epilogue_store<T>(C, (int64_t)row * p.c_sm + col, acc[i][j][r], p.alpha, bv, res, p.act);
       }
     }
   }
@@ -399,8 +401,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
         stage[row * kStagePitch + wn * 64 + j * 32 + li] = acc[i][j][r];
       }
   __syncthreads();
-  T* C = (T*)p.C + (int64_t)z * p.c_sb;
-  const T* res = p.residual ? (const T*)p.residual + (int64_t)z * p.c_sb : nullptr;
+  const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
+  T* C = (T*)p.C + c_off;
+  const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int vid = it * 512 + threadIdx.x;
@@ -416,7 +419,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
       v[4 * h + 2] = x.z + y.z;
       v[4 * h + 3] = x.w + y.w;
     }
-    const int64_t o = (int64_t)(m0 + row) * p.N + n0 + c0;
+    const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
     if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
@@ -590,8 +593,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
     __syncthreads();
   }
-  T* C = (T*)p.C + (int64_t)z * p.c_sb;
-  const T* res = p.residual ? (const T*)p.residual + (int64_t)z * p.c_sb : nullptr;
+  const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
+  T* C = (T*)p.C + c_off;
+  const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int vid = it * 512 + threadIdx.x;
@@ -606,7 +610,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       v[4 * h + 2] = x[2];
       v[4 * h + 3] = x[3];
     }
-    const int64_t o = (int64_t)(m0 + row) * p.N + n0 + c0;
+    const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
     if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
@@ -704,7 +708,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
     static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
     if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
-        tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && (!p.bias || al16(p.bias)) &&
+        tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 && p.c_sm % EPV == 0 && (!p.bias || al16(p.bias)) &&
         (!p.residual || al16(p.residual)))
     {
       // short reductions, or more tiles than one round of workgroups: two workgroups per CU
@@ -788,6 +792,7 @@ extern "C" int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, cons
   p.b_sk = b.stride[0];
   p.b_sn = b.stride[1];
   p.bdiv = 1;
+  p.c_sm = p.N;
   LLC_TRY(fill_epilogue(epi, o, p.N, &p));
   return gemm_dispatch(a.dtype, p, 1, as_stream(stream));
 }
@@ -812,12 +817,21 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
     if (ra == 2 && b.size[1] != bdiv) return set_error(LLC_ERR_SHAPE, "batch_matmul: inner batch extents differ");
     bdiv = b.size[1];
   }
+  if (ro == 2) {
+    if ((ra == 2 || rb == 2) && o.size[1] != bdiv) return set_error(LLC_ERR_SHAPE, "batch_matmul: inner batch extents differ");
+    bdiv = o.size[1];
+  }
   if (nba != nbb || nbo != nba || a.size[ra + 1] != b.size[rb] || o.size[ro] != a.size[ra] || o.size[ro + 1] != b.size[rb + 1] ||
       (bdiv > 0 && nba % (bdiv ? bdiv : 1) != 0))
     return set_error(LLC_ERR_SHAPE, "batch_matmul: [%lld x %lld,%lld] x [%lld x %lld,%lld] -> [%lld x %lld,%lld]", (long long)nba,
                      (long long)a.size[ra], (long long)a.size[ra + 1], (long long)nbb, (long long)b.size[rb], (long long)b.size[rb + 1],
                      (long long)nbo, (long long)o.size[ro], (long long)o.size[ro + 1]);
-  if (!o.contiguous()) return set_error(LLC_ERR_LAYOUT, "batch_matmul: output must be contiguous");
+  // the output is contiguous, or (rank 4) has unit-stride columns and any strides on rows and batches: the
+  // head merge [B, H, S, D] -> [B, S, H*D] is then written in place
+  const bool o_strided = !o.contiguous();
+  if (o_strided && (ro != 2 || o.stride[3] != 1 || o.size[1] != bdiv))
+    return set_error(LLC_ERR_LAYOUT, "batch_matmul: output must be contiguous, or rank 4 with unit-stride columns");
+  if (o_strided && epi && epi->residual) return set_error(LLC_ERR_UNSUPPORTED, "batch_matmul: residual with a strided output");
   if (a.size[ra] > 0x7fffffff || a.size[ra + 1] > 0x7fffffff || b.size[rb + 1] > 0x7fffffff || bdiv > 0x7fffffff)
     return set_error(LLC_ERR_TOO_LARGE, "batch_matmul: extent too large");
   GemmParams p{};
@@ -837,7 +851,15 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
   else { p.b_sb = b.stride[0] * p.bdiv; p.b_sb1 = b.stride[0]; }
   p.b_sk = b.stride[rb];
   p.b_sn = b.stride[rb + 1];
-  p.c_sb = (int64_t)p.M * p.N;
+  if (o_strided) {
+    p.c_sb = o.stride[0];
+    p.c_sb1 = o.stride[1];
+    p.c_sm = o.stride[2];
+  } else {
+    p.c_sb1 = (int64_t)p.M * p.N;
+    p.c_sb = p.c_sb1 * p.bdiv;
+    p.c_sm = p.N;
+  }
   LLC_TRY(fill_epilogue(epi, o, p.N, &p));
   // blockIdx.z carries the batch; larger batches are issued in slices
   hipStream_t s = as_stream(stream);
@@ -850,8 +872,8 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
     const int cnt = (int)((nb - z0) < per ? (nb - z0) : per);
     q.A = p.A + (z0 / p.bdiv) * p.a_sb * (int64_t)a.esize();
     q.B = p.B + (z0 / p.bdiv) * p.b_sb * (int64_t)a.esize();
-    q.C = p.C + z0 * p.c_sb * (int64_t)a.esize();
-    if (p.residual) q.residual = p.residual + z0 * p.c_sb * (int64_t)a.esize();
+    q.C = p.C + (z0 / p.bdiv) * p.c_sb * (int64_t)a.esize();
+    if (p.residual) q.residual = p.residual + (z0 / p.bdiv) * p.c_sb * (int64_t)a.esize();
     LLC_TRY(gemm_dispatch(a.dtype, q, cnt, s));
   }
   return LLC_OK;

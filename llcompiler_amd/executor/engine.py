@@ -197,8 +197,30 @@ class Instance:
                 return x.src
             return materialise(x)
 
+        consumers = {}
+        for st in steps:
+            for v in st.inputs:
+                consumers.setdefault(id(v), []).append(st)
+        skip = set()
+
+        def head_merge(st, nb, m, n):
+            """batch_matmul -> reshape [B0,B1,M,N] -> transpose (0,2,1,3), each read once: returns (reshape step,
+            B0, B1) so that the product can be written in the transposed layout directly."""
+            u = consumers.get(id(st.output), [])
+            if len(u) != 1 or u[0].kind != "view" or u[0].attrs["op"] not in ("reshape", "flatten") or id(st.output) in out_ids:
+                return None
+            shp = _concrete(u[0].output.shape, self.env)
+            if len(shp) != 4 or shp[0] * shp[1] != nb or shp[2] != m or shp[3] != n or id(u[0].output) in out_ids:
+                return None
+            u2 = consumers.get(id(u[0].output), [])
+            if len(u2) != 1 or u2[0].kind != "view" or u2[0].attrs["op"] != "transpose" or tuple(u2[0].attrs["perms"]) != (0, 2, 1, 3):
+                return None
+            return u[0], shp[0], shp[1]
+
         for si, st in enumerate(steps):
             k = st.kind
+            if id(st) in skip:
+                continue
             if k == "batch_matmul":
                 ins = [batched_operand(val[id(v)]) for v in st.inputs]
             else:
@@ -237,6 +259,13 @@ class Instance:
                 if k == "matmul":
                     call = ops.matmul(ins[0], ins[1], epi, out=o, defer=True)
                 elif k == "batch_matmul":
+                    hm = head_merge(st, natural[0], natural[1], natural[2]) if (res is None and len(natural) == 3) else None
+                    if hm is not None:
+                        # the head merge that follows, [B0,B1,M,N] -> [B0,M,B1,N], is done by the kernel's stores
+                        r1, b0, b1 = hm
+                        o = out.view(-1).view(b0, natural[1], b1, natural[2]).permute(0, 2, 1, 3)
+                        val[id(r1.output)] = o
+                        skip.add(id(r1))
                     call = ops.batch_matmul(ins[0], ins[1], epi, out=o, defer=True)
                 else:
                     call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],

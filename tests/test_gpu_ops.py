@@ -402,7 +402,12 @@ def test_batch_matmul_two_level_batches(ops, oracle):
         # one-level lhs with a two-level rhs
         p = r.uniform(0, 1, (B * H, S, S)).astype(np.float32)
         ctx = ops.batch_matmul(dev(rnd(p), dt), v4)
-        close(host(ctx), rnd(oracle.batch_matmul(rnd(p), heads(rnd(v)), "mkn")), "context %s" % dt)
+        want_ctx = rnd(oracle.batch_matmul(rnd(p), heads(rnd(v)), "mkn"))
+        close(host(ctx), want_ctx, "context %s" % dt)
+        # the head merge written in place: out is the [B, H, S, D] view of a [B, S, H*D] buffer
+        merged = torch.zeros(B, S, H * D, dtype=dt, device="cuda")
+        ops.batch_matmul(dev(rnd(p), dt), v4, out=merged.view(B, S, H, D).permute(0, 2, 1, 3))
+        close(host(merged), want_ctx.reshape(B, H, S, D).transpose(0, 2, 1, 3).reshape(B, S, H * D), "merged context %s" % dt)
     del kt
 
 
