@@ -85,7 +85,9 @@ const char* llc_hip_status_string(int status);
 typedef enum llc_activation { LLC_ACT_NONE = 0, LLC_ACT_RELU = 1, LLC_ACT_GELU = 2 } llc_activation;
 typedef struct llc_epilogue {
   float alpha;                /* applied to the fp32 accumulator; 1.0f = none */
-  const llc_tensor* bias;     /* rank 1, one value per output column / filter; may be NULL */
+  const llc_tensor* bias;     /* rank 1, one value per output column / filter; may be NULL.  batch_matmul with two
+                                 batch dims also takes rank 2, [B0, N]: one row per outer batch (an attention
+                                 mask [B,1,1,S] added to scores [B,H,S,S]) */
   const llc_tensor* residual; /* same shape as the output, contiguous; may be NULL */
   int act;                    /* llc_activation */
 } llc_epilogue;

@@ -53,7 +53,8 @@ struct GemmParams {
   const char* A;
   const char* B;
   char* C;
-  const char* bias;      // [N] or null, same type as C
+  const char* bias;      // [N] (or [outer batches, N], row pitch bias_sb) or null, same type as C
+  int64_t bias_sb;       // elements between the bias rows of consecutive outer batches (0: one row for all)
   const char* residual;  // [batch, M, N] contiguous or null, same type as C
   int32_t M, N, K;
   int64_t a_sm, a_sk, a_sb;  // element strides of A along m, k, batch
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
     if (!FULL && col >= p.N) continue;
-    const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, col) : 0.0f;
+    const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, (int64_t)z0 * p.bias_sb + col) : 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
     }
     const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
+    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
     u32x4_t outv;
 #pragma unroll
@@ -612,7 +613,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
     const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + n0 + c0);
+    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
     u32x4_t outv;
 #pragma unroll
@@ -708,7 +709,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
     static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
     if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
-        tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 && p.c_sm % EPV == 0 && (!p.bias || al16(p.bias)) &&
+        tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 && p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) &&
         (!p.residual || al16(p.residual)))
     {
       // short reductions, or more tiles than one round of workgroups: two workgroups per CU
@@ -736,10 +737,12 @@ int gemm_dispatch(int dtype, const GemmParams& p, int batch, hipStream_t s) {
   return set_error(LLC_ERR_DTYPE, "matmul: element type %d (f32, bf16 or f16 expected)", dtype);
 }
 
-int fill_epilogue(const llc_epilogue* epi, const View& o, int64_t n_cols, GemmParams* p) {
+// n_outer: number of outer batches (1 for matmul); a bias of n_outer rows gives every outer batch its own
+int fill_epilogue(const llc_epilogue* epi, const View& o, int64_t n_cols, GemmParams* p, int64_t n_outer = 1) {
   p->alpha = 1.0f;
   p->act = LLC_ACT_NONE;
   p->bias = nullptr;
+  p->bias_sb = 0;
   p->residual = nullptr;
   if (!epi) return LLC_OK;
   p->alpha = epi->alpha;
@@ -749,8 +752,11 @@ int fill_epilogue(const llc_epilogue* epi, const View& o, int64_t n_cols, GemmPa
     View b;
     LLC_TRY(make_view(epi->bias, "epilogue bias", &b));
     if (b.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "epilogue: bias type differs from output");
-    if (b.numel() != n_cols || !b.contiguous()) return set_error(LLC_ERR_SHAPE, "epilogue: bias must hold %lld contiguous values", (long long)n_cols);
+    const bool rows = n_outer > 1 && b.rank == 2 && b.size[0] == n_outer && b.size[1] == n_cols;
+    if ((b.numel() != n_cols && !rows) || !b.contiguous())
+      return set_error(LLC_ERR_SHAPE, "epilogue: bias must hold %lld contiguous values (or one such row per outer batch)", (long long)n_cols);
     p->bias = b.ptr;
+    p->bias_sb = rows ? n_cols : 0;
   }
   if (epi->residual) {
     View r;
@@ -860,7 +866,7 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
     p.c_sb = p.c_sb1 * p.bdiv;
     p.c_sm = p.N;
   }
-  LLC_TRY(fill_epilogue(epi, o, p.N, &p));
+  LLC_TRY(fill_epilogue(epi, o, p.N, &p, nba / p.bdiv));
   // blockIdx.z carries the batch; larger batches are issued in slices
   hipStream_t s = as_stream(stream);
   const int64_t nb = nba;
@@ -874,6 +880,7 @@ extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs
     q.B = p.B + (z0 / p.bdiv) * p.b_sb * (int64_t)a.esize();
     q.C = p.C + (z0 / p.bdiv) * p.c_sb * (int64_t)a.esize();
     if (p.residual) q.residual = p.residual + (z0 / p.bdiv) * p.c_sb * (int64_t)a.esize();
+    if (p.bias) q.bias = p.bias + (z0 / p.bdiv) * p.bias_sb * (int64_t)a.esize();
     LLC_TRY(gemm_dispatch(a.dtype, q, cnt, s));
   }
   return LLC_OK;

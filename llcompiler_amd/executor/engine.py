@@ -248,8 +248,13 @@ class Instance:
                 natural = _concrete(st.attrs["natural_shape"], self.env)
                 bias = materialise(val[id(e["bias"])]) if e["bias"] is not None else None
                 res = materialise(val[id(e["residual"])]) if e["residual"] is not None else None
+                bias_rows = bool(e.get("bias_rows"))
                 if bias is not None:
                     bias = contiguous(bias.reshape(-1) if bias.is_contiguous() else bias).reshape(-1)
+                    if bias_rows:  # [B0,1,1,N] -> [B0,N]; the kernel then needs the 4-D shape of the product
+                        full = _concrete(st.output.shape, self.env)
+                        bias = bias.view(full[0], full[3])
+                        natural = full
                 if res is not None:
                     res = contiguous(res)
                 epi = None

@@ -61,6 +61,10 @@ def _numel_static_one(v):
     return all(isinstance(d, int) and d == 1 for d in v.shape)
 
 
+def _same_extent(a, b):
+    return a == b or str(a) == str(b)
+
+
 class Planner:
     def __init__(self, graph):
         self.g = graph
@@ -69,7 +73,7 @@ class Planner:
         self.steps = []
 
     # ------------------------------------------------------------------ contraction epilogues
-    def _is_bias(self, other, out, channel_dim):
+    def _is_bias(self, other, out, channel_dim):  # noqa: C901
         """`other` broadcasts a rank-1 tensor of out.shape[channel_dim] along channel_dim."""
         root, chain = _strip_views(other)
         n = out.shape[channel_dim]
@@ -129,6 +133,14 @@ class Planner:
                 bias = None
                 if epi["bias"] is None and epi["residual"] is None and not reshaped:
                     bias = self._is_bias(other, v, channel_dim)
+                if bias is None and epi["bias"] is None and epi["residual"] is None and reshaped and \
+                        op.name == "batch_matmul" and v.rank == 4 and other.rank == 4 and _strip_views(other)[0] is other and \
+                        other.dtype == v.dtype and _scalar_const(other) is None and \
+                        _same_extent(other.shape[0], v.shape[0]) and _same_extent(other.shape[3], v.shape[3]) and \
+                        all(isinstance(other.shape[d], int) and other.shape[d] == 1 for d in (1, 2)):
+                    # [B0,1,1,N] added to [B0,B1,M,N] (attention mask): one bias row per outer batch
+                    bias = other
+                    epi["bias_rows"] = True
                 if bias is not None:
                     epi["bias"] = bias
                 elif epi["residual"] is None and tuple(other.shape) == tuple(v.shape) and other.dtype == v.dtype and \

@@ -399,6 +399,11 @@ def test_batch_matmul_two_level_batches(ops, oracle):
         want = oracle.batch_matmul(heads(rnd(q)), np.ascontiguousarray(heads(rnd(k)).transpose(0, 2, 1)), "mkn") * np.float32(0.125)
         assert tuple(scores.shape) == (B * H, S, S)
         close(host(scores), rnd(want), "scores %s" % dt)
+        # an attention mask [B,1,1,S] as one bias row per outer batch
+        mask = rnd(np.where(r.uniform(0, 1, (B, S)) < 0.2, -1e4, 0.0).astype(np.float32))
+        masked = ops.batch_matmul(q4, k4, ops.Epilogue(alpha=0.125, bias=dev(mask, dt)))
+        wantm = want.reshape(B, H, S, S) + mask[:, None, None, :]
+        close(host(masked).reshape(B, H, S, S), rnd(wantm), "masked scores %s" % dt)
         # one-level lhs with a two-level rhs
         p = r.uniform(0, 1, (B * H, S, S)).astype(np.float32)
         ctx = ops.batch_matmul(dev(rnd(p), dt), v4)
