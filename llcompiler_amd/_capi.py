@@ -9,8 +9,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# LLC_HIP_LIB selects another build of the same library (e.g. an instrumented one)
-LIB_PATH = os.environ.get("LLC_HIP_LIB") or os.path.join(_HERE, "lib", "libllc_hip.so")
+LIB_PATH = os.path.join(_HERE, "lib", "libllc_hip.so")
 
 LLC_MAX_RANK = 8
 # element type codes: 0-6 are the reference's enum Type (include/llcompiler/Compiler/Tensor.h:25-33)

@@ -13,16 +13,9 @@
 // wave read consecutive pixels, so loads coalesce for stride 1) and writes its run k-contiguous
 // into the same swizzled LDS tile layout the matmul kernel uses.  Weights go through the shared
 // vector loader.  fp32 tensors use the fp32 MFMA, bf16/f16 the 16-bit MFMA; accumulation is fp32.
-#include <cstdlib>
 
 #include "gemm_core.hpp"
 
-#ifndef LLC_DBG_CONV_GATHER
-#define LLC_DBG_CONV_GATHER 1
-#endif
-#ifndef LLC_DBG_CONV_MMA
-#define LLC_DBG_CONV_MMA 1
-#endif
 namespace llc {
 using namespace gemm;
 namespace {
@@ -158,9 +151,9 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
       la.load(Wg, m0, p.Fg, (kt + 1) * BK, p.Kdim, p.Kdim, 1);
-      if (LLC_DBG_CONV_GATHER) lb.load(p, (kt + 1) * BK);
+      lb.load(p, (kt + 1) * BK);
     }
-    if (LLC_DBG_CONV_MMA) mma_tile<T, TM, TN>(smem + cur * kBufBytes, wm * WTM + li, smem + cur * kBufBytes + kABytes, wn * WTN + li, lh, acc);
+    mma_tile<T, TM, TN>(smem + cur * kBufBytes, wm * WTM + li, smem + cur * kBufBytes + kABytes, wn * WTN + li, lh, acc);
     if (kt + 1 < nk) {
       la.store(smem + (cur ^ 1) * kBufBytes);
       lb.store(smem + (cur ^ 1) * kBufBytes + kABytes);
@@ -504,11 +497,9 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
   const int nk = (p.Kdim + 31) / 32;
   // enough workgroups for two per CU, at least eight k-tiles per split
   int splits = 1;
-  static const int target_env = getenv("LLC_CONV_BLOCKS") ? atoi(getenv("LLC_CONV_BLOCKS")) : 512;  // experiment hook
-  static const int mink_env = getenv("LLC_CONV_MINK") ? atoi(getenv("LLC_CONV_MINK")) : 8;          // experiment hook
-  if (tiles * groups < target_env * 3 / 4) {
-    splits = (int)((target_env + tiles * groups - 1) / (tiles * groups));
-    if (splits > nk / mink_env) splits = nk / mink_env;
+  if (tiles * groups < 384) {
+    splits = (int)((512 + tiles * groups - 1) / (tiles * groups));
+    if (splits > nk / 8) splits = nk / 8;
     if (splits < 1) splits = 1;
   }
   p.splits = splits;
@@ -563,8 +554,7 @@ int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
   const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
   if constexpr (sizeof(T) == 4) {
-    static const bool old_env = getenv("LLC_CONV_OLD") != nullptr;  // experiment hook
-    if (w_vec && !old_env && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
+    if (w_vec && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
         ((uintptr_t)p.X % 4) == 0 && (int64_t)p.N * p.C * p.H * p.Wd < ((int64_t)1 << 30))  // 32-bit byte offsets
       return launch_f32(p, groups, s);
   }

@@ -13,7 +13,6 @@
 // collapses the iteration space to at most four dims so that the common cases (same shape, bias
 // over the last dim, per-channel NCHW, attention mask) need at most three integer divisions per
 // vector.
-#include <cstdlib>
 
 #include "common.hpp"
 
@@ -654,11 +653,11 @@ void launch_vec(const EwKernelParams& p, hipStream_t stream) {
 
 template <typename CT>
 int launch(const EwKernelParams& p, int vec, hipStream_t stream) {
-  static const int u_env = getenv("LLC_EW_U") ? atoi(getenv("LLC_EW_U")) : 1;  // experiment hook; one vector per lane measured best
+  // one vector per lane measured best for the 16-byte widths
   if constexpr (sizeof(CT) == 4) {
     switch (vec) {
-      case 8: if (u_env == 2) launch_vec<8, 2, CT>(p, stream); else launch_vec<8, 1, CT>(p, stream); break;
-      case 4: if (u_env == 1) launch_vec<4, 1, CT>(p, stream); else if (u_env == 4) launch_vec<4, 4, CT>(p, stream); else launch_vec<4, 2, CT>(p, stream); break;
+      case 8: launch_vec<8, 1, CT>(p, stream); break;
+      case 4: launch_vec<4, 1, CT>(p, stream); break;
       case 2: launch_vec<2, 2, CT>(p, stream); break;
       default: launch_vec<1, 2, CT>(p, stream); break;
     }
@@ -769,7 +768,6 @@ extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor*
   bool flat = nc == 1;
   // widest vector: 16 bytes of the output type, shrunk until every access stays aligned and inside a row
   int vec = prog->integer ? 2 : (o.esize() <= 2 ? 8 : 4);
-  if (getenv("LLC_EW_VEC16") && o.esize() <= 2) vec = atoi(getenv("LLC_EW_VEC16"));  // experiment hook
   auto aligned = [](const void* ptr, size_t bytes) { return ((uintptr_t)ptr % bytes) == 0; };
   for (size_t k = 0; k < ne; ++k) {
     p.in[k] = ine[k].ptr;

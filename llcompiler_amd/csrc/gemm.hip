@@ -21,29 +21,8 @@
 // XCDs by the hardware, so ids are first regrouped per XCD and then walked in column-grouped order,
 // which gives each XCD's L2 a compact patch of the output (few distinct A row-panels / B
 // column-panels).
-#include <cstdlib>
 
 #include "gemm_core.hpp"
-
-// experiment switches: drop one phase of the main loop to see what the others cost (results are then wrong)
-#ifndef LLC_DBG_LOAD
-#define LLC_DBG_LOAD 1
-#endif
-#ifndef LLC_DBG_MMA
-#define LLC_DBG_MMA 1
-#endif
-#ifndef LLC_DBG_STORE
-#define LLC_DBG_STORE 1
-#endif
-#ifndef LLC_DBG_DMA
-#define LLC_DBG_DMA 1
-#endif
-#ifndef LLC_DBG_READ
-#define LLC_DBG_READ 1
-#endif
-#ifndef LLC_DBG_EPI
-#define LLC_DBG_EPI 1
-#endif
 
 namespace llc {
 using namespace gemm;
@@ -119,17 +98,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 #define LLC_GEMM_STEP(KT, CUR, LA2, LB2, LA1, LB1, GUARDED)                                                     \
   {                                                                                                             \
     /* LA2/LB2: stage that held tile KT (now in LDS) and receives tile KT+2; LA1/LB1 hold tile KT+1 */          \
-    if (LLC_DBG_LOAD && (!(GUARDED) || (KT) + 2 < nk)) {                                                        \
+    if (!(GUARDED) || (KT) + 2 < nk) {                                                        \
       LA2.template load<FULL>(A, m0, p.M, ((KT) + 2) * BK, p.K, p.a_sm, p.a_sk);                                \
       LB2.template load<FULL>(B, n0, p.N, ((KT) + 2) * BK, p.K, p.b_sn, p.b_sk);                                \
     }                                                                                                           \
     /* keep the loads up here: they must be in flight for two tiles, the scheduler would sink them */         \
     \
-    if (LLC_DBG_MMA)                                                                                            \
-      mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,          \
+    mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,          \
                           wn * WTN + li, lh, acc);                                                              \
     \
-    if (LLC_DBG_STORE && (!(GUARDED) || (KT) + 1 < nk)) {                                                       \
+    if (!(GUARDED) || (KT) + 1 < nk) {                                                       \
       LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
       LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
     }                                                                                                           \
@@ -150,7 +128,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
 
   // ---- epilogue.  32x32 accumulator layout: register r of lane (li, lh) is row 8*(r/4) + 4*lh + r%4,
   //      column li: for fixed r, 32 lanes store 32 consecutive columns of one row. ----
-  if (!LLC_DBG_EPI && p.alpha != 123.0f) return;
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const char* res = p.residual ? p.residual + c_off * (int64_t)sizeof(T) : nullptr;
@@ -266,7 +243,6 @@ struct DmaOperands {
 
   // next k-tile of both operands into `stage`
   __device__ __forceinline__ void issue(char* smem, int stage) {
-    if (!LLC_DBG_DMA) return;
     char* base = smem + stage * kDmaStage;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -312,7 +288,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
 
   auto issue = [&](int stage) { op.issue(smem, stage); };
 #define LLC_DMA_READ(SET, STAGE)                                                                              \
-  if (LLC_DBG_READ) {                                                                                         \
+  {                                                                                                           \
     const char* base = smem + (STAGE) * kDmaStage;                                                            \
     _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i) {             \
       fa[SET][s][i] = *(const u32x4_t*)(base + op.oa[s][i]);                                                     \
@@ -335,7 +311,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
         fb[SET][s][i] = u32x4_t{tb[SET][s][i][0].x, tb[SET][s][i][0].y, tb[SET][s][i][1].x, tb[SET][s][i][1].y}; \
   }
 #define LLC_DMA_MMA(SET)                                                                                      \
-  if (LLC_DBG_MMA) _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i)                 \
+  _Pragma("unroll") for (int s = 0; s < 2; ++s) _Pragma("unroll") for (int i = 0; i < 2; ++i)                 \
       _Pragma("unroll") for (int j = 0; j < 2; ++j) mfma_step<T>(fa[SET][s][i], fb[SET][s][j], acc[i][j]);
 
   const int nk = p.K / 64;
@@ -390,7 +366,6 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   // ---- epilogue: both k halves to LDS as fp32 [half][128][kStagePitch], then row-major 16-byte stores.
   //      No wave reads operand tiles any more (the last fragments were in registers before the last
   //      barrier) and no load is in flight. ----
-  if (!LLC_DBG_EPI && p.alpha != 123.0f) return;
   float* stage = (float*)(smem + ks * kStageHalf);
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -675,11 +650,7 @@ int launch_tiles(const GemmParams& p, int batch, hipStream_t s) {
   // wave tile 32x64) to keep the LDS pipe and the matrix cores busy at once.  Short-K or skinny
   // shapes keep 4 waves and rely on several workgroups per CU.
   const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch;
-  static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
   const bool deep = p.K >= 512;
-  static const int tile_env = getenv("LLC_GEMM_TILE") ? atoi(getenv("LLC_GEMM_TILE")) : 0;  // experiment hook
-  if (tile_env == 64) return launch_cfg<T, 64, 64, 2, 2, LA, LB>(p, batch, s);
-  if (tile_env == 12864) return launch_cfg<T, 128, 64, 2, 2, LA, LB>(p, batch, s);
   if constexpr (sizeof(T) == 4) {
     // fp32 is bound by the (slow) fp32 MFMA, not by LDS or L2: what counts is how evenly the tiles fill the
     // 256 CUs.  A last round that is mostly empty costs more than the ~7% a 64x64 tile loses to a 128x128 one.
@@ -690,7 +661,7 @@ int launch_tiles(const GemmParams& p, int batch, hipStream_t s) {
   }
   if (p.N > 64 && p.M > 64 && t128 >= 128) {
     if constexpr (LA != kLoadGeneric) {  // the element-wise loader needs too many registers for 8 waves
-      if ((deep && cfg_env != 4) || cfg_env == 8) return launch_cfg<T, 128, 128, 4, 2, LA, LB>(p, batch, s);
+      if (deep) return launch_cfg<T, 128, 128, 4, 2, LA, LB>(p, batch, s);
     }
     return launch_cfg<T, 128, 128, 2, 2, LA, LB>(p, batch, s);
   }
@@ -706,15 +677,13 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.B);
   const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.N % EPV == 0 && al16(p.B);
   if constexpr (sizeof(T) == 2) {
-    static const int cfg_env = getenv("LLC_GEMM_CFG") ? atoi(getenv("LLC_GEMM_CFG")) : 0;  // experiment hook
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
-    if (cfg_env == 0 && a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
+    if (a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
         tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 && p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) &&
         (!p.residual || al16(p.residual)))
     {
       // short reductions, or more tiles than one round of workgroups: two workgroups per CU
-      static const int two_env = getenv("LLC_GEMM_TWO") ? atoi(getenv("LLC_GEMM_TWO")) : -1;  // experiment hook
-      const bool two = two_env >= 0 ? two_env != 0 : (p.K <= 1536 && tiles >= 512);
+      const bool two = p.K <= 1536 && tiles >= 512;
       if (two) return b_kvec ? launch_dma2<T, kBKMajor>(p, batch, s) : launch_dma2<T, kBNMajor>(p, batch, s);
       return b_kvec ? launch_dma<T, kBKMajor>(p, batch, s) : launch_dma<T, kBNMajor>(p, batch, s);
     }

@@ -5,7 +5,6 @@
 // when a row spans several waves), and the result is written once.  Statistics are always fp32.
 // Algorithmic traffic is therefore read + write of the tensor, which is what these kernels are
 // measured against.
-#include <cstdlib>
 
 #include "common.hpp"
 
@@ -463,11 +462,6 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
       }
     }
   if (best_cap < 0) return false;
-  if (const char* ft = getenv("LLC_ROW_TPR")) {  // experiment hook
-    int t = atoi(ft);
-    for (int i : {1, 2, 4, 8, 16})
-      if ((int64_t)t * i * VEC >= p.cols) { best_t = t; best_i = i; break; }
-  }
   if (best_t == 16) launch_items<OP, VEC, 16>(p, best_i, s);
   else if (best_t == 64) launch_items<OP, VEC, 64>(p, best_i, s);
   else launch_items<OP, VEC, 256>(p, best_i, s);
