@@ -6,7 +6,12 @@
 // v_mfma_f32_32x32x2_f32 (fp32 products, fp32 accumulate) so that fp32 graphs keep fp32 accuracy.
 // Accumulation is always fp32.
 //
-// Data path per workgroup (256 lanes = 4 waves in a 2x2 grid, macro tile BM x BN):
+// Three kernels share the tile geometry of gemm_core.hpp.  gemm_kernel (any type, any strides, ragged shapes)
+// is described here; gemm_dma_kernel and gemm_dma2_kernel (16-bit operands, complete tiles, operands moved
+// straight into LDS) are described where they are defined.
+//
+// Data path of gemm_kernel per workgroup (4 waves in a 2x2 grid, or 8 waves 4x2 on 128x128 tiles with a deep
+// reduction; macro tile BM x BN):
 //   HBM/L2 --16-byte global loads--> registers --> LDS tile [row][128 bytes of k] whose 16-byte
 //   chunks are XOR-swizzled by the row (no padding; fragment reads, row copies and transposing
 //   stores all spread over the banks) --> ds_read_b128 fragments --> MFMA.  Two LDS buffers and two
