@@ -232,6 +232,65 @@ int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* stream);
 int llc_hip_unpack_params(void* const* params, size_t n_tensors, const size_t* ranks, const size_t* types,
                           llc_tensor* tensors_out, const int64_t** symbols_out);
 
+/* ---- model-level entry: a recorded plan run from the packed block.
+ *
+ * The reference compiles a graph into one `void main(void** params)` (entry type
+ * include/llcompiler/Compiler/Execution.h:23; called at src/Compiler/Execution.cpp:21-66) whose prologue
+ * unpacks the block (AdaptEntryParmsForEngine.cpp:154-242), whose constants are baked into the object and
+ * whose temporaries it allocates itself.  The counterpart here is a plan: the ordered kernel calls of one
+ * graph specialised to concrete extents (one plan per binding of the symbols), recorded once and replayed
+ * by llc_hip_run from the same block.  The caller owns inputs and outputs (Tensor.h:35); the plan owns what
+ * llc_plan_alloc / llc_plan_upload hand out (weights, the arena of intermediates) until llc_plan_destroy.
+ *
+ *   llc_plan_create(&p);
+ *   llc_plan_upload(p, host_weights, bytes, &w);  llc_plan_alloc(p, arena_bytes, &arena);
+ *   llc_plan_declare_io(p, 0, &in0); ...          inputs first, then outputs, in params order
+ *   llc_plan_declare_io(p, 1, &out0); ...
+ *   llc_plan_begin(p);
+ *     llc_hip_matmul(...); llc_hip_elementwise(...); ...   each call runs AND is appended to the plan
+ *   llc_plan_end(p);
+ *   llc_hip_run(p, params, stream);                        any number of times, any input/output addresses
+ *
+ * While recording, an operand whose address lies inside a declared tensor is bound to it and follows the
+ * pointer the block carries at run time; any other address is replayed as recorded.  llc_hip_run launches
+ * only: no allocation, no host-device synchronisation.  One run at a time per plan (runs of one plan are
+ * serialised by a lock; different plans are independent). ---- */
+typedef struct llc_plan llc_plan_t;
+/* The plan belongs to the current device. */
+int llc_plan_create(llc_plan_t** plan);
+/* Frees the plan and the device memory it owns (waits for the device to be done with it). */
+int llc_plan_destroy(llc_plan_t* plan);
+/* Device memory owned by the plan: the stand-in for the reference's baked constants
+ * (src/Dialect/LLH/Transforms/LoadWeight.cpp:58-171) and its malloc'ed temporaries
+ * (include/llcompiler/TransformLibrary/memref_include.mlir:6-8). */
+int llc_plan_alloc(llc_plan_t* plan, size_t bytes, void** device_ptr);
+int llc_plan_upload(llc_plan_t* plan, const void* host, size_t bytes, void** device_ptr);
+/* Declares the next tensor of the params block: type, rank, extents and strides it will have on every run,
+ * and (data + offset) = where it lives while the plan is recorded. */
+int llc_plan_declare_io(llc_plan_t* plan, int is_output, const llc_tensor* like);
+/* The symbol values the plan was specialised for; llc_hip_run then checks params[0] against them
+ * (the reference passes them in slot 0, Execution.cpp:24,46-49). */
+int llc_plan_expect_symbols(llc_plan_t* plan, const int64_t* values, size_t n);
+int llc_plan_begin(llc_plan_t* plan);
+int llc_plan_end(llc_plan_t* plan);
+int64_t llc_plan_num_steps(const llc_plan_t* plan);
+/* Number of slots llc_hip_run reads from `params`: 1 + 5 per declared tensor. */
+int64_t llc_plan_num_params(const llc_plan_t* plan);
+/* Replays the plan.  `params` has the layout described above llc_hip_unpack_params; base/data are device
+ * pointers.  Extents must equal the declared ones and strides too (LLC_ERR_SHAPE / LLC_ERR_LAYOUT
+ * otherwise: the caller then picks or records the plan for that binding). */
+int llc_hip_run(llc_plan_t* plan, void* const* params, void* stream);
+/* The reference's loader resolves a symbol of type void(void**) (Execution.cpp:12-16).  llc_hip_entry has
+ * that type and runs the plan bound with llc_hip_bind_entry (one per process; NULL unbinds) on the stream
+ * given there; like the reference's entry it returns nothing and logs failures
+ * (include/llcompiler/Support/Logger.h:132-134), and llc_hip_entry_status() returns the status of the last
+ * call.  libllc_entry.so exports the same function under the name `main` for a loader that looks that
+ * name up. */
+int llc_hip_bind_entry(llc_plan_t* plan, void* stream);
+void llc_hip_entry(void** params);
+int llc_hip_entry_status(void);
+
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,6 +10,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libllc_hip.so")
+ENTRY_LIB_PATH = os.path.join(_HERE, "lib", "libllc_entry.so")
 
 LLC_MAX_RANK = 8
 # element type codes: 0-6 are the reference's enum Type (include/llcompiler/Compiler/Tensor.h:25-33)
@@ -20,6 +21,8 @@ TORCH_DTYPE_TO_TYPE = {
 }
 TYPE_TO_TORCH_DTYPE = {v: k for k, v in TORCH_DTYPE_TO_TYPE.items()}
 
+OK, ERR_BAD_ARG, ERR_DTYPE, ERR_SHAPE, ERR_LAYOUT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE, ERR_TOO_LARGE = \
+    0, -1, -2, -3, -4, -5, -6, -7, -8
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2
 
@@ -72,6 +75,9 @@ EXPORTS = [
     "llc_hip_layer_norm", "llc_hip_max_pool", "llc_hip_global_avg_pool", "llc_hip_transpose",
     "llc_hip_stride_slice", "llc_hip_broadcast_to", "llc_hip_copy", "llc_hip_gather_rows", "llc_hip_convert",
     "llc_hip_unpack_params",
+    "llc_plan_create", "llc_plan_destroy", "llc_plan_alloc", "llc_plan_upload", "llc_plan_declare_io",
+    "llc_plan_expect_symbols", "llc_plan_begin", "llc_plan_end", "llc_plan_num_steps", "llc_plan_num_params",
+    "llc_hip_run", "llc_hip_bind_entry", "llc_hip_entry", "llc_hip_entry_status",
 ]
 
 
@@ -117,6 +123,22 @@ def lib():
         L.llc_hip_init.argtypes = [ctypes.c_int]
         L.llc_hip_unpack_params.argtypes = [P(vp), ctypes.c_size_t, P(ctypes.c_size_t), P(ctypes.c_size_t), T,
                                             P(i64p)]
+        L.llc_plan_create.argtypes = [P(vp)]
+        L.llc_plan_destroy.argtypes = [vp]
+        L.llc_plan_alloc.argtypes = [vp, ctypes.c_size_t, P(vp)]
+        L.llc_plan_upload.argtypes = [vp, vp, ctypes.c_size_t, P(vp)]
+        L.llc_plan_declare_io.argtypes = [vp, ctypes.c_int, T]
+        L.llc_plan_expect_symbols.argtypes = [vp, i64p, ctypes.c_size_t]
+        L.llc_plan_begin.argtypes = [vp]
+        L.llc_plan_end.argtypes = [vp]
+        L.llc_plan_num_steps.argtypes = [vp]
+        L.llc_plan_num_steps.restype = ctypes.c_int64
+        L.llc_plan_num_params.argtypes = [vp]
+        L.llc_plan_num_params.restype = ctypes.c_int64
+        L.llc_hip_run.argtypes = [vp, P(vp), vp]
+        L.llc_hip_bind_entry.argtypes = [vp, vp]
+        L.llc_hip_entry.argtypes = [P(vp)]
+        L.llc_hip_entry.restype = None
         _lib = L
     return _lib
 

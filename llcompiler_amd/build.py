@@ -17,6 +17,9 @@ CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB = os.path.join(LIB_DIR, "libllc_hip.so")
+# exports `main(void**)`, the symbol the reference's loader resolves, forwarding to libllc_hip.so
+ENTRY_LIB = os.path.join(LIB_DIR, "libllc_entry.so")
+ENTRY_SRC = os.path.join(CSRC, "entry_main.c")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -49,8 +52,8 @@ def build(force=True, jobs=None, verbose=False):
     srcs = sources()
     if not srcs:
         raise RuntimeError("no HIP sources under %s" % CSRC)
-    deps = srcs + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
-    if not force and os.path.exists(LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(d) for d in deps):
+    deps = srcs + [ENTRY_SRC] + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
+    if not force and os.path.exists(LIB) and os.path.exists(ENTRY_LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(d) for d in deps):
         return LIB
     jobs = jobs or min(8, os.cpu_count() or 1, len(srcs))
     with concurrent.futures.ThreadPoolExecutor(jobs) as ex:
@@ -64,6 +67,11 @@ def build(force=True, jobs=None, verbose=False):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    cmd = ["gcc", "-O2", "-shared", "-fPIC", "-Wno-main", "-I", os.path.join(ROOT, "include"), ENTRY_SRC, "-o", ENTRY_LIB,
+           "-L", LIB_DIR, "-lllc_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (ENTRY_LIB, r.stderr))
     return LIB
 
 

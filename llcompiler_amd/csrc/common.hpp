@@ -10,6 +10,7 @@
 #include <cstdio>
 
 #include "llc_hip.h"
+#include "entries.hpp"
 
 namespace llc {
 

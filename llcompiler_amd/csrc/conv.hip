@@ -567,7 +567,7 @@ int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
 
 using namespace llc;
 
-extern "C" int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* at, const llc_epilogue* epi,
+int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* at, const llc_epilogue* epi,
                               llc_tensor* out, void* stream) {
   View a, k, o;
   LLC_TRY(make_view(x, "conv input", &a));

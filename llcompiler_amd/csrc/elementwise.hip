@@ -691,7 +691,7 @@ int launch_chain(const EwKernelParams& p, int vec, hipStream_t stream) {
 
 using namespace llc;
 
-extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor* const* inputs, size_t n_inputs,
+int llc_impl_elementwise(const llc_ew_program* prog, const llc_tensor* const* inputs, size_t n_inputs,
                                    llc_tensor* out, void* stream) {
   if (!prog || !out || (n_inputs && !inputs)) return set_error(LLC_ERR_BAD_ARG, "elementwise: null argument");
   if (n_inputs > LLC_EW_MAX_INPUTS)

@@ -747,7 +747,7 @@ int fill_epilogue(const llc_epilogue* epi, const View& o, int64_t n_cols, GemmPa
 
 using namespace llc;
 
-extern "C" int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+int llc_impl_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                               void* stream) {
   View a, b, o;
   LLC_TRY(make_view(lhs, "matmul lhs", &a));
@@ -777,7 +777,7 @@ extern "C" int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, cons
   return gemm_dispatch(a.dtype, p, 1, as_stream(stream));
 }
 
-extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi,
+int llc_impl_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi,
                                     llc_tensor* out, void* stream) {
   View a, b, o;
   LLC_TRY(make_view(lhs, "batch_matmul lhs", &a));

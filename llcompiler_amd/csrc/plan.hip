@@ -1,0 +1,530 @@
+// Model-level boundary: a plan is a recorded sequence of kernel calls that is replayed from the reference's
+// packed `main(void** params)` block (src/Compiler/Execution.cpp:21-66).
+//
+// The per-op entry points of the C-ABI are defined here as wrappers around the launchers (entries.hpp).
+// Between llc_plan_begin and llc_plan_end every successful call made by the recording thread is also
+// appended to the plan, with deep copies of its descriptors and attributes.  An operand whose address lies
+// inside a declared input or output tensor is bound to that tensor: llc_hip_run re-bases it on the pointer
+// the params block carries for the tensor; every other address (weights uploaded into the plan, its arena,
+// caller-owned constants) is replayed as recorded.  A replay allocates nothing and makes no host-device
+// synchronisation: it is the list of kernel launches, in order, on the given stream.
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include "common.hpp"
+
+using namespace llc;
+
+namespace {
+
+enum OpCode {
+  kMatmul, kBatchMatmul, kConv2d, kElementwise, kReduce, kSoftmax, kLayerNorm, kMaxPool, kGlobalAvgPool,
+  kTranspose, kStrideSlice, kBroadcastTo, kCopy, kGatherRows, kConvert,
+};
+
+// Owned copy of a tensor descriptor.
+struct Operand {
+  llc_tensor t{};
+  size_t size[LLC_MAX_RANK];
+  size_t stride[LLC_MAX_RANK];
+  bool present = false;
+  int io = -1;        // index among the params tensors (inputs, then outputs); -1 = fixed address
+  int64_t delta = 0;  // bytes from that tensor's first element
+
+  // Copies *src; `offset` is folded into the data pointer.  Returns false for a malformed descriptor.
+  bool assign(const llc_tensor* src) {
+    if (!src) return true;  // stays absent
+    const size_t es = dtype_size(src->type);
+    if (src->rank > LLC_MAX_RANK || es == 0 || (src->rank && (!src->size || !src->stride))) return false;
+    present = true;
+    t = *src;
+    for (size_t i = 0; i < src->rank; ++i) {
+      size[i] = src->size[i];
+      stride[i] = src->stride[i];
+    }
+    t.size = size;
+    t.stride = stride;
+    t.data = src->data ? (char*)src->data + src->offset * es : nullptr;
+    t.base = t.data;
+    t.offset = 0;
+    return true;
+  }
+  llc_tensor* ptr() { return present ? &t : nullptr; }
+  // bytes from the first element to one past the last addressed element
+  size_t span_bytes() const {
+    size_t last = 0;
+    for (size_t i = 0; i < t.rank; ++i) {
+      if (size[i] == 0) return 0;
+      last += (size[i] - 1) * stride[i];
+    }
+    return (last + 1) * dtype_size(t.type);
+  }
+};
+
+struct Step {
+  int op = 0;
+  std::vector<Operand> opnd;  // element addresses stay put when the step moves
+  bool has_epi = false;
+  float alpha = 1.0f;
+  int act = 0;
+  int kind = 0;
+  double eps = 0.0;
+  size_t n_ints = 0;
+  int64_t ints[3 * LLC_MAX_RANK];
+  union {
+    llc_conv_attrs conv;
+    llc_pool_attrs pool;
+  };
+  std::unique_ptr<llc_ew_program> prog;
+  Step() { memset(&conv, 0, sizeof(conv)); }
+};
+
+struct Io {
+  Operand like;
+  char* lo = nullptr;  // address range the tensor occupied while the plan was recorded
+  char* hi = nullptr;
+  bool output = false;
+};
+
+struct Overlap {
+  int first, second;
+  int64_t diff;  // recorded address of `second` minus that of `first`
+};
+
+enum State { kOpen, kRecording, kReady, kBroken };
+
+}  // namespace
+
+struct llc_plan {
+  int device = 0;
+  State state = kOpen;
+  std::vector<Io> io;
+  size_t n_inputs = 0;
+  std::vector<Step> steps;
+  std::vector<void*> owned;
+  std::vector<int64_t> symbols;
+  std::vector<Overlap> overlaps;
+  std::vector<char*> bound;  // per run: first element of every params tensor
+  std::mutex mu;
+};
+
+namespace {
+
+thread_local llc_plan* t_rec = nullptr;
+
+// ---- recording ----
+int bind(llc_plan* p, Operand& o) {
+  if (!o.present || !o.t.data) return LLC_OK;
+  char* a = (char*)o.t.data;
+  for (size_t k = 0; k < p->io.size(); ++k) {
+    const Io& io = p->io[k];
+    if (a >= io.lo && a < io.hi) {
+      o.io = (int)k;
+      o.delta = a - io.lo;
+      return LLC_OK;
+    }
+  }
+  return LLC_OK;
+}
+
+struct Recorder {
+  llc_plan* p;
+  Step st;
+  bool ok = true;
+  Recorder(int op, size_t n_operands) : p(t_rec) {
+    st.op = op;
+    st.opnd.resize(n_operands);
+  }
+  void tensor(size_t i, const llc_tensor* t) {
+    if (!st.opnd[i].assign(t)) ok = false;
+    bind(p, st.opnd[i]);
+  }
+  void epilogue(const llc_epilogue* e, size_t bias_at) {
+    if (!e) return;
+    st.has_epi = true;
+    st.alpha = e->alpha;
+    st.act = e->act;
+    tensor(bias_at, e->bias);
+    tensor(bias_at + 1, e->residual);
+  }
+  void ints(const int64_t* v, size_t n) {
+    if (st.n_ints + n > sizeof(st.ints) / sizeof(st.ints[0]) || (n && !v)) {
+      ok = false;
+      return;
+    }
+    for (size_t i = 0; i < n; ++i) st.ints[st.n_ints++] = v[i];
+  }
+  int commit() {
+    if (!ok) {
+      p->state = kBroken;
+      t_rec = nullptr;
+      return set_error(LLC_ERR_BAD_ARG, "plan: a call could not be recorded (descriptor rank or attribute count)");
+    }
+    p->steps.push_back(std::move(st));
+    return LLC_OK;
+  }
+};
+
+// ---- replay ----
+inline void rebase(Step& s, char* const* bound) {
+  for (Operand& o : s.opnd)
+    if (o.io >= 0) o.t.data = o.t.base = bound[o.io] + o.delta;
+}
+
+int replay(Step& s, void* stream) {
+  Operand* o = s.opnd.data();
+  llc_epilogue epi;
+  const llc_epilogue* e = nullptr;
+  switch (s.op) {
+    case kMatmul:
+    case kBatchMatmul:
+    case kConv2d:
+      if (s.has_epi) {
+        epi.alpha = s.alpha;
+        epi.bias = o[2].ptr();
+        epi.residual = o[3].ptr();
+        epi.act = s.act;
+        e = &epi;
+      }
+      if (s.op == kMatmul) return llc_impl_matmul(o[0].ptr(), o[1].ptr(), e, o[4].ptr(), stream);
+      if (s.op == kBatchMatmul) return llc_impl_batch_matmul(o[0].ptr(), o[1].ptr(), e, o[4].ptr(), stream);
+      return llc_impl_conv2d(o[0].ptr(), o[1].ptr(), &s.conv, e, o[4].ptr(), stream);
+    case kElementwise: {
+      const llc_tensor* ins[LLC_EW_MAX_INPUTS];
+      const size_t n = s.opnd.size() - 1;
+      for (size_t i = 0; i < n; ++i) ins[i] = o[i].ptr();
+      return llc_impl_elementwise(s.prog.get(), ins, n, o[n].ptr(), stream);
+    }
+    case kReduce: return llc_impl_reduce(s.kind, o[0].ptr(), s.ints, s.n_ints, o[1].ptr(), stream);
+    case kSoftmax: return llc_impl_softmax(o[0].ptr(), o[1].ptr(), stream);
+    case kLayerNorm: return llc_impl_layer_norm(o[0].ptr(), o[1].ptr(), o[2].ptr(), s.eps, o[3].ptr(), stream);
+    case kMaxPool: return llc_impl_max_pool(o[0].ptr(), &s.pool, o[1].ptr(), stream);
+    case kGlobalAvgPool: return llc_impl_global_avg_pool(o[0].ptr(), o[1].ptr(), stream);
+    case kTranspose: return llc_impl_transpose(o[0].ptr(), s.ints, o[1].ptr(), stream);
+    case kStrideSlice: {
+      const size_t r = s.n_ints / 3;
+      return llc_impl_stride_slice(o[0].ptr(), s.ints, s.ints + r, s.ints + 2 * r, o[1].ptr(), stream);
+    }
+    case kBroadcastTo: return llc_impl_broadcast_to(o[0].ptr(), o[1].ptr(), stream);
+    case kCopy: return llc_impl_copy(o[0].ptr(), o[1].ptr(), stream);
+    case kGatherRows: return llc_impl_gather_rows(o[0].ptr(), o[1].ptr(), o[2].ptr(), stream);
+    case kConvert: return llc_impl_convert(o[0].ptr(), o[1].ptr(), stream);
+  }
+  return set_error(LLC_ERR_BAD_ARG, "plan: unknown step code %d", s.op);
+}
+
+int check_device(llc_plan* p, const char* what) {
+  int dev = -1;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  if (dev != p->device)
+    return set_error(LLC_ERR_BAD_ARG, "%s: the plan belongs to device %d, the current device is %d", what, p->device, dev);
+  return LLC_OK;
+}
+
+}  // namespace
+
+// ---- per-op entry points: launch, then record if a plan is recording on this thread ----
+extern "C" int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+                              void* stream) {
+  LLC_TRY(llc_impl_matmul(lhs, rhs, epi, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kMatmul, 5);
+  r.tensor(0, lhs), r.tensor(1, rhs), r.epilogue(epi, 2), r.tensor(4, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi,
+                                    llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_batch_matmul(lhs, rhs, epi, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kBatchMatmul, 5);
+  r.tensor(0, lhs), r.tensor(1, rhs), r.epilogue(epi, 2), r.tensor(4, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* attrs,
+                              const llc_epilogue* epi, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_conv2d(x, w, attrs, epi, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kConv2d, 5);
+  r.tensor(0, x), r.tensor(1, w), r.epilogue(epi, 2), r.tensor(4, out);
+  r.st.conv = *attrs;
+  return r.commit();
+}
+
+extern "C" int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor* const* inputs, size_t n_inputs,
+                                   llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_elementwise(prog, inputs, n_inputs, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kElementwise, n_inputs + 1);
+  for (size_t i = 0; i < n_inputs; ++i) r.tensor(i, inputs[i]);
+  r.tensor(n_inputs, out);
+  r.st.prog.reset(new llc_ew_program(*prog));
+  return r.commit();
+}
+
+extern "C" int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
+                              void* stream) {
+  LLC_TRY(llc_impl_reduce(kind, x, axes, n_axes, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kReduce, 2);
+  r.tensor(0, x), r.tensor(1, out), r.ints(axes, n_axes);
+  r.st.kind = kind;
+  return r.commit();
+}
+
+extern "C" int llc_hip_softmax(const llc_tensor* x, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_softmax(x, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kSoftmax, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_tensor* bias, double epsilon,
+                                  llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_layer_norm(x, scale, bias, epsilon, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kLayerNorm, 4);
+  r.tensor(0, x), r.tensor(1, scale), r.tensor(2, bias), r.tensor(3, out);
+  r.st.eps = epsilon;
+  return r.commit();
+}
+
+extern "C" int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* attrs, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_max_pool(x, attrs, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kMaxPool, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  r.st.pool = *attrs;
+  return r.commit();
+}
+
+extern "C" int llc_hip_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_global_avg_pool(x, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kGlobalAvgPool, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_transpose(const llc_tensor* x, const int64_t* perms, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_transpose(x, perms, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kTranspose, 2);
+  r.tensor(0, x), r.tensor(1, out), r.ints(perms, x->rank);
+  return r.commit();
+}
+
+extern "C" int llc_hip_stride_slice(const llc_tensor* x, const int64_t* start, const int64_t* end, const int64_t* step,
+                                    llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_stride_slice(x, start, end, step, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kStrideSlice, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  r.ints(start, x->rank), r.ints(end, x->rank), r.ints(step, x->rank);
+  return r.commit();
+}
+
+extern "C" int llc_hip_broadcast_to(const llc_tensor* x, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_broadcast_to(x, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kBroadcastTo, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_copy(const llc_tensor* x, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_copy(x, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kCopy, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_gather_rows(table, idx, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kGatherRows, 3);
+  r.tensor(0, table), r.tensor(1, idx), r.tensor(2, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_convert(x, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kConvert, 2);
+  r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+// ---- plan life cycle ----
+extern "C" int llc_plan_create(llc_plan_t** plan) {
+  if (!plan) return set_error(LLC_ERR_BAD_ARG, "plan_create: null argument");
+  int dev = -1;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  llc_plan* p = new llc_plan();
+  p->device = dev;
+  *plan = p;
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_destroy(llc_plan_t* p) {
+  if (!p) return LLC_OK;
+  if (t_rec == p) t_rec = nullptr;
+  int status = LLC_OK;
+  for (void* m : p->owned) {
+    hipError_t e = hipFree(m);  // waits for the device to finish with the memory
+    if (e != hipSuccess) status = set_error(LLC_ERR_HIP, "plan_destroy: hipFree: %s", hipGetErrorString(e));
+  }
+  delete p;
+  return status;
+}
+
+extern "C" int llc_plan_alloc(llc_plan_t* p, size_t bytes, void** device_ptr) {
+  if (!p || !device_ptr) return set_error(LLC_ERR_BAD_ARG, "plan_alloc: null argument");
+  LLC_TRY(check_device(p, "plan_alloc"));
+  void* m = nullptr;
+  LLC_HIP_TRY(hipMalloc(&m, bytes ? bytes : 1));
+  p->owned.push_back(m);
+  *device_ptr = m;
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_upload(llc_plan_t* p, const void* host, size_t bytes, void** device_ptr) {
+  if (!host && bytes) return set_error(LLC_ERR_BAD_ARG, "plan_upload: null host pointer");
+  LLC_TRY(llc_plan_alloc(p, bytes, device_ptr));
+  if (bytes) LLC_HIP_TRY(hipMemcpy(*device_ptr, host, bytes, hipMemcpyHostToDevice));
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_declare_io(llc_plan_t* p, int is_output, const llc_tensor* like) {
+  if (!p || !like) return set_error(LLC_ERR_BAD_ARG, "plan_declare_io: null argument");
+  if (p->state != kOpen) return set_error(LLC_ERR_BAD_ARG, "plan_declare_io: tensors are declared before recording starts");
+  if (!is_output && p->io.size() != p->n_inputs)
+    return set_error(LLC_ERR_BAD_ARG, "plan_declare_io: inputs are declared before outputs");
+  Io io;
+  if (!io.like.assign(like)) return set_error(LLC_ERR_BAD_ARG, "plan_declare_io: malformed descriptor");
+  io.output = is_output != 0;
+  io.lo = (char*)io.like.t.data;
+  io.hi = io.lo ? io.lo + io.like.span_bytes() : nullptr;
+  p->io.push_back(std::move(io));
+  Io& mine = p->io.back();
+  mine.like.t.size = mine.like.t.stride = nullptr;  // the arrays moved with the copy; only like.size/.stride are read
+  if (!is_output) p->n_inputs++;
+  // a tensor that shares addresses with an earlier one: operands inside the shared range bind to the earlier
+  // tensor, which is only right while the two keep their distance
+  const int k = (int)p->io.size() - 1;
+  for (int j = 0; j < k; ++j) {
+    const Io& other = p->io[j];
+    if (mine.lo && other.lo && mine.lo < other.hi && other.lo < mine.hi)
+      p->overlaps.push_back({j, k, (int64_t)(mine.lo - other.lo)});
+  }
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_expect_symbols(llc_plan_t* p, const int64_t* values, size_t n) {
+  if (!p || (n && !values)) return set_error(LLC_ERR_BAD_ARG, "plan_expect_symbols: null argument");
+  p->symbols.assign(values, values + n);
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_begin(llc_plan_t* p) {
+  if (!p) return set_error(LLC_ERR_BAD_ARG, "plan_begin: null plan");
+  if (t_rec) return set_error(LLC_ERR_BAD_ARG, "plan_begin: this thread is already recording a plan");
+  if (p->state != kOpen) return set_error(LLC_ERR_BAD_ARG, "plan_begin: the plan has been recorded already");
+  LLC_TRY(check_device(p, "plan_begin"));
+  p->state = kRecording;
+  t_rec = p;
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_end(llc_plan_t* p) {
+  if (!p) return set_error(LLC_ERR_BAD_ARG, "plan_end: null plan");
+  if (p->state == kBroken) return set_error(LLC_ERR_BAD_ARG, "plan_end: recording failed earlier");
+  if (t_rec != p || p->state != kRecording) return set_error(LLC_ERR_BAD_ARG, "plan_end: the plan is not recording on this thread");
+  t_rec = nullptr;
+  p->state = kReady;
+  p->bound.assign(p->io.size(), nullptr);
+  return LLC_OK;
+}
+
+extern "C" int64_t llc_plan_num_steps(const llc_plan_t* p) { return p ? (int64_t)p->steps.size() : -1; }
+
+extern "C" int64_t llc_plan_num_params(const llc_plan_t* p) { return p ? (int64_t)(1 + 5 * p->io.size()) : -1; }
+
+// ---- replay from the packed parameter block ----
+extern "C" int llc_hip_run(llc_plan_t* p, void* const* params, void* stream) {
+  if (!p || !params) return set_error(LLC_ERR_BAD_ARG, "run: null argument");
+  if (p->state != kReady) return set_error(LLC_ERR_BAD_ARG, "run: the plan has not been recorded (begin .. end)");
+  if (t_rec) return set_error(LLC_ERR_BAD_ARG, "run: this thread is recording a plan");
+  std::lock_guard<std::mutex> lock(p->mu);
+  if (!p->symbols.empty()) {
+    const int64_t* sym = (const int64_t*)params[0];
+    if (!sym) return set_error(LLC_ERR_BAD_ARG, "run: the plan expects %zu symbol values, slot 0 is null", p->symbols.size());
+    for (size_t i = 0; i < p->symbols.size(); ++i)
+      if (sym[i] != p->symbols[i])
+        return set_error(LLC_ERR_SHAPE, "run: symbol %zu is %lld, the plan was specialised for %lld", i, (long long)sym[i],
+                         (long long)p->symbols[i]);
+  }
+  size_t slot = 1;
+  for (size_t k = 0; k < p->io.size(); ++k, slot += 5) {
+    const Operand& like = p->io[k].like;
+    char* data = (char*)params[slot + 1];
+    const size_t* off = (const size_t*)params[slot + 2];
+    const size_t* size = (const size_t*)params[slot + 3];
+    const size_t* stride = (const size_t*)params[slot + 4];
+    if (!off || (like.t.rank && (!size || !stride)))
+      return set_error(LLC_ERR_BAD_ARG, "run: tensor %zu has a null offset, size or stride slot", k);
+    bool empty = false;
+    for (size_t d = 0; d < like.t.rank; ++d) {
+      if (size[d] != like.size[d])
+        return set_error(LLC_ERR_SHAPE, "run: tensor %zu has extent %zu in dim %zu, the plan was specialised for %zu", k,
+                         size[d], d, like.size[d]);
+      if (size[d] > 1 && stride[d] != like.stride[d])
+        return set_error(LLC_ERR_LAYOUT, "run: tensor %zu has stride %zu in dim %zu, the plan was specialised for %zu", k,
+                         stride[d], d, like.stride[d]);
+      empty |= size[d] == 0;
+    }
+    if (!data && !empty) return set_error(LLC_ERR_BAD_ARG, "run: tensor %zu has a null data pointer", k);
+    p->bound[k] = data ? data + *off * dtype_size(like.t.type) : nullptr;
+  }
+  for (const Overlap& ov : p->overlaps)
+    if (p->bound[ov.second] - p->bound[ov.first] != ov.diff)
+      return set_error(LLC_ERR_LAYOUT, "run: tensors %d and %d shared memory when the plan was recorded and do not now", ov.first,
+                       ov.second);
+  for (Step& s : p->steps) {
+    rebase(s, p->bound.data());
+    LLC_TRY(replay(s, stream));
+  }
+  return LLC_OK;
+}
+
+// ---- `void main(void**)` convention: one plan bound per process ----
+namespace {
+llc_plan* g_entry_plan = nullptr;
+void* g_entry_stream = nullptr;
+int g_entry_status = LLC_OK;
+}  // namespace
+
+extern "C" int llc_hip_bind_entry(llc_plan_t* p, void* stream) {
+  if (p && p->state != kReady) return set_error(LLC_ERR_BAD_ARG, "bind_entry: the plan has not been recorded");
+  g_entry_plan = p;
+  g_entry_stream = stream;
+  g_entry_status = LLC_OK;
+  return LLC_OK;
+}
+
+extern "C" void llc_hip_entry(void** params) {
+  if (!g_entry_plan) {
+    g_entry_status = set_error(LLC_ERR_BAD_ARG, "entry: no plan is bound (llc_hip_bind_entry)");
+  } else {
+    g_entry_status = llc_hip_run(g_entry_plan, params, g_entry_stream);
+  }
+  // the reference's entry returns nothing and its failures are only logged (Logger.h:132-134)
+  if (g_entry_status != LLC_OK) fprintf(stderr, "llc_hip_entry: %s\n", llc_hip_last_error());
+}
+
+extern "C" int llc_hip_entry_status(void) { return g_entry_status; }

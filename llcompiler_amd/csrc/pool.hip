@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void max_pool_kernel(const PoolParams p) {
 
 using namespace llc;
 
-extern "C" int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* at, llc_tensor* out, void* stream) {
+int llc_impl_max_pool(const llc_tensor* x, const llc_pool_attrs* at, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "max_pool input", &a));
   LLC_TRY(make_view(out, "max_pool output", &o));

@@ -496,7 +496,7 @@ int row_dtype_ok(const View& v, const char* what) {
 
 using namespace llc;
 
-extern "C" int llc_hip_softmax(const llc_tensor* x, llc_tensor* out, void* stream) {
+int llc_impl_softmax(const llc_tensor* x, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "softmax input", &a));
   LLC_TRY(make_view(out, "softmax output", &o));
@@ -516,7 +516,7 @@ extern "C" int llc_hip_softmax(const llc_tensor* x, llc_tensor* out, void* strea
   return launch_rows<kSoftmax>(p, as_stream(stream));
 }
 
-extern "C" int llc_hip_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_tensor* bias, double epsilon,
+int llc_impl_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_tensor* bias, double epsilon,
                                   llc_tensor* out, void* stream) {
   View a, o, g, b;
   LLC_TRY(make_view(x, "layer_norm input", &a));
@@ -578,7 +578,7 @@ int reduce_3d(const View& a, const View& o, int kind, int64_t outer, int64_t R, 
 }
 }  // namespace llc
 
-extern "C" int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
+int llc_impl_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
                               void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "reduce input", &a));
@@ -614,7 +614,7 @@ extern "C" int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes
   return reduce_3d(a, o, kind, outer, R, inner, 1.0f, as_stream(stream));
 }
 
-extern "C" int llc_hip_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream) {
+int llc_impl_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "global_avg_pool input", &a));
   LLC_TRY(make_view(out, "global_avg_pool output", &o));

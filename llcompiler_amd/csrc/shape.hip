@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const T* table, const 
 
 using namespace llc;
 
-extern "C" int llc_hip_copy(const llc_tensor* x, llc_tensor* out, void* stream) {
+int llc_impl_copy(const llc_tensor* x, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "copy input", &a));
   LLC_TRY(make_view(out, "copy output", &o));
@@ -257,7 +257,7 @@ extern "C" int llc_hip_copy(const llc_tensor* x, llc_tensor* out, void* stream) 
   return strided_to_contiguous(a.ptr, o.ptr, a.rank, a.size, a.stride, a.esize(), as_stream(stream));
 }
 
-extern "C" int llc_hip_transpose(const llc_tensor* x, const int64_t* perms, llc_tensor* out, void* stream) {
+int llc_impl_transpose(const llc_tensor* x, const int64_t* perms, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "transpose input", &a));
   LLC_TRY(make_view(out, "transpose output", &o));
@@ -279,7 +279,7 @@ extern "C" int llc_hip_transpose(const llc_tensor* x, const int64_t* perms, llc_
   return strided_to_contiguous(a.ptr, o.ptr, a.rank, o.size, st, a.esize(), as_stream(stream));
 }
 
-extern "C" int llc_hip_stride_slice(const llc_tensor* x, const int64_t* start, const int64_t* end, const int64_t* step,
+int llc_impl_stride_slice(const llc_tensor* x, const int64_t* start, const int64_t* end, const int64_t* step,
                                     llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "stride_slice input", &a));
@@ -305,7 +305,7 @@ extern "C" int llc_hip_stride_slice(const llc_tensor* x, const int64_t* start, c
   return strided_to_contiguous(a.ptr + off * (int64_t)a.esize(), o.ptr, a.rank, size, st, a.esize(), as_stream(stream));
 }
 
-extern "C" int llc_hip_broadcast_to(const llc_tensor* x, llc_tensor* out, void* stream) {
+int llc_impl_broadcast_to(const llc_tensor* x, llc_tensor* out, void* stream) {
   View a, o;
   LLC_TRY(make_view(x, "broadcast_to input", &a));
   LLC_TRY(make_view(out, "broadcast_to output", &o));
@@ -321,7 +321,7 @@ extern "C" int llc_hip_broadcast_to(const llc_tensor* x, llc_tensor* out, void* 
   return strided_to_contiguous(a.ptr, o.ptr, a.rank, o.size, st, a.esize(), as_stream(stream));
 }
 
-extern "C" int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream) {
+int llc_impl_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream) {
   View t, i, o;
   LLC_TRY(make_view(table, "gather_rows table", &t));
   LLC_TRY(make_view(idx, "gather_rows indices", &i));
@@ -354,7 +354,7 @@ extern "C" int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* id
   return check_launch("gather_rows_kernel");
 }
 
-extern "C" int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* stream) {
+int llc_impl_convert(const llc_tensor* x, llc_tensor* out, void* stream) {
   if (!x || !out) return set_error(LLC_ERR_BAD_ARG, "convert: null tensor");
   llc_ew_program prog{};
   prog.n_insts = 1;
@@ -366,5 +366,5 @@ extern "C" int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* strea
   prog.insts[0].dst = 0;
   prog.insts[0].a = LLC_EW_IN0;
   const llc_tensor* ins[1] = {x};
-  return llc_hip_elementwise(&prog, ins, 1, out, stream);
+  return llc_impl_elementwise(&prog, ins, 1, out, stream);
 }

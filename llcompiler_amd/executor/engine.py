@@ -23,6 +23,7 @@ from .. import _capi as C
 from .. import ops
 from ..llh.expr import Expr, evaluate
 from ..llh.graph import Value
+from .plan_runner import ParamBlock, Plan
 from .planner import make_plan
 
 # same codes as the reference's map (engine.py:11), extended with bf16 / f16 / i32
@@ -35,10 +36,25 @@ TORCH_DTYPE_TO_TYPE = C.TORCH_DTYPE_TO_TYPE
 # two launches do (57 us against 34 us per call).  It helps a caller that is host-bound for other reasons.
 USE_GRAPHS = os.environ.get("LLC_GRAPHS", "0") == "1"
 MIN_CALLS_FOR_GRAPH = 2
+# The first run of an instance records its kernel calls into a native plan (llc_plan_t); later runs fill the
+# reference's packed parameter block and make one call into the library, which replays the launches.  With
+# False every run launches kernel by kernel from Python (same kernels, same arguments).
+USE_PLAN = True
 
 
 def _concrete(shape, env):
     return tuple(evaluate(d, env) if isinstance(d, Expr) else int(d) for d in shape)
+
+
+def _alias_signature(inputs):
+    """Which inputs share a storage, and at what distance: an instance binds descriptors to inputs by address,
+    so calls that differ in this are different bindings."""
+    first, sig = {}, []
+    for i, t in enumerate(inputs):
+        j = first.setdefault(t.untyped_storage().data_ptr(), i)
+        if j != i:
+            sig.append((j, i, t.data_ptr() - inputs[j].data_ptr()))
+    return tuple(sig)
 
 
 class _Pool:
@@ -350,6 +366,8 @@ class Instance:
         self._last_in_ptrs = None
         self._graph = None
         self._graph_failed = False
+        self._plan = None
+        self._block = None
 
     def _view(self, st, t, contiguous):
         a = st.attrs
@@ -428,8 +446,35 @@ class Instance:
         else:
             outs = [torch.empty(s, dtype=d, device=self.device) for s, d in self.out_specs]
         in_ptrs = [t.data_ptr() for t in inputs]
-        self._patch(in_ptrs, [t.data_ptr() for t in outs])
         stream = C.current_stream(self.device)
+        if self._plan is not None:
+            blk = self._block
+            last = self._last_in_ptrs
+            if in_ptrs != last:
+                for k, p in enumerate(in_ptrs):
+                    if p != last[k]:
+                        blk.set_pointer(k, p)
+                self._last_in_ptrs = in_ptrs
+            n_in = len(in_ptrs)
+            for k, t in enumerate(outs):
+                blk.set_pointer(n_in + k, t.data_ptr())
+            self._plan.run(blk, stream)
+            return self._results(outs)
+        self._patch(in_ptrs, [t.data_ptr() for t in outs])
+        if USE_PLAN and not USE_GRAPHS:
+            # this run launches every kernel as usual and records the calls on the way
+            plan = Plan()
+            for t in inputs:
+                plan.declare_io(t, False)
+            for t in outs:
+                plan.declare_io(t, True)
+            with plan.recording():
+                for c in self.calls:
+                    c.launch(stream)
+            self._block = ParamBlock(list(inputs) + list(outs))
+            self._plan = plan
+            self._last_in_ptrs = in_ptrs
+            return self._results(outs)
         for c in self.calls:
             c.launch(stream)
         # After two eager runs the launch sequence is recorded as a HIP graph: the host then pays one replay
@@ -549,13 +594,17 @@ class Torch_ExecutionEngine(ExecutionEngine):
             device = t.device
         if device is None:
             device = torch.device("cuda", torch.cuda.current_device())
-        key = (tuple(sorted(env.items())), tuple((tuple(t.shape), tuple(t.stride())) for t in inputs), device.index)
+        key = (tuple(sorted(env.items())), tuple((tuple(t.shape), tuple(t.stride())) for t in inputs), device.index,
+               _alias_signature(inputs))
         inst = self.instances.get(key)
         if inst is None:
             C.init(device.index or 0)
             inst = Instance(g, self.steps, env, inputs, device)
             self.instances[key] = inst
-        self._fast[fast_key] = inst
+        if not key[3]:
+            # (an instance built from inputs that share memory is only valid while they do: such calls keep
+            # coming this way, where the key checks it)
+            self._fast[fast_key] = inst
         results = inst.run(inputs)
         if getattr(g, "single_output", len(results) == 1) and len(results) == 1:
             return results[0]

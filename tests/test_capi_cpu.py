@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "llc_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(llc_hip_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(llc_(?:hip|plan)_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_agree():
@@ -74,6 +74,27 @@ def test_unpack_params_follows_execution_run_layout():
     params[0] = None
     used = L.llc_hip_unpack_params(params, 1, ranks, types, out, ctypes.byref(sym_out))
     assert used == 6 and not sym_out
+
+
+def test_plan_entry_points_validate_without_a_gpu():
+    L = C.lib()
+    assert L.llc_hip_run(None, None, None) == C.ERR_BAD_ARG
+    assert L.llc_plan_begin(None) == C.ERR_BAD_ARG
+    assert L.llc_plan_end(None) == C.ERR_BAD_ARG
+    assert L.llc_plan_destroy(None) == 0
+    assert L.llc_plan_num_steps(None) == -1
+    # the void(void**) entry logs and keeps the status when no plan is bound (Execution.h:23 has no return value)
+    assert L.llc_hip_bind_entry(None, None) == 0
+    L.llc_hip_entry(None)
+    assert L.llc_hip_entry_status() == C.ERR_BAD_ARG
+    assert b"no plan is bound" in L.llc_hip_last_error()
+
+
+def test_entry_library_exports_main_for_the_reference_loader():
+    # src/Compiler/Execution.cpp:12-16 resolves "main" in the library it is given
+    assert os.path.exists(C.ENTRY_LIB_PATH), "build the library first: python -m llcompiler_amd.build"
+    E = ctypes.CDLL(C.ENTRY_LIB_PATH)
+    assert hasattr(E, "main")
 
 
 def test_cpu_tensor_is_refused_not_computed():

@@ -1,0 +1,260 @@
+"""The model-level boundary: a plan recorded through the C-ABI and replayed from the reference's packed
+`main(void** params)` block (src/Compiler/Execution.cpp:21-66), checked against the C oracle, and the
+engine's use of it checked bit for bit against kernel-by-kernel launches."""
+import copy
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from tests.util import BF16_RTOL, F32_ATOL, F32_RTOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+
+
+def _stream():
+    from llcompiler_amd import _capi as C
+    return C.current_stream(torch.device("cuda", 0))
+
+
+def _record_two_layer(plan, x, out, w1_host, b1_host, w2_host, hidden):
+    """out = relu(x @ w1 + b1) @ w2 with the weights uploaded into the plan and the hidden layer in its arena."""
+    from llcompiler_amd import _capi as C
+    L = C.lib()
+    M, K = x.shape
+    N = out.shape[1]
+
+    def fixed(ptr, shape):
+        st, s = [], 1
+        for d in reversed(shape):
+            st.insert(0, s)
+            s *= d
+        return C.TensorRef(ptr, C.FLOAT32, shape, st)
+
+    w1 = fixed(plan.upload(w1_host.ctypes.data, w1_host.nbytes), (K, hidden))
+    b1 = fixed(plan.upload(b1_host.ctypes.data, b1_host.nbytes), (hidden,))
+    w2 = fixed(plan.upload(w2_host.ctypes.data, w2_host.nbytes), (hidden, N))
+    h = fixed(plan.alloc(M * hidden * 4), (M, hidden))
+    plan.declare_io(x, False)
+    plan.declare_io(out, True)
+    rx, ro = C.tensor_ref(x), C.tensor_ref(out)
+    epi = C.LlcEpilogue(1.0, b1.ptr, None, C.ACT_RELU)
+    with plan.recording():
+        C.check(L.llc_hip_matmul(rx.ptr, w1.ptr, ctypes.pointer(epi), h.ptr, _stream()))
+        C.check(L.llc_hip_matmul(h.ptr, w2.ptr, None, ro.ptr, _stream()))
+
+
+def test_recorded_plan_replays_from_the_packed_block(oracle):
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    rng = np.random.default_rng(7)
+    M, K, H, N = 48, 80, 96, 24
+    w1 = rng.standard_normal((K, H), dtype=np.float32) * 0.1
+    b1 = rng.standard_normal((H,), dtype=np.float32)
+    w2 = rng.standard_normal((H, N), dtype=np.float32) * 0.1
+    x0 = rng.standard_normal((M, K), dtype=np.float32)
+
+    def want(x):
+        return oracle.matmul(oracle.unary("relu", oracle.matmul(x, w1) + b1), w2)
+
+    plan = Plan()
+    x = torch.from_numpy(x0).cuda()
+    out = torch.empty((M, N), device="cuda")
+    _record_two_layer(plan, x, out, w1, b1, w2, H)
+    assert plan.num_steps == 2 and plan.num_params == 11
+    torch.cuda.synchronize()
+    # recording launches too
+    assert_close(out.cpu().numpy(), want(x0), F32_RTOL, F32_ATOL, "recording run")
+    # replay with other buffers, at other addresses, holding other values
+    for seed in (1, 2):
+        xs = np.random.default_rng(seed).standard_normal((M, K), dtype=np.float32)
+        pad = torch.empty(seed * 1000, device="cuda")  # shifts the next allocations
+        x2 = torch.from_numpy(xs).cuda()
+        out2 = torch.zeros((M, N), device="cuda")
+        assert x2.data_ptr() != x.data_ptr() and out2.data_ptr() != out.data_ptr()
+        plan.run(ParamBlock([x2, out2]), _stream())
+        torch.cuda.synchronize()
+        assert_close(out2.cpu().numpy(), want(xs), F32_RTOL, F32_ATOL, "replay %d" % seed)
+        del pad
+    # the first buffers were not written again
+    assert_close(out.cpu().numpy(), want(x0), F32_RTOL, F32_ATOL, "recording buffers untouched")
+
+    # an input that is a view at an offset inside a larger buffer: data_ptr carries the offset, slot 2 holds 0
+    big = torch.zeros((M + 3, K), device="cuda")
+    big[3:] = torch.from_numpy(x0).cuda()
+    out3 = torch.zeros((M, N), device="cuda")
+    plan.run(ParamBlock([big[3:], out3]), _stream())
+    torch.cuda.synchronize()
+    assert_close(out3.cpu().numpy(), want(x0), F32_RTOL, F32_ATOL, "replay from a view")
+
+    # the offset slot is honoured like the reference's descriptor offset (Tensor.h:42-47), in elements
+    blk = ParamBlock([big, out3])
+    off = ctypes.c_size_t(3 * K)
+    size = (ctypes.c_size_t * 2)(M, K)
+    blk.arr[3] = ctypes.addressof(off)
+    blk.arr[4] = ctypes.addressof(size)
+    out3.zero_()
+    plan.run(blk, _stream())
+    torch.cuda.synchronize()
+    assert_close(out3.cpu().numpy(), want(x0), F32_RTOL, F32_ATOL, "replay with an element offset")
+
+
+def test_plan_refuses_other_extents_strides_and_symbols():
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    rng = np.random.default_rng(3)
+    M, K, H, N = 16, 32, 32, 8
+    plan = Plan()
+    x = torch.zeros((M, K), device="cuda")
+    out = torch.empty((M, N), device="cuda")
+    plan.expect_symbols([M])
+    _record_two_layer(plan, x, out, rng.standard_normal((K, H), dtype=np.float32), np.zeros(H, np.float32),
+                      rng.standard_normal((H, N), dtype=np.float32), H)
+    with pytest.raises(C.LlcHipError) as e:  # slot 0 is NULL but the plan expects a symbol
+        plan.run(ParamBlock([x, out]), _stream())
+    assert e.value.status == C.ERR_BAD_ARG
+    with pytest.raises(C.LlcHipError) as e:
+        plan.run(ParamBlock([x, out], symbols=[M + 1]), _stream())
+    assert e.value.status == C.ERR_SHAPE
+    plan.run(ParamBlock([x, out], symbols=[M]), _stream())
+    with pytest.raises(C.LlcHipError) as e:
+        plan.run(ParamBlock([torch.zeros((M + 1, K), device="cuda"), out], symbols=[M]), _stream())
+    assert e.value.status == C.ERR_SHAPE
+    with pytest.raises(C.LlcHipError) as e:
+        plan.run(ParamBlock([torch.zeros((K, M), device="cuda").t(), out], symbols=[M]), _stream())
+    assert e.value.status == C.ERR_LAYOUT
+    # a plan is recorded once, and ops outside begin/end are not recorded
+    assert C.lib().llc_plan_begin(plan.handle) == C.ERR_BAD_ARG
+    assert plan.num_steps == 2
+    torch.cuda.synchronize()
+
+
+def test_entry_library_main_runs_the_bound_plan(oracle):
+    """What Execution::run does (Execution.cpp:12-16, 21-66): resolve `main`, call it with the packed block."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    rng = np.random.default_rng(11)
+    M, K, H, N = 8, 784, 512, 10  # the reference's own MLP case, batch 8
+    w1 = rng.standard_normal((K, H), dtype=np.float32) * 0.02
+    b1 = rng.standard_normal((H,), dtype=np.float32) * 0.02
+    w2 = rng.standard_normal((H, N), dtype=np.float32) * 0.02
+    plan = Plan()
+    x = torch.zeros((M, K), device="cuda")
+    out = torch.empty((M, N), device="cuda")
+    _record_two_layer(plan, x, out, w1, b1, w2, H)
+    L = C.lib()
+    E = ctypes.CDLL(C.ENTRY_LIB_PATH)
+    E.main.restype = None
+    E.main.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    C.check(L.llc_hip_bind_entry(plan.handle, _stream()))
+    try:
+        xs = rng.standard_normal((M, K), dtype=np.float32)
+        x2 = torch.from_numpy(xs).cuda()
+        out2 = torch.zeros((M, N), device="cuda")
+        blk = ParamBlock([x2, out2])
+        E.main(blk.arr)
+        assert L.llc_hip_entry_status() == 0
+        torch.cuda.synchronize()
+        want = oracle.matmul(oracle.unary("relu", oracle.matmul(xs, w1) + b1), w2)
+        assert_close(out2.cpu().numpy(), want, F32_RTOL, F32_ATOL, "main(void**)")
+    finally:
+        C.check(L.llc_hip_bind_entry(None, None))
+    E.main(blk.arr)  # nothing bound: logged, status kept, no launch
+    assert L.llc_hip_entry_status() == C.ERR_BAD_ARG
+
+
+def _run_both_ways(build, calls):
+    """Runs `calls` (a list of argument tuples) through two engines built by `build`, one replaying native plans,
+    one launching kernel by kernel; returns the two lists of results."""
+    from llcompiler_amd.executor import engine as E
+    got = []
+    for use_plan in (True, False):
+        E.USE_PLAN = use_plan
+        try:
+            fn = build()
+            with torch.no_grad():
+                got.append([fn(*a).clone() for a in calls])
+        finally:
+            E.USE_PLAN = True
+    torch.cuda.synchronize()
+    return got
+
+
+def test_engine_plan_replay_matches_kernel_by_kernel_launches_encoder():
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    enc = EncoderBlock().eval().to(torch.bfloat16)
+    ref = copy.deepcopy(enc).float()
+    (x8,) = make_encoder_inputs(2, 128, dtype=torch.bfloat16)
+
+    def build():
+        return compile_module(copy.deepcopy(enc).cuda(), (x8.cuda(),), dynamic_shapes=({0: torch.export.Dim("batch")},))
+
+    calls = []
+    for B, seed in ((2, 0), (2, 1), (3, 2), (2, 3), (3, 4)):  # first calls record, later ones replay
+        (x,) = make_encoder_inputs(B, 128, seed=seed, dtype=torch.bfloat16)
+        calls.append((x.cuda(),))
+    planned, direct = _run_both_ways(build, calls)
+    for (x,), a, b in zip(calls, planned, direct):
+        assert torch.equal(a, b)
+        assert_close(a.float().cpu().numpy(), ref(x.float().cpu()).detach().numpy(), BF16_RTOL, 2e-2, "encoder via plan")
+
+
+def test_engine_plan_replay_matches_kernel_by_kernel_launches_resnet():
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval()
+
+    def build():
+        torch._dynamo.reset()
+        comp = LLCompiler(mode="inference", target="gfx950", pipeline="hip")
+        return torch.compile(copy.deepcopy(m).cuda(), backend=comp, dynamic=False, fullgraph=True)
+
+    calls = [(make_resnet_inputs(2, 64, seed=s)[0].cuda(),) for s in (0, 1, 2)]
+    planned, direct = _run_both_ways(build, calls)
+    with torch.no_grad():
+        for (x,), a, b in zip(calls, planned, direct):
+            assert torch.equal(a, b)
+            assert_close(a.cpu().numpy(), m(x.cpu()).numpy(), F32_RTOL, F32_ATOL, "resnet via plan")
+
+
+def test_engine_inputs_that_stop_sharing_memory_get_their_own_instance(oracle):
+    """An instance binds descriptors to inputs by address; two inputs that are views of one buffer in the
+    recording call and separate tensors later must not be confused."""
+    from llcompiler_amd.compiler.aot import compile_module
+
+    class AddMul(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.relu(a * 2.0 + b)
+
+    both = torch.arange(32, dtype=torch.float32, device="cuda").reshape(2, 16) - 10.0
+    cm = compile_module(AddMul().cuda(), (both[0], both[1]))
+    r1 = cm(both[0], both[1])
+    r1b = cm(both[0], both[1])
+    a = torch.full((16,), 3.0, device="cuda")
+    b = torch.full((16,), -5.0, device="cuda")
+    r2 = cm(a, b)       # same shapes and strides, no shared memory
+    r2b = cm(a, b)
+    r3 = cm(both[0], both[1])
+    r4 = cm(a, a)       # one tensor twice ...
+    r5 = cm(a, b)       # ... and apart again
+    r6 = cm(b, b)
+    torch.cuda.synchronize()
+    w = both.cpu().numpy()
+    want1 = oracle.unary("relu", w[0] * 2.0 + w[1])
+    for r in (r1, r1b, r3):
+        np.testing.assert_array_equal(r.cpu().numpy(), want1)
+    for r in (r2, r2b, r5):
+        np.testing.assert_array_equal(r.cpu().numpy(), np.full(16, 1.0, np.float32))
+    np.testing.assert_array_equal(r4.cpu().numpy(), np.full(16, 9.0, np.float32))
+    np.testing.assert_array_equal(r6.cpu().numpy(), np.full(16, 0.0, np.float32))
