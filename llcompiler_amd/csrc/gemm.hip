@@ -8,7 +8,8 @@
 //
 // Three kernels share the tile geometry of gemm_core.hpp.  gemm_kernel (any type, any strides, ragged shapes)
 // is described here; gemm_dma_kernel and gemm_dma2_kernel (16-bit operands, complete tiles, operands moved
-// straight into LDS) are described where they are defined.
+// straight into LDS) are described where they are defined.  A fourth, gemm_skinny_kernel, takes products of
+// at most 16 rows without the matrix cores (one pass over the weight, bound by its latency).
 //
 // Data path of gemm_kernel per workgroup (4 waves in a 2x2 grid, or 8 waves 4x2 on 128x128 tiles with a deep
 // reduction; macro tile BM x BN):
@@ -674,6 +675,92 @@ int launch_tiles(const GemmParams& p, int batch, hipStream_t s) {
   return launch_cfg<T, 64, 64, 2, 2, LA, LB>(p, batch, s);
 }
 
+// ---- skinny products: at most 16 rows, both operands contiguous along k (x [M,K] times a linear layer's
+// weight [N,K] read as its transpose).  A tile kernel would leave all but a few CUs idle and walk k in ~30
+// dependent steps; this one is a single pass: one workgroup per NW output columns, its four waves split k in
+// 64-lane vector chunks, every lane keeps MR x NW partial sums that are then added across the wave and
+// across the waves (LDS).  The sums are taken in a fixed order, so results do not vary from run to run.
+template <typename T>
+__device__ __forceinline__ void unpack_vec(const u32x4_t& v, float* f) {
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = __uint_as_float(v[e]);
+  } else if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[2 * e] = __uint_as_float(v[e] << 16);
+      f[2 * e + 1] = __uint_as_float(v[e] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[2 * e] = f16_bits_to_f32((uint16_t)(v[e] & 0xffffu));
+      f[2 * e + 1] = f16_bits_to_f32((uint16_t)(v[e] >> 16));
+    }
+  }
+}
+
+template <typename T, int MR, int NW>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmParams p) {
+  constexpr int VEC = 16 / sizeof(T);
+  __shared__ float red[4][MR * NW];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int n0 = blockIdx.x * NW;
+  const T* A = (const T*)p.A;
+  const T* B = (const T*)p.B;
+  float acc[MR][NW];
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int j = 0; j < NW; ++j) acc[m][j] = 0.0f;
+  for (int k = (int)threadIdx.x * VEC; k < p.K; k += 256 * VEC) {
+    u32x4_t av[MR], bv[NW];
+    // rows and columns past the end re-read the last one; their sums are never stored
+#pragma unroll
+    for (int m = 0; m < MR; ++m) av[m] = *(const u32x4_t*)(A + (int64_t)(m < p.M ? m : p.M - 1) * p.a_sm + k);
+#pragma unroll
+    for (int j = 0; j < NW; ++j) bv[j] = *(const u32x4_t*)(B + (int64_t)(n0 + j < p.N ? n0 + j : p.N - 1) * p.b_sn + k);
+    float bf[NW][VEC];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) unpack_vec<T>(bv[j], bf[j]);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      float af[VEC];
+      unpack_vec<T>(av[m], af);
+#pragma unroll
+      for (int j = 0; j < NW; ++j)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[m][j] = fmaf(af[e], bf[j][e], acc[m][j]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const float v = wave_sum(acc[m][j]);
+      if (lane == 0) red[wave][m * NW + j] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < MR * NW) {
+    const int m = threadIdx.x / NW, n = n0 + threadIdx.x % NW;
+    if (m < p.M && n < p.N) {
+      const float v = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+      const float bias = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, n) : 0.0f;
+      epilogue_store<T>((T*)p.C, (int64_t)m * p.c_sm + n, v, p.alpha, bias, p.residual, p.act);
+    }
+  }
+}
+
+template <typename T>
+int launch_skinny(const GemmParams& p, hipStream_t s) {
+  if (p.M <= 4) {
+    hipLaunchKernelGGL((gemm_skinny_kernel<T, 4, 2>), dim3((unsigned)((p.N + 1) / 2)), dim3(256), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((gemm_skinny_kernel<T, 16, 1>), dim3((unsigned)p.N), dim3(256), 0, s, p);
+  }
+  return check_launch("gemm_skinny_kernel");
+}
+
 template <typename T>
 int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
@@ -681,6 +768,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   const bool a_kvec = p.a_sk == 1 && p.a_sm % EPV == 0 && p.a_sb % EPV == 0 && p.a_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.A);
   const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.B);
   const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.N % EPV == 0 && al16(p.B);
+  if (batch == 1 && p.M <= 16 && a_kvec && b_kvec) return launch_skinny<T>(p, s);
   if constexpr (sizeof(T) == 2) {
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
     if (a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&

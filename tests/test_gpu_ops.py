@@ -338,6 +338,32 @@ def test_matmul_16bit_complete_tiles(ops, oracle, M, N, K):
         assert_close_bf16(host(ops.matmul(da, bt.t(), epi)), bf16_round(w), "NT epilogue " + act)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 100, 256), (4, 512, 784), (4, 10, 512), (3, 33, 1032), (5, 33, 1032), (16, 64, 2048),
+                                   (13, 7, 40), (2, 1, 8)])
+def test_matmul_skinny(ops, oracle, M, N, K):
+    """At most 16 rows times a [N,K] weight read as its transpose (a linear layer on a small batch) takes the
+    single-pass kernel: every dtype, the fused epilogue, rows taken from a wider buffer."""
+    r = rng(M * 5 + N * 11 + K)
+    a = bf16_round(r.uniform(-1, 1, (M, K)))
+    w = bf16_round(r.uniform(-1, 1, (N, K)))
+    bias = bf16_round(r.standard_normal(N))
+    res = bf16_round(r.standard_normal((M, N)))
+    base = oracle.matmul(a, np.ascontiguousarray(w.T), "mkn")
+    wide = np.zeros((M, K + 24), np.float32)
+    wide[:, 8:8 + K] = a
+    for dt, close, rnd in ((torch.float32, assert_close_f32, lambda x: x), (torch.bfloat16, assert_close_bf16, bf16_round),
+                           (torch.float16, assert_close_bf16, lambda x: x)):
+        da, dw = dev(a, dt), dev(w, dt)
+        close(host(ops.matmul(da, dw.t())), rnd(base), "skinny %s" % dt)
+        close(host(ops.matmul(dev(wide, dt)[:, 8:8 + K], dw.t())), rnd(base), "skinny strided rows %s" % dt)
+        for act, alpha in [("none", 1.0), ("relu", 0.5), ("gelu", 0.125)]:
+            want = base * np.float32(alpha) + bias[None, :] + res
+            if act != "none":
+                want = oracle.unary(act, want)
+            epi = ops.Epilogue(alpha=alpha, bias=dev(bias, dt), residual=dev(res, dt), act=act)
+            close(host(ops.matmul(da, dw.t(), epi)), rnd(want), "skinny epilogue %s %s" % (act, dt))
+
+
 def test_batch_matmul_16bit_complete_tiles(ops, oracle):
     r = rng(77)
     a = bf16_round(r.uniform(-1, 1, (8, 512, 256)))
