@@ -118,9 +118,9 @@ def time_gpu(fn, steps, warmup):
 # size gives): profiles/single_op_suite_hbm_counters.md holds the commands and the table.  Counters cannot
 # be read from inside a timed run, so these are carried as measured constants of the kernels as committed.
 MEASURED_TRAFFIC_BYTES = {
-    "matmul_f32": 117758192, "matmul_bf16": 59044501, "batch_matmul_f32": 59286732, "batch_matmul_bf16": 30304309,
-    "add_relu_f32": 805453727, "add_relu_bf16": 402808062, "softmax_f32": 134297839, "softmax_bf16": 67193794,
-    "layernorm_f32": 67269002, "layernorm_bf16": 33671537, "copy_f32": 536870912,
+    "matmul_f32": 117661870, "matmul_bf16": 58942540, "batch_matmul_f32": 59096383, "batch_matmul_bf16": 29560277,
+    "add_relu_f32": 805396346, "add_relu_bf16": 402856019, "softmax_f32": 134281219, "softmax_bf16": 67171380,
+    "layernorm_f32": 67250632, "layernorm_bf16": 33666897, "copy_f32": 536870912,
 }
 
 
