@@ -217,6 +217,17 @@ int llc_hip_copy(const llc_tensor* x, llc_tensor* out, void* stream);
 /* Row gather along dim 0 with int64 indices (aten.embedding / index_select, left to torch eager
  * by the reference): out[i, ...] = table[idx[i], ...]. */
 int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream);
+/* Fused attention: out = softmax(scale * q k^T + mask) v over the key dim, for the op group the importer
+ * produces from an attention layer: llh.batch_matmul (LLHOps.td:446-452) of q with the transposed keys, the
+ * scaling mul/div and the mask add (LLHOps.td:357-393), the softmax chain (amax, sub, exp, sum, div;
+ * llcompiler/compiler/torch_compile_config.py:24) and the llh.batch_matmul with v.  The reference lowers each
+ * of these to its own loop nest; the fused form never writes the [B, H, Sq, Skv] scores.
+ * q, out: [B, H, Sq, 64]; k, v: [B, H, Skv, 64]; bf16 or f16; the last dim contiguous, the other strides
+ * free (multiples of 8 elements), so head-split views of [B, S, H*64] activations are read and written in
+ * place.  mask: NULL or [B, Skv] of the same type, added to every head and query row.  scale > 0. */
+int llc_hip_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask, float scale,
+                      llc_tensor* out, void* stream);
+
 /* llh.convert_to (LLHOps.td:329-335; LLHToHLO.cpp:489) between f32, bf16, f16, i64, i32, i1. */
 int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* stream);
 

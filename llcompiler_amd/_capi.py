@@ -74,6 +74,7 @@ EXPORTS = [
     "llc_hip_batch_matmul", "llc_hip_conv2d", "llc_hip_elementwise", "llc_hip_reduce", "llc_hip_softmax",
     "llc_hip_layer_norm", "llc_hip_max_pool", "llc_hip_global_avg_pool", "llc_hip_transpose",
     "llc_hip_stride_slice", "llc_hip_broadcast_to", "llc_hip_copy", "llc_hip_gather_rows", "llc_hip_convert",
+    "llc_hip_attention",
     "llc_hip_unpack_params",
     "llc_plan_create", "llc_plan_destroy", "llc_plan_alloc", "llc_plan_upload", "llc_plan_declare_io",
     "llc_plan_expect_symbols", "llc_plan_begin", "llc_plan_end", "llc_plan_num_steps", "llc_plan_num_params",
@@ -120,6 +121,7 @@ def lib():
         L.llc_hip_copy.argtypes = [T, T, vp]
         L.llc_hip_gather_rows.argtypes = [T, T, T, vp]
         L.llc_hip_convert.argtypes = [T, T, vp]
+        L.llc_hip_attention.argtypes = [T, T, T, T, ctypes.c_float, T, vp]
         L.llc_hip_init.argtypes = [ctypes.c_int]
         L.llc_hip_unpack_params.argtypes = [P(vp), ctypes.c_size_t, P(ctypes.c_size_t), P(ctypes.c_size_t), T,
                                             P(i64p)]

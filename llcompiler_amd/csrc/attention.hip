@@ -1,0 +1,317 @@
+// Fused attention: out = softmax(scale * Q K^T + mask) V in one pass over the keys.
+//
+// The unfused group (llh.batch_matmul, the mask add folded into its epilogue, the softmax chain,
+// llh.batch_matmul) writes and re-reads the [B, H, Sq, Skv] score tensor four times; it is the largest
+// stream of bytes of an attention layer.  Here a workgroup keeps 128 queries of one head in registers and walks
+// the keys in blocks of 64 with a running maximum and a running sum (the scores never leave the CU):
+//
+//   per wave: 32 queries.  S^T[key, query] = K Q^T on the matrix cores with the K block as the row operand
+//   (read from LDS) and the wave's Q fragments as the column operand (registers, loaded once).  In the
+//   accumulator layout a lane then owns ONE query (lane % 32) and 32 of the 64 keys, so the row maximum and row
+//   sum are in-lane loops plus one exchange with lane ^ 32.  exp2 of the shifted scores, rounded to the storage
+//   type, is already laid out as the column operand of O^T[d, query] += V^T P^T when the key order inside a
+//   16-key step is taken as the accumulator's (keys 4h..4h+3 and 8+4h..8+4h+3 for lane half h); the V block is
+//   read from LDS with the transposing read, which hands a lane four consecutive keys of one d.
+//   O^T keeps the query on the lane, so the rescaling by exp2(m_old - m_new) is one multiplier per lane.
+//
+// LDS per stage: K block [64 keys][128 B] with the row-XOR chunk swizzle of the GEMM tiles, V block
+// [64 keys][128 B] with chunk c stored at c ^ 2 (key & 3) (the four key rows a transposing read touches fall
+// in different banks), and the additive row (mask, -inf past the last key) as fp32.  Two stages: the global
+// loads of block i+1 are issued before the arithmetic of block i and written to the other stage after it; one
+// barrier per block.
+#include "gemm_core.hpp"
+
+namespace llc {
+namespace {
+using namespace gemm;
+
+struct AttnParams {
+  const char* Q;
+  const char* K;
+  const char* V;
+  const char* mask;  // [B, Skv] additive, storage type, or null
+  char* O;
+  int32_t B, H, Sq, Skv;
+  int64_t q_sb, q_sh, q_ss;  // element strides of the [B, H, S, 64] views; the last dim is contiguous
+  int64_t k_sb, k_sh, k_ss;
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int64_t m_sb;
+  float scale_log2e;
+};
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kD = 64;
+constexpr int kBlockQ = 128, kBlockKV = 64;
+constexpr int kTileBytes = kBlockKV * 128;
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, bf2));
+  } else {
+    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+  }
+}
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_tr16(const char* p) {
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
+  return __builtin_bit_cast(uint2, v);
+}
+
+// ADD: scores get the additive LDS row (a mask, and -inf for keys past Skv).  Without it Skv is a multiple of 64.
+template <typename T, bool ADD>
+__global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
+  __shared__ __align__(16) char kt[2][kTileBytes];
+  __shared__ __align__(16) char vt[2][kTileBytes];
+  __shared__ __align__(16) float addrow[2][kBlockKV];
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int li = lane % 32, lh = lane / 32;
+  const int bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
+  const int q0 = blockIdx.x * kBlockQ + wave * 32;
+  const T* Q = (const T*)p.Q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const T* K = (const T*)p.K + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+  const T* V = (const T*)p.V + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+  const T* M = p.mask ? (const T*)p.mask + (int64_t)b * p.m_sb : nullptr;
+
+  // this lane's query row as the column operand of S^T: 8 consecutive d per 16-d step
+  u32x4_t qf[4];
+  {
+    const int qrow = q0 + li < p.Sq ? q0 + li : p.Sq - 1;
+    const T* qp = Q + (int64_t)qrow * p.q_ss + lh * 8;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const u32x4_t*)(qp + ks * 16);
+  }
+
+  // block loader: 512 16-byte chunks of K and of V by 256 lanes
+  int lrow[2], koff[2], voff[2];
+  const int lc = tid % 8;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    lrow[j] = (tid + 256 * j) / 8;
+    koff[j] = lrow[j] * 128 + ((lc ^ lds_swz(lrow[j])) << 4);
+    voff[j] = lrow[j] * 128 + ((lc ^ ((lrow[j] & 3) << 1)) << 4);
+  }
+  u32x4_t kr[2], vr[2];
+  float ar = 0.0f;
+  auto gload = [&](int blk) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      int row = blk * kBlockKV + lrow[j];
+      row = row < p.Skv ? row : p.Skv - 1;
+      kr[j] = *(const u32x4_t*)(K + (int64_t)row * p.k_ss + lc * 8);
+      vr[j] = *(const u32x4_t*)(V + (int64_t)row * p.v_ss + lc * 8);
+    }
+    if constexpr (ADD) {
+      if (tid < kBlockKV) {
+        const int key = blk * kBlockKV + tid;
+        const int kc = key < p.Skv ? key : p.Skv - 1;
+        float mv = 0.0f;
+        if (M) mv = load_as_f32((const char*)M, Elem<T>::kDtype, kc) * kLog2e;
+        ar = key < p.Skv ? mv : -INFINITY;
+      }
+    }
+  };
+  auto lstore = [&](int s) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      *(u32x4_t*)(kt[s] + koff[j]) = kr[j];
+      *(u32x4_t*)(vt[s] + voff[j]) = vr[j];
+    }
+    if constexpr (ADD) {
+      if (tid < kBlockKV) addrow[s][tid] = ar;
+    }
+  };
+
+  // fragment addresses inside a stage
+  int ka[2][4];  // K rows 32 T + li, chunk 2 ks + lh
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int row = 32 * t2 + li;
+      ka[t2][ks] = row * 128 + (((2 * ks + lh) ^ lds_swz(row)) << 4);
+    }
+  // V: a 16-lane group reads a 4 (keys) x 16 (d) patch; lane = 16 g + 4 jj + q addresses key row jj, d chunk q
+  int va[2][2];  // [d tile][which run of four keys]
+  {
+    const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int row = 8 * u + 4 * (g >> 1) + jj;
+        const int c = 4 * dt + 2 * (g & 1) + (q >> 1);
+        va[dt][u] = row * 128 + ((c ^ (jj << 1)) << 4) + (q & 1) * 8;
+      }
+  }
+
+  f32x16_t oacc[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const int nblk = (p.Skv + kBlockKV - 1) / kBlockKV;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int s = blk & 1;
+    if (blk + 1 < nblk) gload(blk + 1);
+    const char* kb = kt[s];
+    const char* vb = vt[s];
+
+    // S^T = K Q^T for 64 keys x 32 queries
+    f32x16_t sacc[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[t2][r] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) mfma_step<T>(*(const u32x4_t*)(kb + ka[t2][ks]), qf[ks], sacc[t2]);
+    }
+    // x = scores in log2 units; accumulator register 4 i + j of tile T is key 32 T + 8 i + 4 lh + j
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (ADD) {
+          const f32x4_t av = *(const f32x4_t*)&addrow[s][32 * t2 + 8 * i + 4 * lh];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sacc[t2][4 * i + j] = fmaf(sacc[t2][4 * i + j], p.scale_log2e, av[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mx = fmaxf(mx, sacc[t2][4 * i + j]);
+      }
+    if constexpr (!ADD) mx *= p.scale_log2e;  // scale > 0: the maximum commutes with it
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    // (a row whose keys so far are all masked with -inf keeps m = -inf: shift by 0 then, so that no inf - inf forms)
+    const float m_max = fmaxf(m_run, mx);
+    const float m_new = m_max == -INFINITY ? 0.0f : m_max;
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_max;
+    float psum = 0.0f;
+    u32x4_t pb[2][2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float pv[2];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            const float x = sacc[t2][8 * t + 2 * e + w];
+            pv[w] = ADD ? __builtin_amdgcn_exp2f(x - m_new) : __builtin_amdgcn_exp2f(fmaf(x, p.scale_log2e, -m_new));
+            psum += pv[w];
+          }
+          pb[t2][t][e] = pack2<T>(pv[0], pv[1]);
+        }
+    l_run = l_run * corr + psum;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    // O^T += V^T P^T, 16 keys per step
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const char* vrow = vb + (32 * t2 + 16 * t) * 128;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          const uint2 lo = lds_tr16(vrow + va[dt][0]), hi = lds_tr16(vrow + va[dt][1]);
+          mfma_step<T>(u32x4_t{lo.x, lo.y, hi.x, hi.y}, pb[t2][t], oacc[dt]);
+        }
+      }
+    if (blk + 1 < nblk) lstore(s ^ 1);
+    __syncthreads();
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  const float inv = 1.0f / l_tot;
+  if (q0 + li < p.Sq) {
+    T* op = (T*)p.O + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)(q0 + li) * p.o_ss;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint2 w;
+        w.x = pack2<T>(oacc[dt][4 * i] * inv, oacc[dt][4 * i + 1] * inv);
+        w.y = pack2<T>(oacc[dt][4 * i + 2] * inv, oacc[dt][4 * i + 3] * inv);
+        *(uint2*)(op + 32 * dt + 8 * i + 4 * lh) = w;
+      }
+  }
+}
+
+int view4(const llc_tensor* t, const char* what, View* v) {
+  LLC_TRY(make_view(t, what, v));
+  if (v->rank != 4) return set_error(LLC_ERR_SHAPE, "%s: rank 4 expected, [B, H, S, D]", what);
+  if (v->size[3] != kD) return set_error(LLC_ERR_UNSUPPORTED, "%s: head dim %lld (64 is implemented)", what, (long long)v->size[3]);
+  if (v->stride[3] != 1 || v->stride[0] % 8 || v->stride[1] % 8 || v->stride[2] % 8 || ((uintptr_t)v->ptr % 16))
+    return set_error(LLC_ERR_LAYOUT, "%s: the head dim must be contiguous and every row 16-byte aligned", what);
+  return LLC_OK;
+}
+
+}  // namespace
+}  // namespace llc
+
+using namespace llc;
+
+int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask, float scale,
+                       llc_tensor* out, void* stream) {
+  View a, b, c, o, m;
+  LLC_TRY(view4(q, "attention q", &a));
+  LLC_TRY(view4(k, "attention k", &b));
+  LLC_TRY(view4(v, "attention v", &c));
+  LLC_TRY(view4(out, "attention out", &o));
+  if (a.dtype != b.dtype || a.dtype != c.dtype || a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "attention: operand types differ");
+  if (a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16)
+    return set_error(LLC_ERR_DTYPE, "attention: bf16 or f16 operands (type %d given)", a.dtype);
+  for (int d = 0; d < 2; ++d)
+    if (a.size[d] != b.size[d] || a.size[d] != c.size[d] || a.size[d] != o.size[d])
+      return set_error(LLC_ERR_SHAPE, "attention: batch dims differ");
+  if (b.size[2] != c.size[2] || o.size[2] != a.size[2]) return set_error(LLC_ERR_SHAPE, "attention: sequence lengths differ");
+  if (!(scale > 0.0f)) return set_error(LLC_ERR_UNSUPPORTED, "attention: scale must be positive");
+  AttnParams p{};
+  p.B = (int)a.size[0];
+  p.H = (int)a.size[1];
+  p.Sq = (int)a.size[2];
+  p.Skv = (int)b.size[2];
+  if (a.size[0] * a.size[1] > 65535 || a.size[2] > 0x7fffff00 || b.size[2] > 0x7fffff00)
+    return set_error(LLC_ERR_TOO_LARGE, "attention: more than 65535 heads in all, or a sequence too long");
+  if (mask) {
+    LLC_TRY(make_view(mask, "attention mask", &m));
+    if (m.dtype != a.dtype) return set_error(LLC_ERR_DTYPE, "attention: mask type differs");
+    if (m.rank != 2 || m.size[0] != a.size[0] || m.size[1] != b.size[2] || (m.size[1] != 1 && m.stride[1] != 1))
+      return set_error(LLC_ERR_SHAPE, "attention: mask must be [B, Skv] with contiguous rows");
+    p.mask = m.ptr;
+    p.m_sb = m.stride[0];
+  }
+  if (o.numel() == 0) return LLC_OK;
+  if (p.Skv == 0) return set_error(LLC_ERR_SHAPE, "attention: no keys");
+  p.Q = a.ptr, p.K = b.ptr, p.V = c.ptr, p.O = o.ptr;
+  p.q_sb = a.stride[0], p.q_sh = a.stride[1], p.q_ss = a.stride[2];
+  p.k_sb = b.stride[0], p.k_sh = b.stride[1], p.k_ss = b.stride[2];
+  p.v_sb = c.stride[0], p.v_sh = c.stride[1], p.v_ss = c.stride[2];
+  p.o_sb = o.stride[0], p.o_sh = o.stride[1], p.o_ss = o.stride[2];
+  p.scale_log2e = scale * kLog2e;
+  const dim3 grid((unsigned)((p.Sq + kBlockQ - 1) / kBlockQ), (unsigned)(p.B * p.H));
+  const bool add = p.mask || p.Skv % kBlockKV != 0;
+  hipStream_t s = as_stream(stream);
+  if (a.dtype == LLC_BFLOAT16) {
+    if (add) hipLaunchKernelGGL((attention_kernel<__bf16, true>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((attention_kernel<__bf16, false>), grid, dim3(256), 0, s, p);
+  } else {
+    if (add) hipLaunchKernelGGL((attention_kernel<_Float16, true>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((attention_kernel<_Float16, false>), grid, dim3(256), 0, s, p);
+  }
+  return check_launch("attention_kernel");
+}

@@ -24,3 +24,5 @@ int llc_impl_broadcast_to(const llc_tensor* x, llc_tensor* out, void* stream);
 int llc_impl_copy(const llc_tensor* x, llc_tensor* out, void* stream);
 int llc_impl_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tensor* out, void* stream);
 int llc_impl_convert(const llc_tensor* x, llc_tensor* out, void* stream);
+int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask, float scale,
+                       llc_tensor* out, void* stream);

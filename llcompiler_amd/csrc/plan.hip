@@ -21,7 +21,7 @@ namespace {
 
 enum OpCode {
   kMatmul, kBatchMatmul, kConv2d, kElementwise, kReduce, kSoftmax, kLayerNorm, kMaxPool, kGlobalAvgPool,
-  kTranspose, kStrideSlice, kBroadcastTo, kCopy, kGatherRows, kConvert,
+  kTranspose, kStrideSlice, kBroadcastTo, kCopy, kGatherRows, kConvert, kAttention,
 };
 
 // Owned copy of a tensor descriptor.
@@ -211,6 +211,7 @@ int replay(Step& s, void* stream) {
     case kCopy: return llc_impl_copy(o[0].ptr(), o[1].ptr(), stream);
     case kGatherRows: return llc_impl_gather_rows(o[0].ptr(), o[1].ptr(), o[2].ptr(), stream);
     case kConvert: return llc_impl_convert(o[0].ptr(), o[1].ptr(), stream);
+    case kAttention: return llc_impl_attention(o[0].ptr(), o[1].ptr(), o[2].ptr(), o[3].ptr(), s.alpha, o[4].ptr(), stream);
   }
   return set_error(LLC_ERR_BAD_ARG, "plan: unknown step code %d", s.op);
 }
@@ -357,6 +358,16 @@ extern "C" int llc_hip_convert(const llc_tensor* x, llc_tensor* out, void* strea
   if (!t_rec) return LLC_OK;
   Recorder r(kConvert, 2);
   r.tensor(0, x), r.tensor(1, out);
+  return r.commit();
+}
+
+extern "C" int llc_hip_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask,
+                                 float scale, llc_tensor* out, void* stream) {
+  LLC_TRY(llc_impl_attention(q, k, v, mask, scale, out, stream));
+  if (!t_rec) return LLC_OK;
+  Recorder r(kAttention, 5);
+  r.tensor(0, q), r.tensor(1, k), r.tensor(2, v), r.tensor(3, mask), r.tensor(4, out);
+  r.st.alpha = scale;
   return r.commit();
 }
 

@@ -40,6 +40,8 @@ MIN_CALLS_FOR_GRAPH = 2
 # reference's packed parameter block and make one call into the library, which replays the launches.  With
 # False every run launches kernel by kernel from Python (same kernels, same arguments).
 USE_PLAN = True
+# batch_matmul -> softmax -> batch_matmul groups of 16-bit attention layers with head dim 64 become one fused kernel
+FUSE_ATTENTION = True
 
 
 def _concrete(shape, env):
@@ -215,9 +217,120 @@ class Instance:
 
         consumers = {}
         for st in steps:
-            for v in st.inputs:
+            reads = list(st.inputs)
+            e = st.attrs.get("epilogue") if isinstance(st.attrs, dict) else None
+            if e:
+                reads += [x for x in (e.get("bias"), e.get("residual")) if x is not None]
+            for v in reads:
                 consumers.setdefault(id(v), []).append(st)
         skip = set()
+
+        def only_consumer(v):
+            u = consumers.get(id(v), [])
+            return u[0] if len(u) == 1 and id(v) not in out_ids else None
+
+        producer = {id(st.output): st for st in steps}
+
+        def resolve_early(v):
+            """Makes val[v] available ahead of its turn when v is only views away from a value that exists."""
+            if id(v) in val:
+                return True
+            st = producer.get(id(v))
+            if st is None or st.kind != "view" or not resolve_early(st.inputs[0]):
+                return False
+            val[id(v)] = self._view(st, materialise(val[id(st.inputs[0])]), contiguous)
+            skip.add(id(st))
+            return True
+
+        def attention_group(st):
+            """scores = batch_matmul(q, k^T) {alpha, mask rows} -> softmax over the keys -> batch_matmul(p, v), every
+            intermediate read once and only reshaped in between: returns (softmax step, second product, the
+            reshapes) or None."""
+            e = st.attrs["epilogue"]
+            if e["act"] or e["residual"] is not None or e["alpha"] <= 0 or (e["bias"] is not None and not e.get("bias_rows")):
+                return None
+            if st.output.dtype not in (torch.bfloat16, torch.float16):
+                return None
+            between = []
+
+            def through_reshapes(v):
+                u = only_consumer(v)
+                while u is not None and u.kind == "view" and u.attrs["op"] in ("reshape", "flatten"):
+                    between.append(u)
+                    v = u.output
+                    u = only_consumer(v)
+                return v, u
+
+            v, u = through_reshapes(st.output)
+            if u is None or u.kind != "softmax":
+                return None
+            n_keys = _concrete(st.attrs["natural_shape"], self.env)[-1]
+            if _concrete(u.inputs[0].shape, self.env)[-1] != n_keys:
+                return None
+            sm = u
+            v, u = through_reshapes(sm.output)
+            if u is None or u.kind != "batch_matmul" or u.inputs[0] is not v or u.inputs[1] is v:
+                return None
+            e2 = u.attrs["epilogue"]
+            if e2["act"] or e2["residual"] is not None or e2["bias"] is not None or e2["alpha"] != 1.0:
+                return None
+            return sm, u, between
+
+        def fused_attention(st):
+            """Emits one attention call for the group that starts at `st` when the operands allow it (head dim 64,
+            16-bit, rows addressable as [B, H, S, 64] views); returns False to leave the group to its own kernels."""
+            grp = attention_group(st)
+            if grp is None:
+                return False
+            sm, second, between = grp
+            if not resolve_early(second.inputs[1]):
+                return False
+            e = st.attrs["epilogue"]
+            qa, ka = (batched_operand(val[id(v)]) for v in st.inputs)
+            va = batched_operand(val[id(second.inputs[1])])
+            nat = _concrete(st.attrs["natural_shape"], self.env)
+            if e.get("bias_rows"):
+                full = _concrete(st.output.shape, self.env)
+                b0, b1 = full[0], full[1]
+            else:
+                four = [t for t in (qa, ka, va) if t.dim() == 4]
+                b0, b1 = (four[0].shape[0], four[0].shape[1]) if four else (nat[0], 1)
+
+            def as4(t):
+                if t.dim() == 4:
+                    return t if tuple(t.shape[:2]) == (b0, b1) else None
+                if t.dim() != 3 or t.shape[0] != b0 * b1:
+                    return None
+                return t.as_strided((b0, b1, t.shape[1], t.shape[2]), (b1 * t.stride(0), t.stride(0), t.stride(1), t.stride(2)))
+
+            q4, k4, v4 = as4(qa), as4(ka), as4(va)
+            if q4 is None or k4 is None or v4 is None:
+                return False
+            k4 = k4.transpose(-1, -2)
+            for t in (q4, k4, v4):
+                if t.shape[3] != 64 or t.stride(3) != 1 or any(s % 8 for s in t.stride()[:3]) or t.data_ptr() % 16:
+                    return False
+            if k4.shape[2] != v4.shape[2] or k4.shape[2] != nat[2] or q4.shape[2] != nat[1] or k4.shape[2] == 0:
+                return False
+            mask = None
+            if e["bias"] is not None:
+                mask = materialise(val[id(e["bias"])])
+                mask = contiguous(mask.reshape(-1) if mask.is_contiguous() else mask).reshape(-1).view(b0, nat[2])
+            out = new_tensor(second.output)
+            sq = nat[1]
+            o4 = out.view(b0, b1, sq, 64)
+            hm = head_merge(second, b0 * b1, sq, 64)
+            if hm is not None and (hm[1], hm[2]) == (b0, b1):
+                # the head merge that follows, [B, H, S, 64] -> [B, S, H, 64], is done by the kernel's stores
+                o4 = out.view(-1).view(b0, sq, b1, 64).permute(0, 2, 1, 3)
+                val[id(hm[0].output)] = o4
+                skip.add(id(hm[0]))
+            if out.numel():
+                self._launch_later(ops.attention(q4, k4, v4, mask, scale=e["alpha"], out=o4, defer=True))
+            val[id(second.output)] = out
+            for x in [sm, second] + between:
+                skip.add(id(x))
+            return True
 
         def head_merge(st, nb, m, n):
             """batch_matmul -> reshape [B0,B1,M,N] -> transpose (0,2,1,3), each read once: returns (reshape step,
@@ -236,6 +349,11 @@ class Instance:
         for si, st in enumerate(steps):
             k = st.kind
             if id(st) in skip:
+                continue
+            if k == "batch_matmul" and FUSE_ATTENTION and fused_attention(st):
+                for buf in temps:
+                    pool.give(buf)
+                del temps[:]
                 continue
             if k == "batch_matmul":
                 ins = [batched_operand(val[id(v)]) for v in st.inputs]

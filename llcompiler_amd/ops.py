@@ -259,3 +259,14 @@ def convert(x, dtype, out=None, defer=False):
         out = torch.empty(tuple(x.shape), dtype=dtype, device=dev)
     rx, ro = C.tensor_ref(x), C.tensor_ref(out)
     return _launch(C.lib().llc_hip_convert, (rx.ptr, ro.ptr), (rx, ro), out, dev, defer)
+
+
+def attention(q, k, v, mask=None, scale=1.0, out=None, defer=False):
+    """softmax(scale * q k^T + mask) v.  q, out: [B, H, Sq, 64]; k, v: [B, H, Skv, 64] (strided views allowed, last
+    dim contiguous); mask: None or [B, Skv]."""
+    dev = _dev(q)
+    if out is None:
+        out = torch.empty(tuple(q.shape), dtype=q.dtype, device=dev)
+    rq, rk, rv, ro, rm = C.tensor_ref(q), C.tensor_ref(k), C.tensor_ref(v), C.tensor_ref(out), C.tensor_ref(mask)
+    return _launch(C.lib().llc_hip_attention, (rq.ptr, rk.ptr, rv.ptr, rm.ptr if rm else None, float(scale), ro.ptr),
+                   (rq, rk, rv, ro, rm), out, dev, defer)

@@ -95,6 +95,45 @@ def test_config5_bert_f32_symbolic_seq():
     assert len(cm.engine.instances) == 3
 
 
+def _kernel_names(engine):
+    return [[c.fn.__name__ for c in inst.calls] for inst in engine.instances.values()]
+
+
+def test_attention_group_becomes_one_kernel_bf16():
+    """Encoder block (no mask) and a 2-layer BERT stack in bf16 (mask rows): the batch_matmul -> softmax ->
+    batch_matmul group runs as llc_hip_attention, and the result equals the unfused plan's within bf16 rounding."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.executor import engine as E
+    from llcompiler_amd.test_models import BertEncoder, EncoderBlock, make_bert_inputs, make_encoder_inputs
+    enc = EncoderBlock().eval().to(torch.bfloat16)
+    (x,) = make_encoder_inputs(2, 256, dtype=torch.bfloat16)
+    bert = BertEncoder(layers=2).eval().to(torch.bfloat16)
+    xb, mb = (t.to(torch.bfloat16) for t in make_bert_inputs(3, 192))
+    results = {}
+    for fuse in (True, False):
+        E.FUSE_ATTENTION = fuse
+        try:
+            with torch.no_grad():
+                ce = compile_module(copy.deepcopy(enc).cuda(), (x.cuda(),))
+                cb = compile_module(copy.deepcopy(bert).cuda(), (xb.cuda(), mb.cuda()))
+                results[fuse] = (ce(x.cuda()).float().cpu().numpy(), cb(xb.cuda(), mb.cuda()).float().cpu().numpy(),
+                                 _kernel_names(ce.engine)[0], _kernel_names(cb.engine)[0])
+        finally:
+            E.FUSE_ATTENTION = True
+    fe, fb, names_e, names_b = results[True]
+    ue, ub, unames_e, unames_b = results[False]
+    assert names_e.count("llc_hip_attention") == 1 and names_e.count("llc_hip_batch_matmul") == 0 and names_e.count("llc_hip_softmax") == 0
+    assert names_b.count("llc_hip_attention") == 2 and names_b.count("llc_hip_batch_matmul") == 0
+    assert unames_e.count("llc_hip_batch_matmul") == 2 and unames_b.count("llc_hip_batch_matmul") == 4
+    with torch.no_grad():
+        want_e = copy.deepcopy(enc).float()(x.float()).numpy()
+        want_b = copy.deepcopy(bert).float()(xb.float(), mb.float()).numpy()
+    assert_close(fe, want_e, BF16_RTOL, 2e-2, "encoder, fused attention")
+    assert_close(ue, want_e, BF16_RTOL, 2e-2, "encoder, unfused")
+    assert_close(fb, want_b, BF16_RTOL, 3e-2, "bert bf16, fused attention")
+    assert_close(ub, want_b, BF16_RTOL, 3e-2, "bert bf16, unfused")
+
+
 def test_dynamic_torch_compile_reuses_one_engine():
     from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
     enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()

@@ -338,6 +338,72 @@ def test_matmul_16bit_complete_tiles(ops, oracle, M, N, K):
         assert_close_bf16(host(ops.matmul(da, bt.t(), epi)), bf16_round(w), "NT epilogue " + act)
 
 
+def _attention_oracle(oracle, q, k, v, mask, scale, rnd):
+    """The unfused op group on the CPU oracle: batch_matmul, scale, mask add, softmax over the keys, the
+    probabilities rounded to the storage type (the fused kernel feeds them to the matrix cores in it), batch_matmul."""
+    B, H, Sq, D = q.shape
+    Skv = k.shape[2]
+    s = oracle.batch_matmul(q.reshape(B * H, Sq, D), np.ascontiguousarray(k.reshape(B * H, Skv, D).transpose(0, 2, 1)), "mkn")
+    s = s.reshape(B, H, Sq, Skv) * np.float32(scale)
+    if mask is not None:
+        s = s + mask[:, None, None, :]
+    p = rnd(oracle.softmax_lastdim(s.reshape(-1, Skv))).reshape(B * H, Sq, Skv)
+    return oracle.batch_matmul(p, v.reshape(B * H, Skv, D), "mkn").reshape(B, H, Sq, D)
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv,masked", [(1, 1, 128, 128, False), (2, 3, 100, 200, True), (1, 2, 64, 64, False),
+                                             (3, 2, 33, 77, False), (1, 1, 1, 1, True), (2, 12, 256, 256, True),
+                                             (1, 2, 130, 448, False)])
+def test_attention(ops, oracle, B, H, Sq, Skv, masked):
+    r = rng(B * 1000 + H * 100 + Sq + Skv)
+    q = bf16_round(r.uniform(-1, 1, (B, H, Sq, 64)))
+    k = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+    v = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+    mask = None
+    if masked:  # per-sample valid length, the tail at -1e4, as a BERT attention mask
+        mask = np.zeros((B, Skv), np.float32)
+        for b in range(B):
+            mask[b, int(r.integers(Skv // 2, Skv)) + 1:] = -1e4
+        mask = bf16_round(mask)
+    scale = 0.125
+    for dt, rnd in ((torch.bfloat16, bf16_round), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+        want = _attention_oracle(oracle, q, k, v, mask, scale, rnd)
+        dm = dev(mask, dt) if masked else None
+        got = ops.attention(dev(q, dt), dev(k, dt), dev(v, dt), dm, scale)
+        assert_close_bf16(host(got), want, "attention %s" % dt)
+    # head-split views of [B, S, H*64] activations in, the merged layout out (no copies on either side)
+    qs = dev(np.ascontiguousarray(q.transpose(0, 2, 1, 3)).reshape(B, Sq, H * 64), torch.bfloat16)
+    ks = dev(np.ascontiguousarray(k.transpose(0, 2, 1, 3)).reshape(B, Skv, H * 64), torch.bfloat16)
+    vs = dev(np.ascontiguousarray(v.transpose(0, 2, 1, 3)).reshape(B, Skv, H * 64), torch.bfloat16)
+    merged = torch.zeros((B, Sq, H, 64), dtype=torch.bfloat16, device="cuda")
+    ops.attention(qs.view(B, Sq, H, 64).permute(0, 2, 1, 3), ks.view(B, Skv, H, 64).permute(0, 2, 1, 3),
+                  vs.view(B, Skv, H, 64).permute(0, 2, 1, 3), dev(mask, torch.bfloat16) if masked else None, scale,
+                  out=merged.permute(0, 2, 1, 3))
+    want = _attention_oracle(oracle, q, k, v, mask, scale, bf16_round)
+    assert_close_bf16(host(merged).transpose(0, 2, 1, 3), want, "attention on head-split views")
+
+
+def test_attention_fully_masked_leading_block_and_errors(ops, oracle):
+    # -inf on the whole first block of keys: the running maximum stays -inf there and must not turn into NaN
+    r = rng(5)
+    q = bf16_round(r.uniform(-1, 1, (1, 1, 32, 64)))
+    k = bf16_round(r.uniform(-1, 1, (1, 1, 192, 64)))
+    v = bf16_round(r.uniform(-1, 1, (1, 1, 192, 64)))
+    mask = np.zeros((1, 192), np.float32)
+    mask[0, :70] = -np.inf
+    got = host(ops.attention(dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(v, torch.bfloat16), dev(mask, torch.bfloat16), 0.125))
+    want = _attention_oracle(oracle, q[:, :, :, :], k[:, :, 70:], v[:, :, 70:], None, 0.125, bf16_round)
+    assert_close_bf16(got, want, "attention with -inf on the first 70 keys")
+    from llcompiler_amd._capi import LlcHipError
+    x = dev(q, torch.bfloat16)
+    with pytest.raises(LlcHipError):  # fp32 operands are not implemented: an error, not another path
+        ops.attention(dev(q), dev(k), dev(v))
+    with pytest.raises(LlcHipError):
+        ops.attention(x, dev(k, torch.bfloat16)[..., :32], dev(v, torch.bfloat16))  # head dim 32
+    with pytest.raises(LlcHipError):
+        ops.attention(x, dev(k, torch.bfloat16), dev(v, torch.bfloat16)[:, :, :100])  # k and v lengths differ
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 100, 256), (4, 512, 784), (4, 10, 512), (3, 33, 1032), (5, 33, 1032), (16, 64, 2048),
                                    (13, 7, 40), (2, 1, 8)])
 def test_matmul_skinny(ops, oracle, M, N, K):
