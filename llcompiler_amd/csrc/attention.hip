@@ -65,7 +65,7 @@ __device__ __forceinline__ uint2 lds_tr16(const char* p) {
 
 // ADD: scores get the additive LDS row (a mask, and -inf for keys past Skv).  Without it Skv is a multiple of 64.
 template <typename T, bool ADD>
-__global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attention_kernel(const AttnParams p) {
   __shared__ __align__(16) char kt[2][kTileBytes];
   __shared__ __align__(16) char vt[2][kTileBytes];
   __shared__ __align__(16) float addrow[2][kBlockKV];
@@ -192,11 +192,23 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
       }
     if constexpr (!ADD) mx *= p.scale_log2e;  // scale > 0: the maximum commutes with it
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    // (a row whose keys so far are all masked with -inf keeps m = -inf: shift by 0 then, so that no inf - inf forms)
-    const float m_max = fmaxf(m_run, mx);
-    const float m_new = m_max == -INFINITY ? 0.0f : m_max;
-    const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_max;
+    // The shift m only has to keep exp2(x - m) in range, it need not be the exact maximum: it is raised (and
+    // the sums rescaled) only when some row of the wave has grown by more than 2^8 over its shift; until
+    // then the probabilities are at most 256 and the final division by the row sum takes the factor out.
+    // (A row whose keys so far are all masked with -inf keeps m = -inf and shifts by 0: no inf - inf forms.)
+    float m_use = m_run == -INFINITY ? 0.0f : m_run;
+    if (__any(mx > m_run + 8.0f)) {
+      const float m_max = fmaxf(m_run, mx);
+      m_use = m_max == -INFINITY ? 0.0f : m_max;
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
+      m_run = m_max;
+      l_run *= corr;
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    }
+    const float m_new = m_use;
     float psum = 0.0f;
     u32x4_t pb[2][2];
 #pragma unroll
@@ -214,11 +226,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
           }
           pb[t2][t][e] = pack2<T>(pv[0], pv[1]);
         }
-    l_run = l_run * corr + psum;
-#pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    l_run += psum;
     // O^T += V^T P^T, 16 keys per step
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2)
