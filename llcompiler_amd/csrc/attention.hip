@@ -259,6 +259,178 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   }
 }
 
+// ---- fp32 operands: v_mfma_f32_32x32x2_f32 takes one k per lane and instruction ----
+// Same plan as above with these differences.  K block [64 keys][256 B] and V block [64 keys][256 B] come straight
+// into LDS (global_load_lds: no staging registers; lane L of a wave load lands at byte 16 L of its 1 KB, so it
+// fetches the chunk that belongs there: K chunk c of row r sits at c ^ (r & 15), V elements of rows with bit 2
+// set sit 32 floats further, which spreads the fragment reads over the banks).  S^T: one 16-byte read of a K row
+// feeds four MFMAs (lane half h owns d = 8c + 4h + s, the same permutation of k on both operands).  The
+// probabilities stay fp32 in the accumulator registers and ARE the column operand of O^T += V^T P^T: in register
+// 4i + j lane half 0 holds key 8i + j and half 1 key 8i + 4 + j, which is one k pair.  V is read 4 bytes per lane
+// and MFMA.  64 or 128 queries per workgroup (2 or 4 waves), whichever gives the CUs more to share.
+constexpr int kF32Tile = kBlockKV * 256;
+
+template <int NW, bool MASK>
+__global__ __launch_bounds__(64 * NW) void attention_f32_kernel(const AttnParams p) {
+  extern __shared__ __align__(16) char smem[];
+  char* kt = smem;                                        // [2][kF32Tile]
+  char* vt = smem + 2 * kF32Tile;                         // [2][kF32Tile]
+  float* addrow = (float*)(smem + 4 * kF32Tile);          // [2][64] raw mask values
+  constexpr int LPW = 16 / NW;  // wave loads of K (and of V) per wave and block
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+  const int li = lane % 32, lh = lane / 32;
+  const int bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
+  const int q0 = blockIdx.x * (32 * NW) + wave * 32;
+  const float* Q = (const float*)p.Q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const float* K = (const float*)p.K + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+  const float* V = (const float*)p.V + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+  const float* M = MASK ? (const float*)p.mask + (int64_t)b * p.m_sb : nullptr;
+
+  f32x4_t qf[8];
+  {
+    const int qrow = q0 + li < p.Sq ? q0 + li : p.Sq - 1;
+    const float* qp = Q + (int64_t)qrow * p.q_ss + 4 * lh;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) qf[c] = *(const f32x4_t*)(qp + 8 * c);
+  }
+
+  auto issue = [&](int blk, int s) {
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+      const int x = wave * LPW + j;            // rows 4x .. 4x + 3 of the block
+      const int r = 4 * x + lane / 16, pos = lane % 16;
+      int row = blk * kBlockKV + r;
+      row = row < p.Skv ? row : p.Skv - 1;
+      const float* ks = K + (int64_t)row * p.k_ss + ((pos ^ (r & 15)) << 2);
+      const float* vs = V + (int64_t)row * p.v_ss + ((pos ^ (((r >> 2) & 1) << 3)) << 2);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ks,
+                                       (__attribute__((address_space(3))) void*)(kt + s * kF32Tile + x * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vs,
+                                       (__attribute__((address_space(3))) void*)(vt + s * kF32Tile + x * 1024), 16, 0, 0);
+    }
+    if constexpr (MASK) {
+      // every wave brings the same 64 values (identical bytes to the same place): no wave is special
+      int key = blk * kBlockKV + lane;
+      key = key < p.Skv ? key : p.Skv - 1;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(M + key),
+                                       (__attribute__((address_space(3))) void*)(addrow + s * kBlockKV), 4, 0, 0);
+    }
+  };
+
+  int ka[2];  // K rows 32 T + li: row offset; the chunk swizzle is applied per read
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2) ka[t2] = (32 * t2 + li) * 256;
+  const int kswz = li & 15;
+  // V element (key, d) sits at key * 256 + 4 * (d ^ 32 * ((key >> 2) & 1)); this lane's keys have (key >> 2) & 1 = lh
+  const int va0 = 4 * lh * 256 + 4 * li + 128 * lh, va1 = 4 * lh * 256 + 4 * li + 128 * (1 - lh);
+
+  f32x16_t oacc[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int nblk = (p.Skv + kBlockKV - 1) / kBlockKV;
+  issue(0, 0);
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int s = blk & 1;
+    // this wave's share of block blk has landed; after the barrier everybody's has, and nobody reads the other stage
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (blk + 1 < nblk) issue(blk + 1, s ^ 1);
+    const char* kb = kt + s * kF32Tile;
+    const char* vb = vt + s * kF32Tile;
+    f32x16_t sacc[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[t2][r] = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const f32x4_t a = *(const f32x4_t*)(kb + ka[t2] + (((2 * c + lh) ^ kswz) << 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sacc[t2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[c][e], sacc[t2], 0, 0, 0);
+      }
+    }
+    // scores in log2 units; register 4 i + j of tile T is key 32 T + 8 i + 4 lh + j
+    const bool tail = blk == nblk - 1 && (p.Skv % kBlockKV) != 0;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f32x4_t av = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (MASK) av = *(const f32x4_t*)&addrow[s * kBlockKV + 32 * t2 + 8 * i + 4 * lh];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float x = MASK ? fmaf(sacc[t2][4 * i + j], p.scale_log2e, av[j] * kLog2e) : sacc[t2][4 * i + j] * p.scale_log2e;
+          if (tail && blk * kBlockKV + 32 * t2 + 8 * i + 4 * lh + j >= p.Skv) x = -INFINITY;
+          sacc[t2][4 * i + j] = x;
+          mx = fmaxf(mx, x);
+        }
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    float m_use = m_run == -INFINITY ? 0.0f : m_run;
+    if (__any(mx > m_run + 8.0f)) {  // see attention_kernel: the shift follows the maximum lazily
+      const float m_max = fmaxf(m_run, mx);
+      m_use = m_max == -INFINITY ? 0.0f : m_max;
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
+      m_run = m_max;
+      l_run *= corr;
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    }
+    float psum = 0.0f;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pv = __builtin_amdgcn_exp2f(sacc[t2][r] - m_use);
+        sacc[t2][r] = pv;
+        psum += pv;
+      }
+    l_run += psum;
+    // O^T += V^T P^T, one k pair (keys 8 i + j and 8 i + 4 + j of tile T) per MFMA
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int koff = (32 * t2 + 8 * (r / 4) + (r % 4)) * 256;
+        const float a0 = *(const float*)(vb + va0 + koff), a1 = *(const float*)(vb + va1 + koff);
+        oacc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, sacc[t2][r], oacc[0], 0, 0, 0);
+        oacc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, sacc[t2][r], oacc[1], 0, 0, 0);
+      }
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  const float inv = 1.0f / l_tot;
+  if (q0 + li < p.Sq) {
+    float* op = (float*)p.O + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)(q0 + li) * p.o_ss;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *(f32x4_t*)(op + 32 * dt + 8 * i + 4 * lh) =
+            f32x4_t{oacc[dt][4 * i] * inv, oacc[dt][4 * i + 1] * inv, oacc[dt][4 * i + 2] * inv, oacc[dt][4 * i + 3] * inv};
+  }
+}
+
+template <int NW, bool MASK>
+int launch_f32(const AttnParams& p, hipStream_t s) {
+  constexpr int lds = 4 * kF32Tile + 2 * kBlockKV * 4;
+  auto kern = attention_f32_kernel<NW, MASK>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)((p.Sq + 32 * NW - 1) / (32 * NW)), (unsigned)(p.B * p.H));
+  hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, p);
+  return check_launch("attention_f32_kernel");
+}
+
 int view4(const llc_tensor* t, const char* what, View* v) {
   LLC_TRY(make_view(t, what, v));
   if (v->rank != 4) return set_error(LLC_ERR_SHAPE, "%s: rank 4 expected, [B, H, S, D]", what);
@@ -281,8 +453,8 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
   LLC_TRY(view4(v, "attention v", &c));
   LLC_TRY(view4(out, "attention out", &o));
   if (a.dtype != b.dtype || a.dtype != c.dtype || a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "attention: operand types differ");
-  if (a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16)
-    return set_error(LLC_ERR_DTYPE, "attention: bf16 or f16 operands (type %d given)", a.dtype);
+  if (a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16 && a.dtype != LLC_FLOAT32)
+    return set_error(LLC_ERR_DTYPE, "attention: f32, bf16 or f16 operands (type %d given)", a.dtype);
   for (int d = 0; d < 2; ++d)
     if (a.size[d] != b.size[d] || a.size[d] != c.size[d] || a.size[d] != o.size[d])
       return set_error(LLC_ERR_SHAPE, "attention: batch dims differ");
@@ -311,9 +483,16 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
   p.v_sb = c.stride[0], p.v_sh = c.stride[1], p.v_ss = c.stride[2];
   p.o_sb = o.stride[0], p.o_sh = o.stride[1], p.o_ss = o.stride[2];
   p.scale_log2e = scale * kLog2e;
+  hipStream_t s = as_stream(stream);
+  if (a.dtype == LLC_FLOAT32) {
+    // 128 queries per workgroup (K and V blocks are then shared by four waves) unless that leaves half the CUs
+    // without work; LDS holds two workgroups per CU either way
+    const bool four = (int64_t)((p.Sq + 127) / 128) * p.B * p.H >= 128;
+    if (four) return p.mask ? launch_f32<4, true>(p, s) : launch_f32<4, false>(p, s);
+    return p.mask ? launch_f32<2, true>(p, s) : launch_f32<2, false>(p, s);
+  }
   const dim3 grid((unsigned)((p.Sq + kBlockQ - 1) / kBlockQ), (unsigned)(p.B * p.H));
   const bool add = p.mask || p.Skv % kBlockKV != 0;
-  hipStream_t s = as_stream(stream);
   if (a.dtype == LLC_BFLOAT16) {
     if (add) hipLaunchKernelGGL((attention_kernel<__bf16, true>), grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL((attention_kernel<__bf16, false>), grid, dim3(256), 0, s, p);

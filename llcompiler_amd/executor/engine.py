@@ -40,7 +40,7 @@ MIN_CALLS_FOR_GRAPH = 2
 # reference's packed parameter block and make one call into the library, which replays the launches.  With
 # False every run launches kernel by kernel from Python (same kernels, same arguments).
 USE_PLAN = True
-# batch_matmul -> softmax -> batch_matmul groups of 16-bit attention layers with head dim 64 become one fused kernel
+# batch_matmul -> softmax -> batch_matmul groups of attention layers with head dim 64 become one fused kernel
 FUSE_ATTENTION = True
 
 
@@ -249,7 +249,7 @@ class Instance:
             e = st.attrs["epilogue"]
             if e["act"] or e["residual"] is not None or e["alpha"] <= 0 or (e["bias"] is not None and not e.get("bias_rows")):
                 return None
-            if st.output.dtype not in (torch.bfloat16, torch.float16):
+            if st.output.dtype not in (torch.bfloat16, torch.float16, torch.float32):
                 return None
             between = []
 
@@ -278,7 +278,7 @@ class Instance:
 
         def fused_attention(st):
             """Emits one attention call for the group that starts at `st` when the operands allow it (head dim 64,
-            16-bit, rows addressable as [B, H, S, 64] views); returns False to leave the group to its own kernels."""
+            rows addressable as [B, H, S, 64] views); returns False to leave the group to its own kernels."""
             grp = attention_group(st)
             if grp is None:
                 return False

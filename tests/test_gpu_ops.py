@@ -366,21 +366,24 @@ def test_attention(ops, oracle, B, H, Sq, Skv, masked):
             mask[b, int(r.integers(Skv // 2, Skv)) + 1:] = -1e4
         mask = bf16_round(mask)
     scale = 0.125
-    for dt, rnd in ((torch.bfloat16, bf16_round), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+    for dt, rnd, close in ((torch.bfloat16, bf16_round, assert_close_bf16),
+                           (torch.float16, lambda x: x.astype(np.float16).astype(np.float32), assert_close_bf16),
+                           (torch.float32, lambda x: x, assert_close_f32)):
         want = _attention_oracle(oracle, q, k, v, mask, scale, rnd)
         dm = dev(mask, dt) if masked else None
         got = ops.attention(dev(q, dt), dev(k, dt), dev(v, dt), dm, scale)
-        assert_close_bf16(host(got), want, "attention %s" % dt)
+        close(host(got), want, "attention %s" % dt)
     # head-split views of [B, S, H*64] activations in, the merged layout out (no copies on either side)
     qs = dev(np.ascontiguousarray(q.transpose(0, 2, 1, 3)).reshape(B, Sq, H * 64), torch.bfloat16)
     ks = dev(np.ascontiguousarray(k.transpose(0, 2, 1, 3)).reshape(B, Skv, H * 64), torch.bfloat16)
     vs = dev(np.ascontiguousarray(v.transpose(0, 2, 1, 3)).reshape(B, Skv, H * 64), torch.bfloat16)
-    merged = torch.zeros((B, Sq, H, 64), dtype=torch.bfloat16, device="cuda")
-    ops.attention(qs.view(B, Sq, H, 64).permute(0, 2, 1, 3), ks.view(B, Skv, H, 64).permute(0, 2, 1, 3),
-                  vs.view(B, Skv, H, 64).permute(0, 2, 1, 3), dev(mask, torch.bfloat16) if masked else None, scale,
-                  out=merged.permute(0, 2, 1, 3))
-    want = _attention_oracle(oracle, q, k, v, mask, scale, bf16_round)
-    assert_close_bf16(host(merged).transpose(0, 2, 1, 3), want, "attention on head-split views")
+    for dt, rnd, close in ((torch.bfloat16, bf16_round, assert_close_bf16), (torch.float32, lambda x: x, assert_close_f32)):
+        merged = torch.zeros((B, Sq, H, 64), dtype=dt, device="cuda")
+        ops.attention(qs.to(dt).view(B, Sq, H, 64).permute(0, 2, 1, 3), ks.to(dt).view(B, Skv, H, 64).permute(0, 2, 1, 3),
+                      vs.to(dt).view(B, Skv, H, 64).permute(0, 2, 1, 3), dev(mask, dt) if masked else None, scale,
+                      out=merged.permute(0, 2, 1, 3))
+        want = _attention_oracle(oracle, q, k, v, mask, scale, rnd)
+        close(host(merged).transpose(0, 2, 1, 3), want, "attention on head-split views %s" % dt)
 
 
 def test_attention_fully_masked_leading_block_and_errors(ops, oracle):
@@ -396,8 +399,10 @@ def test_attention_fully_masked_leading_block_and_errors(ops, oracle):
     assert_close_bf16(got, want, "attention with -inf on the first 70 keys")
     from llcompiler_amd._capi import LlcHipError
     x = dev(q, torch.bfloat16)
-    with pytest.raises(LlcHipError):  # fp32 operands are not implemented: an error, not another path
-        ops.attention(dev(q), dev(k), dev(v))
+    got32 = host(ops.attention(dev(q), dev(k), dev(v), dev(mask), 0.125))
+    assert_close_f32(got32, _attention_oracle(oracle, q, k[:, :, 70:], v[:, :, 70:], None, 0.125, lambda x: x), "fp32, -inf on 70 keys")
+    with pytest.raises(LlcHipError):  # fp64 operands are not implemented: an error, not another path
+        ops.attention(dev(q).double(), dev(k).double(), dev(v).double())
     with pytest.raises(LlcHipError):
         ops.attention(x, dev(k, torch.bfloat16)[..., :32], dev(v, torch.bfloat16))  # head dim 32
     with pytest.raises(LlcHipError):
