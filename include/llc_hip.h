@@ -278,6 +278,18 @@ int llc_plan_destroy(llc_plan_t* plan);
  * (include/llcompiler/TransformLibrary/memref_include.mlir:6-8). */
 int llc_plan_alloc(llc_plan_t* plan, size_t bytes, void** device_ptr);
 int llc_plan_upload(llc_plan_t* plan, const void* host, size_t bytes, void** device_ptr);
+/* llh.weight{weight_file} (LLHOps.td:219-227): the reference's importer saves parameters with np.save
+ * (llcompiler/importer/fx_translate.py:427-430) and its LoadWeight pass (LoadWeight.cpp:58-171) parses the
+ * .npy file ('<f4', '<i8', C order assumed) and bakes the data into the compiled object.  llc_npy_info reads
+ * the header (format versions 1 to 3): element type, rank, extents and where the data starts;
+ * llc_plan_load_npy uploads the data into memory owned by the plan and fills `out` (contiguous, with
+ * size_out / stride_out as its arrays, LLC_MAX_RANK entries each).  Read: f4, i8, f8, f2, i4, i2, i1, b1, and
+ * u2 as bf16 bit patterns when expect_dtype says LLC_BFLOAT16.  expect_dtype < 0 takes what the file says;
+ * otherwise a file of another type is refused (LLC_ERR_DTYPE).  Fortran-ordered files of rank > 1 are refused
+ * (the reference reads them as if they were C ordered). */
+int llc_npy_info(const char* path, int expect_dtype, size_t* dtype, size_t* rank, size_t* size, size_t* data_offset);
+int llc_plan_load_npy(llc_plan_t* plan, const char* path, int expect_dtype, llc_tensor* out, size_t* size_out,
+                      size_t* stride_out);
 /* Declares the next tensor of the params block: type, rank, extents and strides it will have on every run,
  * and (data + offset) = where it lives while the plan is recorded. */
 int llc_plan_declare_io(llc_plan_t* plan, int is_output, const llc_tensor* like);

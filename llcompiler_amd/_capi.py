@@ -79,6 +79,7 @@ EXPORTS = [
     "llc_plan_create", "llc_plan_destroy", "llc_plan_alloc", "llc_plan_upload", "llc_plan_declare_io",
     "llc_plan_expect_symbols", "llc_plan_begin", "llc_plan_end", "llc_plan_num_steps", "llc_plan_num_params",
     "llc_hip_run", "llc_hip_bind_entry", "llc_hip_entry", "llc_hip_entry_status",
+    "llc_npy_info", "llc_plan_load_npy",
 ]
 
 
@@ -141,6 +142,9 @@ def lib():
         L.llc_hip_bind_entry.argtypes = [vp, vp]
         L.llc_hip_entry.argtypes = [P(vp)]
         L.llc_hip_entry.restype = None
+        szp = P(ctypes.c_size_t)
+        L.llc_npy_info.argtypes = [ctypes.c_char_p, ctypes.c_int, szp, szp, szp, szp]
+        L.llc_plan_load_npy.argtypes = [vp, ctypes.c_char_p, ctypes.c_int, T, szp, szp]
         _lib = L
     return _lib
 

@@ -6,6 +6,8 @@ same decompositions, importer and LLH pipeline as the torch.compile backend and 
 whose single plan serves every value of the symbolic dims, batch 1 included.  Every node must be
 translatable: there is no eager fallback on this entry.
 """
+import os
+
 import torch
 from torch._decomp import get_decompositions
 
@@ -29,7 +31,11 @@ class CompiledModule:
         return out
 
 
-def compile_module(model, example_args, dynamic_shapes=None, verbose=False):
+def compile_module(model, example_args, dynamic_shapes=None, verbose=False, weights=None, weight_dir=None):
+    """weights="npy": parameters and buffers are written to .npy files (in weight_dir, or a fresh temporary
+    directory) and enter the graph as llh.weight ops, the reference importer's convention
+    (llcompiler/importer/fx_translate.py:415-435); the engine uploads each file once.  By default they stay
+    torch tensors and are passed to the engine with every call."""
     model = model.eval()
     with torch.no_grad():
         ep = torch.export.export(model, tuple(example_args), dynamic_shapes=dynamic_shapes)
@@ -54,7 +60,20 @@ def compile_module(model, example_args, dynamic_shapes=None, verbose=False):
             lifted.append(t.detach() if isinstance(t, torch.Tensor) else t)
     if any(s.kind.name != "USER_INPUT" for s in sig.input_specs[len(lifted):]):
         raise NotImplementedError("lifted inputs must precede user inputs")
-    graph = torch_translate_to_llh_graph(gm)
+    weight_files = None
+    if weights == "npy":
+        from ..executor.weights import new_weight_dir, save_weight
+        wdir = new_weight_dir(weight_dir)
+        names = [n.name for n in gm.graph.nodes if n.op == "placeholder"][:len(lifted)]
+        weight_files = {}
+        for name, t in zip(names, lifted):
+            if not isinstance(t, torch.Tensor):
+                raise TypeError("weights=\"npy\": %s is not a tensor" % name)
+            weight_files[name] = save_weight(t, os.path.join(wdir, name + ".npy"))
+        lifted = []
+    elif weights is not None:
+        raise ValueError("weights must be None or \"npy\"")
+    graph = torch_translate_to_llh_graph(gm, weight_files)
     run_llh_pipeline(graph)
     if verbose:
         print(graph.dump())

@@ -25,6 +25,7 @@ from ..llh.expr import Expr, evaluate
 from ..llh.graph import Value
 from .plan_runner import ParamBlock, Plan
 from .planner import make_plan
+from .weights import WeightStore
 
 # same codes as the reference's map (engine.py:11), extended with bf16 / f16 / i32
 TORCH_DTYPE_TO_TYPE = C.TORCH_DTYPE_TO_TYPE
@@ -94,8 +95,9 @@ class _LazyReshape:
 class Instance:
     """A plan specialised to concrete extents: a flat list of prepared kernel calls."""
 
-    def __init__(self, graph, steps, env, inputs, device):
+    def __init__(self, graph, steps, env, inputs, device, weights=None):
         self.graph, self.env, self.device = graph, env, device
+        self.weights = weights     # WeightStore of the engine: tensors of llh.weight ops, loaded once
         self.calls = []
         self.patches = []          # (TensorRef, "in"|"out", index, byte offset from that tensor's data_ptr)
         self.keep = []
@@ -370,6 +372,8 @@ class Instance:
                 c = torch.full((1,), st.attrs["value"], dtype=st.output.dtype, device=dev)
                 self.keep.append(c)
                 val[id(st.output)] = c
+            elif k == "weight":
+                val[id(st.output)] = self.weights.get(st.attrs["weight_file"], _concrete(st.output.shape, self.env), st.output.dtype)
             elif k == "ew":
                 out = new_tensor(st.output)
                 prog = ops.make_program(st.attrs["insts"], st.attrs["result"], st.attrs["integer"])
@@ -647,6 +651,7 @@ class ExecutionEngine:
         self.steps = make_plan(graph)
         self.instances = {}
         self._fast = {}
+        self._weights = None
 
     def run(self, *args):
         raise NotImplementedError
@@ -717,7 +722,9 @@ class Torch_ExecutionEngine(ExecutionEngine):
         inst = self.instances.get(key)
         if inst is None:
             C.init(device.index or 0)
-            inst = Instance(g, self.steps, env, inputs, device)
+            if self._weights is None or self._weights.device != device:
+                self._weights = WeightStore(device)
+            inst = Instance(g, self.steps, env, inputs, device, self._weights)
             self.instances[key] = inst
         if not key[3]:
             # (an instance built from inputs that share memory is only valid while they do: such calls keep

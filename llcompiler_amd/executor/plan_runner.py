@@ -5,6 +5,7 @@ the symbol values (or NULL), then five slots per tensor, inputs first: base, dat
 """
 import contextlib
 import ctypes
+import os
 import weakref
 
 from .. import _capi as C
@@ -69,6 +70,14 @@ class Plan:
         p = ctypes.c_void_p()
         C.check(self._lib.llc_plan_upload(self.handle, host_ptr, nbytes, ctypes.byref(p)))
         return p.value
+
+    def load_npy(self, path, expect_dtype=-1):
+        """Uploads the data of a .npy file into memory owned by this plan; returns (device pointer, type code, shape)."""
+        desc = C.LlcTensor()
+        size = (ctypes.c_size_t * C.LLC_MAX_RANK)()
+        stride = (ctypes.c_size_t * C.LLC_MAX_RANK)()
+        C.check(self._lib.llc_plan_load_npy(self.handle, os.fsencode(path), expect_dtype, ctypes.byref(desc), size, stride))
+        return desc.data or 0, int(desc.type), tuple(size[i] for i in range(desc.rank))
 
     @contextlib.contextmanager
     def recording(self):

@@ -10,7 +10,7 @@ A plan is a list of Steps over graph Values:
   view      reshape / transpose / broadcast_to / stride_slice / extract: descriptor changes only
   ew        one fused elementwise chain (a register program for llc_hip_elementwise)
   matmul / batch_matmul / conv      with epilogue {alpha, bias, residual, act}
-  softmax, layer_norm, reduce, max_pool, avg_pool, gather, constant
+  softmax, layer_norm, reduce, max_pool, avg_pool, gather, constant, weight (a .npy file, llh.weight)
 """
 import torch
 
@@ -284,6 +284,8 @@ class Planner:
                 self.steps.append(Step("view", op.operands[:1], r, dict(op.attrs, op=op.name)))
             elif op.name == "constant":
                 self.steps.append(Step("constant", [], r, {"value": op.attrs["value"]}))
+            elif op.name == "weight":
+                self.steps.append(Step("weight", [], r, {"weight_file": op.attrs["weight_file"]}))
             elif op.name == "softmax":
                 self.steps.append(Step("softmax", op.operands, r))
             elif op.name == "layer_norm":

@@ -498,14 +498,23 @@ def is_supported(node):
         return False
 
 
-def torch_translate_to_llh_graph(gm):
-    """Counterpart of torch_translate_to_mlir_module (llcompiler/importer/fx_translate.py:517-521)."""
+def torch_translate_to_llh_graph(gm, weight_files=None):
+    """Counterpart of torch_translate_to_mlir_module (llcompiler/importer/fx_translate.py:517-521).
+
+    weight_files: {placeholder name: .npy path}.  Those placeholders become llh.weight ops that name their file
+    (fx_translate.py:415-435 does this for the parameters of the traced module) instead of run-time inputs."""
     g = Graph()
     ctx = Ctx(g)
+    weight_files = weight_files or {}
     for node in gm.graph.nodes:
         if node.op == "placeholder":
             val = node.meta.get("val", node.meta.get("example_value"))
-            if isinstance(val, torch.Tensor):
+            if node.name in weight_files:
+                if not isinstance(val, torch.Tensor) or any(not isinstance(d, int) for d in meta_shape(val)):
+                    raise TypeError("weight %s must be a tensor of static shape" % node.name)
+                ctx.env[node] = g.add_op("weight", [], {"weight_file": weight_files[node.name]}, shapes=[meta_shape(val)],
+                                         dtypes=[val.dtype])
+            elif isinstance(val, torch.Tensor):
                 ctx.env[node] = g.add_input(meta_shape(val), val.dtype, name=node.name)
             elif isinstance(val, (torch.SymInt, int)):
                 # dynamo passes SymInts as leading int arguments (fx_translate.py:373-406)

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "llc_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(llc_(?:hip|plan)_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(llc_(?:hip|plan|npy)_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_agree():
@@ -102,3 +102,48 @@ def test_cpu_tensor_is_refused_not_computed():
     from llcompiler_amd import ops
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.softmax(torch.zeros(2, 3))
+
+
+def _npy_info(path, expect=-1):
+    import ctypes as ct
+    L = C.lib()
+    dtype, rank, off = ct.c_size_t(), ct.c_size_t(), ct.c_size_t()
+    size = (ct.c_size_t * C.LLC_MAX_RANK)()
+    st = L.llc_npy_info(os.fsencode(path), expect, ct.byref(dtype), ct.byref(rank), size, ct.byref(off))
+    return st, dtype.value, tuple(size[i] for i in range(rank.value)), off.value
+
+
+def test_npy_header_parser_reads_what_np_save_writes(tmp_path):
+    """The weight wire format: np.save output (llcompiler/importer/fx_translate.py:427-430), parsed like
+    src/Dialect/LLH/Transforms/LoadWeight.cpp:58-132: type, shape, and the data right behind the header."""
+    import numpy as np
+    cases = [(np.arange(24, dtype=np.float32).reshape(2, 3, 4), C.FLOAT32), (np.arange(5, dtype=np.int64), C.INT64),
+             (np.float32(3.5).reshape(()), C.FLOAT32), (np.ones((4, 0, 2), np.float16), C.FLOAT16),
+             (np.array([[True, False]]), C.INT1), (np.arange(6, dtype=np.int32).reshape(3, 2), C.INT32)]
+    for k, (arr, code) in enumerate(cases):
+        path = str(tmp_path / ("w%d.npy" % k))
+        np.save(path, arr)
+        st, dtype, shape, off = _npy_info(path)
+        assert (st, dtype, shape) == (0, code, arr.shape), (path, st, C.lib().llc_hip_last_error())
+        raw = open(path, "rb").read()
+        assert raw[off:] == arr.tobytes()          # the data starts where the parser says, in C order
+        assert _npy_info(path, code)[0] == 0 and _npy_info(path, C.INT16)[0] == C.ERR_DTYPE
+    # bf16 travels as its bit patterns: '<u2' is accepted only when the caller expects bf16
+    bits = str(tmp_path / "bits.npy")
+    np.save(bits, np.arange(8, dtype=np.uint16))
+    assert _npy_info(bits)[0] == C.ERR_DTYPE and _npy_info(bits, C.BFLOAT16)[:3] == (0, C.BFLOAT16, (8,))
+    # format version 2 (four-byte header length)
+    v2 = str(tmp_path / "v2.npy")
+    with open(v2, "wb") as f:
+        np.lib.format.write_array(f, np.arange(6, dtype=np.float32).reshape(2, 3), version=(2, 0))
+    assert _npy_info(v2)[:3] == (0, C.FLOAT32, (2, 3))
+    # Fortran order (the reference reads such a file as if it were C ordered), big-endian data, not a .npy file
+    fo = str(tmp_path / "f.npy")
+    np.save(fo, np.asfortranarray(np.arange(6, dtype=np.float32).reshape(2, 3)))
+    assert _npy_info(fo)[0] == C.ERR_LAYOUT
+    be = str(tmp_path / "be.npy")
+    np.save(be, np.arange(4, dtype=">f4"))
+    assert _npy_info(be)[0] == C.ERR_DTYPE
+    junk = str(tmp_path / "junk.npy")
+    open(junk, "wb").write(b"not a numpy file at all")
+    assert _npy_info(junk)[0] == C.ERR_BAD_ARG and _npy_info(str(tmp_path / "missing.npy"))[0] == C.ERR_BAD_ARG

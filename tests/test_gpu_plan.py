@@ -258,3 +258,55 @@ def test_engine_inputs_that_stop_sharing_memory_get_their_own_instance(oracle):
         np.testing.assert_array_equal(r.cpu().numpy(), np.full(16, 1.0, np.float32))
     np.testing.assert_array_equal(r4.cpu().numpy(), np.full(16, 9.0, np.float32))
     np.testing.assert_array_equal(r6.cpu().numpy(), np.full(16, 0.0, np.float32))
+
+
+def test_npy_weights_are_uploaded_into_the_plan(oracle, tmp_path):
+    """llh.weight: a .npy file (np.save, as the reference's importer writes it) read by the library into plan-owned
+    memory, then used by a recorded plan."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    rng = np.random.default_rng(5)
+    M, K, N = 24, 40, 56
+    w = rng.standard_normal((K, N), dtype=np.float32)
+    path = str(tmp_path / "w.npy")
+    np.save(path, w)
+    plan = Plan()
+    ptr, code, shape = plan.load_npy(path, C.FLOAT32)
+    assert (code, shape) == (C.FLOAT32, (K, N)) and ptr
+    with pytest.raises(C.LlcHipError):
+        plan.load_npy(path, C.INT64)
+    wref = C.TensorRef(ptr, C.FLOAT32, (K, N), (N, 1))
+    x = torch.from_numpy(rng.standard_normal((M, K), dtype=np.float32)).cuda()
+    out = torch.empty((M, N), device="cuda")
+    plan.declare_io(x, False)
+    plan.declare_io(out, True)
+    rx, ro = C.tensor_ref(x), C.tensor_ref(out)
+    with plan.recording():
+        C.check(C.lib().llc_hip_matmul(rx.ptr, wref.ptr, None, ro.ptr, _stream()))
+    xs = rng.standard_normal((M, K), dtype=np.float32)
+    out2 = torch.zeros((M, N), device="cuda")
+    plan.run(ParamBlock([torch.from_numpy(xs).cuda(), out2]), _stream())
+    torch.cuda.synchronize()
+    assert_close(out2.cpu().numpy(), oracle.matmul(xs, w), F32_RTOL, F32_ATOL, "matmul with a .npy weight")
+
+
+def test_models_with_npy_weights_match_models_with_tensor_weights(tmp_path):
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import MLP, EncoderBlock, make_encoder_inputs, make_mlp_inputs
+    with torch.no_grad():
+        m = MLP().eval().cuda()
+        (x,) = make_mlp_inputs()
+        a = compile_module(m, (x.cuda(),))
+        b = compile_module(m, (x.cuda(),), weights="npy", weight_dir=str(tmp_path / "mlp"))
+        assert b.lifted == [] and len(b.engine.graph.inputs) == 1
+        for seed in (1, 2, 3):
+            (xs,) = make_mlp_inputs(seed=seed)
+            assert torch.equal(a(xs.cuda()), b(xs.cuda()))
+        enc = EncoderBlock(hidden=128, heads=2, ffn=256).eval().to(torch.bfloat16).cuda()   # bf16 travels as '<u2'
+        (xe,) = make_encoder_inputs(2, 64, 128, dtype=torch.bfloat16)
+        ea = compile_module(enc, (xe.cuda(),))
+        eb = compile_module(enc, (xe.cuda(),), weights="npy", weight_dir=str(tmp_path / "enc"))
+        for seed in (1, 2):
+            (xs,) = make_encoder_inputs(2, 64, 128, seed=seed, dtype=torch.bfloat16)
+            assert torch.equal(ea(xs.cuda()), eb(xs.cuda()))

@@ -224,3 +224,24 @@ def test_engine_argument_convention_and_errors():
         eng.run(torch.zeros(2, 8))
     with pytest.raises(ValueError, match="expected"):
         eng.run(torch.zeros(2, 9).to("meta") if False else torch.zeros(2, 9))
+
+
+def test_parameters_become_weight_ops_naming_npy_files(tmp_path):
+    """weights="npy": the reference importer's convention (llcompiler/importer/fx_translate.py:415-435): every
+    parameter is written with np.save and enters the graph as llh.weight{weight_file}; only the user's tensors
+    remain run-time inputs."""
+    import numpy as np
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    m = MLP().eval()
+    cm = compile_module(m, make_mlp_inputs(), weights="npy", weight_dir=str(tmp_path))
+    g = cm.engine.graph
+    ws = [op for op in g.ops if op.name == "weight"]
+    assert len(ws) == 4 and len(g.inputs) == 1 and cm.lifted == []
+    want = {tuple(p.shape): p.detach().numpy() for p in m.parameters()}
+    for op in ws:
+        arr = np.load(op.attrs["weight_file"])
+        assert arr.dtype == np.float32 and tuple(op.results[0].shape) == arr.shape
+        np.testing.assert_array_equal(arr, want[arr.shape])
+    kinds = [s.kind for s in cm.engine.steps if s.kind != "view"]
+    assert kinds.count("weight") == 4 and kinds.count("matmul") == 2
