@@ -369,7 +369,11 @@ class Instance:
                     # private to this instance (later views of it are not tracked for reuse)
                     self.keep.append(temps.pop())
             elif k == "constant":
-                c = torch.full((1,), st.attrs["value"], dtype=st.output.dtype, device=dev)
+                shape, v = _concrete(st.output.shape, self.env), st.attrs["value"]
+                if isinstance(v, (list, tuple)):  # a dense constant spelt element by element (LLH text)
+                    c = torch.tensor(v, dtype=st.output.dtype).reshape(shape).to(dev)
+                else:
+                    c = torch.full(shape, v, dtype=st.output.dtype, device=dev)
                 self.keep.append(c)
                 val[id(st.output)] = c
             elif k == "weight":

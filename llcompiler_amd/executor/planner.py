@@ -168,6 +168,15 @@ class Planner:
 
     def build_program(self, ops):
         """Register program for a topologically ordered list of elementwise ops whose last op is the output."""
+        prog, inputs = self._build_program(ops, None)
+        if not inputs:
+            # every operand is a one-element constant (a constant expression in LLH text): the kernel wants at
+            # least one tensor to read, so the first constant stays a tensor operand
+            first = next(o for op in ops for o in op.operands if o.producer is None or o.producer not in ops)
+            prog, inputs = self._build_program(ops, id(first))
+        return prog, inputs
+
+    def _build_program(self, ops, keep_as_input):
         produced = {id(op.results[0]): i for i, op in enumerate(ops)}
         last_use = {}
         for i, op in enumerate(ops):
@@ -182,7 +191,7 @@ class Planner:
         def operand(o):
             if id(o) in produced:
                 return "r%d" % reg_of[id(o)]
-            c = _scalar_const(o)
+            c = _scalar_const(o) if id(o) != keep_as_input else None
             if c is not None:
                 return float(c) if not isinstance(c, bool) else float(int(c))
             if id(o) not in in_index:

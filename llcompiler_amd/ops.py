@@ -129,6 +129,8 @@ def make_program(insts, result=0, integer=False):
 
 
 def elementwise(prog, inputs, out_shape, out_dtype, out=None, defer=False):
+    if not inputs:
+        raise ValueError("an elementwise program reads at least one tensor")
     dev = _dev(inputs[0])
     if out is None:
         out = torch.empty(tuple(out_shape), dtype=out_dtype, device=dev)

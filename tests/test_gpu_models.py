@@ -236,3 +236,45 @@ def test_graph_replay_matches_per_kernel_launches():
             inst = next(iter(replayed.engine.instances.values()))
             assert inst._graph is not None and not inst._graph_failed
             eng.USE_GRAPHS = was
+
+
+def test_llh_text_programs_run_on_the_gpu(oracle):
+    """Programs in the reference's text format through reader -> pipeline -> plan -> kernels.  The first two carry
+    the reference's own numeric known answers: abs(dense<-1> : 2xf32) prints [1, 1] (test/RunnerTest/abs.mlir:5-10)
+    and 2 * 2 computed in i64 and converted prints [4] as f32 (test/RunnerTest/mlir-runner.mlir:11-25)."""
+    from llcompiler_amd.executor.engine import Torch_ExecutionEngine
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    from llcompiler_amd.llh.text import parse_llh
+    from tests.test_llh_text_cpu import ABS_RUNNER, CONV_AND_SHAPES
+
+    def engine(text, func=None):
+        g = parse_llh(text, func)
+        run_llh_pipeline(g)
+        return Torch_ExecutionEngine(g)
+
+    torch.cuda.set_device(0)
+    out = engine(ABS_RUNNER).run()
+    np.testing.assert_array_equal(out.cpu().numpy(), np.array([1.0, 1.0], np.float32))
+    mul = '''func.func @main() -> () attributes {entrance} {
+        %two = "llh.constant"() <{value = dense<2> : tensor<1xi64>}> : () -> tensor<1xi64>
+        %sq = "llh.mul"(%two, %two) : (tensor<1xi64>, tensor<1xi64>) -> tensor<1xi64>
+        %f = "llh.convert_to"(%sq) : (tensor<1xi64>) -> tensor<1xf32>
+        "llh.print"(%f) <{prefix_description = "mul"}> : (tensor<1xf32>) -> ()
+        return
+    }'''
+    out = engine(mul).run()
+    assert out.dtype == torch.float32
+    np.testing.assert_array_equal(out.cpu().numpy(), np.array([4.0], np.float32))
+    # dynamic shapes: one engine, two bindings
+    conv = engine(CONV_AND_SHAPES, "conv_nchw_fchw")
+    r = np.random.default_rng(0)
+    w = r.standard_normal((4, 3, 5, 5)).astype(np.float32)
+    for n, h, wd in ((2, 21, 30), (1, 33, 18)):
+        x = r.standard_normal((n, 3, h, wd)).astype(np.float32)
+        got = conv.run(torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda())
+        want = oracle.conv2d(x, w, pad=(2, 2, 2, 2), stride=(2, 2), dilation=(2, 2))
+        assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, "conv from text %s" % ((n, h, wd),))
+    sl = engine(CONV_AND_SHAPES, "slice_reshape_broadcast")
+    x = r.standard_normal((3, 4, 5, 6)).astype(np.float32)
+    got = sl.run(torch.from_numpy(x).cuda())
+    np.testing.assert_array_equal(got.cpu().numpy(), x[0:1] * np.float32(2.0))

@@ -1,0 +1,106 @@
+"""The LLH text reader and printer (MLIR generic op syntax, the wire format between the reference's importer and its
+compiler and the language of its lit tests).  The programs below are written in that syntax after the reference's own
+test inputs (test/RunnerTest/abs.mlir, test/Conversion/LLHToHLO/llh_to_hlo.mlir, preprocessing_llh_to_hlo.mlir):
+same ops, same attribute spellings, same scalar (i64) side."""
+import pytest
+import torch
+
+from llcompiler_amd.executor.planner import make_plan
+from llcompiler_amd.llh.expr import Expr, evaluate
+from llcompiler_amd.llh.passes import run_llh_pipeline
+from llcompiler_amd.llh.text import LLHSyntaxError, parse_llh, print_llh
+
+ABS_RUNNER = '''
+module{
+    func.func @main() -> () attributes {entrance} {
+        %const = "llh.constant"() <{value = dense<-1.000000e+00> : tensor<2xf32>}> : () -> tensor<2xf32>
+        %0 = "llh.abs"(%const) : (tensor<2xf32>) -> tensor<2xf32>
+        // CHECK-NEXT: [1,  1]
+        "llh.print"(%0) <{prefix_description = "abs"}>: (tensor<2xf32>) -> ()
+        return
+  }
+}'''
+
+CONV_AND_SHAPES = '''
+// -----
+func.func @conv_nchw_fchw(%arg0: tensor<4x3x5x5xf32> , %arg1: tensor<?x3x?x?xf32>) -> tensor<?x4x?x?xf32> attributes {entrance} {
+    %2 = "llh.conv"(%arg1, %arg0) <{dilation = array<i64: 2, 2>, group = 1 : i64, kernel_shape = array<i64: 5, 5>, layout = #llh.Layout<NCHW>, pad = array<i64: 2, 2, 2, 2>, stride = array<i64: 2, 2>}> : (tensor<?x3x?x?xf32>, tensor<4x3x5x5xf32>) -> tensor<?x4x?x?xf32>
+    return %2 : tensor<?x4x?x?xf32>
+}
+// -----
+func.func @slice_reshape_broadcast(%arg0: tensor<?x?x?x?xf32>) -> tensor<1x?x?x?xf32> attributes {entrance} {
+  %c0_i64 = "llh.constant"() <{value = 0 : i64}> : () -> i64
+  %c1_i64 = "llh.constant"() <{value = 1 : i64}> : () -> i64
+  %c2_i64 = "llh.constant"() <{value = 2 : i64}> : () -> i64
+  %c3_i64 = "llh.constant"() <{value = 3 : i64}> : () -> i64
+  %0 = "llh.dim"(%arg0, %c1_i64) <{symbol = @s1}> : (tensor<?x?x?x?xf32>, i64) -> i64
+  %1 = "llh.dim"(%arg0, %c2_i64) : (tensor<?x?x?x?xf32>, i64) -> i64
+  %2 = "llh.dim"(%arg0, %c3_i64) : (tensor<?x?x?x?xf32>, i64) -> i64
+  %3 = "llh.stride_slice"(%arg0, %c0_i64, %c0_i64, %c0_i64, %c0_i64, %c1_i64, %0, %1, %2, %c1_i64, %c1_i64, %c1_i64, %c1_i64) <{operandSegmentSizes = array<i32: 1, 4, 4, 4>}> : (tensor<?x?x?x?xf32>, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64) -> tensor<1x?x?x?xf32>
+  %4 = "llh.constant"() <{value = dense<2.000000e+00> : tensor<1xf32>}> : () -> tensor<1xf32>
+  %5 = "llh.reshape"(%4, %c1_i64, %c1_i64, %c1_i64, %c1_i64) : (tensor<1xf32>, i64, i64, i64, i64) -> tensor<1x1x1x1xf32>
+  %10 = "llh.broadcast_to"(%5, %c1_i64, %0, %1, %2) <{cast_dims = array<i64: 0, 1, 2, 3>}> : (tensor<1x1x1x1xf32>, i64, i64, i64, i64) -> tensor<1x?x?x?xf32>
+  %11 = "llh.mul"(%3, %10) : (tensor<1x?x?x?xf32>, tensor<1x?x?x?xf32>) -> tensor<1x?x?x?xf32>
+  return %11 : tensor<1x?x?x?xf32>
+}
+'''
+
+
+def test_runner_program_parses_to_constant_abs_and_returns_what_it_prints():
+    g = parse_llh(ABS_RUNNER)
+    assert g.op_names() == ["constant", "abs"] and g.inputs == []
+    const = g.ops[0]
+    assert tuple(const.results[0].shape) == (2,) and const.attrs["value"] == -1.0 and const.results[0].dtype == torch.float32
+    assert g.outputs == [g.ops[1].results[0]]          # no func result: the printed value is the observable
+
+
+def test_conv_attributes_and_symbolic_result_shape():
+    g = parse_llh(CONV_AND_SHAPES, func="conv_nchw_fchw")
+    (conv,) = g.ops
+    assert conv.name == "conv" and [v.name for v in conv.operands] == ["arg1", "arg0"]
+    assert conv.attrs == {"dilation": (2, 2), "kernel_shape": (5, 5), "pad": (2, 2, 2, 2), "stride": (2, 2), "group": 1}
+    n, f, oh, ow = conv.results[0].shape
+    assert f == 4 and isinstance(n, Expr) and isinstance(oh, Expr)
+    # out = (in + 2 + 2 - 2 * (5 - 1) - 1) / 2 + 1 (src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:257-268)
+    x = g.inputs[1]
+    env = {x.shape[0].args[0]: 3, x.shape[2].args[0]: 33, x.shape[3].args[0]: 18}
+    assert (evaluate(n, env), evaluate(oh, env), evaluate(ow, env)) == (3, (33 + 4 - 8 - 1) // 2 + 1, (18 + 4 - 8 - 1) // 2 + 1)
+
+
+def test_scalar_side_becomes_symbolic_extents():
+    g = parse_llh(CONV_AND_SHAPES, func="slice_reshape_broadcast")
+    assert g.op_names() == ["stride_slice", "constant", "reshape", "broadcast_to", "mul"]
+    x = g.inputs[0]
+    sl = g.ops[0]
+    assert sl.attrs["start"] == (0, 0, 0, 0) and sl.attrs["stride"] == (1, 1, 1, 1)
+    assert sl.attrs["end"] == (1,) + tuple(x.shape[1:])          # llh.dim(%arg0, k) is the k-th extent of %arg0
+    assert tuple(sl.results[0].shape) == (1,) + tuple(x.shape[1:])
+    assert tuple(g.ops[2].results[0].shape) == (1, 1, 1, 1)
+    assert tuple(g.ops[3].results[0].shape) == (1,) + tuple(x.shape[1:])
+    # and the graph lowers: slice and broadcast are views, the multiply by a one-element constant one kernel
+    run_llh_pipeline(g)
+    kinds = [s.kind for s in make_plan(g) if s.kind not in ("view", "constant")]
+    assert kinds == ["ew"]
+
+
+def test_printer_round_trip_of_an_imported_model():
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    g = compile_module(MLP().eval(), make_mlp_inputs(), weights="npy").engine.graph
+    text = print_llh(g)
+    assert '"llh.weight"() <{weight_file = "' in text and '"llh.matmul"' in text
+    g2 = parse_llh(text)
+    assert g2.op_names() == g.op_names()
+    for a, b in zip(g.ops, g2.ops):
+        assert tuple(a.results[0].shape) == tuple(b.results[0].shape) and a.results[0].dtype == b.results[0].dtype
+        assert {k: v for k, v in a.attrs.items() if k != "cast_dims"} == {k: v for k, v in b.attrs.items() if k != "cast_dims"}
+    assert print_llh(g2).replace("%arg", "%x") .count("llh.") == text.count("llh.")
+
+
+def test_syntax_errors_are_reported():
+    with pytest.raises(LLHSyntaxError):
+        parse_llh("module {}")
+    with pytest.raises(LLHSyntaxError):
+        parse_llh('func.func @main() -> () { %0 = "llh.abs"(%nope) : (tensor<2xf32>) -> tensor<2xf32> return }')
+    with pytest.raises(NotImplementedError):
+        parse_llh('func.func @main(%a: tensor<2xf32>) -> () { %0 = "stablehlo.abs"(%a) : (tensor<2xf32>) -> tensor<2xf32> return }')
