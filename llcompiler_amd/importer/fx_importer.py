@@ -398,7 +398,13 @@ def _softmax(ctx, node):
     return ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
 
 
-@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm.default, check=lambda n: len(n.args[1]) == 1)
+def _first_result_only(node):
+    """The translators of multi-result ATen ops produce the first result only (the output; not the saved
+    statistics or pooling indices a backward graph asks for): a node whose other results are used stays in eager."""
+    return all(u.op == "call_function" and u.target is operator.getitem and u.args[1] == 0 for u in node.users)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm.default, check=lambda n: len(n.args[1]) == 1 and _first_result_only(n))
 def _layer_norm(ctx, node):
     x, shape, w, b, eps = node.args
     ops = [ctx.val(x)] + [ctx.val(t) for t in (w, b) if t is not None]
@@ -407,7 +413,7 @@ def _layer_norm(ctx, node):
     return (y, None, None)
 
 
-@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._native_batch_norm_legit_no_training.default)
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._native_batch_norm_legit_no_training.default, check=_first_result_only)
 def _batch_norm(ctx, node):
     x, w, b, mean, var, momentum, eps = node.args
     xv = ctx.val(x)
@@ -420,7 +426,7 @@ def _batch_norm(ctx, node):
 
 
 def _bn_eval_only(node):
-    return node.args[5] is False
+    return node.args[5] is False and _first_result_only(node)
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_batch_norm.default, aten._native_batch_norm_legit.default,
@@ -445,7 +451,7 @@ def _ones_like_channels(ctx, c, dtype, value):
 
 def _maxpool_ok(node):
     a = list(node.args) + [None] * 6
-    return not a[5]  # ceil_mode
+    return not a[5] and _first_result_only(node)  # no ceil_mode, no indices
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.max_pool2d_with_indices.default, check=_maxpool_ok)

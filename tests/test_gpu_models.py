@@ -278,3 +278,75 @@ def test_llh_text_programs_run_on_the_gpu(oracle):
     x = r.standard_normal((3, 4, 5, 6)).astype(np.float32)
     got = sl.run(torch.from_numpy(x).cuda())
     np.testing.assert_array_equal(got.cpu().numpy(), x[0:1] * np.float32(2.0))
+
+
+def test_training_mode_compiles_forward_and_backward_graphs():
+    """mode="training": AOT-autograd's backward graph goes through the same backend (the reference tests static and
+    dynamic x inference and training, llcompiler/test_models/utility.py:128-138).  MLP: the backward of the two
+    Linear layers is matmuls on transposed views, a sum over the batch for the bias, and the relu mask as one
+    elementwise program; gradients are compared with torch eager's."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    torch._dynamo.reset()
+    m = MLP().cuda()
+    ref = copy.deepcopy(m)
+    comp = LLCompiler(mode="training", target="gfx950", pipeline="hip")
+    opt = torch.compile(m, backend=comp, dynamic=False)
+    (x,) = make_mlp_inputs(batch=32)
+    x = x.cuda()
+    for step in range(2):
+        for mod in (m, ref):
+            mod.zero_grad()
+        out = opt(x)
+        out.square().mean().backward()
+        want = ref(x)
+        want.square().mean().backward()
+        assert_close(out.detach().cpu().numpy(), want.detach().cpu().numpy(), F32_RTOL, F32_ATOL, "training forward")
+        for (name, p), (_, q) in zip(m.named_parameters(), ref.named_parameters()):
+            assert p.grad is not None, name
+            assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-6, "grad of %s" % name)
+    assert comp.compile_count >= 2          # a forward and a backward partition at least
+    names = [k for e in comp.engines for s in e.steps for k in [s.kind] if k != "view"]
+    assert names.count("matmul") >= 5       # 2 forward, 3 backward (dW1, dW2, dX of the second layer)
+
+
+class _SmallConvNet(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1 = torch.nn.Conv2d(3, 8, 3, padding=1)
+        self.c2 = torch.nn.Conv2d(8, 8, 3, padding=1)
+        self.fc = torch.nn.Linear(8, 5)
+
+    def forward(self, x):
+        y = torch.relu(self.c1(x))
+        y = torch.relu(self.c2(y) + y)
+        return self.fc(y.mean((2, 3)))
+
+
+@pytest.mark.parametrize("which", ["convnet", "encoder"])
+def test_training_mode_with_eager_fallbacks(which):
+    """Backward graphs contain nodes without a translator (convolution_backward, the layer-norm, softmax and gelu
+    backward ops, and forward ops whose saved statistics the backward graph reads): they stay in torch eager, the
+    rest runs on the kernels, and the gradients match eager's."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    torch._dynamo.reset()
+    torch.manual_seed(0)
+    if which == "convnet":
+        m, x = _SmallConvNet().cuda(), torch.randn(4, 3, 16, 16).cuda()
+    else:
+        m, x = EncoderBlock(hidden=128, heads=2, ffn=256).cuda(), make_encoder_inputs(2, 64, 128)[0].cuda()
+    ref = copy.deepcopy(m)
+    comp = LLCompiler(mode="training", target="gfx950", pipeline="hip")
+    opt = torch.compile(m, backend=comp, dynamic=False)
+    out = opt(x)
+    out.square().mean().backward()
+    want = ref(x)
+    want.square().mean().backward()
+    assert_close(out.detach().cpu().numpy(), want.detach().cpu().numpy(), F32_RTOL, F32_ATOL, "training forward")
+    scale = max(q.grad.abs().max().item() for q in ref.parameters())
+    for (name, p), (_, q) in zip(m.named_parameters(), ref.named_parameters()):
+        # (the gradient of an attention key bias is zero in exact arithmetic: an absolute bar on the common scale)
+        assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-5 * scale, "grad of %s" % name)
+    kinds = [s.kind for e in comp.engines for s in e.steps]
+    assert kinds.count("matmul") >= 3 and len(comp.engines) >= 2
