@@ -20,11 +20,12 @@ from .torch_compile_config import LLC_DECOMPOSITIONS
 class CompiledModule:
     def __init__(self, engine, lifted, n_user):
         self.engine, self.lifted, self.n_user = engine, lifted, n_user
+        self._run = engine.bind_leading(lifted) if all(isinstance(t, torch.Tensor) for t in lifted) else None
 
     def __call__(self, *args):
         if len(args) != self.n_user:
             raise ValueError("expected %d inputs, got %d" % (self.n_user, len(args)))
-        out = self.engine.run(*self.lifted, *args)
+        out = self._run(*args) if self._run is not None else self.engine.run(*self.lifted, *args)
         # export always returns a tuple; a single result is handed back bare, like the module would
         if isinstance(out, (list, tuple)) and len(out) == 1:
             return out[0]

@@ -692,6 +692,26 @@ class Torch_ExecutionEngine(ExecutionEngine):
             env.setdefault(name, inputs[i].shape[d])
         return env
 
+    def bind_leading(self, tensors):
+        """run() with `tensors` fixed as the first arguments (the parameters an ahead-of-time compiled module
+        passes with every call): their part of the call signature is computed once, not per call."""
+        lead = tuple(tensors)
+        lead_key = tuple((a.dtype, a.shape, a.stride(), a.device) for a in lead)
+        lead_list = list(lead)
+        fast = self._fast
+
+        def run(*args):
+            key = lead_key + tuple(a if not isinstance(a, torch.Tensor) else (a.dtype, a.shape, a.stride(), a.device) for a in args)
+            hit = fast.get(key)
+            if hit is None:
+                return self.run(*lead, *args)
+            results = hit.run(lead_list + [a for a in args if isinstance(a, torch.Tensor)])
+            if getattr(self.graph, "single_output", len(results) == 1) and len(results) == 1:
+                return results[0]
+            return results
+
+        return run
+
     def run(self, *args):
         # ([inputs...]) case, as in the reference
         if len(args) == 1 and isinstance(args[0], (list, tuple)):
