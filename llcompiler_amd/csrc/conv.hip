@@ -522,6 +522,235 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
   return LLC_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Channels-last (NHWC) fp32 convolution: x [N,C,H,W] with strides (HWC, 1, WC, C), weight [F,C,KH,KW] with
+// strides (KH KW C, 1, KW C, C), output and residual channels-last too.
+//
+// In this layout the im2col matrix needs no gather arithmetic: with k ordered (kh, kw, c) a row of it is, per
+// filter tap, a run of C contiguous floats of the input, and a k-tile of 32 floats (C % 32 == 0) lies inside
+// one tap.  So the convolution is the GEMM  out[pixel, f] = sum_k im2col[pixel, k] * weight[f, k]  with both
+// operands contiguous along k and the output row-major [pixels, F], i.e. channels-last again, and it runs on
+// the tile machinery of gemm_kernel (LDS layout, fragment reads, MFMA loop, two register stages).  What is
+// specific is the loader of the pixel operand: every lane keeps, for each of its rows, the offset of the
+// window origin and one validity bit per tap, computed once; a k-tile adds one scalar offset (tap, channel
+// block) to them.  A lane spends a handful of integer instructions per 16-byte vector where the NCHW kernel
+// spends about forty on (c, kh, kw) bookkeeping, window clamping and border shifts.
+template <int BM, int NT>
+struct NhwcLoader {
+  static constexpr int kIters = BM * 8 / NT;
+  static_assert(BM * 8 % NT == 0 && kIters >= 1 && kIters <= 32, "whole vectors per lane");
+  u32x4_t v[kIters];
+  uint32_t okm = 0;
+  int base[kIters];       // element offset of (n, oh*sh - ph, ow*sw - pw, channel 0) from X; may be negative
+  uint64_t taps[kIters];  // bit kh*KW + kw: that tap of the row's window lies inside the image
+
+  __device__ __forceinline__ void init(const ConvParams& p, int m0) {
+    const int ohw = p.OH * p.OW;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int m = m0 + ((i * NT + (int)threadIdx.x) >> 3);
+      base[i] = 0;
+      taps[i] = 0;
+      if (m < p.ncols) {
+        const int n = m / ohw, rem = m - n * ohw;
+        const int oh = rem / p.OW, ow = rem - oh * p.OW;
+        const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
+        base[i] = ((n * p.H + ih0) * p.Wd + iw0) * p.C;
+        uint64_t bits = 0;
+        for (int kh = 0; kh < p.KH; ++kh)
+          for (int kw = 0; kw < p.KW; ++kw) {
+            const int ih = ih0 + kh * p.dh, iw = iw0 + kw * p.dw;
+            if (ih >= 0 && ih < p.H && iw >= 0 && iw < p.Wd) bits |= (uint64_t)1 << (kh * p.KW + kw);
+          }
+        taps[i] = bits;
+      }
+    }
+  }
+  // all loads are issued, from offset 0 where the tap falls outside; what was outside is zeroed in store()
+  __device__ __forceinline__ void load(const float* X, const ConvParams& p, int k0) {
+    const int tap = k0 / p.C, c0 = k0 - tap * p.C;
+    const int kh = tap / p.KW, kw = tap - kh * p.KW;
+    const int toff = (kh * p.dh * p.Wd + kw * p.dw) * p.C + c0;
+    okm = 0;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int kv = (i * NT + (int)threadIdx.x) & 7;
+      const uint32_t ok = (uint32_t)(taps[i] >> tap) & 1u;
+      const int off = ok ? base[i] + toff + kv * 4 : 0;
+      v[i] = *(const u32x4_t*)(X + off);
+      okm |= ok << i;
+    }
+  }
+  __device__ __forceinline__ void store(char* lds) const {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int vid = i * NT + (int)threadIdx.x;
+      const uint32_t m = 0u - ((okm >> i) & 1u);
+      *(u32x4_t*)(lds + lds_off(vid >> 3, (vid & 7) * 16)) = u32x4_t{v[i][0] & m, v[i][1] & m, v[i][2] & m, v[i][3] & m};
+    }
+  }
+};
+
+template <int BM, int BN, int WM, int WN, bool BFULL>
+__global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvParams p) {
+  constexpr int NT = 64 * WM * WN;
+  constexpr int BK = 32;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int kABytes = BM * kRowStride, kBBytes = BN * kRowStride;
+  constexpr int kBufBytes = kABytes + kBBytes;
+  extern __shared__ __align__(16) char smem[];
+  int tile_m, tile_n;
+  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const float* X = (const float*)p.X;
+  const float* Wt = (const float*)p.W;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int wm = wave / WN, wn = wave % WN;
+  const int li = lane % 32, lh = lane / 32;
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // k-tiles of this split
+  const int nk_all = p.Kdim / BK;
+  const int split = blockIdx.y;
+  const int kt0 = (int)((int64_t)split * nk_all / p.splits), nk = (int)((int64_t)(split + 1) * nk_all / p.splits) - kt0;
+  NhwcLoader<BM, NT> la0, la1;
+  TileLoader<float, BN, kLoadKVec, NT> lb0, lb1;
+  la0.init(p, m0);
+#pragma unroll
+  for (int i = 0; i < NhwcLoader<BM, NT>::kIters; ++i) {
+    la1.base[i] = la0.base[i];
+    la1.taps[i] = la0.taps[i];
+  }
+  la0.load(X, p, kt0 * BK);
+  lb0.template load<BFULL>(Wt, n0, p.F, kt0 * BK, p.Kdim, p.Kdim, 1);
+  if (nk > 1) {
+    la1.load(X, p, (kt0 + 1) * BK);
+    lb1.template load<BFULL>(Wt, n0, p.F, (kt0 + 1) * BK, p.Kdim, p.Kdim, 1);
+  }
+  la0.store(smem);
+  lb0.store(smem + kABytes);
+  __syncthreads();
+#define LLC_NHWC_STEP(KT, CUR, LA2, LB2, LA1, LB1)                                                              \
+  {                                                                                                             \
+    if ((KT) + 2 < nk) {                                                                                        \
+      LA2.load(X, p, (kt0 + (KT) + 2) * BK);                                                                    \
+      LB2.template load<BFULL>(Wt, n0, p.F, (kt0 + (KT) + 2) * BK, p.Kdim, p.Kdim, 1);                          \
+    }                                                                                                           \
+    mma_tile<float, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,        \
+                            wn * WTN + li, lh, acc);                                                            \
+    if ((KT) + 1 < nk) {                                                                                        \
+      LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
+      LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
+    }                                                                                                           \
+    __syncthreads();                                                                                            \
+  }
+  for (int kt = 0; kt < nk; kt += 2) {
+    LLC_NHWC_STEP(kt, 0, la0, lb0, la1, lb1)
+    if (kt + 1 < nk) LLC_NHWC_STEP(kt + 1, 1, la1, lb1, la0, lb0)
+  }
+#undef LLC_NHWC_STEP
+
+  // ---- epilogue: register r of lane (li, lh) is row 8 (r/4) + 4 lh + r%4, column li: 32 lanes store 32 consecutive
+  //      filters of one pixel ----
+  float* Y = p.splits > 1 ? (float*)p.partial + (int64_t)split * p.ncols * p.F : (float*)p.Y;
+  const char* res = p.splits > 1 ? nullptr : p.residual;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * WTN + j * 32 + li;
+    if (!BFULL && col >= p.F) continue;
+    const float bv = (p.bias && p.splits == 1) ? ((const float*)p.bias)[col] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+        if (row >= p.ncols) continue;
+        const int64_t o = (int64_t)row * p.F + col;
+        if (p.splits > 1) Y[o] = acc[i][j][r];
+        else epilogue_store<float>(Y, o, acc[i][j][r], p.alpha, bv, res, p.act);
+      }
+  }
+}
+
+// Sums the split partials [splits][pixels][F] in split order and applies the epilogue (channels-last output).
+__global__ __launch_bounds__(256) void nhwc_split_reduce_kernel(const ConvParams p) {
+  const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int64_t total = (int64_t)p.ncols * p.F;
+  if (i4 >= total) return;  // F % 4 == 0: a vector never straddles the end
+  const float* part = (const float*)p.partial + i4;
+  f32x4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k = 0; k < p.splits; ++k) s += *(const f32x4_t*)(part + (int64_t)k * total);
+  const int f = (int)(i4 % p.F);
+  f32x4_t b = {0.0f, 0.0f, 0.0f, 0.0f}, r = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (p.bias) b = *(const f32x4_t*)((const float*)p.bias + f);
+  if (p.residual) r = *(const f32x4_t*)((const float*)p.residual + i4);
+  f32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float v = s[e] * p.alpha + b[e] + r[e];
+    if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
+    else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
+    o[e] = v;
+  }
+  *(f32x4_t*)((float*)p.Y + i4) = o;
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
+  ConvParams p = p0;
+  p.tiles_m = (p.ncols + BM - 1) / BM;
+  p.tiles_n = (p.F + BN - 1) / BN;
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "conv: grid too large");
+  const int nk = p.Kdim / 32;
+  // too few tiles for 256 CUs: split the reduction (at least eight k-tiles per split)
+  int splits = 1;
+  if (tiles < 384) {
+    splits = (int)((512 + tiles - 1) / tiles);
+    if (splits > nk / 8) splits = nk / 8;
+    if (splits < 1) splits = 1;
+  }
+  p.splits = splits;
+  if (splits > 1) {
+    void* ws = nullptr;
+    LLC_TRY(get_workspace((size_t)splits * p.ncols * p.F * sizeof(float), &ws));
+    p.partial = (char*)ws;
+  }
+  const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
+  const bool bfull = p.F % BN == 0;
+  auto kern = bfull ? conv_nhwc_f32_kernel<BM, BN, WM, WN, true> : conv_nhwc_f32_kernel<BM, BN, WM, WN, false>;
+  static bool attr_set[2] = {false, false};
+  if (!attr_set[bfull]) {
+    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set[bfull] = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)splits, 1), dim3(64 * WM * WN), lds, s, p);
+  LLC_TRY(check_launch("conv_nhwc_f32_kernel"));
+  if (splits > 1) {
+    const int64_t total4 = (int64_t)p.ncols * p.F / 4;
+    hipLaunchKernelGGL(nhwc_split_reduce_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, s, p);
+    LLC_TRY(check_launch("nhwc_split_reduce_kernel"));
+  }
+  return LLC_OK;
+}
+
+#ifndef LLC_NHWC_CFG64
+#define LLC_NHWC_CFG64 128, 64, 4, 2
+#define LLC_NHWC_CFG128 128, 128, 4, 2
+#endif
+int launch_nhwc_f32(const ConvParams& p, hipStream_t s) {
+  if (p.F <= 64) return launch_nhwc_cfg<LLC_NHWC_CFG64>(p, s);
+  return launch_nhwc_cfg<LLC_NHWC_CFG128>(p, s);
+}
+
 template <typename T, int BM, int BN, int LA>
 int launch_cfg(const ConvParams& p0, int groups, hipStream_t s) {
   ConvParams p = p0;
@@ -578,7 +807,15 @@ int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_att
   if (a.dtype != LLC_FLOAT32 && a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16)
     return set_error(LLC_ERR_DTYPE, "conv: element type %d (LLH_FloatTensor expected)", a.dtype);
   if (a.rank != 4 || k.rank != 4 || o.rank != 4) return set_error(LLC_ERR_SHAPE, "conv: NCHW x FCHW -> NCHW expected");
-  if (!a.contiguous() || !k.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "conv: contiguous tensors expected");
+  // Layout travels in the strides, as in torch: all tensors NCHW-contiguous, or all channels-last (NHWC in memory).
+  auto channels_last = [](const View& v) {
+    const int64_t C = v.size[1], H = v.size[2], W = v.size[3];
+    return (C == 1 || v.stride[1] == 1) && (W == 1 || v.stride[3] == C) && (H == 1 || v.stride[2] == W * C) &&
+           (v.size[0] == 1 || v.stride[0] == H * W * C);
+  };
+  const bool nhwc = !(a.contiguous() && k.contiguous() && o.contiguous()) && channels_last(a) && channels_last(k) && channels_last(o);
+  if (!nhwc && (!a.contiguous() || !k.contiguous() || !o.contiguous()))
+    return set_error(LLC_ERR_LAYOUT, "conv: tensors must all be contiguous (NCHW) or all channels-last");
   const int64_t group = at->group;
   for (int i = 0; i < 2; ++i)
     if (at->stride[i] <= 0 || at->dilation[i] <= 0 || at->pad[i] < 0 || at->pad[i + 2] < 0)
@@ -638,11 +875,20 @@ int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_att
       View r;
       LLC_TRY(make_view(epi->residual, "conv residual", &r));
       if (r.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "conv: residual type differs from output");
-      if (r.numel() != o.numel() || !r.contiguous()) return set_error(LLC_ERR_SHAPE, "conv: residual must match the output and be contiguous");
+      bool same = r.rank == 4 && r.numel() == o.numel();
+      for (int d = 0; same && d < 4; ++d) same = r.size[d] == o.size[d];
+      if (!(nhwc ? same && channels_last(r) : r.numel() == o.numel() && r.contiguous()))
+        return set_error(LLC_ERR_SHAPE, "conv: residual must match the output in shape and layout");
       p.residual = r.ptr;
     }
   }
   hipStream_t s = as_stream(stream);
+  if (nhwc) {
+    if (a.dtype != LLC_FLOAT32 || group != 1 || p.C % 32 != 0 || p.KH * p.KW > 64 || p.F % 4 != 0 ||
+        ((uintptr_t)p.X | (uintptr_t)p.W | (uintptr_t)p.Y | (uintptr_t)p.residual | (uintptr_t)p.bias) % 16 != 0)
+      return set_error(LLC_ERR_UNSUPPORTED, "conv: channels-last tensors need fp32, group 1, C %% 32 == 0, F %% 4 == 0, at most 64 taps and 16-byte alignment");
+    return launch_nhwc_f32(p, s);
+  }
   switch (a.dtype) {
     case LLC_FLOAT32: return launch_loaders<float>(p, (int)group, s);
     case LLC_BFLOAT16: return launch_loaders<__bf16>(p, (int)group, s);

@@ -43,6 +43,10 @@ MIN_CALLS_FOR_GRAPH = 2
 USE_PLAN = True
 # batch_matmul -> softmax -> batch_matmul groups of attention layers with head dim 64 become one fused kernel
 FUSE_ATTENTION = True
+# fp32 convolutions with C % 32 == 0 run on channels-last (NHWC) copies of their operands: the kernel for that
+# layout needs no gather arithmetic.  Results keep the layout as strided views (logical shape NCHW), so a chain of
+# convolutions converts once; anything that needs NCHW memory copies back through the usual contiguity path.
+CHANNELS_LAST = True
 
 
 def _concrete(shape, env):
@@ -99,6 +103,9 @@ class Instance:
         self.graph, self.env, self.device = graph, env, device
         self.weights = weights     # WeightStore of the engine: tensors of llh.weight ops, loaded once
         self.calls = []
+        self.prep_calls = []       # run before `calls` when an input listed in prep_inputs changed
+        self.prep_inputs = []
+        self._prep_key = None
         self.patches = []          # (TensorRef, "in"|"out", index, byte offset from that tensor's data_ptr)
         self.keep = []
         self._roots = {}           # storage data_ptr -> ("in"|"out", index, base data_ptr)
@@ -115,6 +122,24 @@ class Instance:
         for item in call.keep:
             self._scan(item)
         self.calls.append(call)
+
+    def _prepare_later(self, call, input_index):
+        """A call whose result depends only on graph input `input_index` (a layout copy of a weight): it runs
+        before the instance's other calls, and again only when that input's address or version counter changed."""
+        for item in call.keep:
+            self._scan(item)
+        self.prep_calls.append(call)
+        if input_index not in self.prep_inputs:
+            self.prep_inputs.append(input_index)
+
+    def _channels_last_ok(self, st, ins, out, natural):
+        if not CHANNELS_LAST or out.dtype != torch.float32 or st.attrs["group"] != 1 or len(natural) != 4:
+            return False
+        x, w = ins
+        if tuple(natural) != tuple(out.shape) or not out.numel() or x.dim() != 4 or w.dim() != 4:
+            return False
+        return x.shape[1] % 32 == 0 and w.shape[0] % 4 == 0 and w.shape[2] * w.shape[3] <= 64 and \
+            x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
     def _scan(self, item):
         if isinstance(item, C.TensorRef):
@@ -217,6 +242,30 @@ class Instance:
                 return x.src
             return materialise(x)
 
+        cl_copies = {}   # id(value) -> its channels-last copy
+
+        def to_channels_last(v, t):
+            """`t` (the tensor of value `v`, logical NCHW) as a channels-last tensor: itself if it already is, else a
+            copy made once per value.  Copies of graph inputs (weights) are made by the instance's preparation
+            calls, which run again only when such an input moved or was written to."""
+            if t.is_contiguous(memory_format=torch.channels_last):
+                return t
+            c = cl_copies.get(id(v))
+            if c is None:
+                n = t.numel()
+                buf = pool.take(n * t.dtype.itemsize)
+                self.keep.append(buf)
+                nhwc = buf[: n * t.dtype.itemsize].view(t.dtype).view(t.shape[0], t.shape[2], t.shape[3], t.shape[1])
+                call = ops.copy(t.permute(0, 2, 3, 1), out=nhwc, defer=True)
+                root = self._roots.get(t.untyped_storage().data_ptr())
+                if root is not None and root[0] == "in" and id(v) in input_ids:
+                    self._prepare_later(call, root[1])
+                else:
+                    self._launch_later(call)
+                c = cl_copies[id(v)] = nhwc.permute(0, 3, 1, 2)
+            return c
+
+        input_ids = set(id(v) for v in g.inputs)
         consumers = {}
         for st in steps:
             reads = list(st.inputs)
@@ -397,7 +446,8 @@ class Instance:
                         full = _concrete(st.output.shape, self.env)
                         bias = bias.view(full[0], full[3])
                         natural = full
-                if res is not None:
+                cl = k == "conv" and self._channels_last_ok(st, ins, out, natural)
+                if res is not None and not cl:
                     res = contiguous(res)
                 epi = None
                 if bias is not None or res is not None or e["act"] or e["alpha"] != 1.0:
@@ -414,6 +464,16 @@ class Instance:
                         val[id(r1.output)] = o
                         skip.add(id(r1))
                     call = ops.batch_matmul(ins[0], ins[1], epi, out=o, defer=True)
+                elif cl:
+                    xc = to_channels_last(st.inputs[0], ins[0])
+                    wc = to_channels_last(st.inputs[1], ins[1])
+                    if res is not None:
+                        epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=to_channels_last(e["residual"], res),
+                                           act=e["act"] or "none")
+                    n_, f_, oh_, ow_ = natural
+                    out = out.view(-1).view(n_, oh_, ow_, f_).permute(0, 3, 1, 2)  # NCHW shape over NHWC memory
+                    call = ops.conv2d(xc, wc, pad=st.attrs["pad"], stride=st.attrs["stride"], dilation=st.attrs["dilation"],
+                                      group=1, epilogue=epi, out=out, defer=True)
                 else:
                     call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],
                                       dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi, out=o, defer=True)
@@ -573,6 +633,13 @@ class Instance:
             outs = [torch.empty(s, dtype=d, device=self.device) for s, d in self.out_specs]
         in_ptrs = [t.data_ptr() for t in inputs]
         stream = C.current_stream(self.device)
+        if self.prep_calls:
+            key = [(in_ptrs[i], inputs[i]._version) for i in self.prep_inputs]
+            if key != self._prep_key:
+                self._patch(in_ptrs, [t.data_ptr() for t in outs])
+                for c in self.prep_calls:
+                    c.launch(stream)
+                self._prep_key = key
         if self._plan is not None:
             blk = self._block
             last = self._last_in_ptrs

@@ -350,3 +350,26 @@ def test_training_mode_with_eager_fallbacks(which):
         assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-5 * scale, "grad of %s" % name)
     kinds = [s.kind for e in comp.engines for s in e.steps]
     assert kinds.count("matmul") >= 3 and len(comp.engines) >= 2
+
+
+def test_channels_last_weight_copies_follow_the_weights():
+    """ResNet convolutions run on channels-last copies of their weights, made by preparation calls that run again
+    when a weight is written in place or replaced; the stem (3 channels) and everything else stay NCHW."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval().cuda()
+    (x,) = make_resnet_inputs(2, 64)
+    x = x.cuda()
+    with torch.no_grad():
+        cm = compile_module(m, (x,))
+        first = cm(x)
+        assert_close(first.cpu().numpy(), m(x).cpu().numpy(), F32_RTOL, F32_ATOL, "resnet, first run")
+        inst = list(cm.engine.instances.values())[0]
+        # every conv but the stem; the three 1x1 downsample weights are channels-last as they are
+        assert len(inst.prep_calls) == 16 and len(inst.prep_inputs) == 16
+        again = cm(x)
+        assert torch.equal(first, again)
+        for p in m.parameters():       # in place: same addresses, new version counters
+            if p.dim() == 4:
+                p.mul_(0.5)
+        assert_close(cm(x).cpu().numpy(), m(x).cpu().numpy(), F32_RTOL, F32_ATOL, "resnet, weights scaled in place")

@@ -563,6 +563,55 @@ def test_conv2d(ops, oracle, case):
                       "conv bf16 %s" % (case,))
 
 
+NHWC_CASES = [
+    # N, C, H, W, F, KH, KW, pad(h_lo, w_lo, h_hi, w_hi), stride, dil
+    (2, 64, 14, 14, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # basic-block conv
+    (2, 64, 15, 13, 128, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),     # stride 2, odd extents
+    (2, 64, 14, 14, 128, 1, 1, (0, 0, 0, 0), (2, 2), (1, 1)),     # 1x1 stride-2 downsample
+    (1, 32, 20, 20, 68, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilated; 68 filters: a partial filter tile
+    (3, 32, 9, 11, 8, 5, 3, (2, 0, 1, 2), (1, 2), (1, 1)),        # asymmetric window, pad and stride
+    (4, 256, 7, 7, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # few pixels, deep reduction: split over k
+    (1, 96, 5, 5, 4, 7, 7, (3, 3, 3, 3), (1, 1), (1, 1)),         # 49 taps, windows larger than the image
+]
+
+
+@pytest.mark.parametrize("case", NHWC_CASES)
+def test_conv2d_channels_last(ops, oracle, case):
+    """The same entry point with the layout in the strides: x, weight, output and residual channels-last (NHWC in
+    memory, logical shape NCHW) take the kernel that reads the im2col rows as contiguous runs."""
+    N, C, H, W, Fo, KH, KW, pad, s, d = case
+    r = rng(sum(case[:7]) + 1)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((Fo, C, KH, KW)) / np.sqrt(C * KH * KW)).astype(np.float32)
+    b = r.standard_normal(Fo).astype(np.float32)
+    want = oracle.conv2d(x, w, None, pad=pad, stride=s, dilation=d)
+    cl = torch.channels_last
+    dx, dw = dev(x).contiguous(memory_format=cl), dev(w).contiguous(memory_format=cl)
+    out = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
+    got = ops.conv2d(dx, dw, pad=pad, stride=s, dilation=d, out=out)
+    assert got.is_contiguous(memory_format=cl)
+    assert_close_f32(host(got), want, "channels-last conv %s" % (case,))
+    res = r.standard_normal(want.shape).astype(np.float32)
+    want2 = oracle.unary("relu", oracle.conv2d(x, w, b, pad=pad, stride=s, dilation=d) * np.float32(1.0) + res)
+    epi = ops.Epilogue(bias=dev(b), residual=dev(res).contiguous(memory_format=cl), act="relu")
+    out2 = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
+    assert_close_f32(host(ops.conv2d(dx, dw, pad=pad, stride=s, dilation=d, epilogue=epi, out=out2)), want2,
+                     "channels-last conv+bias+res+relu %s" % (case,))
+
+
+def test_conv2d_layouts_must_agree(ops):
+    from llcompiler_amd._capi import LlcHipError
+    cl = torch.channels_last
+    x = torch.zeros((1, 32, 6, 6), device="cuda")
+    w = torch.zeros((8, 32, 3, 3), device="cuda")
+    with pytest.raises(LlcHipError):  # channels-last input, NCHW weight and output
+        ops.conv2d(x.contiguous(memory_format=cl), w, pad=(1, 1, 1, 1))
+    x48 = torch.zeros((1, 48, 6, 6), device="cuda").contiguous(memory_format=cl)  # 48 channels: not a multiple of 32
+    w48 = torch.zeros((8, 48, 3, 3), device="cuda").contiguous(memory_format=cl)
+    with pytest.raises(LlcHipError):
+        ops.conv2d(x48, w48, pad=(1, 1, 1, 1), out=torch.empty((1, 8, 6, 6), device="cuda").contiguous(memory_format=cl))
+
+
 def test_conv2d_asymmetric_pad(ops, oracle):
     r = rng(31)
     x = r.standard_normal((1, 2, 6, 7)).astype(np.float32)
