@@ -122,7 +122,8 @@ typedef struct llc_conv_attrs {
   int64_t stride[2];
   int64_t group;
 } llc_conv_attrs;
-/* Cross-correlation as implicit GEMM (LLHToHLO.cpp:214-270).  conv_bias is `epi->bias`.  * Layout travels in the strides, as in torch: either every tensor (x, w, out, epilogue residual) is contiguous
+/* Cross-correlation as implicit GEMM (LLHToHLO.cpp:214-270).  conv_bias is `epi->bias`.
+ * Layout travels in the strides, as in torch: either every tensor (x, w, out, epilogue residual) is contiguous
  * NCHW / FCHW, or every one is channels-last (NHWC in memory: strides (H W C, 1, W C, C) under the same
  * logical shape), which takes a kernel of its own (fp32, group 1, C % 32 == 0, F % 4 == 0, at most 64 taps;
  * LLC_ERR_UNSUPPORTED otherwise).  Mixed layouts are refused (LLC_ERR_LAYOUT). */
