@@ -713,7 +713,7 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   const int nk = p.Kdim / 32;
   // too few tiles for 256 CUs: split the reduction (at least eight k-tiles per split)
   int splits = 1;
-  if (tiles < 384) {
+  if (tiles < 256 || (BM == 128 && tiles < 384)) {
     splits = (int)((512 + tiles - 1) / tiles);
     if (splits > nk / 8) splits = nk / 8;
     if (splits < 1) splits = 1;
@@ -742,13 +742,15 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   return LLC_OK;
 }
 
-#ifndef LLC_NHWC_CFG64
-#define LLC_NHWC_CFG64 128, 64, 4, 2
-#define LLC_NHWC_CFG128 128, 128, 4, 2
-#endif
 int launch_nhwc_f32(const ConvParams& p, hipStream_t s) {
-  if (p.F <= 64) return launch_nhwc_cfg<LLC_NHWC_CFG64>(p, s);
-  return launch_nhwc_cfg<LLC_NHWC_CFG128>(p, s);
+  // 128-pixel tiles when they fill the chip by themselves; else 64 x 64 tiles if those are numerous enough to need
+  // no split of the reduction (a split costs a pass over the partial sums: the middle layers of a ResNet); the
+  // last layers split either way and do better on the large tiles
+  const int64_t bn = p.F <= 64 ? 64 : 128;
+  const int64_t t128 = (int64_t)((p.ncols + 127) / 128) * ((p.F + bn - 1) / bn);
+  const int64_t t64 = (int64_t)((p.ncols + 63) / 64) * ((p.F + 63) / 64);
+  if (t128 < 384 && t64 >= 256) return launch_nhwc_cfg<64, 64, 2, 2>(p, s);
+  return p.F <= 64 ? launch_nhwc_cfg<128, 64, 4, 2>(p, s) : launch_nhwc_cfg<128, 128, 4, 2>(p, s);
 }
 
 template <typename T, int BM, int BN, int LA>
