@@ -172,13 +172,15 @@ def cpu_baseline():
             "per_op_ms": {k: round(v * 1e3, 1) for k, v in parts.items()}}
 
 
-def model_latencies():
+MODELS = ("mlp", "resnet18", "encoder", "bert")
+
+
+def model_latencies(which=MODELS):
     """End-to-end latency per batch of the other four configurations (whole compiled graphs through the
     executor, inputs resident on the GPU, synchronised wall clock over repeated calls): an MLP, ResNet-18
     with folded batch norm, a bf16 encoder block compiled once with a symbolic batch, and a 12-layer BERT-base
     shaped encoder compiled once with a symbolic sequence length.  Reported next to the suite, not part of
-    `value`."""
-    import copy
+    `value`.  `which` selects a subset (for profiling one model's kernels at a time)."""
     import warnings
     from llcompiler_amd.compiler.aot import compile_module
     from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18Folded, make_bert_inputs,
@@ -197,22 +199,27 @@ def model_latencies():
 
     res = {}
     with torch.no_grad():
-        x = make_mlp_inputs()[0].cuda()
-        cm = compile_module(MLP().cuda(), (x,))
-        res["mlp_f32_batch4_ms"] = timed(lambda: cm(x), 200, 20)
-        xs = make_resnet_inputs(16, 224)[0].cuda()
-        cr = compile_module(ResNet18Folded().cuda(), (xs,))
-        res["resnet18_f32_batch16_ms"] = timed(lambda: cr(xs), 20, 3)
-        xe = make_encoder_inputs(8, 512)[0].to(torch.bfloat16).cuda()
-        ce = compile_module(EncoderBlock().to(torch.bfloat16).cuda(), (xe,), dynamic_shapes=({0: torch.export.Dim("batch")},))
-        for b in (1, 8, 32):
-            xb = make_encoder_inputs(b, 512, seed=b)[0].to(torch.bfloat16).cuda()
-            res["encoder_block_bf16_seq512_batch%d_ms" % b] = timed(lambda: ce(xb), 50, 5)
-        cb = compile_module(BertEncoder().cuda(), tuple(t.cuda() for t in make_bert_inputs(8, 128)),
-                            dynamic_shapes=({1: torch.export.Dim("seq")}, {3: torch.export.Dim("seq")}))
-        for sl in (128, 256, 512):
-            xi, mi = (t.cuda() for t in make_bert_inputs(8, sl, seed=sl))
-            res["bert_base_f32_batch8_seq%d_ms" % sl] = timed(lambda: cb(xi, mi), 10, 2)
+        if "mlp" in which:
+            x = make_mlp_inputs()[0].cuda()
+            cm = compile_module(MLP().cuda(), (x,))
+            res["mlp_f32_batch4_ms"] = timed(lambda: cm(x), 200, 20)
+        if "resnet18" in which:
+            xs = make_resnet_inputs(16, 224)[0].cuda()
+            cr = compile_module(ResNet18Folded().cuda(), (xs,))
+            res["resnet18_f32_batch16_ms"] = timed(lambda: cr(xs), 20, 3)
+        if "encoder" in which:
+            xe = make_encoder_inputs(8, 512)[0].to(torch.bfloat16).cuda()
+            ce = compile_module(EncoderBlock().to(torch.bfloat16).cuda(), (xe,),
+                                dynamic_shapes=({0: torch.export.Dim("batch")},))
+            for b in (1, 8, 32):
+                xb = make_encoder_inputs(b, 512, seed=b)[0].to(torch.bfloat16).cuda()
+                res["encoder_block_bf16_seq512_batch%d_ms" % b] = timed(lambda: ce(xb), 50, 5)
+        if "bert" in which:
+            cb = compile_module(BertEncoder().cuda(), tuple(t.cuda() for t in make_bert_inputs(8, 128)),
+                                dynamic_shapes=({1: torch.export.Dim("seq")}, {3: torch.export.Dim("seq")}))
+            for sl in (128, 256, 512):
+                xi, mi = (t.cuda() for t in make_bert_inputs(8, sl, seed=sl))
+                res["bert_base_f32_batch8_seq%d_ms" % sl] = timed(lambda: cb(xi, mi), 10, 2)
     return res
 
 
@@ -223,6 +230,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-models", action="store_true", help="skip the end-to-end latencies of the model configurations")
+    ap.add_argument("--models", default="", help="comma-separated subset of %s whose end-to-end latencies to "
+                    "measure (default: all of them, or none when --only is given)" % ",".join(MODELS))
     ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
                     "these cases, for profiling one kernel at a time (`all` = the whole suite, `copy_f32` adds the "
                     "counter calibration copy); the JSON line then describes that subset")
@@ -234,6 +243,9 @@ def main():
     from llcompiler_amd import ops
     device = torch.device("cuda", 0)
     only = [n for n in args.only.split(",") if n]
+    models = tuple(n for n in args.models.split(",") if n) or (() if only else MODELS)
+    if set(models) - set(MODELS):
+        sys.exit("--models takes names from %s" % ",".join(MODELS))
     cases = build_cases(ops, device, only)
 
     def step(i):
@@ -256,9 +268,9 @@ def main():
         "dominant_kernel": dominant["kernel"],
         "kernels": kernels,
     }
-    if not args.no_models and not only:
+    if not args.no_models and models:
         try:
-            out["model_latency_ms"] = model_latencies()
+            out["model_latency_ms"] = model_latencies(models)
         except Exception as e:  # the suite's line is still worth printing
             out["model_latency_ms"] = {"error": "%s: %s" % (type(e).__name__, e)}
     if not args.no_cpu_baseline:

@@ -761,6 +761,73 @@ int launch_skinny(const GemmParams& p, hipStream_t s) {
   return check_launch("gemm_skinny_kernel");
 }
 
+// ---- fp32 products with a long reduction and too few output tiles to fill the chip (a transformer's second
+// feed-forward layer at a short sequence: 1024 x 768 x 3072 is 192 tiles of 64x64).  The reduction is cut into
+// `splits` equal chunks that run as the batches of one batched product into fp32 partial results
+// [splits][M][N] in the workspace; a second kernel sums them in chunk order (the same order on every run)
+// and applies the epilogue.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int splits, int64_t mn,
+                                                            int n, float alpha, const float* __restrict__ bias,
+                                                            const float* __restrict__ residual, int act,
+                                                            float* __restrict__ out) {
+  const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i4 >= mn) return;
+  f32x4_t acc = *(const f32x4_t*)(part + i4);
+  for (int z = 1; z < splits; ++z) {
+    const f32x4_t v = *(const f32x4_t*)(part + (int64_t)z * mn + i4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] += v[j];
+  }
+  const int col = (int)(i4 % n);  // n is a multiple of 4: the four values share a row
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    epilogue_store<float>(out, i4 + j, acc[j], alpha, bias ? bias[col + j] : 0.0f, (const char*)residual, act);
+}
+
+// Number of reduction chunks for an fp32 product, 1 = no split.  A split pays when the 64x64 tiles cover less
+// than two rounds of the 256 CUs and the reduction is long (measured: 1024 x 768 x 3072 goes from 64 to 50 us
+// in four chunks, 2048 x 768 x 3072 from 110 to 94 us in two; at K = 768 every split loses to the plain kernel).
+// The smallest chunk count that gives three workgroups per CU is taken, chunks of at least 256.
+inline int splitk_chunks(const GemmParams& p) {
+  const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
+  if (p.K < 1536 || t64 >= 512 || p.M <= 64 || p.N <= 64 || p.N % 4 != 0 || p.c_sm != p.N) return 1;
+  int best = 1;
+  for (int sp = 2; sp <= 8; ++sp) {
+    if (p.K % (sp * 32) != 0 || p.K / sp < 256) continue;
+    if (t64 * sp > 1024) break;
+    best = sp;
+    if (t64 * sp >= 768) break;
+  }
+  return best;
+}
+
+template <int LB>
+int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
+  const int64_t mn = (int64_t)p.M * p.N;
+  void* ws = nullptr;
+  LLC_TRY(get_workspace((size_t)splits * mn * sizeof(float), &ws));
+  GemmParams q = p;
+  q.K = p.K / splits;
+  q.a_sb = (int64_t)q.K * p.a_sk;
+  q.b_sb = (int64_t)q.K * p.b_sk;
+  q.a_sb1 = q.b_sb1 = 0;
+  q.bdiv = 1;
+  q.C = (char*)ws;
+  q.c_sb = mn;
+  q.c_sb1 = 0;
+  q.c_sm = p.N;
+  q.bias = nullptr;
+  q.bias_sb = 0;
+  q.residual = nullptr;
+  q.alpha = 1.0f;
+  q.act = LLC_ACT_NONE;
+  LLC_TRY((launch_tiles<float, kLoadKVec, LB>(q, splits, s)));
+  const int64_t blocks = (mn / 4 + 255) / 256;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const float*)ws, splits, mn, p.N,
+                     p.alpha, (const float*)p.bias, (const float*)p.residual, p.act, (float*)p.C);
+  return check_launch("splitk_reduce_kernel");
+}
+
 template <typename T>
 int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
@@ -769,6 +836,12 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.B);
   const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.N % EPV == 0 && al16(p.B);
   if (batch == 1 && p.M <= 16 && a_kvec && b_kvec) return launch_skinny<T>(p, s);
+  if constexpr (sizeof(T) == 4) {
+    if (batch == 1 && a_kvec && (b_kvec || b_rvec) && al16(p.C) && (!p.residual || al16(p.residual))) {
+      const int splits = splitk_chunks(p);
+      if (splits > 1) return b_kvec ? launch_splitk<kLoadKVec>(p, splits, s) : launch_splitk<kLoadRVec>(p, splits, s);
+    }
+  }
   if constexpr (sizeof(T) == 2) {
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
     if (a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&

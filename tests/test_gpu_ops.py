@@ -461,6 +461,29 @@ def test_matmul_epilogue(ops, oracle):
         assert_close_f32(host(ops.matmul(dev(a), dev(b), epi)), want, "epilogue " + act)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 192, 2048), (200, 132, 1536), (448, 768, 3072)])
+def test_matmul_f32_long_reduction_few_tiles(ops, oracle, M, N, K):
+    """fp32 products whose reduction is cut into chunks (few output tiles, K >= 1536): the chunk sums are added
+    in a fixed order and the epilogue runs once, after the sum.  Both weight layouts, with and without epilogue."""
+    r = rng(M + N + K)
+    a = r.uniform(-1, 1, (M, K)).astype(np.float32) * 0.25
+    b = r.uniform(-1, 1, (K, N)).astype(np.float32) * 0.25
+    bias = r.standard_normal(N).astype(np.float32)
+    res = r.standard_normal((M, N)).astype(np.float32)
+    base = oracle.matmul(a, b, "mkn")
+    bt = dev(np.ascontiguousarray(b.T))
+    assert_close_f32(host(ops.matmul(dev(a), dev(b))), base, "NN %s" % ((M, N, K),))
+    first = host(ops.matmul(dev(a), bt.t()))
+    assert_close_f32(first, base, "NT %s" % ((M, N, K),))
+    np.testing.assert_array_equal(host(ops.matmul(dev(a), bt.t())), first)  # the same bits on every run
+    for act, alpha in [("none", 1.0), ("relu", 0.5), ("gelu", 0.125)]:
+        want = base * np.float32(alpha) + bias[None, :] + res
+        if act != "none":
+            want = oracle.unary(act, want)
+        epi = ops.Epilogue(alpha=alpha, bias=dev(bias), residual=dev(res), act=act)
+        assert_close_f32(host(ops.matmul(dev(a), bt.t(), epi)), want, "NT epilogue %s %s" % (act, (M, N, K)))
+
+
 @pytest.mark.parametrize("B,M,N,K", [(3, 9, 4, 6), (4, 64, 64, 64), (6, 128, 128, 64), (5, 100, 64, 100), (2, 130, 70, 36)])
 def test_batch_matmul(ops, oracle, B, M, N, K):
     r = rng(B + M + N + K)
