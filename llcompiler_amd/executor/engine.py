@@ -47,6 +47,9 @@ FUSE_ATTENTION = True
 # layout needs no gather arithmetic.  Results keep the layout as strided views (logical shape NCHW), so a chain of
 # convolutions converts once; anything that needs NCHW memory copies back through the usual contiguity path.
 CHANNELS_LAST = True
+# linear layers that read the same rows with weights that are graph inputs (q, k, v projections) run as one
+# product against a stacked copy of the weights
+FUSE_PROJECTIONS = True
 
 
 def _concrete(shape, env):
@@ -253,12 +256,18 @@ class Instance:
             c = cl_copies.get(id(v))
             if c is None:
                 n = t.numel()
-                buf = pool.take(n * t.dtype.itemsize)
-                self.keep.append(buf)
-                nhwc = buf[: n * t.dtype.itemsize].view(t.dtype).view(t.shape[0], t.shape[2], t.shape[3], t.shape[1])
-                call = ops.copy(t.permute(0, 2, 3, 1), out=nhwc, defer=True)
                 root = self._roots.get(t.untyped_storage().data_ptr())
-                if root is not None and root[0] == "in" and id(v) in input_ids:
+                prepared = root is not None and root[0] == "in" and id(v) in input_ids
+                if prepared:
+                    # written ahead of every other call and kept: never a buffer that earlier steps have used
+                    nhwc = torch.empty((t.shape[0], t.shape[2], t.shape[3], t.shape[1]), dtype=t.dtype, device=dev)
+                    self.keep.append(nhwc)
+                else:
+                    buf = pool.take(n * t.dtype.itemsize)
+                    self.keep.append(buf)
+                    nhwc = buf[: n * t.dtype.itemsize].view(t.dtype).view(t.shape[0], t.shape[2], t.shape[3], t.shape[1])
+                call = ops.copy(t.permute(0, 2, 3, 1), out=nhwc, defer=True)
+                if prepared:
                     self._prepare_later(call, root[1])
                 else:
                     self._launch_later(call)
@@ -397,9 +406,108 @@ class Instance:
                 return None
             return u[0], shp[0], shp[1]
 
+        def weight_like(t, shape):
+            """A tensor of the given shape that lies contiguous in a graph input's storage (a parameter)."""
+            if not isinstance(t, torch.Tensor) or tuple(t.shape) != tuple(shape) or not t.is_contiguous():
+                return None
+            root = self._roots.get(t.untyped_storage().data_ptr())
+            return root[1] if root is not None and root[0] == "in" else None
+
+        def fused_projections(st, si):
+            """Several linear layers over the same rows (the q, k and v projections of an attention block) run as one
+            product against the stacked weights: [M,K] x [K, N1+N2+..].  The stacked weight and bias are copies made
+            by the instance's preparation calls; every layer's result is a column slice of the one output."""
+            e = st.attrs["epilogue"]
+            if e["residual"] is not None or e.get("bias_rows") or id(st.output) in out_ids:
+                return False
+            nat = _concrete(st.attrs["natural_shape"], self.env)
+            if len(nat) != 2 or nat[0] == 0:
+                return False
+            x = materialise(val[id(st.inputs[0])])
+            if x.dim() != 2:
+                return False
+            m, kdim = x.shape
+
+            def member(s2):
+                """(weight as [N,K], its input index, bias, its input index) when s2 can join, else None."""
+                e2 = s2.attrs["epilogue"]
+                if s2.kind != "matmul" or id(s2) in skip or id(s2.output) in out_ids or s2.output.dtype != st.output.dtype:
+                    return None
+                if e2["residual"] is not None or e2.get("bias_rows") or e2["act"] != e["act"] or e2["alpha"] != e["alpha"] or \
+                        (e2["bias"] is None) != (e["bias"] is None):
+                    return None
+                n2 = _concrete(s2.attrs["natural_shape"], self.env)
+                if len(n2) != 2 or n2[0] != m or not resolve_early(s2.inputs[0]) or not resolve_early(s2.inputs[1]):
+                    return None
+                x2, w2 = val[id(s2.inputs[0])], val[id(s2.inputs[1])]
+                if not isinstance(x2, torch.Tensor) or not isinstance(w2, torch.Tensor) or x2.data_ptr() != x.data_ptr() or \
+                        tuple(x2.shape) != tuple(x.shape) or x2.stride() != x.stride() or w2.dim() != 2:
+                    return None
+                wi = weight_like(w2.t(), (n2[1], kdim))
+                if wi is None:
+                    return None
+                b2, bi = None, None
+                if e2["bias"] is not None:
+                    if not resolve_early(e2["bias"]):
+                        return None
+                    b2 = val[id(e2["bias"])]
+                    b2 = b2.reshape(-1) if isinstance(b2, torch.Tensor) and b2.is_contiguous() else None
+                    bi = weight_like(b2, (n2[1],))
+                    if bi is None:
+                        return None
+                try:
+                    # the result will be a column slice (row pitch > N): its shape must be a view of that
+                    torch.empty_strided((m, n2[1]), (n2[1] + 16, 1), dtype=x.dtype, device="meta").view(
+                        _concrete(s2.output.shape, self.env))
+                except RuntimeError:
+                    return None
+                return w2.t(), wi, b2, bi, n2[1]
+
+            group = []
+            for s2 in [st] + [s for s in steps[si + 1: si + 1 + 24] if s.kind == "matmul"]:
+                mem = member(s2)
+                if mem is not None:
+                    group.append((s2, mem))
+                elif s2 is st:
+                    return False
+            if len(group) < 2:
+                return False
+            dt, isz = st.output.dtype, st.output.dtype.itemsize
+            ntot = sum(mem[4] for _, mem in group)
+            if (ntot * isz) % 16 or any((mem[4] * isz) % 16 for _, mem in group):
+                return False
+            # written by the preparation calls, ahead of every other call: never a buffer of the reuse pool
+            wcat = torch.empty((ntot, kdim), dtype=dt, device=dev)
+            bcat = torch.empty((ntot,), dtype=dt, device=dev) if e["bias"] is not None else None
+            self.keep.append((wcat, bcat))
+            obuf = pool.take(m * ntot * isz)
+            owner[id(st.output)] = obuf
+            cat = obuf[: m * ntot * isz].view(dt).view(m, ntot)
+            off = 0
+            for s2, (w2, wi, b2, bi, n2) in group:
+                self._prepare_later(ops.copy(w2, out=wcat[off:off + n2], defer=True), wi)
+                if bcat is not None:
+                    self._prepare_later(ops.copy(b2, out=bcat[off:off + n2], defer=True), bi)
+                val[id(s2.output)] = cat[:, off:off + n2].view(_concrete(s2.output.shape, self.env))
+                rid = id(s2.output)
+                last_use[id(st.output)] = max(last_use.get(id(st.output), si), last_use.get(rid, si))
+                if s2 is not st:
+                    skip.add(id(s2))
+                off += n2
+            epi = None
+            if bcat is not None or e["act"] or e["alpha"] != 1.0:
+                epi = ops.Epilogue(alpha=e["alpha"], bias=bcat, residual=None, act=e["act"] or "none")
+            self._launch_later(ops.matmul(x, wcat.t(), epi, out=cat, defer=True))
+            return True
+
         for si, st in enumerate(steps):
             k = st.kind
             if id(st) in skip:
+                continue
+            if k == "matmul" and FUSE_PROJECTIONS and fused_projections(st, si):
+                for buf in temps:
+                    pool.give(buf)
+                del temps[:]
                 continue
             if k == "batch_matmul" and FUSE_ATTENTION and fused_attention(st):
                 for buf in temps:

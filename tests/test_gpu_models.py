@@ -352,6 +352,38 @@ def test_training_mode_with_eager_fallbacks(which):
     assert kinds.count("matmul") >= 3 and len(comp.engines) >= 2
 
 
+def test_projections_of_the_same_rows_run_as_one_product():
+    """The q, k and v layers of every attention block read the same rows: one product against stacked copies of
+    their weights and biases (made by preparation calls, redone when a weight is written), each result a column
+    slice of the one output.  Three layers at 576 rows: an intermediate of the first layers has exactly the size
+    of a stacked weight, which must nevertheless not share its buffer."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.executor import engine as E
+    from llcompiler_amd.test_models import BertEncoder, make_bert_inputs
+    bert = BertEncoder(layers=3).eval().cuda()
+    xb, mb = (t.cuda() for t in make_bert_inputs(3, 192))
+    with torch.no_grad():
+        want = bert(xb, mb).cpu().numpy()
+        cm = compile_module(bert, (xb, mb))
+        got = cm(xb, mb)
+        inst = list(cm.engine.instances.values())[0]
+        names = [c.fn.__name__ for c in inst.calls]
+        assert names.count("llc_hip_matmul") == 4 * 3 and len(inst.prep_calls) == 6 * 3
+        assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, "bert, stacked q/k/v weights")
+        E.FUSE_PROJECTIONS = False
+        try:
+            plain = compile_module(bert, (xb, mb))
+            ref = plain(xb, mb)
+            assert [c.fn.__name__ for c in list(plain.engine.instances.values())[0].calls].count("llc_hip_matmul") == 6 * 3
+        finally:
+            E.FUSE_PROJECTIONS = True
+        assert_close(got.cpu().numpy(), ref.cpu().numpy(), F32_RTOL, F32_ATOL, "stacked against separate products")
+        assert torch.equal(cm(xb, mb), got)
+        bert.layers[1].attn.k.weight.mul_(1.5)   # in place: the stacked copy must follow
+        bert.layers[2].attn.v.bias.add_(0.25)
+        assert_close(cm(xb, mb).cpu().numpy(), bert(xb, mb).cpu().numpy(), F32_RTOL, F32_ATOL, "after writing a weight and a bias")
+
+
 def test_channels_last_weight_copies_follow_the_weights():
     """ResNet convolutions run on channels-last copies of their weights, made by preparation calls that run again
     when a weight is written in place or replaced; the stem (3 channels) and everything else stay NCHW."""
