@@ -97,7 +97,9 @@ typedef struct llc_epilogue {
  * fp32 accumulate.  f32, bf16 or f16 operands (all three the same type).  Either operand may be a
  * transposed view (stride[0] == 1), which is how llh.transpose{perms=[1,0]} of a weight
  * (llcompiler/importer/fx_op_translate/transpose.py:39-48) is consumed without a copy.
- * `epi` may be NULL. */
+ * `epi` may be NULL.  fp32 products with a long reduction and few output tiles sum the reduction in
+ * chunks through the library's per-device scratch buffer (grown on demand by this call); the order
+ * of the sum is fixed, so results are the same bits on every run. */
 int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                    void* stream);
 
