@@ -104,3 +104,49 @@ def test_syntax_errors_are_reported():
         parse_llh('func.func @main() -> () { %0 = "llh.abs"(%nope) : (tensor<2xf32>) -> tensor<2xf32> return }')
     with pytest.raises(NotImplementedError):
         parse_llh('func.func @main(%a: tensor<2xf32>) -> () { %0 = "stablehlo.abs"(%a) : (tensor<2xf32>) -> tensor<2xf32> return }')
+
+
+LINEAR_RELU = '''
+func.func @main(%x: tensor<8x784xf32>, %w: tensor<512x784xf32>, %b: tensor<512xf32>, %w2: tensor<10x512xf32>) -> tensor<8x10xf32> attributes {entrance} {
+  %wt = "llh.transpose"(%w) <{perms = array<i64: 1, 0>}> : (tensor<512x784xf32>) -> tensor<784x512xf32>
+  %0 = "llh.matmul"(%x, %wt) : (tensor<8x784xf32>, tensor<784x512xf32>) -> tensor<8x512xf32>
+  %c1 = "llh.constant"() <{value = 1 : i64}> : () -> i64
+  %c512 = "llh.constant"() <{value = 512 : i64}> : () -> i64
+  %br = "llh.reshape"(%b, %c1, %c512) : (tensor<512xf32>, i64, i64) -> tensor<1x512xf32>
+  %1 = "llh.add"(%0, %br) : (tensor<8x512xf32>, tensor<1x512xf32>) -> tensor<8x512xf32>
+  %2 = "llh.relu"(%1) : (tensor<8x512xf32>) -> tensor<8x512xf32>
+  %w2t = "llh.transpose"(%w2) <{perms = array<i64: 1, 0>}> : (tensor<10x512xf32>) -> tensor<512x10xf32>
+  %3 = "llh.matmul"(%2, %w2t) : (tensor<8x512xf32>, tensor<512x10xf32>) -> tensor<8x10xf32>
+  %4 = "llh.exp"(%3) : (tensor<8x10xf32>) -> tensor<8x10xf32>
+  %5 = "llh.abs"(%4) : (tensor<8x10xf32>) -> tensor<8x10xf32>
+  return %5 : tensor<8x10xf32>
+}
+'''
+
+
+def test_llh_plan_tool_prints_the_fused_plan(tmp_path, capsys):
+    """The stand-in for `llc-opt ... | FileCheck`: text in, kernel plan out, checked line by line."""
+    from llcompiler_amd.llh import plan_tool
+    f = tmp_path / "linear.mlir"
+    f.write_text(LINEAR_RELU)
+    assert plan_tool.main([str(f)]) == 0
+    lines = [l.strip() for l in capsys.readouterr().out.splitlines()]
+    assert lines[0] == "plan(%x: tensor<8x784xf32>, %w: tensor<512x784xf32>, %b: tensor<512xf32>, %w2: tensor<10x512xf32>) {"
+    mm = [l for l in lines if "= matmul(" in l]
+    assert len(mm) == 2 and mm[0].endswith("{bias=%b, act=relu} : tensor<8x512xf32>") and mm[0].split("(")[1].startswith("%x, ")
+    assert mm[1].endswith(": tensor<8x10xf32>") and "{" not in mm[1]
+    assert any(l.split(" = ")[1].startswith("ew[exp abs](") for l in lines if " = " in l)
+    assert not any("= ew[add" in l or "= ew[relu" in l for l in lines)      # both went into the first product
+    assert lines[-2].startswith("return %") and lines[-1] == "}"
+    # --emit llh prints the graph back in the input syntax, and that text plans the same way
+    assert plan_tool.main([str(f), "--emit", "llh"]) == 0
+    again = tmp_path / "again.mlir"
+    again.write_text(capsys.readouterr().out)
+    assert plan_tool.main([str(again)]) == 0
+    assert [l.strip() for l in capsys.readouterr().out.splitlines()] == lines
+    # one of several functions, as in the reference's split test files
+    multi = tmp_path / "multi.mlir"
+    multi.write_text(CONV_AND_SHAPES)
+    assert plan_tool.main([str(multi), "--func", "conv_nchw_fchw"]) == 0
+    out = capsys.readouterr().out
+    assert "= conv(%arg1, %arg0) : tensor<?x4x?x?xf32>" in out
