@@ -311,6 +311,16 @@ int64_t llc_plan_num_params(const llc_plan_t* plan);
  * pointers.  Extents must equal the declared ones and strides too (LLC_ERR_SHAPE / LLC_ERR_LAYOUT
  * otherwise: the caller then picks or records the plan for that binding). */
 int llc_hip_run(llc_plan_t* plan, void* const* params, void* stream);
+/* Plans on disk.  The reference's compile step leaves a shared object with the weights baked in
+ * (src/Compiler/Compiler.cpp:306-330: the object is named after a hash of the module text) that a later process
+ * loads and runs (src/Compiler/Execution.cpp:21-66).  llc_plan_save writes a recorded plan: the declared tensors,
+ * the expected symbol values, the steps, and the device memory the steps address outside the declared tensors
+ * (constants and weights with their contents as they are now; memory that every run writes before it reads
+ * it, i.e. intermediates, only by size).  llc_plan_load gives a plan of its own memory on the current device
+ * that llc_hip_run replays like the original.  A file written by another ABI version is refused
+ * (LLC_ERR_UNSUPPORTED), a truncated or malformed one LLC_ERR_BAD_ARG. */
+int llc_plan_save(llc_plan_t* plan, const char* path);
+int llc_plan_load(const char* path, llc_plan_t** plan);
 /* The reference's loader resolves a symbol of type void(void**) (Execution.cpp:12-16).  llc_hip_entry has
  * that type and runs the plan bound with llc_hip_bind_entry (one per process; NULL unbinds) on the stream
  * given there; like the reference's entry it returns nothing and logs failures

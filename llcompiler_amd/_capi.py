@@ -79,7 +79,7 @@ EXPORTS = [
     "llc_plan_create", "llc_plan_destroy", "llc_plan_alloc", "llc_plan_upload", "llc_plan_declare_io",
     "llc_plan_expect_symbols", "llc_plan_begin", "llc_plan_end", "llc_plan_num_steps", "llc_plan_num_params",
     "llc_hip_run", "llc_hip_bind_entry", "llc_hip_entry", "llc_hip_entry_status",
-    "llc_npy_info", "llc_plan_load_npy",
+    "llc_npy_info", "llc_plan_load_npy", "llc_plan_save", "llc_plan_load",
 ]
 
 
@@ -145,6 +145,8 @@ def lib():
         szp = P(ctypes.c_size_t)
         L.llc_npy_info.argtypes = [ctypes.c_char_p, ctypes.c_int, szp, szp, szp, szp]
         L.llc_plan_load_npy.argtypes = [vp, ctypes.c_char_p, ctypes.c_int, T, szp, szp]
+        L.llc_plan_save.argtypes = [vp, ctypes.c_char_p]
+        L.llc_plan_load.argtypes = [ctypes.c_char_p, P(vp)]
         _lib = L
     return _lib
 

@@ -8,9 +8,12 @@
 // the params block carries for the tensor; every other address (weights uploaded into the plan, its arena,
 // caller-owned constants) is replayed as recorded.  A replay allocates nothing and makes no host-device
 // synchronisation: it is the list of kernel launches, in order, on the given stream.
+#include <algorithm>
+#include <cstdio>
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <utility>
 #include <vector>
 
 #include "common.hpp"
@@ -539,3 +542,320 @@ extern "C" void llc_hip_entry(void** params) {
 }
 
 extern "C" int llc_hip_entry_status(void) { return g_entry_status; }
+
+// ---- plans on disk --------------------------------------------------------------------------------------
+// The reference's compile step leaves a shared object with the weights baked in, which Execution loads and
+// runs later (src/Compiler/Compiler.cpp:306-330, src/Compiler/Execution.cpp:21-66).  The counterpart here is
+// a plan file: the recorded steps, the declared tensors, and the device memory the steps address outside
+// those tensors.  That memory is cut into regions (maximal runs of overlapping operand ranges); a region
+// whose every byte is written by a step before a step reads it is scratch and only its size is kept, any
+// other region (constants, weights uploaded into the plan) is stored with its contents as they are when the
+// plan is saved.  Loading allocates the regions in memory owned by the new plan, at the same address modulo
+// 256, and points the operands into them.
+namespace {
+
+constexpr char kPlanMagic[8] = {'L', 'L', 'C', 'P', 'L', 'A', 'N', '1'};
+
+struct Region {
+  char* lo;
+  char* hi;
+  bool keep = false;                                // contents are part of the plan
+  std::vector<std::pair<char*, char*>> written;     // ranges known to be fully written by earlier steps
+};
+
+struct Writer {
+  FILE* f;
+  bool ok = true;
+  void raw(const void* p, size_t n) {
+    if (ok && n && fwrite(p, 1, n, f) != n) ok = false;
+  }
+  template <typename T>
+  void pod(const T& v) { raw(&v, sizeof(T)); }
+  void u64(uint64_t v) { pod(v); }
+  void i64(int64_t v) { pod(v); }
+};
+
+struct Reader {
+  FILE* f;
+  bool ok = true;
+  void raw(void* p, size_t n) {
+    if (ok && n && fread(p, 1, n, f) != n) ok = false;
+  }
+  template <typename T>
+  void pod(T& v) { raw(&v, sizeof(T)); }
+  uint64_t u64() {
+    uint64_t v = 0;
+    pod(v);
+    return v;
+  }
+  int64_t i64() {
+    int64_t v = 0;
+    pod(v);
+    return v;
+  }
+};
+
+void write_operand_shape(Writer& w, const Operand& o) {
+  w.u64(o.present ? 1 : 0);
+  if (!o.present) return;
+  w.u64(o.t.type);
+  w.u64(o.t.rank);
+  for (size_t i = 0; i < o.t.rank; ++i) w.u64(o.size[i]), w.u64(o.stride[i]);
+}
+
+bool read_operand_shape(Reader& r, Operand& o) {
+  o.present = r.u64() != 0;
+  if (!o.present) return r.ok;
+  memset(&o.t, 0, sizeof(o.t));
+  o.t.type = (size_t)r.u64();
+  o.t.rank = (size_t)r.u64();
+  if (!r.ok || o.t.rank > LLC_MAX_RANK || dtype_size(o.t.type) == 0) return false;
+  for (size_t i = 0; i < o.t.rank; ++i) o.size[i] = (size_t)r.u64(), o.stride[i] = (size_t)r.u64();
+  o.t.size = o.size;
+  o.t.stride = o.stride;
+  return r.ok;
+}
+
+bool covered(const Region& g, char* lo, char* hi) {
+  // written ranges are few (one per intermediate): a linear walk over the sorted, merged list
+  for (const auto& w : g.written)
+    if (w.first <= lo && hi <= w.second) return true;
+  return false;
+}
+
+void add_written(Region& g, char* lo, char* hi) {
+  g.written.emplace_back(lo, hi);
+  std::sort(g.written.begin(), g.written.end());
+  std::vector<std::pair<char*, char*>> merged;
+  for (const auto& w : g.written) {
+    if (!merged.empty() && w.first <= merged.back().second) merged.back().second = std::max(merged.back().second, w.second);
+    else merged.push_back(w);
+  }
+  g.written.swap(merged);
+}
+
+// index of the last operand of a step that is written (the result); everything before it is read
+inline size_t result_index(const Step& s) { return s.opnd.size() - 1; }
+
+}  // namespace
+
+extern "C" int llc_plan_save(llc_plan_t* p, const char* path) {
+  if (!p || !path) return set_error(LLC_ERR_BAD_ARG, "plan_save: null argument");
+  if (p->state != kReady) return set_error(LLC_ERR_BAD_ARG, "plan_save: the plan has not been recorded (begin .. end)");
+  LLC_TRY(check_device(p, "plan_save"));
+  std::lock_guard<std::mutex> lock(p->mu);
+  // regions of fixed-address memory
+  std::vector<std::pair<char*, char*>> spans;
+  for (const Step& s : p->steps)
+    for (const Operand& o : s.opnd)
+      if (o.present && o.io < 0 && o.t.data && o.span_bytes()) spans.emplace_back((char*)o.t.data, (char*)o.t.data + o.span_bytes());
+  std::sort(spans.begin(), spans.end());
+  std::vector<Region> regions;
+  for (const auto& sp : spans) {
+    if (!regions.empty() && sp.first < regions.back().hi) regions.back().hi = std::max(regions.back().hi, sp.second);
+    else regions.push_back(Region{sp.first, sp.second});
+  }
+  auto region_of = [&](const char* a) -> int {
+    size_t lo = 0, hi = regions.size();
+    while (lo < hi) {
+      const size_t mid = (lo + hi) / 2;
+      if (regions[mid].hi <= a) lo = mid + 1;
+      else hi = mid;
+    }
+    return (lo < regions.size() && regions[lo].lo <= a) ? (int)lo : -1;
+  };
+  // which regions are read before they are written
+  for (const Step& s : p->steps) {
+    const size_t res = result_index(s);
+    for (size_t i = 0; i < s.opnd.size(); ++i) {
+      const Operand& o = s.opnd[i];
+      if (!o.present || o.io >= 0 || !o.t.data || !o.span_bytes()) continue;
+      Region& g = regions[region_of((char*)o.t.data)];
+      char* lo = (char*)o.t.data;
+      char* hi = lo + o.span_bytes();
+      if (i != res) {
+        if (!covered(g, lo, hi)) g.keep = true;
+      } else {
+        size_t n = dtype_size(o.t.type);
+        for (size_t d = 0; d < o.t.rank; ++d) n *= o.size[d];
+        if (n == o.span_bytes()) add_written(g, lo, hi);  // a dense result covers its range; a strided one may leave gaps
+      }
+    }
+  }
+  LLC_HIP_TRY(hipDeviceSynchronize());
+  FILE* f = fopen(path, "wb");
+  if (!f) return set_error(LLC_ERR_BAD_ARG, "plan_save: cannot open %s for writing", path);
+  Writer w{f};
+  w.raw(kPlanMagic, 8);
+  w.u64((uint64_t)LLC_HIP_ABI_VERSION);
+  w.u64(p->io.size());
+  w.u64(p->n_inputs);
+  for (const Io& io : p->io) {
+    write_operand_shape(w, io.like);
+    w.u64(io.output ? 1 : 0);
+  }
+  w.u64(p->symbols.size());
+  for (int64_t v : p->symbols) w.i64(v);
+  w.u64(p->overlaps.size());
+  for (const Overlap& ov : p->overlaps) w.i64(ov.first), w.i64(ov.second), w.i64(ov.diff);
+  w.u64(regions.size());
+  std::vector<char> host;
+  for (const Region& g : regions) {
+    const size_t bytes = (size_t)(g.hi - g.lo);
+    w.u64(bytes);
+    w.u64((uint64_t)((uintptr_t)g.lo % 256));
+    w.u64(g.keep ? 1 : 0);
+    if (g.keep) {
+      host.resize(bytes);
+      const hipError_t e = hipMemcpy(host.data(), g.lo, bytes, hipMemcpyDeviceToHost);
+      if (e != hipSuccess) {
+        fclose(f);
+        return set_error(LLC_ERR_HIP, "plan_save: reading %zu bytes of device memory failed: %s", bytes, hipGetErrorString(e));
+      }
+      w.raw(host.data(), bytes);
+    }
+  }
+  w.u64(p->steps.size());
+  for (const Step& s : p->steps) {
+    w.i64(s.op);
+    w.u64(s.has_epi ? 1 : 0);
+    w.pod(s.alpha);
+    w.i64(s.act);
+    w.i64(s.kind);
+    w.pod(s.eps);
+    w.u64(s.n_ints);
+    for (size_t i = 0; i < s.n_ints; ++i) w.i64(s.ints[i]);
+    w.pod(s.conv);
+    w.pod(s.pool);
+    w.u64(s.prog ? 1 : 0);
+    if (s.prog) w.pod(*s.prog);
+    w.u64(s.opnd.size());
+    for (const Operand& o : s.opnd) {
+      write_operand_shape(w, o);
+      if (!o.present) continue;
+      w.i64(o.io);
+      w.i64(o.delta);
+      int reg = -1;
+      int64_t off = 0;
+      if (o.io < 0 && o.t.data && o.span_bytes()) {
+        reg = region_of((char*)o.t.data);
+        off = (char*)o.t.data - regions[reg].lo;
+      }
+      w.i64(reg);
+      w.i64(off);
+    }
+  }
+  const bool ok = w.ok && fclose(f) == 0;
+  if (!ok) return set_error(LLC_ERR_BAD_ARG, "plan_save: writing %s failed", path);
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
+  if (!path || !out) return set_error(LLC_ERR_BAD_ARG, "plan_load: null argument");
+  *out = nullptr;
+  FILE* f = fopen(path, "rb");
+  if (!f) return set_error(LLC_ERR_BAD_ARG, "plan_load: cannot open %s", path);
+  struct Closer {
+    FILE* f;
+    ~Closer() { fclose(f); }
+  } closer{f};
+  Reader r{f};
+  char magic[8] = {0};
+  r.raw(magic, 8);
+  if (!r.ok || memcmp(magic, kPlanMagic, 8) != 0) return set_error(LLC_ERR_BAD_ARG, "plan_load: %s is not a plan file", path);
+  const uint64_t abi = r.u64();
+  if (abi != (uint64_t)LLC_HIP_ABI_VERSION)
+    return set_error(LLC_ERR_UNSUPPORTED, "plan_load: %s was written by ABI version %llu, this library is version %d", path,
+                     (unsigned long long)abi, LLC_HIP_ABI_VERSION);
+  llc_plan_t* p = nullptr;
+  LLC_TRY(llc_plan_create(&p));
+  std::unique_ptr<llc_plan_t, int (*)(llc_plan_t*)> guard(p, llc_plan_destroy);
+  auto bad = [&](const char* what) { return set_error(LLC_ERR_BAD_ARG, "plan_load: %s: %s", path, what); };
+  const uint64_t n_io = r.u64();
+  p->n_inputs = (size_t)r.u64();
+  if (!r.ok || n_io > (1u << 20) || p->n_inputs > n_io) return bad("truncated or corrupt header");
+  p->io.resize((size_t)n_io);
+  for (Io& io : p->io) {
+    if (!read_operand_shape(r, io.like) || !io.like.present) return bad("malformed tensor declaration");
+    io.like.t.size = io.like.t.stride = nullptr;  // as after llc_plan_declare_io: only like.size / like.stride are read
+    io.output = r.u64() != 0;
+  }
+  const uint64_t n_sym = r.u64();
+  if (!r.ok || n_sym > (1u << 20)) return bad("truncated symbol list");
+  p->symbols.resize((size_t)n_sym);
+  for (int64_t& v : p->symbols) v = r.i64();
+  const uint64_t n_ov = r.u64();
+  if (!r.ok || n_ov > (1u << 20)) return bad("truncated overlap list");
+  for (uint64_t i = 0; i < n_ov; ++i) {
+    Overlap ov;
+    ov.first = (int)r.i64(), ov.second = (int)r.i64(), ov.diff = r.i64();
+    if (!r.ok || ov.first < 0 || ov.second < 0 || (uint64_t)ov.first >= n_io || (uint64_t)ov.second >= n_io) return bad("malformed overlap entry");
+    p->overlaps.push_back(ov);
+  }
+  const uint64_t n_reg = r.u64();
+  if (!r.ok || n_reg > (1u << 24)) return bad("truncated region list");
+  std::vector<std::pair<char*, size_t>> regions;
+  std::vector<char> host;
+  for (uint64_t i = 0; i < n_reg; ++i) {
+    const uint64_t bytes = r.u64(), mis = r.u64(), keep = r.u64();
+    if (!r.ok || mis >= 256 || bytes > ((uint64_t)1 << 40)) return bad("malformed region entry");
+    void* m = nullptr;
+    LLC_TRY(llc_plan_alloc(p, (size_t)(bytes + mis), &m));
+    char* base = (char*)m + mis;
+    if (keep) {
+      host.resize((size_t)bytes);
+      r.raw(host.data(), (size_t)bytes);
+      if (!r.ok) return bad("truncated region contents");
+      if (bytes) LLC_HIP_TRY(hipMemcpy(base, host.data(), (size_t)bytes, hipMemcpyHostToDevice));
+    } else if (bytes) {
+      LLC_HIP_TRY(hipMemset(base, 0, (size_t)bytes));
+    }
+    regions.emplace_back(base, (size_t)bytes);
+  }
+  const uint64_t n_steps = r.u64();
+  if (!r.ok || n_steps > (1u << 24)) return bad("truncated step list");
+  p->steps.resize((size_t)n_steps);
+  for (Step& s : p->steps) {
+    s.op = (int)r.i64();
+    s.has_epi = r.u64() != 0;
+    r.pod(s.alpha);
+    s.act = (int)r.i64();
+    s.kind = (int)r.i64();
+    r.pod(s.eps);
+    s.n_ints = (size_t)r.u64();
+    if (!r.ok || s.n_ints > sizeof(s.ints) / sizeof(s.ints[0]) || s.op < kMatmul || s.op > kAttention) return bad("malformed step");
+    for (size_t i = 0; i < s.n_ints; ++i) s.ints[i] = r.i64();
+    llc_conv_attrs conv;
+    llc_pool_attrs pool;
+    r.pod(conv);
+    r.pod(pool);
+    if (s.op == kMaxPool) s.pool = pool;
+    else s.conv = conv;
+    if (r.u64()) {
+      s.prog.reset(new llc_ew_program);
+      r.pod(*s.prog);
+    }
+    const uint64_t n_op = r.u64();
+    if (!r.ok || n_op == 0 || n_op > LLC_EW_MAX_INPUTS + 8) return bad("malformed operand list");
+    if ((s.op == kElementwise) != (s.prog != nullptr)) return bad("elementwise step without a program (or a program elsewhere)");
+    s.opnd.resize((size_t)n_op);
+    for (Operand& o : s.opnd) {
+      if (!read_operand_shape(r, o)) return bad("malformed operand");
+      if (!o.present) continue;
+      o.io = (int)r.i64();
+      o.delta = r.i64();
+      const int64_t reg = r.i64(), off = r.i64();
+      if (!r.ok || o.io >= (int64_t)n_io) return bad("operand bound to an undeclared tensor");
+      if (o.io < 0 && reg >= 0) {
+        if ((uint64_t)reg >= regions.size() || off < 0 || (uint64_t)off + o.span_bytes() > regions[(size_t)reg].second)
+          return bad("operand outside its memory region");
+        o.t.data = o.t.base = regions[(size_t)reg].first + off;
+      }
+    }
+  }
+  if (!r.ok) return bad("truncated file");
+  p->state = kReady;
+  p->bound.assign(p->io.size(), nullptr);
+  *out = guard.release();
+  return LLC_OK;
+}

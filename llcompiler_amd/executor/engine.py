@@ -872,6 +872,46 @@ class Torch_ExecutionEngine(ExecutionEngine):
             env.setdefault(name, inputs[i].shape[d])
         return env
 
+    def save_plan(self, path, *args):
+        """Runs the graph for `args` (so that the plan for those extents exists and is recorded), writes that plan
+        to `path` and a description of its parameter block to `path + ".json"`: the tensors in block order
+        (inputs, then outputs) with type, shape and strides, the symbol values it is specialised for, and the
+        output views.  Another process loads the file with `Plan.load` (or `llc_plan_load` from C) and runs it
+        with a block of that layout: the counterpart of the reference's compile-to-shared-object followed by
+        `ExecutionEngine.load` (src/Compiler/Compiler.cpp:306-330, llcompiler/executor/engine.py:15-26).  Weights
+        that are graph inputs stay parameters of the block; weights taken from .npy files are part of the file.
+        Returns the description."""
+        import json
+        if not USE_PLAN or USE_GRAPHS:
+            raise RuntimeError("save_plan needs the recorded-plan execution path (engine.USE_PLAN)")
+        self.run(*args)
+        self.run(*args)
+        tensors = [a for a in self.trans_to_tensor(*args)]
+        env = self.bind_symbols(args, tensors)
+        device = tensors[0].device if tensors else torch.device("cuda", torch.cuda.current_device())
+        key = (tuple(sorted(env.items())), tuple((tuple(t.shape), tuple(t.stride())) for t in tensors), device.index,
+               _alias_signature(tensors))
+        inst = self.instances[key]
+        if inst._plan is None:
+            raise RuntimeError("the instance has no recorded plan")
+        if inst.prep_calls:
+            torch.cuda.synchronize(device)  # prepared weight copies are part of the file: they must be complete
+        inst._plan.save(path)
+
+        def describe(t):
+            return {"dtype": str(t.dtype).replace("torch.", ""), "shape": list(t.shape), "stride": list(t.stride())}
+        meta = {"symbols": {k: int(v) for k, v in sorted(env.items())},
+                "inputs": [dict(describe(t), name=v.name) for v, t in zip(self.graph.inputs, tensors)],
+                "outputs": [{"dtype": str(d).replace("torch.", ""), "shape": list(s), "stride": list(torch.empty(s, device="meta").stride())}
+                            for s, d in inst.out_specs],
+                "results": [list(spec) if spec[0] != "tensor" else
+                            {"output": spec[1], "shape": list(spec[2]), "stride": list(spec[3]), "offset": spec[4]}
+                            for spec in inst.output_plan],
+                "steps": int(inst._plan.num_steps)}
+        with open(str(path) + ".json", "w") as f:
+            json.dump(meta, f, indent=1)
+        return meta
+
     def bind_leading(self, tensors):
         """run() with `tensors` fixed as the first arguments (the parameters an ahead-of-time compiled module
         passes with every call): their part of the call signature is computed once, not per call."""

@@ -44,13 +44,27 @@ class ParamBlock:
 class Plan:
     """Owns an llc_plan_t.  Usage: declare the tensors of the block, record the kernel calls once, run."""
 
-    def __init__(self):
+    def __init__(self, _handle=None):
         self._lib = C.lib()
-        h = ctypes.c_void_p()
-        C.check(self._lib.llc_plan_create(ctypes.byref(h)))
+        h = _handle
+        if h is None:
+            h = ctypes.c_void_p()
+            C.check(self._lib.llc_plan_create(ctypes.byref(h)))
         self.handle = h
         self._refs = []
         weakref.finalize(self, self._lib.llc_plan_destroy, h)
+
+    def save(self, path):
+        """Writes the recorded plan to `path`: steps, declared tensors, and the device memory the steps address
+        outside those tensors (constants with their contents, intermediates by size)."""
+        C.check(self._lib.llc_plan_save(self.handle, os.fsencode(path)))
+
+    @classmethod
+    def load(cls, path):
+        """A plan read back from a file written by `save`, with memory of its own on the current device."""
+        h = ctypes.c_void_p()
+        C.check(C.lib().llc_plan_load(os.fsencode(path), ctypes.byref(h)))
+        return cls(_handle=h)
 
     def declare_io(self, t, is_output):
         r = C.tensor_ref(t)

@@ -147,3 +147,24 @@ def test_npy_header_parser_reads_what_np_save_writes(tmp_path):
     junk = str(tmp_path / "junk.npy")
     open(junk, "wb").write(b"not a numpy file at all")
     assert _npy_info(junk)[0] == C.ERR_BAD_ARG and _npy_info(str(tmp_path / "missing.npy"))[0] == C.ERR_BAD_ARG
+
+
+def test_plan_files_are_checked_before_anything_touches_a_device(tmp_path):
+    """llc_plan_load refuses what is not a plan file (missing, wrong magic, another ABI version) and
+    llc_plan_save refuses null arguments: all of it host logic."""
+    import ctypes
+    import struct
+    from llcompiler_amd import _capi as C
+    L = C.lib()
+    h = ctypes.c_void_p()
+    assert L.llc_plan_load(str(tmp_path / "missing.llcplan").encode(), ctypes.byref(h)) == C.ERR_BAD_ARG
+    assert b"cannot open" in L.llc_hip_last_error()
+    junk = tmp_path / "junk.llcplan"
+    junk.write_bytes(b"not a plan at all, just bytes")
+    assert L.llc_plan_load(str(junk).encode(), ctypes.byref(h)) == C.ERR_BAD_ARG and not h.value
+    assert b"not a plan file" in L.llc_hip_last_error()
+    other = tmp_path / "other_abi.llcplan"
+    other.write_bytes(b"LLCPLAN1" + struct.pack("<Q", 10 ** 6))
+    assert L.llc_plan_load(str(other).encode(), ctypes.byref(h)) == C.ERR_UNSUPPORTED and not h.value
+    assert L.llc_plan_save(None, b"x") == C.ERR_BAD_ARG
+    assert L.llc_plan_load(None, ctypes.byref(h)) == C.ERR_BAD_ARG

@@ -310,3 +310,139 @@ def test_models_with_npy_weights_match_models_with_tensor_weights(tmp_path):
         for seed in (1, 2):
             (xs,) = make_encoder_inputs(2, 64, 128, seed=seed, dtype=torch.bfloat16)
             assert torch.equal(ea(xs.cuda()), eb(xs.cuda()))
+
+
+def test_plan_file_round_trip(oracle, tmp_path):
+    """A recorded plan written to a file and read back replays like the original, from memory of its own: the
+    uploaded weights travel with their contents, the hidden layer (written before it is read) only by size."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    rng = np.random.default_rng(11)
+    M, K, H, N = 40, 72, 2048, 24
+    w1 = rng.standard_normal((K, H), dtype=np.float32) * 0.1
+    b1 = rng.standard_normal((H,), dtype=np.float32)
+    w2 = rng.standard_normal((H, N), dtype=np.float32) * 0.1
+    x0 = rng.standard_normal((M, K), dtype=np.float32)
+    plan = Plan()
+    x = torch.from_numpy(x0).cuda()
+    out = torch.empty((M, N), device="cuda")
+    _record_two_layer(plan, x, out, w1, b1, w2, H)
+    path = tmp_path / "two_layer.llcplan"
+    plan.save(path)
+    size = path.stat().st_size
+    weights = w1.nbytes + b1.nbytes + w2.nbytes
+    assert weights < size < weights + 4096, "the file holds the weights and no intermediate (%d bytes)" % size
+    loaded = Plan.load(path)
+    assert loaded.num_steps == 2 and loaded.num_params == 11
+    del plan                                     # the original and its memory go away
+    import gc
+    gc.collect()
+    filler = torch.full((4 * (K * H + H * N),), float("nan"), device="cuda")   # whatever reuses that memory is poison
+    for seed in (3, 4):
+        xs = np.random.default_rng(seed).standard_normal((M, K), dtype=np.float32)
+        x2, out2 = torch.from_numpy(xs).cuda(), torch.zeros((M, N), device="cuda")
+        loaded.run(ParamBlock([x2, out2]), _stream())
+        torch.cuda.synchronize()
+        want = oracle.matmul(oracle.unary("relu", oracle.matmul(xs, w1) + b1), w2)
+        assert_close(out2.cpu().numpy(), want, F32_RTOL, F32_ATOL, "loaded plan, seed %d" % seed)
+    del filler
+    # the loaded plan checks its block like any other
+    with pytest.raises(C.LlcHipError):
+        loaded.run(ParamBlock([torch.zeros((M + 1, K), device="cuda"), torch.zeros((M, N), device="cuda")]), _stream())
+    # files that are not plans
+    junk = tmp_path / "junk.llcplan"
+    junk.write_bytes(b"LLCPLAN1" + bytes(5))
+    with pytest.raises(C.LlcHipError):
+        Plan.load(junk)
+    cut = tmp_path / "cut.llcplan"
+    cut.write_bytes(path.read_bytes()[: size // 2])
+    with pytest.raises(C.LlcHipError):
+        Plan.load(cut)
+
+
+@pytest.mark.parametrize("which", ["encoder_bf16", "resnet"])
+def test_engine_plans_survive_a_file(which, tmp_path):
+    """The plan an engine instance records (fused attention, stacked projections, channels-last convolutions with
+    their prepared weight copies, constants) written to a file and read back gives the engine's result bit for bit."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    from llcompiler_amd.test_models import EncoderBlock, ResNet18Folded, make_encoder_inputs, make_resnet_inputs
+    if which == "resnet":
+        m = ResNet18Folded().eval().cuda()
+        (x,) = make_resnet_inputs(2, 64)
+        x = x.cuda()
+    else:
+        m = EncoderBlock().eval().to(torch.bfloat16).cuda()
+        x = make_encoder_inputs(2, 128)[0].to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        cm = compile_module(m, (x,))
+        cm(x)
+        inst = list(cm.engine.instances.values())[0]
+        seen, run = {}, inst.run
+
+        def spy(inputs):                               # the tensors of the block: lifted parameters, then x
+            seen["inputs"] = list(inputs)
+            return run(inputs)
+        inst.run = spy
+        want = cm(x)                                   # second run: the recorded plan
+        assert inst._plan is not None and seen["inputs"][-1] is x
+        path = tmp_path / (which + ".llcplan")
+        inst._plan.save(path)
+        loaded = Plan.load(path)
+        assert loaded.num_steps == inst._plan.num_steps
+    blk_inputs = seen["inputs"]
+    out = torch.zeros_like(want)
+    loaded.run(ParamBlock(list(blk_inputs) + [out]), _stream())
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    # intermediates are not in the file: it is smaller than the weights' prepared copies plus a margin
+    n_param_bytes = sum(p.numel() * p.element_size() for p in m.parameters())
+    assert path.stat().st_size < n_param_bytes + (4 << 20)
+
+
+_RUN_PLAN_FILE = '''
+import json, sys
+import numpy as np
+import torch
+from llcompiler_amd import _capi as C
+from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+C.init(0)
+path, x_file, out_file = sys.argv[1:4]
+meta = json.load(open(path + ".json"))
+plan = Plan.load(path)
+assert plan.num_steps == meta["steps"]
+x = torch.from_numpy(np.load(x_file)).cuda()
+assert [list(x.shape)] == [i["shape"] for i in meta["inputs"]]
+outs = [torch.empty(o["shape"], dtype=getattr(torch, o["dtype"]), device="cuda") for o in meta["outputs"]]
+plan.run(ParamBlock([x] + outs), C.current_stream(torch.device("cuda", 0)))
+torch.cuda.synchronize()
+np.save(out_file, outs[0].cpu().numpy())
+'''
+
+
+def test_saved_plan_with_baked_weights_runs_in_another_process(tmp_path):
+    """Compile with the weights taken from .npy files, save the plan: the file is self-contained (the weights are
+    part of it, as in the reference's compiled object) and a fresh process that never saw the model gets the same
+    bits from it, given only the input."""
+    import os
+    import subprocess
+    import sys
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    m = MLP().eval().cuda()
+    (x,) = make_mlp_inputs(seed=5)
+    with torch.no_grad():
+        cm = compile_module(m, (x.cuda(),), weights="npy", weight_dir=str(tmp_path / "w"))
+        want = cm(x.cuda()).cpu().numpy()
+        path = str(tmp_path / "mlp.llcplan")
+        meta = cm.engine.save_plan(path, x.cuda())
+    assert len(meta["inputs"]) == 1 and len(meta["outputs"]) == 1 and meta["steps"] == 2
+    n_weight_bytes = sum(p.numel() * 4 for p in m.parameters())
+    assert n_weight_bytes <= os.path.getsize(path) < n_weight_bytes + 8192
+    np.save(tmp_path / "x.npy", x.numpy())
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", _RUN_PLAN_FILE, path, str(tmp_path / "x.npy"), str(tmp_path / "out.npy")],
+                       cwd=root, timeout=110, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    np.testing.assert_array_equal(np.load(tmp_path / "out.npy"), want)
