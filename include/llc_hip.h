@@ -321,6 +321,15 @@ int llc_hip_run(llc_plan_t* plan, void* const* params, void* stream);
  * (LLC_ERR_UNSUPPORTED), a truncated or malformed one LLC_ERR_BAD_ARG. */
 int llc_plan_save(llc_plan_t* plan, const char* path);
 int llc_plan_load(const char* path, llc_plan_t** plan);
+/* What a host needs to run a plan it did not record (the reference's Execution gets the same from the
+ * tensors its caller passes, Execution.cpp:21-45): how many tensors the block holds, and type, rank, extents
+ * and strides of each (index < n_inputs: an input).  `like` is filled with size_out / stride_out as its
+ * arrays (LLC_MAX_RANK entries each) and a null data pointer. */
+int llc_plan_num_io(const llc_plan_t* plan, size_t* n_inputs, size_t* n_outputs);
+int llc_plan_io_info(const llc_plan_t* plan, size_t index, llc_tensor* like, size_t* size_out, size_t* stride_out);
+/* Waits for `stream`, then copies device memory to the host: results for a host that has no GPU runtime of
+ * its own (the counterpart of llc_plan_upload). */
+int llc_hip_download(void* host, const void* device, size_t bytes, void* stream);
 /* The reference's loader resolves a symbol of type void(void**) (Execution.cpp:12-16).  llc_hip_entry has
  * that type and runs the plan bound with llc_hip_bind_entry (one per process; NULL unbinds) on the stream
  * given there; like the reference's entry it returns nothing and logs failures

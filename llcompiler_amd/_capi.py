@@ -80,6 +80,7 @@ EXPORTS = [
     "llc_plan_expect_symbols", "llc_plan_begin", "llc_plan_end", "llc_plan_num_steps", "llc_plan_num_params",
     "llc_hip_run", "llc_hip_bind_entry", "llc_hip_entry", "llc_hip_entry_status",
     "llc_npy_info", "llc_plan_load_npy", "llc_plan_save", "llc_plan_load",
+    "llc_plan_num_io", "llc_plan_io_info", "llc_hip_download",
 ]
 
 
@@ -147,6 +148,9 @@ def lib():
         L.llc_plan_load_npy.argtypes = [vp, ctypes.c_char_p, ctypes.c_int, T, szp, szp]
         L.llc_plan_save.argtypes = [vp, ctypes.c_char_p]
         L.llc_plan_load.argtypes = [ctypes.c_char_p, P(vp)]
+        L.llc_plan_num_io.argtypes = [vp, szp, szp]
+        L.llc_plan_io_info.argtypes = [vp, ctypes.c_size_t, T, szp, szp]
+        L.llc_hip_download.argtypes = [vp, vp, ctypes.c_size_t, vp]
         _lib = L
     return _lib
 

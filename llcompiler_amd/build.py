@@ -20,6 +20,9 @@ LIB = os.path.join(LIB_DIR, "libllc_hip.so")
 # exports `main(void**)`, the symbol the reference's loader resolves, forwarding to libllc_hip.so
 ENTRY_LIB = os.path.join(LIB_DIR, "libllc_entry.so")
 ENTRY_SRC = os.path.join(CSRC, "entry_main.c")
+# a host in plain C that loads a plan file and runs it through the C-ABI alone
+RUN_PLAN = os.path.join(LIB_DIR, "llc_run_plan")
+RUN_PLAN_SRC = os.path.join(CSRC, "run_plan_main.c")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -52,8 +55,8 @@ def build(force=True, jobs=None, verbose=False):
     srcs = sources()
     if not srcs:
         raise RuntimeError("no HIP sources under %s" % CSRC)
-    deps = srcs + [ENTRY_SRC] + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
-    if not force and os.path.exists(LIB) and os.path.exists(ENTRY_LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(d) for d in deps):
+    deps = srcs + [ENTRY_SRC, RUN_PLAN_SRC] + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
+    if not force and os.path.exists(LIB) and os.path.exists(ENTRY_LIB) and os.path.exists(RUN_PLAN) and all(os.path.getmtime(LIB) >= os.path.getmtime(d) for d in deps):
         return LIB
     jobs = jobs or min(8, os.cpu_count() or 1, len(srcs))
     with concurrent.futures.ThreadPoolExecutor(jobs) as ex:
@@ -72,6 +75,11 @@ def build(force=True, jobs=None, verbose=False):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("building %s failed:\n%s" % (ENTRY_LIB, r.stderr))
+    cmd = ["gcc", "-O2", "-std=c11", "-Wall", "-I", os.path.join(ROOT, "include"), RUN_PLAN_SRC, "-o", RUN_PLAN,
+           "-L", LIB_DIR, "-lllc_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (RUN_PLAN, r.stderr))
     return LIB
 
 

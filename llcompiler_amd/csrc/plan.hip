@@ -859,3 +859,31 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
   *out = guard.release();
   return LLC_OK;
 }
+
+// ---- what a host needs to run a loaded plan without any other description of it ----
+extern "C" int llc_plan_num_io(const llc_plan_t* p, size_t* n_inputs, size_t* n_outputs) {
+  if (!p || !n_inputs || !n_outputs) return set_error(LLC_ERR_BAD_ARG, "plan_num_io: null argument");
+  *n_inputs = p->n_inputs;
+  *n_outputs = p->io.size() - p->n_inputs;
+  return LLC_OK;
+}
+
+extern "C" int llc_plan_io_info(const llc_plan_t* p, size_t index, llc_tensor* like, size_t* size_out, size_t* stride_out) {
+  if (!p || !like || !size_out || !stride_out) return set_error(LLC_ERR_BAD_ARG, "plan_io_info: null argument");
+  if (index >= p->io.size()) return set_error(LLC_ERR_BAD_ARG, "plan_io_info: the plan declares %zu tensors, index %zu", p->io.size(), index);
+  const Operand& o = p->io[index].like;
+  memset(like, 0, sizeof(*like));
+  like->type = o.t.type;
+  like->rank = o.t.rank;
+  for (size_t d = 0; d < o.t.rank; ++d) size_out[d] = o.size[d], stride_out[d] = o.stride[d];
+  like->size = size_out;
+  like->stride = stride_out;
+  return LLC_OK;
+}
+
+extern "C" int llc_hip_download(void* host, const void* device, size_t bytes, void* stream) {
+  if (bytes && (!host || !device)) return set_error(LLC_ERR_BAD_ARG, "download: null pointer");
+  LLC_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+  if (bytes) LLC_HIP_TRY(hipMemcpy(host, device, bytes, hipMemcpyDeviceToHost));
+  return LLC_OK;
+}

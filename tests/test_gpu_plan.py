@@ -446,3 +446,13 @@ def test_saved_plan_with_baked_weights_runs_in_another_process(tmp_path):
                        cwd=root, timeout=110, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
     np.testing.assert_array_equal(np.load(tmp_path / "out.npy"), want)
+    # and the same file through the host written in plain C (no Python, no torch: the C-ABI alone)
+    from llcompiler_amd.build import RUN_PLAN
+    assert os.path.exists(RUN_PLAN), "llc_run_plan is built with the library (python -m llcompiler_amd.build)"
+    r = subprocess.run([RUN_PLAN, path, str(tmp_path / "x.npy"), "-o", str(tmp_path / "out_c.npy")], timeout=110,
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    np.testing.assert_array_equal(np.load(tmp_path / "out_c.npy"), want)
+    r = subprocess.run([RUN_PLAN, path, str(tmp_path / "x.npy"), str(tmp_path / "x.npy"), "-o", str(tmp_path / "o.npy")],
+                       timeout=110, capture_output=True, text=True)
+    assert r.returncode == 1 and "takes 1 inputs" in r.stderr
