@@ -150,9 +150,9 @@ def cpu_baseline():
         fn()
         return time.perf_counter() - t0
 
-    a = r.uniform(-1, 1, (48, 2048)).astype(np.float32)
+    a = r.uniform(-1, 1, (256, 2048)).astype(np.float32)
     b = r.uniform(-1, 1, (2048, 2048)).astype(np.float32)
-    parts["matmul"] = timed(lambda: ref.matmul(a, b, "mnk")) * (2048 / 48)
+    parts["matmul"] = timed(lambda: ref.matmul(a, b, "mnk")) * (2048 / 256)
     a3 = r.uniform(-1, 1, (4, 512, 64)).astype(np.float32)
     b3 = r.uniform(-1, 1, (4, 64, 512)).astype(np.float32)
     parts["batch_matmul"] = timed(lambda: ref.batch_matmul(a3, b3, "mnk")) * (32 / 4)
@@ -165,11 +165,27 @@ def cpu_baseline():
     g = np.ones(1024, np.float32)
     parts["layernorm"] = timed(lambda: ref.layernorm_lastdim(l, g, np.zeros(1024, np.float32))) * (8192 / 2048)
     total_ms = sum(parts.values()) * 1e3
+    # the same five fp32 ops, full size, in torch eager on all host threads: what the reference checks its
+    # results against and runs the nodes it does not compile with (one pass each after one warm-up pass)
+    eager = {}
+    ta, tb = torch.from_numpy(r.uniform(-1, 1, (2048, 2048)).astype(np.float32)), torch.from_numpy(b)
+    t3a = torch.from_numpy(r.uniform(-1, 1, (32, 512, 64)).astype(np.float32))
+    t3b = torch.from_numpy(r.uniform(-1, 1, (32, 64, 512)).astype(np.float32))
+    tx = torch.from_numpy(r.uniform(-1, 1, (64, 1024, 1024)).astype(np.float32))
+    ts = torch.from_numpy(r.uniform(-1, 1, (4096, 4096)).astype(np.float32))
+    tl = torch.from_numpy(r.uniform(-1, 1, (8192, 1024)).astype(np.float32))
+    for name, fn in (("matmul", lambda: ta @ tb), ("batch_matmul", lambda: torch.bmm(t3a, t3b)),
+                     ("add_relu", lambda: torch.relu(tx + tx)), ("softmax", lambda: torch.softmax(ts, -1)),
+                     ("layernorm", lambda: torch.nn.functional.layer_norm(tl, (1024,)))):
+        fn()
+        eager[name] = timed(fn)
     return {"value": round(total_ms, 1), "unit": "ms", "cores": 1, "kind": "port",
-            "sample": "fp32 half of the suite on the C oracle, 1 thread: matmul 48 of 2048 rows, batch_matmul 4 of 32 "
+            "sample": "fp32 half of the suite on the C oracle, 1 thread: matmul 256 of 2048 rows, batch_matmul 4 of 32 "
                       "batches, add+relu 8 of 64 slabs, softmax 1024 of 4096 rows, layernorm 2048 of 8192 rows; each "
                       "extrapolated linearly and summed (the bf16 half has no CPU path in the reference)",
-            "per_op_ms": {k: round(v * 1e3, 1) for k, v in parts.items()}}
+            "per_op_ms": {k: round(v * 1e3, 1) for k, v in parts.items()},
+            "torch_cpu_eager": {"value": round(sum(eager.values()) * 1e3, 2), "unit": "ms", "threads": torch.get_num_threads(),
+                                "per_op_ms": {k: round(v * 1e3, 2) for k, v in eager.items()}}}
 
 
 MODELS = ("mlp", "resnet18", "encoder", "bert")
