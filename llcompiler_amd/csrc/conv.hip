@@ -745,11 +745,14 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
 int launch_nhwc_f32(const ConvParams& p, hipStream_t s) {
   // 128-pixel tiles when they fill the chip by themselves; else 64 x 64 tiles if those are numerous enough to need
   // no split of the reduction (a split costs a pass over the partial sums: the middle layers of a ResNet); the
-  // last layers split either way and do better on the large tiles
+  // last layers split either way and do better on the large tiles, unless their reduction is too short to split
+  // (1x1 downsampling convolutions: 3136 x 256 x 128 is 50 large tiles and 18 us, 196 small ones and 9 us)
   const int64_t bn = p.F <= 64 ? 64 : 128;
   const int64_t t128 = (int64_t)((p.ncols + 127) / 128) * ((p.F + bn - 1) / bn);
   const int64_t t64 = (int64_t)((p.ncols + 63) / 64) * ((p.F + 63) / 64);
   if (t128 < 384 && t64 >= 256) return launch_nhwc_cfg<64, 64, 2, 2>(p, s);
+  const int64_t max_splits = std::max<int64_t>(1, (p.Kdim / 32) / 8);
+  if (t128 * max_splits < 192 && t64 > t128 * max_splits) return launch_nhwc_cfg<64, 64, 2, 2>(p, s);
   return p.F <= 64 ? launch_nhwc_cfg<128, 64, 4, 2>(p, s) : launch_nhwc_cfg<128, 128, 4, 2>(p, s);
 }
 
