@@ -14,6 +14,10 @@
  *  - the caller owns every input and output buffer (Tensor.h:35: the descriptor allocates nothing).
  *  - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Calls only enqueue
  *    work; the caller synchronises.
+ *  - the library keeps one scratch buffer per device for kernels that split a reduction (convolutions with few
+ *    output tiles, fp32 matmuls with a long K): it grows on demand, which is the only allocation an op entry
+ *    point ever makes, and it is shared: such calls may follow each other on one stream, but issuing them on
+ *    several streams of one device at the same time lets them overwrite each other's partial sums.
  *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
  *    llc_hip_last_error() (thread local).  The reference only logs on failure
  *    (include/llcompiler/Support/Logger.h:132-134); returning a status is a deliberate tightening.
