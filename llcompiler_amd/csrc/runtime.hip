@@ -2,6 +2,8 @@
 // the unpacking of the reference's packed `main(void**)` parameter array.
 #include <cstring>
 
+#include <mutex>
+
 #include "common.hpp"
 
 namespace llc {
@@ -52,6 +54,8 @@ int get_workspace(size_t bytes, void** out) {
   int dev = 0;
   LLC_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "workspace: device %d", dev);
+  static std::mutex mu;  // host threads may launch at the same time; the buffer itself is shared per device
+  std::lock_guard<std::mutex> lock(mu);
   if (bytes > g_ws_cap[dev]) {
     if (g_ws[dev]) {
       LLC_HIP_TRY(hipDeviceSynchronize());
