@@ -161,6 +161,82 @@ def test_int64_elementwise(ops, oracle):
         np.testing.assert_array_equal(host(got), oracle.binary(name, a, b), err_msg=name)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_programs_bit_exact(ops, oracle, seed):
+    """Randomly drawn straight-line and branching programs over exactly rounded ops (add, sub, mul, max, min, relu,
+    abs, neg, with immediates on either side and inputs broadcast along leading, inner or all dims), in fp32, bf16
+    storage and int64: every rewrite the library applies (accumulator form, swapped operands of sub, seed input moved
+    to slot 0) must leave the bits the oracle computes op by op."""
+    r = rng(100 + seed)
+    shape = [(5, 7, 33), (130, 66), (3, 1, 257), (2, 3, 4, 40), (1, 513), (64, 64)][seed]
+    binary, unary = ["add", "sub", "mul", "max", "min"], ["relu", "abs", "neg"]
+    for trial in range(12):
+        integer = trial % 4 == 3
+        n_in = int(r.integers(1, 5))
+        in_shapes, inputs = [], []
+        for _ in range(n_in):
+            kind = int(r.integers(0, 4))
+            shp = list(shape)
+            if kind == 1:
+                shp = [1] * (len(shape) - 1) + [shape[-1]]            # a row broadcast over the leading dims
+            elif kind == 2 and len(shape) > 1:
+                shp[-1] = 1                                             # a column broadcast along the last dim
+            elif kind == 3:
+                shp = [1] * len(shape)                                  # a scalar tensor
+            in_shapes.append(tuple(shp))
+            if integer:
+                inputs.append(r.integers(-50, 50, shp).astype(np.int64))
+            else:
+                inputs.append((r.integers(-64, 64, shp) / 8.0).astype(np.float32))   # exact in bf16 too
+        in_shapes[0], inputs[0] = tuple(shape), (r.integers(-50, 50, shape).astype(np.int64) if integer else
+                                                 (r.integers(-64, 64, shape) / 8.0).astype(np.float32))
+        n_regs = int(r.integers(1, 4))
+        insts, env, written = [], {}, []
+
+        def operand(allow_imm=True):
+            c = int(r.integers(0, 3 if allow_imm else 2))
+            if c == 0 or not written:
+                k = int(r.integers(0, n_in))
+                return "in%d" % k, np.broadcast_to(inputs[k], shape)
+            if c == 1:
+                k = written[int(r.integers(0, len(written)))]
+                return k, env[k]
+            v = float(r.integers(-4, 5)) if integer else float(r.integers(-16, 17)) / 4.0
+            return v, np.full(shape, v, np.int64 if integer else np.float32)
+        for _ in range(int(r.integers(1, 9))):
+            dst = "r%d" % int(r.integers(0, n_regs))
+            if r.random() < 0.3 and not integer:
+                name = unary[int(r.integers(0, len(unary)))]
+                a, av = operand(allow_imm=False)
+                insts.append((name, dst, a))
+                val = oracle.unary(name, np.ascontiguousarray(av))
+            else:
+                name = binary[int(r.integers(0, len(binary)))]
+                a, av = operand()
+                b, bv = operand(allow_imm=not isinstance(a, float))
+                insts.append((name, dst, a, b))
+                val = oracle.binary(name, np.ascontiguousarray(av), np.ascontiguousarray(bv))
+                if not integer:
+                    # keep magnitudes small so that products stay exactly representable in fp32 and bf16
+                    val = np.clip(val, -16.0, 16.0).astype(np.float32)
+                    insts.append(("min", dst, dst, 16.0))
+                    insts.append(("max", dst, dst, -16.0))
+            env[dst] = val
+            if dst not in written:
+                written.append(dst)
+        result = written[int(r.integers(0, len(written)))]
+        prog = ops.make_program(insts, result, integer=integer)
+        if integer:
+            got = ops.elementwise(prog, [dev(t) for t in inputs], tuple(shape), torch.int64)
+            np.testing.assert_array_equal(host(got), env[result], err_msg="int64 %s -> %s" % (insts, result))
+        else:
+            got = ops.elementwise(prog, [dev(t) for t in inputs], tuple(shape), torch.float32)
+            np.testing.assert_array_equal(host(got), env[result], err_msg="f32 %s -> %s" % (insts, result))
+            # bf16 storage: the inputs are exact in bf16, the arithmetic is fp32, the result is rounded once
+            gotb = ops.elementwise(prog, [dev(t, torch.bfloat16) for t in inputs], tuple(shape), torch.bfloat16)
+            np.testing.assert_array_equal(host(gotb), bf16_round(env[result]), err_msg="bf16 %s -> %s" % (insts, result))
+
+
 def test_elementwise_empty_and_errors(ops):
     prog = ops.make_program([("relu", "r0", "in0")], "r0")
     out = ops.elementwise(prog, [torch.empty(0, 4, device="cuda")], (0, 4), torch.float32)
