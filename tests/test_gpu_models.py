@@ -405,3 +405,155 @@ def test_channels_last_weight_copies_follow_the_weights():
             if p.dim() == 4:
                 p.mul_(0.5)
         assert_close(cm(x).cpu().numpy(), m(x).cpu().numpy(), F32_RTOL, F32_ATOL, "resnet, weights scaled in place")
+
+
+class _RandomNet(torch.nn.Module):
+    """A seeded stack of blocks drawn from what the five configurations are made of, wired with residuals and
+    shape changes in random places: linear (+bias) with relu / gelu / nothing, layer norm, softmax over the last
+    dim, scaling by constants, residual adds with any earlier activation of the same shape, a head-split style
+    reshape + transpose round trip, and a row-wise max / sum normalisation."""
+
+    def __init__(self, seed, width=96):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.width = width
+        self.kinds = []
+        self.mods = torch.nn.ModuleList()
+        names = ["linear", "linear_relu", "linear_gelu", "norm", "softmax", "scale", "residual", "heads", "rownorm"]
+        for _ in range(int(torch.randint(4, 9, (1,), generator=g))):
+            kind = names[int(torch.randint(0, len(names), (1,), generator=g))]
+            self.kinds.append(kind)
+            if kind.startswith("linear"):
+                lin = torch.nn.Linear(width, width, bias=bool(torch.randint(0, 2, (1,), generator=g)))
+                with torch.no_grad():
+                    lin.weight.copy_(torch.randn(width, width, generator=g) * 0.1)
+                    if lin.bias is not None:
+                        lin.bias.copy_(torch.randn(width, generator=g) * 0.1)
+                self.mods.append(lin)
+            elif kind == "norm":
+                ln = torch.nn.LayerNorm(width)
+                with torch.no_grad():
+                    ln.weight.copy_(1 + 0.1 * torch.randn(width, generator=g))
+                    ln.bias.copy_(0.1 * torch.randn(width, generator=g))
+                self.mods.append(ln)
+            else:
+                self.mods.append(torch.nn.Identity())
+        self.picks = [int(torch.randint(0, 1 << 30, (1,), generator=g)) for _ in self.kinds]
+
+    def forward(self, x):
+        seen = [x]
+        for kind, mod, pick in zip(self.kinds, self.mods, self.picks):
+            if kind == "linear":
+                x = mod(x)
+            elif kind == "linear_relu":
+                x = torch.relu(mod(x))
+            elif kind == "linear_gelu":
+                x = torch.nn.functional.gelu(mod(x))
+            elif kind == "norm":
+                x = mod(x)
+            elif kind == "softmax":
+                x = torch.softmax(x, dim=-1)
+            elif kind == "scale":
+                x = x * (0.5 + (pick % 7) * 0.25) - 0.125
+            elif kind == "residual":
+                x = x + seen[pick % len(seen)]
+            elif kind == "heads":
+                b, s, w = x.shape
+                h = x.view(b, s, 4, w // 4).permute(0, 2, 1, 3)
+                h = torch.relu(h) + 0.5 * h
+                x = h.permute(0, 2, 1, 3).reshape(b, s, w)
+            elif kind == "rownorm":
+                x = (x - x.amax(dim=-1, keepdim=True)) / (x.abs().sum(dim=-1, keepdim=True) + 1.0)
+            seen.append(x)
+        return x
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_networks_match_eager(seed):
+    """Whatever the planner fuses (epilogues, elementwise groups, softmax re-fusion, stacked projections) and whatever
+    the engine turns into views, a randomly wired network gives torch eager's result at the fp32 tolerance, from
+    the torch.compile backend and from the export entry, kernel by kernel and through the recorded plan."""
+    from llcompiler_amd.compiler.aot import compile_module
+    net = _RandomNet(seed).eval()
+    x = torch.randn(3, 40, net.width, generator=torch.Generator().manual_seed(1000 + seed))
+    with torch.no_grad():
+        want = net(x).numpy()
+        opt, comp = _compile(net)
+        got = opt(x.cuda()).cpu().numpy()
+        cm = compile_module(copy.deepcopy(net).cuda(), (x.cuda(),))
+        first = cm(x.cuda())
+        second = cm(x.cuda())
+    what = "random net %d: %s" % (seed, " ".join(net.kinds))
+    assert_close(got, want, F32_RTOL, F32_ATOL, what + " (backend)")
+    assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what + " (export entry)")
+    assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
+
+
+class _RandomConvNet(torch.nn.Module):
+    """A seeded chain of convolutions whose channel counts switch between those the channels-last kernel takes
+    (multiples of 32) and those it does not, with 1x1 / 3x3 kernels, strides, eval-mode batch norm, relu,
+    residual adds where shapes allow, a max-pool somewhere, then global average pooling and a linear layer: layout
+    changes in both directions, residuals in either layout, epilogues with and without bias."""
+
+    def __init__(self, seed):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+
+        def pick(options):
+            return options[int(torch.randint(0, len(options), (1,), generator=g))]
+        c = pick([8, 32])
+        self.stem = torch.nn.Conv2d(3, c, 3, padding=1, bias=True)
+        self.blocks = torch.nn.ModuleList()
+        self.kinds = []
+        for _ in range(int(torch.randint(3, 7, (1,), generator=g))):
+            kind = pick(["conv", "conv_bn", "pool", "residual_conv"])
+            if kind == "pool":
+                self.blocks.append(torch.nn.MaxPool2d(pick([2, 3]), stride=2, padding=pick([0, 1])))
+            else:
+                k = pick([1, 3])
+                out = c if kind == "residual_conv" else pick([16, 32, 64, 96])
+                stride = 1 if kind == "residual_conv" else pick([1, 1, 2])
+                conv = torch.nn.Conv2d(c, out, k, stride=stride, padding=k // 2, bias=kind != "conv_bn")
+                mods = [conv]
+                if kind == "conv_bn":
+                    bn = torch.nn.BatchNorm2d(out)
+                    with torch.no_grad():
+                        bn.running_mean.copy_(0.1 * torch.randn(out, generator=g))
+                        bn.running_var.copy_(0.5 + torch.rand(out, generator=g))
+                        bn.weight.copy_(1 + 0.1 * torch.randn(out, generator=g))
+                        bn.bias.copy_(0.1 * torch.randn(out, generator=g))
+                    mods.append(bn)
+                self.blocks.append(torch.nn.Sequential(*mods))
+                c = out
+            self.kinds.append(kind)
+        self.fc = torch.nn.Linear(c, 10)
+        for p in self.parameters():
+            if p.dim() == 4:
+                with torch.no_grad():
+                    p.copy_(torch.randn(p.shape, generator=g) * (2.0 / (p.shape[1] * p.shape[2] * p.shape[3])) ** 0.5)
+
+    def forward(self, x):
+        x = torch.relu(self.stem(x))
+        for kind, block in zip(self.kinds, self.blocks):
+            if kind == "pool":
+                x = block(x)
+            elif kind == "residual_conv":
+                x = torch.relu(block(x) + x)
+            else:
+                x = torch.relu(block(x))
+        return self.fc(x.mean(dim=(2, 3)))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_conv_networks_match_eager(seed):
+    from llcompiler_amd.compiler.aot import compile_module
+    net = _RandomConvNet(seed).eval()
+    x = torch.randn(2, 3, 40, 36, generator=torch.Generator().manual_seed(2000 + seed))
+    with torch.no_grad():
+        want = net(x).numpy()
+        cm = compile_module(copy.deepcopy(net).cuda(), (x.cuda(),))
+        first = cm(x.cuda())
+        second = cm(x.cuda())
+    what = "random conv net %d: %s" % (seed, " ".join(net.kinds))
+    assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what)
+    assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
