@@ -557,3 +557,26 @@ def test_random_conv_networks_match_eager(seed):
     what = "random conv net %d: %s" % (seed, " ".join(net.kinds))
     assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what)
     assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_networks_symbolic_batch_and_sequence(seed):
+    """One compiled graph with symbolic batch and sequence extents serves every binding: the same random networks,
+    exported once, run at several (batch, sequence) pairs, in fp32 and with bf16 storage."""
+    from llcompiler_amd.compiler.aot import compile_module
+    net = _RandomNet(seed).eval()
+    example = torch.randn(2, 12, net.width)
+    dims = ({0: torch.export.Dim("batch"), 1: torch.export.Dim("seq")},)
+    with torch.no_grad():
+        cm = compile_module(copy.deepcopy(net).cuda(), (example.cuda(),), dynamic_shapes=dims)
+        cb = compile_module(copy.deepcopy(net).to(torch.bfloat16).cuda(), (example.to(torch.bfloat16).cuda(),), dynamic_shapes=dims)
+        for b, s in [(1, 8), (3, 40), (5, 17), (2, 128)]:
+            x = torch.randn(b, s, net.width, generator=torch.Generator().manual_seed(seed * 100 + b * 10 + s))
+            what = "random net %d (%s) at batch %d, seq %d" % (seed, " ".join(net.kinds), b, s)
+            assert_close(cm(x.cuda()).cpu().numpy(), net(x).numpy(), F32_RTOL, F32_ATOL, what)
+            xb = x.to(torch.bfloat16)
+            want = copy.deepcopy(net).to(torch.bfloat16)(xb).float().numpy()   # eager bf16: the same roundings between ops
+            got = cb(xb.cuda()).float().cpu().numpy()
+            scale = max(1.0, float(np.abs(want).max()))
+            assert_close(got, want, 4e-2, 4e-2 * scale, what + ", bf16")
+    assert len(cm.engine.instances) == 4
