@@ -42,6 +42,7 @@ struct View {
   bool contiguous() const {
     int64_t s = 1;
     for (int i = rank - 1; i >= 0; --i) {
+      if (size[i] == 0) return true;  // no elements: nothing is addressed, whatever the strides say
       if (size[i] != 1 && stride[i] != s) return false;
       s *= size[i];
     }

@@ -300,6 +300,47 @@ def test_reduce(ops, oracle, shape, axes):
     assert host(ops.reduce("max", dev(neg), axes)).max() < 0
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_random_rowwise_and_shape_cases(ops, oracle, seed):
+    """Randomly drawn softmax / layer_norm / reduce shapes (rows from one element to tens of thousands, any number
+    of rows) and random transposes, strided slices and copies of permuted or sliced views, the data movement bit
+    exact against numpy indexing."""
+    r = rng(900 + seed)
+    for _ in range(10):
+        cols = int(r.choice([1, 2, 7, 64, 100, 257, 768, 1000, 4096, 5003, 33000]))
+        rows = int(r.integers(1, max(2, min(70, 200000 // cols))))
+        lead = (rows,) if r.random() < 0.6 else (int(r.integers(1, 4)), rows)
+        shape = lead + (cols,)
+        x = (r.standard_normal(shape) * 2).astype(np.float32)
+        assert_close_f32(host(ops.softmax(dev(x))), oracle.softmax_lastdim(x), "softmax %s" % (shape,))
+        g, b = r.uniform(-1, 1, cols).astype(np.float32), r.uniform(-1, 1, cols).astype(np.float32)
+        if cols > 1:
+            assert_close_f32(host(ops.layer_norm(dev(x), dev(g), dev(b), 1e-5)), oracle.layernorm_lastdim(x, g, b, 1e-5),
+                             "layer_norm %s" % (shape,))
+        xb = bf16_round(x)
+        assert_close_bf16(host(ops.softmax(dev(xb, torch.bfloat16))), bf16_round(oracle.softmax_lastdim(xb)), "softmax bf16 %s" % (shape,))
+        axes = [len(shape) - 1] if r.random() < 0.5 else [0] if len(shape) == 2 else [0, 1]
+        np.testing.assert_array_equal(host(ops.reduce("max", dev(x), axes)), oracle.reduce("max", x, axes))
+        assert_close_f32(host(ops.reduce("sum", dev(x), axes)), oracle.reduce("sum", x, axes), "reduce_sum %s %s" % (shape, axes))
+    for _ in range(12):
+        rank = int(r.integers(2, 5))
+        shape = tuple(int(v) for v in r.choice([1, 2, 3, 5, 8, 17, 33, 64, 70], rank))
+        dtype = [np.float32, np.int64, np.float16, np.int8][int(r.integers(0, 4))]
+        x = r.integers(-100, 100, shape).astype(dtype)
+        perms = tuple(int(v) for v in r.permutation(rank))
+        np.testing.assert_array_equal(host(ops.transpose(dev(x), perms)), np.ascontiguousarray(x.transpose(perms)),
+                                      err_msg="transpose %s %s %s" % (shape, perms, dtype))
+        start = tuple(int(r.integers(0, n)) for n in shape)
+        end = tuple(int(r.integers(st, n + 1)) for st, n in zip(start, shape))
+        step = tuple(int(r.integers(1, 4)) for _ in shape)
+        want = x[tuple(slice(a, b, c) for a, b, c in zip(start, end, step))]
+        got = ops.stride_slice(dev(x), start, end, step)
+        assert tuple(got.shape) == want.shape, "slice %s %s %s %s" % (shape, start, end, step)
+        np.testing.assert_array_equal(host(got), want, err_msg="slice %s %s %s %s" % (shape, start, end, step))
+        view = dev(x).permute(*perms)[tuple(slice(None, None, int(r.integers(1, 3))) for _ in shape)]
+        np.testing.assert_array_equal(host(ops.copy(view)), view.cpu().numpy(), err_msg="copy of a strided view %s %s" % (shape, perms))
+
+
 def test_reduce_rejects_split_axes(ops):
     from llcompiler_amd._capi import LlcHipError
     with pytest.raises(LlcHipError, match="adjacent"):
@@ -537,6 +578,54 @@ def test_matmul_epilogue(ops, oracle):
         assert_close_f32(host(ops.matmul(dev(a), dev(b), epi)), want, "epilogue " + act)
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_random_matmul_cases(ops, oracle, seed):
+    """Randomly drawn products: extents on both sides of every dispatch threshold (16 rows, complete 128-tiles,
+    K of 1536 and more with few tiles), each operand plain or a transposed view, rows taken from a wider buffer,
+    every storage type, random epilogues."""
+    r = rng(500 + seed)
+    dims_m = [1, 3, 16, 17, 64, 100, 128, 200, 256, 384]
+    dims_n = [1, 8, 24, 64, 72, 128, 136, 256, 384]
+    dims_k = [1, 8, 40, 64, 96, 256, 320, 1536, 2048]
+    for trial in range(14):
+        M, N, K = (int(d[r.integers(0, len(d))]) for d in (dims_m, dims_n, dims_k))
+        if M * N * K > 60e6:
+            K = 256
+        dt, close, rnd = [(torch.float32, assert_close_f32, lambda x: x), (torch.bfloat16, assert_close_bf16, bf16_round),
+                          (torch.float16, assert_close_bf16, lambda x: x)][int(r.integers(0, 3))]
+        a = bf16_round(r.uniform(-1, 1, (M, K)))
+        b = bf16_round(r.uniform(-1, 1, (K, N)))
+        base = oracle.matmul(a, b, "mkn")
+        lay_a, lay_b = int(r.integers(0, 3)), int(r.integers(0, 2))
+        if lay_a == 0:
+            da = dev(a, dt)
+        elif lay_a == 1:
+            da = dev(np.ascontiguousarray(a.T), dt).t()
+        else:                                        # rows of a wider buffer: row pitch K + 16, 16-byte aligned start
+            wide = np.zeros((M, K + 16), np.float32)
+            wide[:, 8:8 + K] = a
+            da = dev(wide, dt)[:, 8:8 + K]
+        db = dev(b, dt) if lay_b == 0 else dev(np.ascontiguousarray(b.T), dt).t()
+        epi, want = None, base
+        if r.random() < 0.6:
+            alpha = float(r.choice([1.0, 0.5, 0.125]))
+            bias = bf16_round(r.standard_normal(N)) if r.random() < 0.7 else None
+            res = bf16_round(r.standard_normal((M, N))) if r.random() < 0.5 else None
+            act = str(r.choice(["none", "relu", "gelu"]))
+            want = base * np.float32(alpha)
+            if bias is not None:
+                want = want + bias[None, :]
+            if res is not None:
+                want = want + res
+            if act != "none":
+                want = oracle.unary(act, want.astype(np.float32))
+            epi = ops.Epilogue(alpha=alpha, bias=None if bias is None else dev(bias, dt),
+                               residual=None if res is None else dev(res, dt), act=act)
+        got = ops.matmul(da, db, epi)
+        close(host(got), rnd(want.astype(np.float32)), "M=%d N=%d K=%d %s A-layout %d B-layout %d epilogue %s" % (
+            M, N, K, dt, lay_a, lay_b, None if epi is None else (alpha, bias is not None, res is not None, act)))
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 192, 2048), (200, 132, 1536), (448, 768, 3072)])
 def test_matmul_f32_long_reduction_few_tiles(ops, oracle, M, N, K):
     """fp32 products whose reduction is cut into chunks (few output tiles, K >= 1536): the chunk sums are added
@@ -696,6 +785,52 @@ def test_conv2d_channels_last(ops, oracle, case):
     out2 = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
     assert_close_f32(host(ops.conv2d(dx, dw, pad=pad, stride=s, dilation=d, epilogue=epi, out=out2)), want2,
                      "channels-last conv+bias+res+relu %s" % (case,))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_conv_cases(ops, oracle, seed):
+    """Randomly drawn convolutions: window, stride, dilation, asymmetric pads, groups, channel and filter counts on
+    both sides of what each kernel takes (reduction a multiple of 4 or not, channels a multiple of 32 or not), NCHW
+    and channels-last, fp32 and bf16, with and without the epilogue."""
+    r = rng(700 + seed)
+    cl = torch.channels_last
+    done = 0
+    while done < 10:
+        g = int(r.choice([1, 1, 1, 2, 4]))
+        C = g * int(r.choice([1, 2, 3, 8, 16, 32]))
+        Fo = g * int(r.choice([1, 2, 4, 5, 16, 33, 64]))
+        if g == 1 and r.random() < 0.4:
+            C = int(r.choice([32, 64, 96]))
+        KH, KW = int(r.choice([1, 2, 3, 5])), int(r.choice([1, 2, 3, 5]))
+        s = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+        d = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+        pad = tuple(int(v) for v in r.integers(0, 3, 4))
+        N, H, W = int(r.integers(1, 4)), int(r.integers(4, 19)), int(r.integers(4, 19))
+        oh = (H + pad[0] + pad[2] - d[0] * (KH - 1) - 1) // s[0] + 1
+        ow = (W + pad[1] + pad[3] - d[1] * (KW - 1) - 1) // s[1] + 1
+        if oh < 1 or ow < 1:
+            continue
+        done += 1
+        x = r.standard_normal((N, C, H, W)).astype(np.float32)
+        w = (r.standard_normal((Fo, C // g, KH, KW)) / np.sqrt((C // g) * KH * KW)).astype(np.float32)
+        b = r.standard_normal(Fo).astype(np.float32)
+        what = "N%d C%d %dx%d F%d k%dx%d s%s d%s pad%s g%d" % (N, C, H, W, Fo, KH, KW, s, d, pad, g)
+        want = oracle.conv2d(x, w, None, pad=pad, stride=s, dilation=d, group=g)
+        res = r.standard_normal(want.shape).astype(np.float32)
+        kw = dict(pad=pad, stride=s, dilation=d, group=g)
+        assert_close_f32(host(ops.conv2d(dev(x), dev(w), **kw)), want, what)
+        # the epilogue is act(alpha * acc + bias + residual): bias is added after the scaling
+        want3 = oracle.unary("relu", want * np.float32(0.5) + b[None, :, None, None] + res)
+        epi = ops.Epilogue(alpha=0.5, bias=dev(b), residual=dev(res), act="relu")
+        assert_close_f32(host(ops.conv2d(dev(x), dev(w), epilogue=epi, **kw)), want3, what + " with epilogue")
+        xb, wb = bf16_round(x), bf16_round(w)
+        gotb = ops.conv2d(dev(xb, torch.bfloat16), dev(wb, torch.bfloat16), **kw)
+        assert_close_bf16(host(gotb), bf16_round(oracle.conv2d(xb, wb, None, pad=pad, stride=s, dilation=d, group=g)), what + " bf16")
+        if g == 1 and C % 32 == 0 and Fo % 4 == 0 and KH * KW <= 64:
+            dx, dw = dev(x).contiguous(memory_format=cl), dev(w).contiguous(memory_format=cl)
+            out = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
+            epi = ops.Epilogue(alpha=0.5, bias=dev(b), residual=dev(res).contiguous(memory_format=cl), act="relu")
+            assert_close_f32(host(ops.conv2d(dx, dw, epilogue=epi, out=out, **kw)), want3, what + " channels-last")
 
 
 def test_conv2d_layouts_must_agree(ops):
