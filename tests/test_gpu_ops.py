@@ -503,6 +503,73 @@ def test_attention(ops, oracle, B, H, Sq, Skv, masked):
         close(host(merged).transpose(0, 2, 1, 3), want, "attention on head-split views %s" % dt)
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_random_bmm_attention_pool_gather_cases(ops, oracle, seed):
+    """Randomly drawn batched products (rank 3 and the rank-4 head-split form, either operand a transposed view,
+    every storage type), attention shapes (ragged query and key counts, masks, any batch and head count), max-pool
+    windows and row gathers."""
+    r = rng(1100 + seed)
+    types = [(torch.float32, assert_close_f32, lambda x: x), (torch.bfloat16, assert_close_bf16, bf16_round),
+             (torch.float16, assert_close_bf16, lambda x: x)]
+    for _ in range(10):
+        B = int(r.choice([1, 2, 5, 12]))
+        M, N, K = (int(r.choice(d)) for d in ([1, 7, 64, 128, 130, 256], [1, 8, 64, 72, 128, 256], [1, 8, 64, 96, 128, 200]))
+        dt, close, rnd = types[int(r.integers(0, 3))]
+        a = bf16_round(r.uniform(-1, 1, (B, M, K)))
+        b = bf16_round(r.uniform(-1, 1, (B, K, N)))
+        want = rnd(oracle.batch_matmul(a, b, "mkn"))
+        da = dev(a, dt) if r.random() < 0.5 else dev(np.ascontiguousarray(a.transpose(0, 2, 1)), dt).transpose(1, 2)
+        db = dev(b, dt) if r.random() < 0.5 else dev(np.ascontiguousarray(b.transpose(0, 2, 1)), dt).transpose(1, 2)
+        close(host(ops.batch_matmul(da, db)), want, "bmm B%d %dx%dx%d %s" % (B, M, N, K, dt))
+        if B % 2 == 0 or B == 12:                      # [B0, B1, rows, cols] operands cut out of [B0, rows, B1*cols]
+            b1 = 2 if B % 2 == 0 and B != 12 else 3
+            b0 = B // b1
+            a4 = np.ascontiguousarray(a.reshape(b0, b1, M, K).transpose(0, 2, 1, 3))      # [b0, M, b1, K] in memory
+            d4 = dev(a4, dt).permute(0, 2, 1, 3)                                            # logical [b0, b1, M, K]
+            out = torch.empty((b0, M, b1, N), dtype=dt, device="cuda").permute(0, 2, 1, 3)  # merged layout written in place
+            ops.batch_matmul(d4, db.reshape(b0, b1, K, N) if db.is_contiguous() else dev(b, dt).view(b0, b1, K, N), out=out)
+            close(host(out).reshape(B, M, N), want, "bmm rank 4 B%d=%dx%d %dx%dx%d %s" % (B, b0, b1, M, N, K, dt))
+    for _ in range(6):
+        B, H = int(r.integers(1, 4)), int(r.integers(1, 5))
+        Sq, Skv = int(r.choice([1, 5, 32, 100, 128, 129, 300])), int(r.choice([1, 17, 64, 65, 128, 200, 333]))
+        q = bf16_round(r.uniform(-1, 1, (B, H, Sq, 64)))
+        k = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+        v = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+        mask = None
+        if r.random() < 0.5:
+            mask = np.zeros((B, Skv), np.float32)
+            for bb in range(B):
+                mask[bb, int(r.integers(Skv // 2, Skv)) + 1:] = -1e4
+            mask = bf16_round(mask)
+        scale = float(r.choice([0.125, 0.25, 0.5]))   # (sharper distributions leave bf16 rounding noise of the
+                                                      # probabilities above the absolute floor on outputs near 0)
+        for dt, close, rnd in types:
+            rr = rnd if dt != torch.float16 else (lambda x: x.astype(np.float16).astype(np.float32))
+            want = _attention_oracle(oracle, q, k, v, mask, scale, rr)
+            got = ops.attention(dev(q, dt), dev(k, dt), dev(v, dt), None if mask is None else dev(mask, dt), scale)
+            close(host(got), want, "attention B%d H%d Sq%d Skv%d mask %s scale %g %s" % (B, H, Sq, Skv, mask is not None, scale, dt))
+    for _ in range(8):
+        N, Cc, H, W = int(r.integers(1, 4)), int(r.integers(1, 9)), int(r.integers(3, 30)), int(r.integers(3, 30))
+        kern = (int(r.integers(1, 5)), int(r.integers(1, 5)))
+        st = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+        dil = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+        pad = tuple(int(min(v, (kk - 1) * dd // 2)) for v, kk, dd in zip(r.integers(0, 3, 4), kern + kern, dil + dil))
+        if (H + pad[0] + pad[2] - dil[0] * (kern[0] - 1) - 1) < 0 or (W + pad[1] + pad[3] - dil[1] * (kern[1] - 1) - 1) < 0:
+            continue
+        x = r.standard_normal((N, Cc, H, W)).astype(np.float32)
+        for iz in (False, True):
+            np.testing.assert_array_equal(host(ops.max_pool(dev(x), kern, pad=pad, stride=st, dilation=dil, init_zero=iz)),
+                                          oracle.maxpool2d(x, kern, pad=pad, stride=st, dilation=dil, init_zero=iz),
+                                          err_msg="max_pool %s k%s s%s d%s pad%s init_zero=%s" % (x.shape, kern, st, dil, pad, iz))
+    for _ in range(6):
+        rows, width = int(r.integers(1, 200)), int(r.choice([1, 3, 8, 64, 100, 768]))
+        table = r.standard_normal((rows, width)).astype(np.float32)
+        idx = r.integers(0, rows, tuple(int(v) for v in r.integers(1, 9, int(r.integers(1, 3))))).astype(np.int64)
+        np.testing.assert_array_equal(host(ops.gather_rows(dev(table), dev(idx))), oracle.gather_rows(table, idx))
+        tb = bf16_round(table)
+        np.testing.assert_array_equal(host(ops.gather_rows(dev(tb, torch.bfloat16), dev(idx))), oracle.gather_rows(tb, idx))
+
+
 def test_attention_fully_masked_leading_block_and_errors(ops, oracle):
     # -inf on the whole first block of keys: the running maximum stays -inf there and must not turn into NaN
     r = rng(5)
