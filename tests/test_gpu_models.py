@@ -407,6 +407,30 @@ def test_channels_last_weight_copies_follow_the_weights():
         assert_close(cm(x).cpu().numpy(), m(x).cpu().numpy(), F32_RTOL, F32_ATOL, "resnet, weights scaled in place")
 
 
+def _plan_file_round_trip(cm, args, path):
+    """Saves the plan of the (single) instance of an export-compiled module, loads it back and runs it on the
+    tensors the engine passes for `args`; returns the outputs of that run."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    inst = list(cm.engine.instances.values())[-1]
+    seen, run = {}, inst.run
+
+    def spy(inputs):
+        seen["inputs"] = list(inputs)
+        return run(inputs)
+    inst.run = spy
+    try:
+        want = cm(*args)
+    finally:
+        del inst.run
+    inst._plan.save(path)
+    loaded = Plan.load(path)
+    outs = [torch.zeros(s, dtype=d, device="cuda") for s, d in inst.out_specs]
+    loaded.run(ParamBlock(seen["inputs"] + outs), C.current_stream(torch.device("cuda", 0)))
+    torch.cuda.synchronize()
+    return want, inst._results(outs)[0]
+
+
 class _RandomNet(torch.nn.Module):
     """A seeded stack of blocks drawn from what the five configurations are made of, wired with residuals and
     shape changes in random places: linear (+bias) with relu / gelu / nothing, layer norm, softmax over the last
@@ -469,7 +493,7 @@ class _RandomNet(torch.nn.Module):
 
 
 @pytest.mark.parametrize("seed", range(16))
-def test_random_networks_match_eager(seed):
+def test_random_networks_match_eager(seed, tmp_path):
     """Whatever the planner fuses (epilogues, elementwise groups, softmax re-fusion, stacked projections) and whatever
     the engine turns into views, a randomly wired network gives torch eager's result at the fp32 tolerance, from
     the torch.compile backend and from the export entry, kernel by kernel and through the recorded plan."""
@@ -487,6 +511,9 @@ def test_random_networks_match_eager(seed):
     assert_close(got, want, F32_RTOL, F32_ATOL, what + " (backend)")
     assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what + " (export entry)")
     assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
+    with torch.no_grad():
+        want_again, from_file = _plan_file_round_trip(cm, (x.cuda(),), tmp_path / "net.llcplan")
+    assert torch.equal(want_again, first) and torch.equal(from_file, first), what + ": the plan read back from a file differs"
 
 
 class _RandomConvNet(torch.nn.Module):
@@ -545,7 +572,7 @@ class _RandomConvNet(torch.nn.Module):
 
 
 @pytest.mark.parametrize("seed", range(12))
-def test_random_conv_networks_match_eager(seed):
+def test_random_conv_networks_match_eager(seed, tmp_path):
     from llcompiler_amd.compiler.aot import compile_module
     net = _RandomConvNet(seed).eval()
     x = torch.randn(2, 3, 40, 36, generator=torch.Generator().manual_seed(2000 + seed))
@@ -557,6 +584,9 @@ def test_random_conv_networks_match_eager(seed):
     what = "random conv net %d: %s" % (seed, " ".join(net.kinds))
     assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what)
     assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
+    with torch.no_grad():
+        want_again, from_file = _plan_file_round_trip(cm, (x.cuda(),), tmp_path / "convnet.llcplan")
+    assert torch.equal(want_again, first) and torch.equal(from_file, first), what + ": the plan read back from a file differs"
 
 
 @pytest.mark.parametrize("seed", range(8))
