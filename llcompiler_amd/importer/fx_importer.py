@@ -358,15 +358,24 @@ def _reduce(name):
     return tr
 
 
-TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amax.default)(_reduce("reduce_max"))
-TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amin.default)(_reduce("reduce_min"))
-TORCH_FUNCTION_TRANSLATE_REGISTER(aten.sum.dim_IntList)(_reduce("reduce_sum"))
+def _float_reduce(node):
+    """The reduce kernels take f32, bf16 and f16 and give the same type back: a sum over a bool mask (int64 in
+    torch; the backward of amax makes one) or over integers stays in eager."""
+    v = node.args[0].meta.get("val")
+    out = node.meta.get("val")
+    floats = (torch.float32, torch.bfloat16, torch.float16)
+    return isinstance(v, torch.Tensor) and v.dtype in floats and isinstance(out, torch.Tensor) and out.dtype == v.dtype
+
+
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amax.default, check=_float_reduce)(_reduce("reduce_max"))
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amin.default, check=_float_reduce)(_reduce("reduce_min"))
+TORCH_FUNCTION_TRANSLATE_REGISTER(aten.sum.dim_IntList, check=_float_reduce)(_reduce("reduce_sum"))
 
 
 def _mean_ok(node):
     shape = node.args[0].meta["val"].shape
     dims = node.args[1]
-    return all(isinstance(shape[d], int) for d in dims)
+    return all(isinstance(shape[d], int) for d in dims) and _float_reduce(node)
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.mean.dim, check=_mean_ok)

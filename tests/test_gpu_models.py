@@ -610,3 +610,32 @@ def test_random_networks_symbolic_batch_and_sequence(seed):
             scale = max(1.0, float(np.abs(want).max()))
             assert_close(got, want, 4e-2, 4e-2 * scale, what + ", bf16")
     assert len(cm.engine.instances) == 4
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_networks_training_mode(seed):
+    """The random dense networks under mode="training": forward and backward graphs go through the backend (nodes
+    without a translator stay in eager), two optimisation-free steps, gradients of every parameter against eager."""
+    from llcompiler_amd import LLCompiler
+    torch._dynamo.reset()
+    net = _RandomNet(seed).train().cuda()
+    ref = copy.deepcopy(net)
+    comp = LLCompiler(mode="training", target="gfx950", pipeline="hip")
+    opt = torch.compile(net, backend=comp, dynamic=False)
+    what = "random net %d (%s)" % (seed, " ".join(net.kinds))
+    for step in range(2):
+        x = torch.randn(3, 24, net.width, generator=torch.Generator().manual_seed(3000 + 10 * seed + step)).cuda()
+        for mod in (net, ref):
+            mod.zero_grad()
+        out = opt(x)
+        out.square().mean().backward()
+        want = ref(x)
+        want.square().mean().backward()
+        assert_close(out.detach().cpu().numpy(), want.detach().cpu().numpy(), F32_RTOL, F32_ATOL, what + " forward")
+        grads = [q.grad for q in ref.parameters() if q.grad is not None]
+        scale = max([g.abs().max().item() for g in grads] + [1e-30])
+        for (name, p), (_, q) in zip(net.named_parameters(), ref.named_parameters()):
+            if q.grad is None:
+                assert p.grad is None, name
+                continue
+            assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-5 * scale, what + " grad of %s, step %d" % (name, step))
