@@ -325,12 +325,25 @@ def _where(ctx, node):
     return out
 
 
-@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.scalar_tensor.default, aten.full.default)
+def _fill_value_ok(node):
+    if node.target in (aten.full.default, aten.full_like.default):
+        return isinstance(node.args[1], (int, float, bool))
+    return True
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.scalar_tensor.default, aten.full.default, aten.full_like.default, aten.zeros_like.default,
+                                   aten.ones_like.default, aten.zeros.default, aten.ones.default, check=_fill_value_ok)
 def _full(ctx, node):
+    """Tensors filled with one value (the reference's alloc translators, fx_op_translate/alloc_ops.py:46-103, make a
+    constant and broadcast it the same way)."""
     if node.target is aten.scalar_tensor.default:
         value = node.args[0]
-    else:
+    elif node.target in (aten.full.default, aten.full_like.default):
         value = node.args[1]
+    elif node.target in (aten.ones_like.default, aten.ones.default):
+        value = 1
+    else:
+        value = 0
     dt = _out_dtype(node)
     c = ctx.g.constant(value, dt)
     shape = _out_shape(node)
@@ -340,6 +353,17 @@ def _full(ctx, node):
     if all(isinstance(d, int) and d == 1 for d in shape):
         return c
     return ctx.g.add_op("broadcast_to", [c], {"shape": shape, "cast_dims": tuple(range(len(shape)))})
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.sign.default, aten.sgn.default,
+                                   check=lambda n: n.meta["val"].dtype in (torch.float32, torch.bfloat16, torch.float16))
+def _sign(ctx, node):
+    """sign(x) = (x > 0) - (x < 0) in x's type (NaN gives 0 here, NaN in torch)."""
+    x = ctx.val(node.args[0])
+    zero = ctx.g.constant(0.0, x.dtype)
+    pos = ctx.g.add_op("convert_to", [ctx.g.add_op("compare", [x, zero], {"kind": "GT"})], {"dtype": x.dtype})
+    neg = ctx.g.add_op("convert_to", [ctx.g.add_op("compare", [x, zero], {"kind": "LT"})], {"dtype": x.dtype})
+    return ctx.g.add_op("sub", [pos, neg])
 
 
 # ---------------------------------------------------------------- reductions / normalisation / pooling

@@ -435,7 +435,8 @@ class _RandomNet(torch.nn.Module):
     """A seeded stack of blocks drawn from what the five configurations are made of, wired with residuals and
     shape changes in random places: linear (+bias) with relu / gelu / nothing, layer norm, softmax over the last
     dim, scaling by constants, residual adds with any earlier activation of the same shape, a head-split style
-    reshape + transpose round trip, and a row-wise max / sum normalisation."""
+    reshape + transpose round trip, a row-wise max / sum normalisation, and compare / where / masked_fill steps
+    (bool intermediates)."""
 
     def __init__(self, seed, width=96):
         super().__init__()
@@ -443,7 +444,8 @@ class _RandomNet(torch.nn.Module):
         self.width = width
         self.kinds = []
         self.mods = torch.nn.ModuleList()
-        names = ["linear", "linear_relu", "linear_gelu", "norm", "softmax", "scale", "residual", "heads", "rownorm"]
+        names = ["linear", "linear_relu", "linear_gelu", "norm", "softmax", "scale", "residual", "heads", "rownorm",
+                 "where", "masked_fill", "clamp_abs"]
         for _ in range(int(torch.randint(4, 9, (1,), generator=g))):
             kind = names[int(torch.randint(0, len(names), (1,), generator=g))]
             self.kinds.append(kind)
@@ -488,6 +490,12 @@ class _RandomNet(torch.nn.Module):
                 x = h.permute(0, 2, 1, 3).reshape(b, s, w)
             elif kind == "rownorm":
                 x = (x - x.amax(dim=-1, keepdim=True)) / (x.abs().sum(dim=-1, keepdim=True) + 1.0)
+            elif kind == "where":
+                x = torch.where(x > 0.1, x, 0.5 * x)
+            elif kind == "masked_fill":
+                x = x.masked_fill(seen[0] < -0.5, -2.0)
+            elif kind == "clamp_abs":
+                x = torch.minimum(x.abs(), torch.full_like(x, 3.0)) * torch.sign(seen[0]).abs()
             seen.append(x)
         return x
 
@@ -624,15 +632,17 @@ def test_random_networks_training_mode(seed):
     opt = torch.compile(net, backend=comp, dynamic=False)
     what = "random net %d (%s)" % (seed, " ".join(net.kinds))
     for step in range(2):
-        x = torch.randn(3, 24, net.width, generator=torch.Generator().manual_seed(3000 + 10 * seed + step)).cuda()
+        x = torch.randn(3, 24, net.width, generator=torch.Generator().manual_seed(3000 + 10 * seed + step)).cuda().requires_grad_()
+        xr = x.detach().clone().requires_grad_()     # (a net drawn without any layer with parameters still has this gradient)
         for mod in (net, ref):
             mod.zero_grad()
         out = opt(x)
         out.square().mean().backward()
-        want = ref(x)
+        want = ref(xr)
         want.square().mean().backward()
         assert_close(out.detach().cpu().numpy(), want.detach().cpu().numpy(), F32_RTOL, F32_ATOL, what + " forward")
-        grads = [q.grad for q in ref.parameters() if q.grad is not None]
+        grads = [q.grad for q in ref.parameters() if q.grad is not None] + [xr.grad]
+        assert_close(x.grad.cpu().numpy(), xr.grad.cpu().numpy(), 1e-4, 1e-5 * max(xr.grad.abs().max().item(), 1e-30), what + " grad of the input")
         scale = max([g.abs().max().item() for g in grads] + [1e-30])
         for (name, p), (_, q) in zip(net.named_parameters(), ref.named_parameters()):
             if q.grad is None:
