@@ -445,7 +445,7 @@ class _RandomNet(torch.nn.Module):
         self.kinds = []
         self.mods = torch.nn.ModuleList()
         names = ["linear", "linear_relu", "linear_gelu", "norm", "softmax", "scale", "residual", "heads", "rownorm",
-                 "where", "masked_fill", "clamp_abs"]
+                 "where", "masked_fill", "clamp_abs", "colscale", "gram", "first_row", "smooth", "gates"]
         for _ in range(int(torch.randint(4, 9, (1,), generator=g))):
             kind = names[int(torch.randint(0, len(names), (1,), generator=g))]
             self.kinds.append(kind)
@@ -462,6 +462,11 @@ class _RandomNet(torch.nn.Module):
                     ln.weight.copy_(1 + 0.1 * torch.randn(width, generator=g))
                     ln.bias.copy_(0.1 * torch.randn(width, generator=g))
                 self.mods.append(ln)
+            elif kind == "colscale":
+                holder = torch.nn.Module()
+                holder.scale = torch.nn.Parameter(1 + 0.2 * torch.randn(width, generator=g))
+                holder.shift = torch.nn.Parameter(0.2 * torch.randn(1, 1, width, generator=g))
+                self.mods.append(holder)
             else:
                 self.mods.append(torch.nn.Identity())
         self.picks = [int(torch.randint(0, 1 << 30, (1,), generator=g)) for _ in self.kinds]
@@ -490,6 +495,17 @@ class _RandomNet(torch.nn.Module):
                 x = h.permute(0, 2, 1, 3).reshape(b, s, w)
             elif kind == "rownorm":
                 x = (x - x.amax(dim=-1, keepdim=True)) / (x.abs().sum(dim=-1, keepdim=True) + 1.0)
+            elif kind == "colscale":
+                x = x * mod.scale + mod.shift
+            elif kind == "gram":                       # an attention-like group whose inner extent is not 64
+                p = torch.softmax(torch.matmul(x, x.transpose(1, 2)) / self.width, dim=-1)
+                x = torch.matmul(p, x)
+            elif kind == "first_row":
+                x = x - 0.5 * x[:, :1, :]
+            elif kind == "smooth":
+                x = torch.rsqrt(x * x + 1.0) * x + torch.exp(-x.abs()) - torch.sqrt(x.abs() + 1.0) * 0.25
+            elif kind == "gates":
+                x = torch.sigmoid(x) * torch.tanh(seen[pick % len(seen)])
             elif kind == "where":
                 x = torch.where(x > 0.1, x, 0.5 * x)
             elif kind == "masked_fill":
