@@ -431,6 +431,23 @@ def _plan_file_round_trip(cm, args, path):
     return want, inst._results(outs)[0]
 
 
+def _assert_as_close_as_eager(got, want32, want64, rtol, atol, what):
+    """`got` against the float64 evaluation `want64`, at the stated tolerance plus what torch's own fp32 evaluation
+    `want32` misses it by: a randomly wired network can be ill-conditioned (a layer norm over nearly constant rows
+    multiplies every rounding error before it by hundreds), and then no fp32 evaluation meets a fixed bar; ours must
+    be as good as eager's, up to a factor."""
+    got, want32, want64 = (np.asarray(t, dtype=np.float64) for t in (got, want32, want64))
+    assert got.shape == want64.shape, "%s: shape %s vs %s" % (what, got.shape, want64.shape)
+    noise = float(np.abs(want32 - want64).max())
+    err = np.abs(got - want64)
+    bar = atol + rtol * np.abs(want64) + 4.0 * noise
+    bad = ~(err <= bar)
+    if bad.any():
+        i = np.unravel_index(np.argmax(np.where(bad, err, 0)), err.shape)
+        raise AssertionError("%s: %d of %d elements outside rtol=%g atol=%g + 4 x eager's own error %.3g; worst at %s: got %r "
+                             "want %r" % (what, int(bad.sum()), bad.size, rtol, atol, noise, i, got[i], want64[i]))
+
+
 class _RandomNet(torch.nn.Module):
     """A seeded stack of blocks drawn from what the five configurations are made of, wired with residuals and
     shape changes in random places: linear (+bias) with relu / gelu / nothing, layer norm, softmax over the last
@@ -516,7 +533,7 @@ class _RandomNet(torch.nn.Module):
         return x
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(28))
 def test_random_networks_match_eager(seed, tmp_path):
     """Whatever the planner fuses (epilogues, elementwise groups, softmax re-fusion, stacked projections) and whatever
     the engine turns into views, a randomly wired network gives torch eager's result at the fp32 tolerance, from
@@ -526,14 +543,15 @@ def test_random_networks_match_eager(seed, tmp_path):
     x = torch.randn(3, 40, net.width, generator=torch.Generator().manual_seed(1000 + seed))
     with torch.no_grad():
         want = net(x).numpy()
+        want64 = copy.deepcopy(net).double()(x.double()).numpy()
         opt, comp = _compile(net)
         got = opt(x.cuda()).cpu().numpy()
         cm = compile_module(copy.deepcopy(net).cuda(), (x.cuda(),))
         first = cm(x.cuda())
         second = cm(x.cuda())
     what = "random net %d: %s" % (seed, " ".join(net.kinds))
-    assert_close(got, want, F32_RTOL, F32_ATOL, what + " (backend)")
-    assert_close(first.cpu().numpy(), want, F32_RTOL, F32_ATOL, what + " (export entry)")
+    _assert_as_close_as_eager(got, want, want64, F32_RTOL, F32_ATOL, what + " (backend)")
+    _assert_as_close_as_eager(first.cpu().numpy(), want, want64, F32_RTOL, F32_ATOL, what + " (export entry)")
     assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
     with torch.no_grad():
         want_again, from_file = _plan_file_round_trip(cm, (x.cuda(),), tmp_path / "net.llcplan")
@@ -595,7 +613,7 @@ class _RandomConvNet(torch.nn.Module):
         return self.fc(x.mean(dim=(2, 3)))
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(16))
 def test_random_conv_networks_match_eager(seed, tmp_path):
     from llcompiler_amd.compiler.aot import compile_module
     net = _RandomConvNet(seed).eval()
@@ -613,7 +631,7 @@ def test_random_conv_networks_match_eager(seed, tmp_path):
     assert torch.equal(want_again, first) and torch.equal(from_file, first), what + ": the plan read back from a file differs"
 
 
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(27))
 def test_random_networks_symbolic_batch_and_sequence(seed):
     """One compiled graph with symbolic batch and sequence extents serves every binding: the same random networks,
     exported once, run at several (batch, sequence) pairs, in fp32 and with bf16 storage."""
@@ -627,16 +645,19 @@ def test_random_networks_symbolic_batch_and_sequence(seed):
         for b, s in [(1, 8), (3, 40), (5, 17), (2, 128)]:
             x = torch.randn(b, s, net.width, generator=torch.Generator().manual_seed(seed * 100 + b * 10 + s))
             what = "random net %d (%s) at batch %d, seq %d" % (seed, " ".join(net.kinds), b, s)
-            assert_close(cm(x.cuda()).cpu().numpy(), net(x).numpy(), F32_RTOL, F32_ATOL, what)
+            _assert_as_close_as_eager(cm(x.cuda()).cpu().numpy(), net(x).numpy(), copy.deepcopy(net).double()(x.double()).numpy(),
+                                      F32_RTOL, F32_ATOL, what)
             xb = x.to(torch.bfloat16)
-            want = copy.deepcopy(net).to(torch.bfloat16)(xb).float().numpy()   # eager bf16: the same roundings between ops
+            netb = copy.deepcopy(net).to(torch.bfloat16)
+            want = netb(xb).float().numpy()                 # eager bf16: a rounding after every op
+            want64 = netb.double()(xb.double()).numpy()     # the bf16 weights and input evaluated exactly
             got = cb(xb.cuda()).float().cpu().numpy()
-            scale = max(1.0, float(np.abs(want).max()))
-            assert_close(got, want, 4e-2, 4e-2 * scale, what + ", bf16")
+            scale = max(1.0, float(np.abs(want64).max()))
+            _assert_as_close_as_eager(got, want, want64, 4e-2, 4e-2 * scale, what + ", bf16")
     assert len(cm.engine.instances) == 4
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(27))
 def test_random_networks_training_mode(seed):
     """The random dense networks under mode="training": forward and backward graphs go through the backend (nodes
     without a translator stay in eager), two optimisation-free steps, gradients of every parameter against eager."""
@@ -644,24 +665,31 @@ def test_random_networks_training_mode(seed):
     torch._dynamo.reset()
     net = _RandomNet(seed).train().cuda()
     ref = copy.deepcopy(net)
+    ref64 = copy.deepcopy(net).double()
     comp = LLCompiler(mode="training", target="gfx950", pipeline="hip")
     opt = torch.compile(net, backend=comp, dynamic=False)
     what = "random net %d (%s)" % (seed, " ".join(net.kinds))
     for step in range(2):
         x = torch.randn(3, 24, net.width, generator=torch.Generator().manual_seed(3000 + 10 * seed + step)).cuda().requires_grad_()
         xr = x.detach().clone().requires_grad_()     # (a net drawn without any layer with parameters still has this gradient)
-        for mod in (net, ref):
+        xd = x.detach().double().requires_grad_()
+        for mod in (net, ref, ref64):
             mod.zero_grad()
         out = opt(x)
         out.square().mean().backward()
         want = ref(xr)
         want.square().mean().backward()
-        assert_close(out.detach().cpu().numpy(), want.detach().cpu().numpy(), F32_RTOL, F32_ATOL, what + " forward")
-        grads = [q.grad for q in ref.parameters() if q.grad is not None] + [xr.grad]
-        assert_close(x.grad.cpu().numpy(), xr.grad.cpu().numpy(), 1e-4, 1e-5 * max(xr.grad.abs().max().item(), 1e-30), what + " grad of the input")
+        want64 = ref64(xd)
+        want64.square().mean().backward()
+
+        def host(t):
+            return t.detach().cpu().numpy()
+        _assert_as_close_as_eager(host(out), host(want), host(want64), F32_RTOL, F32_ATOL, what + " forward")
+        grads = [q.grad for q in ref64.parameters() if q.grad is not None] + [xd.grad]
         scale = max([g.abs().max().item() for g in grads] + [1e-30])
-        for (name, p), (_, q) in zip(net.named_parameters(), ref.named_parameters()):
+        _assert_as_close_as_eager(host(x.grad), host(xr.grad), host(xd.grad), 1e-4, 1e-5 * scale, what + " grad of the input")
+        for (name, p), (_, q), (_, d) in zip(net.named_parameters(), ref.named_parameters(), ref64.named_parameters()):
             if q.grad is None:
                 assert p.grad is None, name
                 continue
-            assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-5 * scale, what + " grad of %s, step %d" % (name, step))
+            _assert_as_close_as_eager(host(p.grad), host(q.grad), host(d.grad), 1e-4, 1e-5 * scale, what + " grad of %s, step %d" % (name, step))
