@@ -15,7 +15,7 @@
  *  - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Calls only enqueue
  *    work; the caller synchronises.
  *  - the library keeps one scratch buffer per device for kernels that split a reduction (convolutions with few
- *    output tiles, fp32 matmuls with a long K): it grows on demand, which is the only allocation an op entry
+ *    output tiles, matmuls with a long K): it grows on demand, which is the only allocation an op entry
  *    point ever makes, and it is shared: such calls may follow each other on one stream, but issuing them on
  *    several streams of one device at the same time lets them overwrite each other's partial sums.
  *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
@@ -101,7 +101,7 @@ typedef struct llc_epilogue {
  * fp32 accumulate.  f32, bf16 or f16 operands (all three the same type).  Either operand may be a
  * transposed view (stride[0] == 1), which is how llh.transpose{perms=[1,0]} of a weight
  * (llcompiler/importer/fx_op_translate/transpose.py:39-48) is consumed without a copy.
- * `epi` may be NULL.  fp32 products with a long reduction and few output tiles sum the reduction in
+ * `epi` may be NULL.  Products with a long reduction and few output tiles sum the reduction in
  * chunks through the library's per-device scratch buffer (grown on demand by this call); the order
  * of the sum is fixed, so results are the same bits on every run. */
 int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,

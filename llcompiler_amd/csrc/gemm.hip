@@ -53,6 +53,7 @@ struct GemmParams {
   float alpha;
   int32_t act;
   int32_t tiles_m, tiles_n;
+  int32_t c_f32;  // gemm_kernel only: C holds raw fp32 sums whatever T is (the chunks of a split reduction)
 };
 
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB, bool FULL>
@@ -148,7 +149,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
         if (!FULL && row >= p.M) continue;
-        epilogue_store<T>(C, (int64_t)row * p.c_sm + col, acc[i][j][r], p.alpha, bv, res, p.act);
+        if (sizeof(T) != 4 && p.c_f32) ((float*)p.C)[c_off + (int64_t)row * p.c_sm + col] = acc[i][j][r];
+        else epilogue_store<T>(C, (int64_t)row * p.c_sm + col, acc[i][j][r], p.alpha, bv, res, p.act);
       }
     }
   }
@@ -761,15 +763,15 @@ int launch_skinny(const GemmParams& p, hipStream_t s) {
   return check_launch("gemm_skinny_kernel");
 }
 
-// ---- fp32 products with a long reduction and too few output tiles to fill the chip (a transformer's second
-// feed-forward layer at a short sequence: 1024 x 768 x 3072 is 192 tiles of 64x64).  The reduction is cut into
+// ---- products with a long reduction and too few output tiles to fill the chip (a transformer's second
+// feed-forward layer at a short sequence: 1024 x 768 x 3072 is 192 tiles of 64x64), any storage type.  The reduction is cut into
 // `splits` equal chunks that run as the batches of one batched product into fp32 partial results
 // [splits][M][N] in the workspace; a second kernel sums them in chunk order (the same order on every run)
 // and applies the epilogue.
+template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int splits, int64_t mn,
-                                                            int n, float alpha, const float* __restrict__ bias,
-                                                            const float* __restrict__ residual, int act,
-                                                            float* __restrict__ out) {
+                                                            int n, float alpha, const char* __restrict__ bias,
+                                                            const char* __restrict__ residual, int act, T* __restrict__ out) {
   const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i4 >= mn) return;
   f32x4_t acc = *(const f32x4_t*)(part + i4);
@@ -781,27 +783,30 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   const int col = (int)(i4 % n);  // n is a multiple of 4: the four values share a row
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    epilogue_store<float>(out, i4 + j, acc[j], alpha, bias ? bias[col + j] : 0.0f, (const char*)residual, act);
+    epilogue_store<T>(out, i4 + j, acc[j], alpha, bias ? load_as_f32(bias, Elem<T>::kDtype, col + j) : 0.0f, residual, act);
 }
 
-// Number of reduction chunks for an fp32 product, 1 = no split.  A split pays when the 64x64 tiles cover less
-// than two rounds of the 256 CUs and the reduction is long (measured: 1024 x 768 x 3072 goes from 64 to 50 us
-// in four chunks, 2048 x 768 x 3072 from 110 to 94 us in two; at K = 768 every split loses to the plain kernel).
-// The smallest chunk count that gives three workgroups per CU is taken, chunks of at least 256.
-inline int splitk_chunks(const GemmParams& p) {
+// Number of reduction chunks, 1 = no split; bk = elements of a k-tile (32 for fp32, 64 for the 16-bit types).  A
+// split pays when the 64x64 tiles cover less than two rounds of the 256 CUs and the reduction is long (measured,
+// fp32: 1024 x 768 x 3072 goes from 64 to 50 us in four chunks, 2048 x 768 x 3072 from 110 to 94 us in two; bf16:
+// 512 x 768 x 3072 from 22 to 15 us, 1024 x 768 x 3072 from 23 to 18.5 us; at K = 768 every split loses to the plain
+// kernel).  The smallest chunk count that gives three (fp32) or two (16-bit, whose tiles are done sooner)
+// workgroups per CU is taken, chunks of at least 256.
+inline int splitk_chunks(const GemmParams& p, int bk) {
   const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
   if (p.K < 1536 || t64 >= 512 || p.M <= 64 || p.N <= 64 || p.N % 4 != 0 || p.c_sm != p.N) return 1;
+  const int64_t enough = bk == 32 ? 768 : 512;
   int best = 1;
   for (int sp = 2; sp <= 8; ++sp) {
-    if (p.K % (sp * 32) != 0 || p.K / sp < 256) continue;
+    if (p.K % (sp * bk) != 0 || p.K / sp < 256) continue;
     if (t64 * sp > 1024) break;
     best = sp;
-    if (t64 * sp >= 768) break;
+    if (t64 * sp >= enough) break;
   }
   return best;
 }
 
-template <int LB>
+template <typename T, int LB>
 int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
   const int64_t mn = (int64_t)p.M * p.N;
   void* ws = nullptr;
@@ -816,15 +821,16 @@ int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
   q.c_sb = mn;
   q.c_sb1 = 0;
   q.c_sm = p.N;
+  q.c_f32 = 1;
   q.bias = nullptr;
   q.bias_sb = 0;
   q.residual = nullptr;
   q.alpha = 1.0f;
   q.act = LLC_ACT_NONE;
-  LLC_TRY((launch_tiles<float, kLoadKVec, LB>(q, splits, s)));
+  LLC_TRY((launch_tiles<T, kLoadKVec, LB>(q, splits, s)));
   const int64_t blocks = (mn / 4 + 255) / 256;
-  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const float*)ws, splits, mn, p.N,
-                     p.alpha, (const float*)p.bias, (const float*)p.residual, p.act, (float*)p.C);
+  hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, (const float*)ws, splits, mn, p.N,
+                     p.alpha, p.bias, p.residual, p.act, (T*)p.C);
   return check_launch("splitk_reduce_kernel");
 }
 
@@ -836,11 +842,9 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   const bool b_kvec = p.b_sk == 1 && p.b_sn % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.K % EPV == 0 && al16(p.B);
   const bool b_rvec = p.b_sn == 1 && p.b_sk % EPV == 0 && p.b_sb % EPV == 0 && p.b_sb1 % EPV == 0 && p.N % EPV == 0 && al16(p.B);
   if (batch == 1 && p.M <= 16 && a_kvec && b_kvec) return launch_skinny<T>(p, s);
-  if constexpr (sizeof(T) == 4) {
-    if (batch == 1 && a_kvec && (b_kvec || b_rvec) && al16(p.C) && (!p.residual || al16(p.residual))) {
-      const int splits = splitk_chunks(p);
-      if (splits > 1) return b_kvec ? launch_splitk<kLoadKVec>(p, splits, s) : launch_splitk<kLoadRVec>(p, splits, s);
-    }
+  if (batch == 1 && a_kvec && (b_kvec || b_rvec) && al16(p.C) && (!p.residual || al16(p.residual))) {
+    const int splits = splitk_chunks(p, kRowBytes / (int)sizeof(T));
+    if (splits > 1) return b_kvec ? launch_splitk<T, kLoadKVec>(p, splits, s) : launch_splitk<T, kLoadRVec>(p, splits, s);
   }
   if constexpr (sizeof(T) == 2) {
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;

@@ -695,8 +695,9 @@ def test_random_matmul_cases(ops, oracle, seed):
 
 @pytest.mark.parametrize("M,N,K", [(256, 192, 2048), (200, 132, 1536), (448, 768, 3072)])
 def test_matmul_f32_long_reduction_few_tiles(ops, oracle, M, N, K):
-    """fp32 products whose reduction is cut into chunks (few output tiles, K >= 1536): the chunk sums are added
-    in a fixed order and the epilogue runs once, after the sum.  Both weight layouts, with and without epilogue."""
+    """Products whose reduction is cut into chunks (few output tiles, K >= 1536): the chunk sums (fp32 whatever the
+    storage type) are added in a fixed order and the epilogue runs once, after the sum.  Both weight layouts, with
+    and without epilogue, every storage type."""
     r = rng(M + N + K)
     a = r.uniform(-1, 1, (M, K)).astype(np.float32) * 0.25
     b = r.uniform(-1, 1, (K, N)).astype(np.float32) * 0.25
@@ -714,6 +715,18 @@ def test_matmul_f32_long_reduction_few_tiles(ops, oracle, M, N, K):
             want = oracle.unary(act, want)
         epi = ops.Epilogue(alpha=alpha, bias=dev(bias), residual=dev(res), act=act)
         assert_close_f32(host(ops.matmul(dev(a), bt.t(), epi)), want, "NT epilogue %s %s" % (act, (M, N, K)))
+    # the 16-bit types split the same way (fp32 partial sums, one rounding at the end)
+    ab, bb, biasb, resb = bf16_round(a), bf16_round(b), bf16_round(bias), bf16_round(res)
+    baseb = oracle.matmul(ab, bb, "mkn")
+    for dt, rnd in ((torch.bfloat16, bf16_round), (torch.float16, lambda x: x)):
+        btd = dev(np.ascontiguousarray(bb.T), dt)
+        firstb = host(ops.matmul(dev(ab, dt), btd.t()))
+        assert_close_bf16(firstb, rnd(baseb), "NT %s %s" % (dt, (M, N, K)))
+        np.testing.assert_array_equal(host(ops.matmul(dev(ab, dt), btd.t())), firstb)
+        assert_close_bf16(host(ops.matmul(dev(ab, dt), dev(bb, dt))), rnd(baseb), "NN %s %s" % (dt, (M, N, K)))
+        want = oracle.unary("gelu", baseb * np.float32(0.125) + biasb[None, :] + resb)
+        epi = ops.Epilogue(alpha=0.125, bias=dev(biasb, dt), residual=dev(resb, dt), act="gelu")
+        assert_close_bf16(host(ops.matmul(dev(ab, dt), btd.t(), epi)), rnd(want), "NT epilogue %s %s" % (dt, (M, N, K)))
 
 
 @pytest.mark.parametrize("B,M,N,K", [(3, 9, 4, 6), (4, 64, 64, 64), (6, 128, 128, 64), (5, 100, 64, 100), (2, 130, 70, 36)])
