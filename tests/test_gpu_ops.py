@@ -804,6 +804,9 @@ CONV_CASES = [
     (1, 16, 20, 20, 32, 3, 3, (2, 2), (1, 1), (2, 2), 1),   # dilated, stride 1
     (2, 8, 12, 16, 16, 3, 3, (1, 1), (1, 1), (1, 1), 2),    # groups, stride 1
     (4, 256, 7, 7, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1),   # few pixels, deep reduction: split over k
+    (2, 3, 32, 224, 64, 7, 7, (3, 3), (2, 2), (1, 1), 1),   # an image network's first layer: 3 channels, 7x7 window, stride 2
+    (3, 3, 8, 192, 64, 7, 7, (3, 3), (2, 2), (1, 1), 1),    # the same on images of 8 rows: mostly padding rows
+    (1, 3, 20, 236, 64, 7, 7, (2, 2), (2, 2), (1, 1), 1),   # pad 2, rows of 117 outputs
 ]
 
 
