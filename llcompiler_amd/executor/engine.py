@@ -688,6 +688,9 @@ class Instance:
                               st_) for s, e, st_ in zip(a["start"], a["end"], a["stride"]))
             return t[idx]
         if op == "extract":
+            if t.dim() == 1:  # one element of a vector stays a tensor<1> (LLHinfersymbolShape.cpp:513-516)
+                i = a["index"] % t.shape[0]
+                return t[i:i + 1]
             return t[a["index"]]
         raise NotImplementedError(op)
 

@@ -200,7 +200,9 @@ def _select(ctx, node):
     x = ctx.val(node.args[0])
     dim, index = node.args[1] % x.rank, node.args[2]
     if dim == 0:
-        return ctx.g.add_op("extract", [x], {"index": int(index)})
+        r = ctx.g.add_op("extract", [x], {"index": int(index)})
+        # llh.extract of a vector gives tensor<1>, torch a 0-d tensor
+        return r if x.rank > 1 else _reshape_to(ctx, r, _out_shape(node))
     if index < 0:
         index += x.shape[dim]
     start = [0] * x.rank

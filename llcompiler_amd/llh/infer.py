@@ -86,8 +86,8 @@ def infer(name, operands, attrs):
         return [tuple(attrs["shape"])], [dt]
     if name == "stride_slice":  # size = ceildiv(end - start, stride), StablehlotoLinalgExtension.cpp:68-118
         return [tuple(ceildiv(e - s, st) for s, e, st in zip(attrs["start"], attrs["end"], attrs["stride"]))], [dt]
-    if name == "extract":
-        return [tuple(shapes[0][1:])], [dt]
+    if name == "extract":  # the row of dim 0 with the dim dropped; a rank-1 input keeps one element as tensor<1>
+        return [tuple(shapes[0][1:]) if len(shapes[0]) > 1 else (1,)], [dt]  # (LLHinfersymbolShape.cpp:504-529)
     if name == "gather":
         return [tuple(shapes[1]) + tuple(shapes[0][1:])], [dt]
     raise NotImplementedError("no shape rule for llh.%s" % name)

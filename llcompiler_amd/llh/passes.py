@@ -1,8 +1,9 @@
 """LLH-level rewrites run before kernel planning.  Counterparts of the reference's
 src/Dialect/LLH/Transforms passes and canonicalisers, on the Python graph:
 
-  canonicalize           no-op reshape / broadcast / convert / identity folds, x*1, x+0
-                         (LLHCanonicalize.cpp:378-455, LLHFolder.cpp:33-330)
+  canonicalize           no-op reshape / broadcast / convert / identity folds, abs(abs x), reshape of a constant,
+                         x*1, x/1, x+0, 0+x, x-0, c-c (LLHCanonicalize.cpp:378-455, LLHFolder.cpp:33-330).  x*0 is not
+                         folded (the reference does): the product is NaN where x is NaN or infinite
   decompose_batch_norm   batch_norm_inference -> add, sqrt, reshape, broadcast_to x4, sub, mul, div, add
                          (DecomposeOps.cpp:110-148; op order pinned by test/Dialect/LLH/decompose_ops.mlir:10-20)
   fuse_softmax           reduce_max -> sub -> exp -> reduce_sum -> div  ==>  softmax
@@ -26,6 +27,21 @@ def _through_broadcast(v):
     return v
 
 
+def _splat(v):
+    """The value every element of v has when v is a constant filled with one number (seen through reshape and
+    broadcast_to), else None."""
+    v = _through_broadcast(v)
+    if v.const is not None:
+        return float(v.const)
+    if v.producer is not None and v.producer.name == "constant" and not isinstance(v.producer.attrs.get("value"), (list, tuple)):
+        return float(v.producer.attrs["value"])
+    return None
+
+
+def _static(shape):
+    return all(isinstance(d, int) for d in shape)
+
+
 def canonicalize(g):
     changed = True
     while changed:
@@ -47,15 +63,63 @@ def canonicalize(g):
                 src.users.append(op)
                 changed = True
                 continue
+            elif op.name == "broadcast_to" and op.operands[0].rank == r.rank and \
+                    sorted(op.attrs.get("noexpand_dims", ())) == list(range(r.rank)):
+                # the importer's hint that no dim expands (LLHCanonicalize.cpp: fold of broadcast_to, pinned by
+                # test/Dialect/LLH/canonicalize.mlir fold_broadcast)
+                rep = op.operands[0]
             elif op.name == "transpose" and tuple(op.attrs["perms"]) == tuple(range(r.rank)):
                 rep = op.operands[0]
-            elif op.name in ("mul", "div") and _is_const(_through_broadcast(op.operands[1]), 1.0) and \
-                    tuple(op.operands[0].shape) == tuple(r.shape) and op.operands[0].dtype == r.dtype:
-                rep = op.operands[0]
-            elif op.name == "mul" and _is_const(_through_broadcast(op.operands[0]), 1.0) and \
+            elif op.name == "abs" and op.operands[0].producer is not None and op.operands[0].producer.name == "abs":
+                rep = op.operands[0]      # abs(abs(x)) (canonicalize.mlir fold_two_abs)
+            elif op.name == "reshape" and _static(r.shape) and op.operands[0].producer is not None and \
+                    op.operands[0].producer.name == "constant" and op.operands[0].const is None and \
+                    not isinstance(op.operands[0].producer.attrs["value"], (list, tuple)):
+                # reshape of a constant filled with one value is that constant in the new shape (fold_reshape)
+                idx = g.ops.index(op)
+                tail = g.ops[idx:]
+                del g.ops[idx:]
+                rep = g.add_op("constant", [], {"value": op.operands[0].producer.attrs["value"]}, shapes=[tuple(r.shape)], dtypes=[r.dtype])
+                g.ops += tail
+            elif op.name == "reshape" and _static(r.shape) and op.operands[0].producer is not None and \
+                    op.operands[0].producer.name == "constant" and isinstance(op.operands[0].producer.attrs["value"], (list, tuple)):
+                idx = g.ops.index(op)
+                tail = g.ops[idx:]
+                del g.ops[idx:]
+                rep = g.add_op("constant", [], {"value": list(op.operands[0].producer.attrs["value"])}, shapes=[tuple(r.shape)], dtypes=[r.dtype])
+                g.ops += tail
+            elif op.name == "sub" and op.operands[0] is op.operands[1] and _static(r.shape) and r.dtype.is_floating_point and \
+                    _splat(op.operands[0]) is not None:
+                # c - c for a constant c (fold.mlir sub_same_fold; for a general x the difference is NaN where x is)
+                idx = g.ops.index(op)
+                tail = g.ops[idx:]
+                del g.ops[idx:]
+                rep = g.add_op("constant", [], {"value": 0.0}, shapes=[tuple(r.shape)], dtypes=[r.dtype])
+                g.ops += tail
+            elif op.name in ("add", "sub", "mul", "div") and r.dtype == torch.float32 and _static(r.shape) and \
+                    all(o.producer is not None and o.producer.name == "constant" and tuple(o.shape) == tuple(r.shape)
+                        for o in op.operands) and _splat(op.operands[0]) is not None and _splat(op.operands[1]) is not None and \
+                    not (op.name == "div" and _splat(op.operands[1]) == 0.0):
+                # two constants filled with one value each: the result is such a constant (fold.mlir mul_fold, div_fold),
+                # computed in fp32 like the kernel would
+                import numpy as np
+                a, b = np.float32(_splat(op.operands[0])), np.float32(_splat(op.operands[1]))
+                val = a + b if op.name == "add" else a - b if op.name == "sub" else a * b if op.name == "mul" else a / b
+                idx = g.ops.index(op)
+                tail = g.ops[idx:]
+                del g.ops[idx:]
+                rep = g.add_op("constant", [], {"value": float(val)}, shapes=[tuple(r.shape)], dtypes=[r.dtype])
+                g.ops += tail
+            elif op.name == "add" and _splat(op.operands[0]) == 0.0 and \
                     tuple(op.operands[1].shape) == tuple(r.shape) and op.operands[1].dtype == r.dtype:
                 rep = op.operands[1]
-            elif op.name in ("add", "sub") and _is_const(_through_broadcast(op.operands[1]), 0.0) and \
+            elif op.name in ("mul", "div") and _splat(op.operands[1]) == 1.0 and \
+                    tuple(op.operands[0].shape) == tuple(r.shape) and op.operands[0].dtype == r.dtype:
+                rep = op.operands[0]
+            elif op.name == "mul" and _splat(op.operands[0]) == 1.0 and \
+                    tuple(op.operands[1].shape) == tuple(r.shape) and op.operands[1].dtype == r.dtype:
+                rep = op.operands[1]
+            elif op.name in ("add", "sub") and _splat(op.operands[1]) == 0.0 and \
                     tuple(op.operands[0].shape) == tuple(r.shape) and op.operands[0].dtype == r.dtype:
                 rep = op.operands[0]
             if rep is not None:

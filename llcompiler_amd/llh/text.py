@@ -127,8 +127,8 @@ def _split_top(text, sep=","):
 
 # ------------------------------------------------------------------------------------------ types
 class _Type:
-    def __init__(self, kind, shape=(), dtype=None, symbols=None):
-        self.kind, self.shape, self.dtype, self.symbols = kind, tuple(shape), dtype, symbols
+    def __init__(self, kind, shape=(), dtype=None, symbols=None, ranked=True):
+        self.kind, self.shape, self.dtype, self.symbols, self.ranked = kind, tuple(shape), dtype, symbols, ranked
 
 
 def _parse_type(text):
@@ -148,6 +148,8 @@ def _parse_type(text):
     dtype = _DTYPES.get(toks[-1].strip())
     if dtype is None:
         raise LLHSyntaxError("element type in %r" % text)
+    if toks[0].strip() == "*":  # tensor<*xf32>: rank and extents are whatever shape inference says
+        return _Type("tensor", (), dtype, None, ranked=False)
     dims = []
     for t in toks[:-1]:
         t = t.strip()
@@ -260,7 +262,7 @@ class _Reader:
         for k, d in enumerate(ty.shape):
             if d is not None:
                 shape.append(d)
-            elif ty.symbols and k < len(ty.symbols) and not re.fullmatch(r"c\d+", ty.symbols[k]):
+            elif ty.symbols and k < len(ty.symbols) and ty.symbols[k] and not re.fullmatch(r"c\d+", ty.symbols[k]):
                 shape.append(Expr.sym(ty.symbols[k]))
             else:
                 shape.append(Expr.sym(self.fresh_symbol()))
@@ -298,12 +300,15 @@ class _Reader:
             return t.shape[k % t.rank]
         if rt.kind == "scalar" and name in ("add", "sub", "mul", "div"):
             a, b = (self.scalar(o) for o in operands)
+            if name == "div" and not isinstance(b, Expr) and b == 0:
+                raise NotImplementedError("llh.div of scalars by the constant 0")
             return {"add": lambda: a + b, "sub": lambda: a - b, "mul": lambda: a * b, "div": lambda: a // b}[name]()
         if name == "print":
             self.printed.append(self.tensor(operands[0]))
             return None
         if name == "weight":
-            return g.add_op("weight", [], {"weight_file": attrs["weight_file"]}, shapes=[tuple(rt.shape)], dtypes=[rt.dtype])
+            shape = tuple(rt.shape) if len(rt.shape) else (1,)  # tensor<f32> is refined to tensor<1xf32>
+            return g.add_op("weight", [], {"weight_file": attrs["weight_file"]}, shapes=[shape], dtypes=[rt.dtype])
         if name in UNARY_OPS or name in BINARY_OPS or name in ("where", "matmul", "batch_matmul", "softmax", "identity", "gather"):
             ins = [self.tensor(o) for o in operands]
             return g.add_op(name, ins, {"axis": ins[0].rank - 1} if name == "softmax" else {})
@@ -344,6 +349,8 @@ class _Reader:
             a = {"shape": shape}
             if name == "broadcast_to":
                 a["cast_dims"] = tuple(attrs.get("cast_dims", range(len(shape))))
+                if "noexpand_dims" in attrs:
+                    a["noexpand_dims"] = tuple(attrs["noexpand_dims"])
                 return g.add_op(name, [x], a)
             return g.add_op(name, [x], a, shapes=[_resolve(x, shape)], dtypes=[x.dtype])
         if name == "stride_slice":
@@ -357,9 +364,13 @@ class _Reader:
             return g.add_op(name, [x], {"start": tuple(st), "end": tuple(en), "stride": tuple(sp)})
         if name == "extract":
             idx = self.scalar(operands[1]) if len(operands) > 1 else attrs["index"]
+            if isinstance(idx, Expr):
+                raise NotImplementedError("llh.extract with a symbolic index")
             return g.add_op(name, [self.tensor(operands[0])], {"index": int(idx)})
         if name == "flatten":
             x = self.tensor(operands[0])
+            if not rt.ranked:
+                raise NotImplementedError("llh.flatten with an unranked result type")
             return g.add_op("reshape", [x], {"shape": tuple(rt.shape)}, shapes=[_resolve(x, tuple(-1 if d is None else d for d in rt.shape))],
                             dtypes=[x.dtype])
         raise NotImplementedError("llh.%s has no reader" % name)
@@ -373,6 +384,11 @@ class _Reader:
                 if not c.take(","):
                     break
             c.expect("=")
+        m = c.match(r"(?:arith|index)\.constant\s*(?:\{[^}]*\}\s*)?(-?\d+)(?:\s*:\s*(?:i64|i32|index))?")
+        if m:  # the scalar side also appears in MLIR's custom syntax: %c3 = arith.constant 3 : i64
+            if results:
+                self.env[results[0]] = int(m.group(1))
+            return
         m = c.match(r'"([\w.]+)"')
         if not m:
             raise LLHSyntaxError("operation expected at ...%s" % c.s[c.i:c.i + 40].replace("\n", " "))
@@ -399,7 +415,11 @@ class _Reader:
             raise NotImplementedError("operation %s (only the llh dialect is read)" % full)
         value = self.emit(full[4:], operands, attrs, rtypes)
         if results:
-            if isinstance(value, Value) and rtypes and rtypes[0].kind == "tensor" and len(rtypes[0].shape) != value.rank:
+            # (a printed tensor<f32> for a one-element result is what the importer writes; the reference's
+            # legalisation refines it to tensor<1xf32>, Operationlegalization.cpp:152-193)
+            scalar_as_1 = isinstance(value, Value) and rtypes and len(rtypes[0].shape) == 0 and tuple(value.shape) == (1,)
+            if isinstance(value, Value) and rtypes and rtypes[0].kind == "tensor" and rtypes[0].ranked and not scalar_as_1 and \
+                    len(rtypes[0].shape) != value.rank:
                 raise LLHSyntaxError("%%%s: printed type has rank %d, inferred rank %d" % (results[0], len(rtypes[0].shape), value.rank))
             self.env[results[0]] = value
 
@@ -409,8 +429,9 @@ def _resolve(x, shape):
     return resolve_reshape(x.shape, shape)
 
 
-def parse_llh(text, func=None):
-    """Parses the (first, or named) func.func of `text` into a Graph."""
+def parse_llh(text, func=None, ssa=None):
+    """Parses the (first, or named) func.func of `text` into a Graph.  `ssa`, if given, is a dict that is filled with what every
+    SSA name of the function stands for (a graph Value, an int, or a symbolic extent)."""
     text = _strip_comments(text)
     pat = r"func\.func\s+(?:private\s+|public\s+)?@(%s)\s*\(" % (re.escape(func) if func else r"[\w.$-]+")
     m = re.search(pat, text)
@@ -423,7 +444,13 @@ def parse_llh(text, func=None):
         am = re.match(r"%([\w.$-]+)\s*:\s*(.*?)(\s*\{.*\})?$", arg, re.S)
         if not am:
             raise LLHSyntaxError("argument %r" % arg)
-        r.add_argument(am.group(1), _parse_type(am.group(2)))
+        ty = _parse_type(am.group(2))
+        if am.group(3) and ty.kind == "tensor" and not ty.symbols:
+            # {func.input_symbol_0 = "s0", ...}: which symbol every extent of the argument is (fx_translate.py:197-224)
+            bound = dict((int(k), v) for k, v in re.findall(r'func\.input_symbol_(\d+)\s*=\s*"([^"]+)"', am.group(3)))
+            if bound:
+                ty.symbols = [bound.get(k, "") for k in range(len(ty.shape))]
+        r.add_argument(am.group(1), ty)
     if c.take("->"):
         if c.peek("("):
             c.bracketed("(", ")")
@@ -450,6 +477,8 @@ def parse_llh(text, func=None):
             break
         r.statement(body)
     outs = returned if returned else r.printed
+    if ssa is not None:
+        ssa.update(r.env)
     r.g.set_outputs(list(outs))
     r.g.single_output = len(outs) == 1
     return r.g

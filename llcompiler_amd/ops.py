@@ -216,12 +216,17 @@ def stride_slice(x, start, end, step, out=None, defer=False):
 
 def extract(x, index, out=None, defer=False):
     """llh.extract: row `index` of dim 0 with the dim dropped; a negative index counts from the end
-    (src/Dialect/LLH/IR/LLHCanonicalize.cpp:337-354)."""
+    (src/Dialect/LLH/IR/LLHCanonicalize.cpp:337-354); one element of a vector comes back as tensor<1>
+    (src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:513-516)."""
     dev = _dev(x)
     if index < 0:
         index += x.shape[0]
     if out is None:
-        out = torch.empty(tuple(x.shape[1:]), dtype=x.dtype, device=dev)
+        out = torch.empty(tuple(x.shape[1:]) if x.dim() > 1 else (1,), dtype=x.dtype, device=dev)
+    if x.dim() == 1:
+        rx, ro = C.tensor_ref(x), C.tensor_ref(out)
+        a, b, c = C.i64_array([index]), C.i64_array([index + 1]), C.i64_array([1])
+        return _launch(C.lib().llc_hip_stride_slice, (rx.ptr, a, b, c, ro.ptr), (rx, ro, a, b, c), out, dev, defer)
     start = [index] + [0] * (x.dim() - 1)
     end = [index + 1] + list(x.shape[1:])
     ro = C.tensor_ref(out, (1,) + tuple(out.shape), (max(out.numel(), 1),) + tuple(out.stride()))

@@ -200,7 +200,8 @@ def stride_slice(x, start, end, step):
 
 def extract(x, index):
     x = np.ascontiguousarray(x)
-    y = np.empty(x.shape[1:], x.dtype)
+    # (one element of a vector stays a tensor<1>: LLHinfersymbolShape.cpp:513-516)
+    y = np.empty(x.shape[1:] if x.ndim > 1 else (1,), x.dtype)
     lib().llc_ref_extract(_p(x), _p(y), x.ndim, _i64v(x.shape), _c64(index), x.itemsize)
     return y
 

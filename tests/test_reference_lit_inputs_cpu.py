@@ -1,0 +1,174 @@
+"""The reference's own lit test inputs, read where they lie (nothing of them is copied into this repository), fed to
+the LLH text reader and to this build's shape inference.  The reference tree is only present on the build machine:
+without it these tests skip.
+
+test/Dialect/LLH/symbol_infer/infer_symbol_shape.mlir gives every op an unranked result type (tensor<*xf32>) and
+holds, in its CHECK-SAME lines, the type the reference's --infer-symbol-shape pass must produce: those are known
+answers for llh/infer.py, including which extents are static and which dynamic extents are the same symbol."""
+import glob
+import os
+import re
+
+import pytest
+
+from llcompiler_amd.llh.expr import Expr
+from llcompiler_amd.llh.graph import Value
+from llcompiler_amd.llh.text import LLHSyntaxError, parse_llh
+
+REF_TESTS = "/root/reference/test"
+pytestmark = pytest.mark.skipif(not os.path.isdir(REF_TESTS), reason="the reference tree is not on this machine")
+
+
+def _functions(path):
+    """(function name, text of its split) for every func.func of a lit file (splits are separated by // -----)."""
+    for chunk in re.split(r"//\s*-----", open(path).read()):
+        for name in re.findall(r"func\.func\s+@([\w\-.]+)", chunk):
+            yield name, chunk
+
+
+def test_reader_takes_the_reference_lit_inputs():
+    """Every function of every lit file either parses or is refused for a stated reason (ops of other dialects in
+    custom syntax, ops the backend has no counterpart for, NHWC convolutions): never a crash, and the LLH dialect's
+    own test files parse almost completely."""
+    parsed, refused = [], []
+    for path in sorted(glob.glob(REF_TESTS + "/**/*.mlir", recursive=True)):
+        for name, chunk in _functions(path):
+            where = "%s:@%s" % (path[len(REF_TESTS) + 1:], name)
+            try:
+                parse_llh(chunk, func=name)
+                parsed.append(where)
+            except (LLHSyntaxError, NotImplementedError) as e:
+                refused.append((where, str(e)))
+    assert len(parsed) >= 85, "only %d of %d functions parsed" % (len(parsed), len(parsed) + len(refused))
+    llh_dialect = [w for w in parsed if w.startswith("Dialect/LLH/") and "/symbol_infer/" not in w]
+    llh_refused = [w for w, _ in refused if w.startswith("Dialect/LLH/") and "/symbol_infer/" not in w]
+    assert len(llh_dialect) >= 30 and len(llh_refused) <= 3, (llh_refused,)
+    for where, why in refused:
+        assert why, where
+
+
+def _expected_types(chunk):
+    """SSA name -> (op, dims, symbols) from `// CHECK: llh.<op>` / `// CHECK-SAME: [->] tensor<...>` pairs: the type
+    belongs to the next statement of that op."""
+    lines = chunk.splitlines()
+    out = {}
+    for i, line in enumerate(lines):
+        m = re.match(r"\s*//\s*CHECK-SAME:\s*(?:->\s*)?tensor<([^,>]*)(?:,\s*#llh\.encoding<shapes\s*=\s*([^>]*)>)?>\s*$", line)
+        if not m or i == 0:
+            continue
+        op = re.match(r"\s*//\s*CHECK:\s*llh\.(\w+)", lines[i - 1])
+        if not op:
+            continue
+        for later in lines[i + 1:]:
+            st = re.match(r'\s*%([\w.$-]+)\s*=\s*"llh\.(\w+)"', later)
+            if st and st.group(2) == op.group(1) and st.group(1) not in out:
+                dims = m.group(1).split("x")[:-1]
+                syms = [t.strip().lstrip("@") for t in m.group(2).split(",")] if m.group(2) else None
+                out[st.group(1)] = (op.group(1), dims, syms)
+                break
+    return out
+
+
+def test_shape_inference_agrees_with_the_reference_known_answers():
+    path = REF_TESTS + "/Dialect/LLH/symbol_infer/infer_symbol_shape.mlir"
+    checked, ops_seen = 0, set()
+    for name, chunk in _functions(path):
+        ssa = {}
+        try:
+            parse_llh(chunk, func=name, ssa=ssa)
+        except NotImplementedError:
+            continue          # llh.empty, llh.batch_norm (training form): no counterpart here
+        expected = _expected_types(chunk)
+        by_symbol = {}
+        for ssa_name, (op, dims, syms) in expected.items():
+            v = ssa.get(ssa_name)
+            assert isinstance(v, Value), "@%s %%%s (%s): not a tensor here" % (name, ssa_name, op)
+            mine = ["?" if isinstance(d, Expr) else str(d) for d in v.shape]
+            assert mine == dims, "@%s %%%s = llh.%s: the reference infers %s, this build %s" % (name, ssa_name, op, dims, v.shape)
+            checked += 1
+            ops_seen.add(op)
+            # extents the reference gives the same symbol must be the same expression here
+            for d, s in zip(v.shape, syms or []):
+                if isinstance(d, Expr) and re.fullmatch(r"s\d+", s):
+                    by_symbol.setdefault(s, []).append((ssa_name, d))
+        for s, uses in by_symbol.items():
+            first = uses[0][1]
+            for ssa_name, d in uses[1:]:
+                assert str(d) == str(first), "@%s: the reference calls both extents @%s; here %s vs %s (%%%s)" % (name, s, first, d, ssa_name)
+    assert checked >= 20, checked
+    assert {"transpose", "max_pool", "reshape", "adaptive_average_pool", "matmul", "batch_matmul", "stride_slice", "conv",
+            "broadcast_to", "extract", "where", "reduce_max"} <= ops_seen, ops_seen
+
+
+def _filecheck_lite(printed, directives):
+    """The reference's CHECK / CHECK-NOT / CHECK-COUNT-n / CHECK-SAME lines, restricted to those that name an
+    llh op, against the printed graph: CHECK finds the next line with the pattern, CHECK-SAME looks at the same
+    line, CHECK-NOT forbids the pattern between its neighbours' matches (or up to the end)."""
+    lines = printed.splitlines()
+    pos, pending_not = 0, []
+    for kind, pat in directives:
+        if kind == "CHECK-NOT":
+            pending_not.append(pat)
+            continue
+        if kind == "CHECK-SAME":
+            assert pos > 0 and pat in lines[pos - 1], "CHECK-SAME %r not on line %r" % (pat, lines[pos - 1] if pos else None)
+            continue
+        count = int(kind.split("-")[-1]) if kind.startswith("CHECK-COUNT") else 1
+        for _ in range(count):
+            hit = next((k for k in range(pos, len(lines)) if pat in lines[k]), None)
+            assert hit is not None, "CHECK %r not found after line %d of:\n%s" % (pat, pos, printed)
+            for bad in pending_not:
+                assert not any(bad in l for l in lines[pos:hit]), "CHECK-NOT %r violated in:\n%s" % (bad, printed)
+            pending_not = []
+            pos = hit + 1
+    for bad in pending_not:
+        assert not any(bad in l for l in lines[pos:]), "CHECK-NOT %r violated in:\n%s" % (bad, printed)
+
+
+# (file, function, which of its directives apply here: all those naming these op spellings)
+_PASS_LEVEL = [
+    ("Dialect/LLH/canonicalize.mlir", "fold_two_abs", ("llh.abs",)),
+    ("Dialect/LLH/canonicalize.mlir", "fold_reshape", ("llh.reshape",)),
+    ("Dialect/LLH/canonicalize.mlir", "fold_broadcast", ("llh.broadcast_to",)),
+    ("Dialect/LLH/canonicalize.mlir", "fold_convert_to", ("llh.convert_to",)),
+    ("Dialect/LLH/fold.mlir", "add_zore_fold", ("llh.add",)),
+    ("Dialect/LLH/fold.mlir", "sub_same_fold", ("llh.sub",)),
+    ("Dialect/LLH/fold.mlir", "mul_fold", ("llh.mul",)),
+    ("Dialect/LLH/decompose_ops.mlir", "batch_norm", ("llh.add", "llh.sqrt", "llh.reshape", "llh.broadcast_to", "llh.sub", "llh.mul",
+                                                      "llh.div", "llh.batch_norm_inference")),
+    ("Dialect/LLH/operation-legalization.mlir", "extract", ("llh.extract", "-> tensor<1xf32>")),
+    ("Dialect/LLH/operation-legalization.mlir", "weight_refine", ("llh.weight", "-> tensor<1xf32>")),
+]
+
+
+@pytest.mark.parametrize("path,func,patterns", _PASS_LEVEL)
+def test_rewrites_satisfy_the_reference_check_lines(path, func, patterns):
+    """The reference's pass-level expectations (its FileCheck lines) hold for this build's rewrites of the same input,
+    for the passes it has a counterpart of: canonicalisation and folding, batch-norm decomposition, and the
+    refinement of one-element results to tensor<1xT>."""
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    from llcompiler_amd.llh.text import _type_str
+
+    def listing(g):   # one line per op: name and result type, in the reference's spelling
+        return "\n".join('%%%s = "llh.%s"(%s) -> %s' % (op.results[0].name, op.name, ", ".join("%" + o.name for o in op.operands),
+                                                      _type_str(op.results[0])) for op in g.ops)
+    ran = 0
+    for name, chunk in _functions(REF_TESTS + "/" + path):
+        if name != func:
+            continue
+        body = chunk[chunk.index("@" + func):]
+        directives = []
+        for kind, pat in re.findall(r"//\s*(CHECK(?:-NOT|-COUNT-\d+|-SAME)?):\s*(.*)", body):
+            pat = pat.strip()
+            if any(pat == p or (p.startswith("->") and pat == p) for p in patterns):
+                directives.append((kind, pat))
+        try:
+            g = parse_llh(chunk, func=func)
+        except NotImplementedError:
+            continue          # (a second function of the same name with scalar-only content)
+        if not any(op.results[0].rank >= 0 for op in g.ops) and not directives:
+            continue
+        run_llh_pipeline(g)
+        _filecheck_lite(listing(g), directives)
+        ran += 1
+    assert ran >= 1, "no function @%s in %s" % (func, path)
