@@ -159,9 +159,12 @@ def _view(ctx, node):
     return _reshape_to(ctx, ctx.val(node.args[0]), _out_shape(node))
 
 
+# (prims.inductor_force_stride_order asks for a memory layout, not for other values: layouts travel in the
+# strides here; the reference rebuilds the shape from the strides, reshape_ops.py:110-140)
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.clone.default, aten.contiguous.default, aten.alias.default,
                                    aten.detach.default, aten.lift_fresh_copy.default, aten._to_copy.default,
-                                   prims.convert_element_type.default)
+                                   prims.convert_element_type.default, prims.clone.default,
+                                   prims.inductor_force_stride_order.default)
 def _identity_or_convert(ctx, node):
     x = ctx.val(node.args[0])
     dt = _out_dtype(node)
@@ -396,6 +399,13 @@ def _float_reduce(node):
 TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amax.default, check=_float_reduce)(_reduce("reduce_max"))
 TORCH_FUNCTION_TRANSLATE_REGISTER(aten.amin.default, check=_float_reduce)(_reduce("reduce_min"))
 TORCH_FUNCTION_TRANSLATE_REGISTER(aten.sum.dim_IntList, check=_float_reduce)(_reduce("reduce_sum"))
+TORCH_FUNCTION_TRANSLATE_REGISTER(prims.sum.default, check=_float_reduce)(_reduce("reduce_sum"))  # (x, dims): never keepdim
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(prims.collapse_view.default)
+def _collapse_view(ctx, node):
+    """Dims start .. end (inclusive) become one (fx_op_translate/reshape_ops.py:89-107)."""
+    return _reshape_to(ctx, ctx.val(node.args[0]), _out_shape(node))
 
 
 def _mean_ok(node):

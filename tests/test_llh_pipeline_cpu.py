@@ -245,3 +245,27 @@ def test_parameters_become_weight_ops_naming_npy_files(tmp_path):
         np.testing.assert_array_equal(arr, want[arr.shape])
     kinds = [s.kind for s in cm.engine.steps if s.kind != "view"]
     assert kinds.count("weight") == 4 and kinds.count("matmul") == 2
+
+
+def test_prims_level_nodes_are_translated():
+    """Graphs that arrive at prims level (what inductor's decompositions leave): prims.collapse_view, prims.sum,
+    prims.clone and prims.inductor_force_stride_order have translators like in the reference
+    (fx_op_translate/reshape_ops.py:89-140, reduce_ops.py:85-118, identity.py:51-59)."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from llcompiler_amd.importer.fx_importer import torch_translate_to_llh_graph
+    prims = torch.ops.prims
+
+    def f(x):
+        y = prims.collapse_view(x, 1, 2)
+        z = prims.sum(y, [1])
+        return prims.clone(prims.inductor_force_stride_order(z, (5, 1)))
+
+    gm = make_fx(f, tracing_mode="fake")(torch.zeros(3, 4, 6, 5))
+    g = torch_translate_to_llh_graph(gm)
+    names = g.op_names()
+    assert names.count("reshape") == 1 and names.count("reduce_sum") == 1, names
+    shapes = {op.name: tuple(op.results[0].shape) for op in g.ops}
+    assert shapes["reshape"] == (3, 24, 5) and shapes["reduce_sum"] == (3, 5)
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    run_llh_pipeline(g)
+    assert g.op_names() == ["reshape", "reduce_sum"]          # the identities are gone
