@@ -163,14 +163,24 @@ def _view(ctx, node):
 # strides here; the reference rebuilds the shape from the strides, reshape_ops.py:110-140)
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.clone.default, aten.contiguous.default, aten.alias.default,
                                    aten.detach.default, aten.lift_fresh_copy.default, aten._to_copy.default,
-                                   prims.convert_element_type.default, prims.clone.default,
-                                   prims.inductor_force_stride_order.default)
+                                   prims.convert_element_type.default, prims.clone.default)
 def _identity_or_convert(ctx, node):
     x = ctx.val(node.args[0])
     dt = _out_dtype(node)
     if dt != x.dtype:
         return ctx.g.add_op("convert_to", [x], {"dtype": dt})
     return ctx.g.add_op("identity", [x])
+
+
+def register_inductor_prims():
+    """prims.inductor_force_stride_order only exists once torch._inductor has been imported (it defines the op): called
+    at import time here and again by the backend before it translates a graph."""
+    op = getattr(prims, "inductor_force_stride_order", None) if "inductor_force_stride_order" in dir(prims) else None
+    if op is not None:
+        TORCH_FUNCTION_TRANSLATE[op.default] = _identity_or_convert
+
+
+register_inductor_prims()
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(prims.broadcast_in_dim.default)
@@ -541,6 +551,8 @@ def is_supported(node):
     if node.target in _SYMBOLIC_TARGETS:
         return True
     if node.target not in TORCH_FUNCTION_TRANSLATE:
+        register_inductor_prims()
+    if node.target not in TORCH_FUNCTION_TRANSLATE:
         return False
     chk = _SUPPORT_CHECKS.get(node.target)
     try:
@@ -554,6 +566,7 @@ def torch_translate_to_llh_graph(gm, weight_files=None):
 
     weight_files: {placeholder name: .npy path}.  Those placeholders become llh.weight ops that name their file
     (fx_translate.py:415-435 does this for the parameters of the traced module) instead of run-time inputs."""
+    register_inductor_prims()
     g = Graph()
     ctx = Ctx(g)
     weight_files = weight_files or {}

@@ -253,6 +253,9 @@ def test_prims_level_nodes_are_translated():
     (fx_op_translate/reshape_ops.py:89-140, reduce_ops.py:85-118, identity.py:51-59)."""
     from torch.fx.experimental.proxy_tensor import make_fx
     from llcompiler_amd.importer.fx_importer import torch_translate_to_llh_graph
+    import torch._inductor.inductor_prims  # noqa: F401  (defines prims.inductor_force_stride_order)
+    from llcompiler_amd.importer.fx_importer import register_inductor_prims
+    register_inductor_prims()
     prims = torch.ops.prims
 
     def f(x):
