@@ -5,7 +5,8 @@ import torch.nn.functional as F
 
 __all__ = ["Add", "Sub", "Mul", "Div", "Abs", "Relu", "ElewiseFusion1", "Matmul", "BatchMatmul", "Linear", "Conv2D_NCHW_FCHW",
            "MaxPool2D", "ReduceFusion1", "Where", "Transpose", "Slice", "BatchNorm2D_Inference", "LayerNorm", "Softmax", "Gelu",
-           "Extract", "Embedding"]
+           "Extract", "Embedding", "Braodcast", "Unsqueeze", "RecudeMax", "RecudeSum", "Sqrt", "Exp", "EQ", "Drop",
+           "BatchNorm1D_Inference", "Decompose_BatchNorm", "Where3", "Slice2", "Extract3", "MaxPool2D_Twice"]
 
 
 class Add(nn.Module):
@@ -155,3 +156,112 @@ class Embedding(nn.Module):
 
     def forward(self, idx):
         return self.emb(idx) * 2
+
+
+# ---- the remaining modules of the reference's llcompiler/test_models/ops/*.py, by behaviour (names as there) ----
+class Braodcast(nn.Module):
+    """A [M,N] tensor added to itself viewed as [1,M,N] and as [M,1,N] (braodcast.py: rank-extending broadcasts)."""
+
+    def forward(self, x):
+        a = x + x.reshape(1, x.shape[0], x.shape[1])
+        b = x + x.reshape(x.shape[0], 1, x.shape[1])
+        return a + b
+
+
+class Unsqueeze(nn.Module):
+    def forward(self, x):
+        return x.unsqueeze(1) + x.unsqueeze(1)
+
+
+class RecudeMax(nn.Module):
+    """amax over dim rank-of-batch-1 with and without keepdim (squeezed), then over the last dim (reduce.py)."""
+
+    def forward(self, x):
+        d = x.shape[0] - 1
+        y = x.amax(d, keepdim=False) + x.amax(d, keepdim=True).squeeze(d)
+        return y.amax(-1, keepdim=True)
+
+
+class RecudeSum(nn.Module):
+    def forward(self, x):
+        d = x.shape[0] - 1
+        y = x.sum(d, keepdim=False) + x.sum(d, keepdim=True).squeeze(d)
+        return y.sum(-1, keepdim=True)
+
+
+class Sqrt(nn.Module):
+    def forward(self, x):
+        return x.sqrt()          # NaN for negative inputs, in eager and compiled alike
+
+
+class Exp(nn.Module):
+    def forward(self, x):
+        return x.exp()
+
+
+class EQ(nn.Module):
+    def forward(self, x):
+        return (x == x) == 2     # a bool compared with 2: all False
+
+
+class Drop(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.drop = nn.Dropout()
+
+    def forward(self, x):
+        return self.drop(x)      # identity in inference
+
+
+class BatchNorm1D_Inference(nn.Module):
+    def __init__(self, c=3):
+        super().__init__()
+        self.bn = nn.BatchNorm1d(c)
+        gen = torch.Generator().manual_seed(1)
+        self.bn.running_mean.data = torch.randn(c, generator=gen)
+        self.bn.running_var.data = torch.rand(c, generator=gen) + 0.5
+
+    def forward(self, x):
+        for _ in range(4):
+            x = self.bn(x)
+        return x
+
+
+class Decompose_BatchNorm(nn.Module):
+    """linear -> batch norm -> relu, twice, then flatten (decompose.py)."""
+
+    def __init__(self):
+        super().__init__()
+        self.l1, self.b1 = nn.Linear(224, 100), nn.BatchNorm1d(100)
+        self.l2, self.b2 = nn.Linear(100, 10), nn.BatchNorm1d(10)
+
+    def forward(self, x):
+        x = F.relu(self.b1(self.l1(x)))
+        x = F.relu(self.b2(self.l2(x)))
+        return torch.flatten(x, 1)
+
+
+class Where3(nn.Module):
+    """where.py: x.where(pred, y) + y with the predicate as an input."""
+
+    def forward(self, pred, x, y):
+        return x.where(pred, y) + y
+
+
+class Slice2(nn.Module):
+    def forward(self, x):
+        return x[0:3] + x[3:6]
+
+
+class Extract3(nn.Module):
+    def forward(self, x):
+        return x[1] + x[-2] + x[0]
+
+
+class MaxPool2D_Twice(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.pool = nn.MaxPool2d(5, 1, 2, 2)
+
+    def forward(self, x):
+        return self.pool(self.pool(x))

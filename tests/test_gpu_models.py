@@ -693,3 +693,56 @@ def test_random_networks_training_mode(seed):
                 assert p.grad is None, name
                 continue
             _assert_as_close_as_eager(host(p.grad), host(q.grad), host(d.grad), 1e-4, 1e-5 * scale, what + " grad of %s, step %d" % (name, step))
+
+
+# The reference's python op tests (test/python/ops/*.py): module, input shapes, and which of the four modes
+# check_model / check_static_model / check_static_model_inference runs there (utility.py:79-138).
+_REFERENCE_OP_TESTS = [
+    ("Abs", [(3, 3, 224, 224)], "all"), ("Add", [(3, 3, 224, 224)], "all"), ("BatchMatmul", [(3, 224, 112), (3, 224, 112)], "all"),
+    ("BatchNorm1D_Inference", [(3, 3, 224)], "static_inference"), ("BatchNorm2D_Inference", [(3, 3, 224, 224)], "static_inference"),
+    ("Braodcast", [(224, 112)], "all"), ("Conv2D_NCHW_FCHW", [(3, 3, 224, 224)], "static"), ("Div", [(3, 3, 100)], "all"),
+    ("Extract3", [(3, 3, 224, 224)], "all"), ("Linear", [(10, 100000)], "all"), ("Matmul", [(3, 3), (3, 3)], "all"),
+    ("MaxPool2D_Twice", [(3, 3, 224, 224)], "static"), ("Mul", [(3, 3, 224, 224)], "all"), ("RecudeMax", [(3, 3, 224, 224)], "all"),
+    ("RecudeSum", [(3, 3, 224, 224)], "all"), ("Relu", [(3, 3, 224, 224)], "all"), ("Sqrt", [(3, 3, 224, 224)], "all"),
+    ("Sub", [(3, 3, 224, 224)], "all"), ("Unsqueeze", [(3, 3, 224, 224)], "all"), ("Where3", [(1000, 224), (1000, 224), (1000, 224)], "all"),
+    ("Exp", [(3, 3, 24, 24)], "all"), ("EQ", [(3, 3, 24, 24)], "static_inference"), ("Drop", [(3, 3, 24, 24)], "static_inference"),
+    ("Decompose_BatchNorm", [(6, 224)], "static_inference"), ("Slice2", [(6, 5, 9)], "all"),
+]
+
+
+@pytest.mark.parametrize("name,shapes,modes", _REFERENCE_OP_TESTS, ids=[t[0] for t in _REFERENCE_OP_TESTS])
+def test_reference_op_tests_in_their_four_modes(name, shapes, modes):
+    """static / dynamic x inference / training, each compared with eager like the reference's check_model does (forward
+    outputs, NaNs equal), at the reference's input shapes.  Its tolerance is 1e-5; sums over 1e5 products (Linear) and
+    over 224 values need this build's fp32 bar."""
+    from llcompiler_amd import LLCompiler
+    import llcompiler_amd.test_models as tm
+    gen = torch.Generator().manual_seed(11)
+    inputs = [torch.randn(s, generator=gen) for s in shapes]
+    if name == "Where3":
+        inputs[0] = torch.ones(shapes[0], dtype=torch.bool)
+        inputs[0][::3] = False
+    kwargs = {"n_in": 100000} if name == "Linear" else {}
+    base = getattr(tm, name)(**kwargs)
+    plan = {"all": [(False, "inference"), (False, "training"), (True, "inference"), (True, "training")],
+            "static": [(False, "inference"), (False, "training")], "static_inference": [(False, "inference")]}[modes]
+    for dynamic, mode in plan:
+        torch._dynamo.reset()
+        m = copy.deepcopy(base).train(mode == "training").cuda()
+        ref = copy.deepcopy(base).train(mode == "training")
+        comp = LLCompiler(mode=mode, target="gfx950", pipeline="hip")
+        opt = torch.compile(m, backend=comp, dynamic=dynamic, fullgraph=True)
+        if mode == "inference":
+            with torch.no_grad():
+                want = ref(*inputs)
+                got = opt(*[t.cuda() for t in inputs])
+        else:
+            want = ref(*inputs)
+            got = opt(*[t.cuda() for t in inputs])
+        what = "%s, %s %s" % (name, "dynamic" if dynamic else "static", mode)
+        if want.dtype == torch.bool:
+            assert torch.equal(got.cpu(), want), what
+        else:
+            scale = max(1.0, float(want.detach().abs().nan_to_num(0.0, 0.0, 0.0).max()))
+            assert_close(got.detach().cpu().numpy(), want.detach().numpy(), F32_RTOL, F32_ATOL * scale, what)
+        assert comp.compile_count >= 1, what
