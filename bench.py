@@ -223,6 +223,11 @@ def model_latencies(which=MODELS):
             xs = make_resnet_inputs(16, 224)[0].cuda()
             cr = compile_module(ResNet18Folded().cuda(), (xs,))
             res["resnet18_f32_batch16_ms"] = timed(lambda: cr(xs), 20, 3)
+            # the same network in bf16 storage (not one of the five configurations: its convolutions run on the
+            # bf16 matrix instructions, which the fp32 configuration cannot show)
+            xh = xs.to(torch.bfloat16)
+            ch = compile_module(ResNet18Folded().to(torch.bfloat16).cuda(), (xh,))
+            res["resnet18_bf16_batch16_ms"] = timed(lambda: ch(xh), 20, 3)
         if "encoder" in which:
             xe = make_encoder_inputs(8, 512)[0].to(torch.bfloat16).cuda()
             ce = compile_module(EncoderBlock().to(torch.bfloat16).cuda(), (xe,),

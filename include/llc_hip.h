@@ -131,8 +131,8 @@ typedef struct llc_conv_attrs {
 /* Cross-correlation as implicit GEMM (LLHToHLO.cpp:214-270).  conv_bias is `epi->bias`.
  * Layout travels in the strides, as in torch: either every tensor (x, w, out, epilogue residual) is contiguous
  * NCHW / FCHW, or every one is channels-last (NHWC in memory: strides (H W C, 1, W C, C) under the same
- * logical shape), which takes a kernel of its own (fp32, group 1, C % 32 == 0, F % 4 == 0, at most 64 taps;
- * LLC_ERR_UNSUPPORTED otherwise).  Mixed layouts are refused (LLC_ERR_LAYOUT). */
+ * logical shape), which takes a kernel of its own (group 1, C a multiple of 128 bytes' worth of values: 32 fp32,
+ * 64 bf16 / f16; F % 4 == 0, at most 64 taps; LLC_ERR_UNSUPPORTED otherwise).  Mixed layouts are refused (LLC_ERR_LAYOUT). */
 int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* attrs, const llc_epilogue* epi,
                    llc_tensor* out, void* stream);
 

@@ -523,20 +523,21 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Channels-last (NHWC) fp32 convolution: x [N,C,H,W] with strides (HWC, 1, WC, C), weight [F,C,KH,KW] with
-// strides (KH KW C, 1, KW C, C), output and residual channels-last too.
+// Channels-last (NHWC) convolution, fp32 and the 16-bit types: x [N,C,H,W] with strides (HWC, 1, WC, C), weight
+// [F,C,KH,KW] with strides (KH KW C, 1, KW C, C), output and residual channels-last too.
 //
 // In this layout the im2col matrix needs no gather arithmetic: with k ordered (kh, kw, c) a row of it is, per
-// filter tap, a run of C contiguous floats of the input, and a k-tile of 32 floats (C % 32 == 0) lies inside
-// one tap.  So the convolution is the GEMM  out[pixel, f] = sum_k im2col[pixel, k] * weight[f, k]  with both
+// filter tap, a run of C contiguous values of the input, and a k-tile of 128 bytes (32 floats, 64 16-bit values;
+// C a multiple of that) lies inside one tap.  So the convolution is the GEMM  out[pixel, f] = sum_k im2col[pixel, k] * weight[f, k]  with both
 // operands contiguous along k and the output row-major [pixels, F], i.e. channels-last again, and it runs on
 // the tile machinery of gemm_kernel (LDS layout, fragment reads, MFMA loop, two register stages).  What is
 // specific is the loader of the pixel operand: every lane keeps, for each of its rows, the offset of the
 // window origin and one validity bit per tap, computed once; a k-tile adds one scalar offset (tap, channel
 // block) to them.  A lane spends a handful of integer instructions per 16-byte vector where the NCHW kernel
 // spends about forty on (c, kh, kw) bookkeeping, window clamping and border shifts.
-template <int BM, int NT>
+template <typename T, int BM, int NT>
 struct NhwcLoader {
+  static constexpr int EPV = 16 / (int)sizeof(T);
   static constexpr int kIters = BM * 8 / NT;
   static_assert(BM * 8 % NT == 0 && kIters >= 1 && kIters <= 32, "whole vectors per lane");
   u32x4_t v[kIters];
@@ -567,7 +568,7 @@ struct NhwcLoader {
     }
   }
   // all loads are issued, from offset 0 where the tap falls outside; what was outside is zeroed in store()
-  __device__ __forceinline__ void load(const float* X, const ConvParams& p, int k0) {
+  __device__ __forceinline__ void load(const T* X, const ConvParams& p, int k0) {
     const int tap = k0 / p.C, c0 = k0 - tap * p.C;
     const int kh = tap / p.KW, kw = tap - kh * p.KW;
     const int toff = (kh * p.dh * p.Wd + kw * p.dw) * p.C + c0;
@@ -576,7 +577,7 @@ struct NhwcLoader {
     for (int i = 0; i < kIters; ++i) {
       const int kv = (i * NT + (int)threadIdx.x) & 7;
       const uint32_t ok = (uint32_t)(taps[i] >> tap) & 1u;
-      const int off = ok ? base[i] + toff + kv * 4 : 0;
+      const int off = ok ? base[i] + toff + kv * EPV : 0;
       v[i] = *(const u32x4_t*)(X + off);
       okm |= ok << i;
     }
@@ -591,10 +592,10 @@ struct NhwcLoader {
   }
 };
 
-template <int BM, int BN, int WM, int WN, bool BFULL>
-__global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvParams p) {
+template <typename T, int BM, int BN, int WM, int WN, bool BFULL>
+__global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_kernel(const ConvParams p) {
   constexpr int NT = 64 * WM * WN;
-  constexpr int BK = 32;
+  constexpr int BK = kRowBytes / (int)sizeof(T);
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int kABytes = BM * kRowStride, kBBytes = BN * kRowStride;
@@ -603,8 +604,8 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvP
   int tile_m, tile_n;
   tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const float* X = (const float*)p.X;
-  const float* Wt = (const float*)p.W;
+  const T* X = (const T*)p.X;
+  const T* Wt = (const T*)p.W;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int wm = wave / WN, wn = wave % WN;
   const int li = lane % 32, lh = lane / 32;
@@ -621,11 +622,11 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvP
   const int nk_all = p.Kdim / BK;
   const int split = blockIdx.y;
   const int kt0 = (int)((int64_t)split * nk_all / p.splits), nk = (int)((int64_t)(split + 1) * nk_all / p.splits) - kt0;
-  NhwcLoader<BM, NT> la0, la1;
-  TileLoader<float, BN, kLoadKVec, NT> lb0, lb1;
+  NhwcLoader<T, BM, NT> la0, la1;
+  TileLoader<T, BN, kLoadKVec, NT> lb0, lb1;
   la0.init(p, m0);
 #pragma unroll
-  for (int i = 0; i < NhwcLoader<BM, NT>::kIters; ++i) {
+  for (int i = 0; i < NhwcLoader<T, BM, NT>::kIters; ++i) {
     la1.base[i] = la0.base[i];
     la1.taps[i] = la0.taps[i];
   }
@@ -644,8 +645,8 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvP
       LA2.load(X, p, (kt0 + (KT) + 2) * BK);                                                                    \
       LB2.template load<BFULL>(Wt, n0, p.F, (kt0 + (KT) + 2) * BK, p.Kdim, p.Kdim, 1);                          \
     }                                                                                                           \
-    mma_tile<float, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,        \
-                            wn * WTN + li, lh, acc);                                                            \
+    mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,            \
+                        wn * WTN + li, lh, acc);                                                                \
     if ((KT) + 1 < nk) {                                                                                        \
       LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
       LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
@@ -660,13 +661,13 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvP
 
   // ---- epilogue: register r of lane (li, lh) is row 8 (r/4) + 4 lh + r%4, column li: 32 lanes store 32 consecutive
   //      filters of one pixel ----
-  float* Y = p.splits > 1 ? (float*)p.partial + (int64_t)split * p.ncols * p.F : (float*)p.Y;
+  float* part = (float*)p.partial + (int64_t)split * p.ncols * p.F;
   const char* res = p.splits > 1 ? nullptr : p.residual;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
     if (!BFULL && col >= p.F) continue;
-    const float bv = (p.bias && p.splits == 1) ? ((const float*)p.bias)[col] : 0.0f;
+    const float bv = (p.bias && p.splits == 1) ? load_as_f32(p.bias, Elem<T>::kDtype, col) : 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -674,13 +675,14 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_f32_kernel(const ConvP
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
         if (row >= p.ncols) continue;
         const int64_t o = (int64_t)row * p.F + col;
-        if (p.splits > 1) Y[o] = acc[i][j][r];
-        else epilogue_store<float>(Y, o, acc[i][j][r], p.alpha, bv, res, p.act);
+        if (p.splits > 1) part[o] = acc[i][j][r];
+        else epilogue_store<T>((T*)p.Y, o, acc[i][j][r], p.alpha, bv, res, p.act);
       }
   }
 }
 
 // Sums the split partials [splits][pixels][F] in split order and applies the epilogue (channels-last output).
+template <typename T>
 __global__ __launch_bounds__(256) void nhwc_split_reduce_kernel(const ConvParams p) {
   const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   const int64_t total = (int64_t)p.ncols * p.F;
@@ -689,28 +691,34 @@ __global__ __launch_bounds__(256) void nhwc_split_reduce_kernel(const ConvParams
   f32x4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
   for (int k = 0; k < p.splits; ++k) s += *(const f32x4_t*)(part + (int64_t)k * total);
   const int f = (int)(i4 % p.F);
-  f32x4_t b = {0.0f, 0.0f, 0.0f, 0.0f}, r = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (p.bias) b = *(const f32x4_t*)((const float*)p.bias + f);
-  if (p.residual) r = *(const f32x4_t*)((const float*)p.residual + i4);
-  f32x4_t o;
+  if constexpr (sizeof(T) == 4) {
+    f32x4_t b = {0.0f, 0.0f, 0.0f, 0.0f}, r = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (p.bias) b = *(const f32x4_t*)((const float*)p.bias + f);
+    if (p.residual) r = *(const f32x4_t*)((const float*)p.residual + i4);
+    f32x4_t o;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    float v = s[e] * p.alpha + b[e] + r[e];
-    if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
-    else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
-    o[e] = v;
+    for (int e = 0; e < 4; ++e) {
+      float v = s[e] * p.alpha + b[e] + r[e];
+      if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
+      else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
+      o[e] = v;
+    }
+    *(f32x4_t*)((float*)p.Y + i4) = o;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      epilogue_store<T>((T*)p.Y, i4 + e, s[e], p.alpha, p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, f + e) : 0.0f, p.residual, p.act);
   }
-  *(f32x4_t*)((float*)p.Y + i4) = o;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <typename T, int BM, int BN, int WM, int WN>
 int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   ConvParams p = p0;
   p.tiles_m = (p.ncols + BM - 1) / BM;
   p.tiles_n = (p.F + BN - 1) / BN;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "conv: grid too large");
-  const int nk = p.Kdim / 32;
+  const int nk = p.Kdim / (kRowBytes / (int)sizeof(T));
   // too few tiles for 256 CUs: split the reduction (at least eight k-tiles per split)
   int splits = 1;
   if (tiles < 256 || (BM == 128 && tiles < 384)) {
@@ -726,23 +734,24 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   }
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
   const bool bfull = p.F % BN == 0;
-  auto kern = bfull ? conv_nhwc_f32_kernel<BM, BN, WM, WN, true> : conv_nhwc_f32_kernel<BM, BN, WM, WN, false>;
+  auto kern = bfull ? conv_nhwc_kernel<T, BM, BN, WM, WN, true> : conv_nhwc_kernel<T, BM, BN, WM, WN, false>;
   static bool attr_set[2] = {false, false};
   if (!attr_set[bfull]) {
     LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set[bfull] = true;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)splits, 1), dim3(64 * WM * WN), lds, s, p);
-  LLC_TRY(check_launch("conv_nhwc_f32_kernel"));
+  LLC_TRY(check_launch("conv_nhwc_kernel"));
   if (splits > 1) {
     const int64_t total4 = (int64_t)p.ncols * p.F / 4;
-    hipLaunchKernelGGL(nhwc_split_reduce_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(nhwc_split_reduce_kernel<T>, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, s, p);
     LLC_TRY(check_launch("nhwc_split_reduce_kernel"));
   }
   return LLC_OK;
 }
 
-int launch_nhwc_f32(const ConvParams& p, hipStream_t s) {
+template <typename T>
+int launch_nhwc(const ConvParams& p, hipStream_t s) {
   // 128-pixel tiles when they fill the chip by themselves; else 64 x 64 tiles if those are numerous enough to need
   // no split of the reduction (a split costs a pass over the partial sums: the middle layers of a ResNet); the
   // last layers split either way and do better on the large tiles, unless their reduction is too short to split
@@ -750,10 +759,10 @@ int launch_nhwc_f32(const ConvParams& p, hipStream_t s) {
   const int64_t bn = p.F <= 64 ? 64 : 128;
   const int64_t t128 = (int64_t)((p.ncols + 127) / 128) * ((p.F + bn - 1) / bn);
   const int64_t t64 = (int64_t)((p.ncols + 63) / 64) * ((p.F + 63) / 64);
-  if (t128 < 384 && t64 >= 256) return launch_nhwc_cfg<64, 64, 2, 2>(p, s);
-  const int64_t max_splits = std::max<int64_t>(1, (p.Kdim / 32) / 8);
-  if (t128 * max_splits < 192 && t64 > t128 * max_splits) return launch_nhwc_cfg<64, 64, 2, 2>(p, s);
-  return p.F <= 64 ? launch_nhwc_cfg<128, 64, 4, 2>(p, s) : launch_nhwc_cfg<128, 128, 4, 2>(p, s);
+  if (t128 < 384 && t64 >= 256) return launch_nhwc_cfg<T, 64, 64, 2, 2>(p, s);
+  const int64_t max_splits = std::max<int64_t>(1, (p.Kdim / (kRowBytes / (int)sizeof(T))) / 8);
+  if (t128 * max_splits < 192 && t64 > t128 * max_splits) return launch_nhwc_cfg<T, 64, 64, 2, 2>(p, s);
+  return p.F <= 64 ? launch_nhwc_cfg<T, 128, 64, 4, 2>(p, s) : launch_nhwc_cfg<T, 128, 128, 4, 2>(p, s);
 }
 
 template <typename T, int BM, int BN, int LA>
@@ -889,10 +898,15 @@ int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_att
   }
   hipStream_t s = as_stream(stream);
   if (nhwc) {
-    if (a.dtype != LLC_FLOAT32 || group != 1 || p.C % 32 != 0 || p.KH * p.KW > 64 || p.F % 4 != 0 ||
+    const int ktile = 128 / (int)a.esize();  // values in the 128 bytes of a k-tile: they must share a tap
+    if (group != 1 || p.C % ktile != 0 || p.KH * p.KW > 64 || p.F % 4 != 0 ||
         ((uintptr_t)p.X | (uintptr_t)p.W | (uintptr_t)p.Y | (uintptr_t)p.residual | (uintptr_t)p.bias) % 16 != 0)
-      return set_error(LLC_ERR_UNSUPPORTED, "conv: channels-last tensors need fp32, group 1, C %% 32 == 0, F %% 4 == 0, at most 64 taps and 16-byte alignment");
-    return launch_nhwc_f32(p, s);
+      return set_error(LLC_ERR_UNSUPPORTED, "conv: channels-last tensors need group 1, C %% %d == 0, F %% 4 == 0, at most 64 taps and 16-byte alignment", ktile);
+    switch (a.dtype) {
+      case LLC_FLOAT32: return launch_nhwc<float>(p, s);
+      case LLC_BFLOAT16: return launch_nhwc<__bf16>(p, s);
+      default: return launch_nhwc<_Float16>(p, s);
+    }
   }
   switch (a.dtype) {
     case LLC_FLOAT32: return launch_loaders<float>(p, (int)group, s);

@@ -43,8 +43,8 @@ MIN_CALLS_FOR_GRAPH = 2
 USE_PLAN = True
 # batch_matmul -> softmax -> batch_matmul groups of attention layers with head dim 64 become one fused kernel
 FUSE_ATTENTION = True
-# fp32 convolutions with C % 32 == 0 run on channels-last (NHWC) copies of their operands: the kernel for that
-# layout needs no gather arithmetic.  Results keep the layout as strided views (logical shape NCHW), so a chain of
+# convolutions whose channel count is a multiple of 128 bytes' worth of values (32 fp32, 64 bf16 / f16) run on
+# channels-last (NHWC) copies of their operands: the kernel for that layout needs no gather arithmetic.  Results keep the layout as strided views (logical shape NCHW), so a chain of
 # convolutions converts once; anything that needs NCHW memory copies back through the usual contiguity path.
 CHANNELS_LAST = True
 # linear layers that read the same rows with weights that are graph inputs (q, k, v projections) run as one
@@ -136,12 +136,13 @@ class Instance:
             self.prep_inputs.append(input_index)
 
     def _channels_last_ok(self, st, ins, out, natural):
-        if not CHANNELS_LAST or out.dtype != torch.float32 or st.attrs["group"] != 1 or len(natural) != 4:
+        if not CHANNELS_LAST or out.dtype not in (torch.float32, torch.bfloat16, torch.float16) or \
+                st.attrs["group"] != 1 or len(natural) != 4:
             return False
         x, w = ins
         if tuple(natural) != tuple(out.shape) or not out.numel() or x.dim() != 4 or w.dim() != 4:
             return False
-        return x.shape[1] % 32 == 0 and w.shape[0] % 4 == 0 and w.shape[2] * w.shape[3] <= 64 and \
+        return x.shape[1] % (128 // out.dtype.itemsize) == 0 and w.shape[0] % 4 == 0 and w.shape[2] * w.shape[3] <= 64 and \
             x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
     def _scan(self, item):

@@ -407,6 +407,28 @@ def test_channels_last_weight_copies_follow_the_weights():
         assert_close(cm(x).cpu().numpy(), m(x).cpu().numpy(), F32_RTOL, F32_ATOL, "resnet, weights scaled in place")
 
 
+def test_resnet18_in_bf16_runs_channels_last():
+    """The ResNet configuration in bf16 storage: every convolution but the stem has a multiple of 64 channels and
+    takes the channels-last kernel on the bf16 matrix instructions.  Compared with a float64 evaluation of the same
+    (bf16-valued) weights at the bf16 bar plus what torch's own bf16 evaluation misses it by."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval().to(torch.bfloat16)
+    (x,) = make_resnet_inputs(2, 64)
+    x = x.to(torch.bfloat16)
+    with torch.no_grad():
+        want64 = copy.deepcopy(m).double()(x.double())
+        eager = m(x)
+        mg = copy.deepcopy(m).cuda()
+        cm = compile_module(mg, (x.cuda(),))
+        got = cm(x.cuda())
+        inst = list(cm.engine.instances.values())[0]
+        assert len(inst.prep_calls) == 16      # channels-last weight copies, as in fp32
+        assert got.dtype == torch.bfloat16
+        _assert_as_close_as_eager(got.float().cpu().numpy(), eager.float().numpy(), want64.numpy(), BF16_RTOL, BF16_ATOL, "resnet18 bf16")
+        assert torch.equal(cm(x.cuda()), got)
+
+
 def _plan_file_round_trip(cm, args, path):
     """Saves the plan of the (single) instance of an export-compiled module, loads it back and runs it on the
     tensors the engine passes for `args`; returns the outputs of that run."""

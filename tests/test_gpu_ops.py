@@ -843,6 +843,8 @@ NHWC_CASES = [
     (3, 32, 9, 11, 8, 5, 3, (2, 0, 1, 2), (1, 2), (1, 1)),        # asymmetric window, pad and stride
     (4, 256, 7, 7, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # few pixels, deep reduction: split over k
     (1, 96, 5, 5, 4, 7, 7, (3, 3, 3, 3), (1, 1), (1, 1)),         # 49 taps, windows larger than the image
+    (2, 128, 28, 28, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),    # 1568 pixels: 64-pixel tiles, no split
+    (1, 192, 6, 9, 36, 3, 3, (1, 0, 2, 1), (1, 1), (1, 1)),       # 16-bit k-tiles of 64 in 192 channels, partial filter tile
 ]
 
 
@@ -868,6 +870,22 @@ def test_conv2d_channels_last(ops, oracle, case):
     out2 = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
     assert_close_f32(host(ops.conv2d(dx, dw, pad=pad, stride=s, dilation=d, epilogue=epi, out=out2)), want2,
                      "channels-last conv+bias+res+relu %s" % (case,))
+    if C % 64:
+        return
+    # the 16-bit types: a k-tile is 64 channels of one tap; products of the rounded operands summed in fp32
+    xb, wb, bb, rb = bf16_round(x), bf16_round(w), bf16_round(b), bf16_round(res)
+    wantb = oracle.conv2d(xb, wb, None, pad=pad, stride=s, dilation=d)
+    wantb2 = oracle.unary("relu", wantb * np.float32(1.0) + bb[None, :, None, None] + rb)
+    for dt in (torch.bfloat16, torch.float16):
+        tx, tw = dev(xb, dt).contiguous(memory_format=cl), dev(wb, dt).contiguous(memory_format=cl)
+        o = torch.empty(want.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        g = ops.conv2d(tx, tw, pad=pad, stride=s, dilation=d, out=o)
+        assert g.is_contiguous(memory_format=cl)
+        assert_close_bf16(host(g), wantb, "channels-last conv %s %s" % (dt, case))
+        epi = ops.Epilogue(bias=dev(bb, dt), residual=dev(rb, dt).contiguous(memory_format=cl), act="relu")
+        o2 = torch.empty(want.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        assert_close_bf16(host(ops.conv2d(tx, tw, pad=pad, stride=s, dilation=d, epilogue=epi, out=o2)), wantb2,
+                          "channels-last conv+bias+res+relu %s %s" % (dt, case))
 
 
 @pytest.mark.parametrize("seed", range(4))
@@ -883,7 +901,7 @@ def test_random_conv_cases(ops, oracle, seed):
         C = g * int(r.choice([1, 2, 3, 8, 16, 32]))
         Fo = g * int(r.choice([1, 2, 4, 5, 16, 33, 64]))
         if g == 1 and r.random() < 0.4:
-            C = int(r.choice([32, 64, 96]))
+            C = int(r.choice([32, 64, 96, 128]))
         KH, KW = int(r.choice([1, 2, 3, 5])), int(r.choice([1, 2, 3, 5]))
         s = (int(r.integers(1, 3)), int(r.integers(1, 3)))
         d = (int(r.integers(1, 3)), int(r.integers(1, 3)))
@@ -914,6 +932,11 @@ def test_random_conv_cases(ops, oracle, seed):
             out = torch.empty(want.shape, device="cuda").contiguous(memory_format=cl)
             epi = ops.Epilogue(alpha=0.5, bias=dev(b), residual=dev(res).contiguous(memory_format=cl), act="relu")
             assert_close_f32(host(ops.conv2d(dx, dw, epilogue=epi, out=out, **kw)), want3, what + " channels-last")
+            if C % 64 == 0:
+                tx, tw = dev(xb, torch.bfloat16).contiguous(memory_format=cl), dev(wb, torch.bfloat16).contiguous(memory_format=cl)
+                o = torch.empty(want.shape, device="cuda", dtype=torch.bfloat16).contiguous(memory_format=cl)
+                assert_close_bf16(host(ops.conv2d(tx, tw, out=o, **kw)),
+                                  bf16_round(oracle.conv2d(xb, wb, None, pad=pad, stride=s, dilation=d, group=g)), what + " channels-last bf16")
 
 
 def test_conv2d_layouts_must_agree(ops):
@@ -927,6 +950,11 @@ def test_conv2d_layouts_must_agree(ops):
     w48 = torch.zeros((8, 48, 3, 3), device="cuda").contiguous(memory_format=cl)
     with pytest.raises(LlcHipError):
         ops.conv2d(x48, w48, pad=(1, 1, 1, 1), out=torch.empty((1, 8, 6, 6), device="cuda").contiguous(memory_format=cl))
+    # 32 channels of a 16-bit type are half a k-tile
+    xh = torch.zeros((1, 32, 6, 6), device="cuda", dtype=torch.bfloat16).contiguous(memory_format=cl)
+    wh = torch.zeros((8, 32, 3, 3), device="cuda", dtype=torch.bfloat16).contiguous(memory_format=cl)
+    with pytest.raises(LlcHipError):
+        ops.conv2d(xh, wh, pad=(1, 1, 1, 1), out=torch.empty((1, 8, 6, 6), device="cuda", dtype=torch.bfloat16).contiguous(memory_format=cl))
 
 
 def test_conv2d_asymmetric_pad(ops, oracle):
