@@ -610,7 +610,14 @@ bool read_operand_shape(Reader& r, Operand& o) {
   o.t.type = (size_t)r.u64();
   o.t.rank = (size_t)r.u64();
   if (!r.ok || o.t.rank > LLC_MAX_RANK || dtype_size(o.t.type) == 0) return false;
-  for (size_t i = 0; i < o.t.rank; ++i) o.size[i] = (size_t)r.u64(), o.stride[i] = (size_t)r.u64();
+  // extents and strides small enough that the byte span below cannot wrap: a file is not trusted
+  unsigned __int128 last = 0;
+  for (size_t i = 0; i < o.t.rank; ++i) {
+    o.size[i] = (size_t)r.u64(), o.stride[i] = (size_t)r.u64();
+    if (o.size[i] > ((uint64_t)1 << 40) || o.stride[i] > ((uint64_t)1 << 40)) return false;
+    if (o.size[i]) last += (unsigned __int128)(o.size[i] - 1) * o.stride[i];
+  }
+  if (last > ((uint64_t)1 << 44)) return false;
   o.t.size = o.size;
   o.t.stride = o.stride;
   return r.ok;
@@ -760,6 +767,12 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
     ~Closer() { fclose(f); }
   } closer{f};
   Reader r{f};
+  uint64_t file_bytes = 0;
+  if (fseek(f, 0, SEEK_END) == 0) {
+    const long end = ftell(f);
+    file_bytes = end > 0 ? (uint64_t)end : 0;
+  }
+  rewind(f);
   char magic[8] = {0};
   r.raw(magic, 8);
   if (!r.ok || memcmp(magic, kPlanMagic, 8) != 0) return set_error(LLC_ERR_BAD_ARG, "plan_load: %s is not a plan file", path);
@@ -798,7 +811,7 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
   std::vector<char> host;
   for (uint64_t i = 0; i < n_reg; ++i) {
     const uint64_t bytes = r.u64(), mis = r.u64(), keep = r.u64();
-    if (!r.ok || mis >= 256 || bytes > ((uint64_t)1 << 40)) return bad("malformed region entry");
+    if (!r.ok || mis >= 256 || bytes > ((uint64_t)1 << 40) || (keep && bytes > file_bytes)) return bad("malformed region entry");
     void* m = nullptr;
     LLC_TRY(llc_plan_alloc(p, (size_t)(bytes + mis), &m));
     char* base = (char*)m + mis;
@@ -846,10 +859,19 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
       o.delta = r.i64();
       const int64_t reg = r.i64(), off = r.i64();
       if (!r.ok || o.io >= (int64_t)n_io) return bad("operand bound to an undeclared tensor");
-      if (o.io < 0 && reg >= 0) {
+      if (o.io >= 0) {
+        // bound at run time to a tensor of the parameter block, `delta` bytes into it: it starts inside that
+        // tensor, and ends inside it too unless tensors of the block share memory (then it may run on into the next)
+        const uint64_t io_bytes = p->io[(size_t)o.io].like.span_bytes();
+        if (o.delta < 0 || (o.span_bytes() && (uint64_t)o.delta >= io_bytes) ||
+            (p->overlaps.empty() && (uint64_t)o.delta + o.span_bytes() > io_bytes))
+          return bad("operand outside the tensor it is bound to");
+      } else if (reg >= 0) {
         if ((uint64_t)reg >= regions.size() || off < 0 || (uint64_t)off + o.span_bytes() > regions[(size_t)reg].second)
           return bad("operand outside its memory region");
         o.t.data = o.t.base = regions[(size_t)reg].first + off;
+      } else if (o.span_bytes()) {
+        return bad("operand with elements but no memory");
       }
     }
   }

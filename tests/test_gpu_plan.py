@@ -359,6 +359,20 @@ def test_plan_file_round_trip(oracle, tmp_path):
     cut.write_bytes(path.read_bytes()[: size // 2])
     with pytest.raises(C.LlcHipError):
         Plan.load(cut)
+    # a damaged description (the part after the weights: steps, operands, offsets) is refused or loads, never
+    # crashes the loader; an absurd extent, stride or offset in particular is refused.  Nothing loaded here is run.
+    good = path.read_bytes()
+    tail = size - 1400
+    refused = 0
+    for pos in range(tail - tail % 8, size - 8, 8):
+        for word in ((1 << 62).to_bytes(8, "little"), (2 ** 64 - 5).to_bytes(8, "little")):
+            bad = tmp_path / "bad.llcplan"
+            bad.write_bytes(good[:pos] + word + good[pos + 8:])
+            try:
+                Plan.load(bad)
+            except C.LlcHipError:
+                refused += 1
+    assert refused > 100, refused
 
 
 @pytest.mark.parametrize("which", ["encoder_bf16", "resnet"])
