@@ -113,6 +113,23 @@ def time_gpu(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def launch_spread_us(fn, n=100):
+    """p10 / median / p90 of single launches in microseconds, each between its own pair of events with the device
+    idle before it: what one isolated call costs, launch latency included (the averages above are of launches
+    issued back to back, where that latency is hidden behind the previous kernel)."""
+    times = []
+    for i in range(n):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        fn(i)
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b) * 1e3)
+    times.sort()
+    return {"p10": round(times[n // 10], 2), "median": round(times[n // 2], 2), "p90": round(times[(9 * n) // 10], 2)}
+
+
 # HBM bytes per launch (reads + writes) of each case's kernel, from two rocprofv3 counter runs over this
 # same workload (FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain copy of known
 # size gives): profiles/single_op_suite_hbm_counters.md holds the commands and the table.  Counters cannot
@@ -279,6 +296,8 @@ def main():
     # a few milliseconds of work after an idle period run below the sustained clocks (the fp32 matmul reads 155 us
     # over 20 launches and 134 us over 100)
     kernels = [roofline_of(c, time_gpu(c.run, max(args.steps, 100), max(args.warmup, 20))) for c in cases]
+    for c, k in zip(cases, kernels):
+        k["single_launch_us"] = launch_spread_us(c.run)
     dominant = max(kernels, key=lambda k: k["avg_ms"])
     out = {
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
