@@ -639,23 +639,35 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_kernel(const ConvParam
   la0.store(smem);
   lb0.store(smem + kABytes);
   __syncthreads();
-#define LLC_NHWC_STEP(KT, CUR, LA2, LB2, LA1, LB1)                                                              \
+#define LLC_NHWC_STEP(KT, CUR, LA2, LB2, LA1, LB1, GUARDED)                                                     \
   {                                                                                                             \
-    if ((KT) + 2 < nk) {                                                                                        \
+    if (!(GUARDED) || (KT) + 2 < nk) {                                                                          \
       LA2.load(X, p, (kt0 + (KT) + 2) * BK);                                                                    \
       LB2.template load<BFULL>(Wt, n0, p.F, (kt0 + (KT) + 2) * BK, p.Kdim, p.Kdim, 1);                          \
     }                                                                                                           \
+    /* nothing moves across: left alone, the scheduler sinks the loads into the MFMAs and lifts the masking of  \
+       the previous tile's vectors (and with it the wait for them) above the MFMAs */                           \
+    __builtin_amdgcn_sched_barrier(0);                                                                          \
     mma_tile<T, TM, TN>(smem + (CUR) * kBufBytes, wm * WTM + li, smem + (CUR) * kBufBytes + kABytes,            \
                         wn * WTN + li, lh, acc);                                                                \
-    if ((KT) + 1 < nk) {                                                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                          \
+    if (!(GUARDED) || (KT) + 1 < nk) {                                                                          \
       LA1.store(smem + ((CUR) ^ 1) * kBufBytes);                                                                \
       LB1.store(smem + ((CUR) ^ 1) * kBufBytes + kABytes);                                                      \
     }                                                                                                           \
     __syncthreads();                                                                                            \
   }
-  for (int kt = 0; kt < nk; kt += 2) {
-    LLC_NHWC_STEP(kt, 0, la0, lb0, la1, lb1)
-    if (kt + 1 < nk) LLC_NHWC_STEP(kt + 1, 1, la1, lb1, la0, lb0)
+  // steady state without control flow in the body: with the guards inside, the compiler must assume at the top of
+  // an iteration that the loads of either register stage may still be in flight and waits for all of them before
+  // it issues the next ones, which puts the memory latency of every k-tile in front of its MFMAs
+  int kt = 0;
+  for (; kt + 3 < nk; kt += 2) {
+    LLC_NHWC_STEP(kt, 0, la0, lb0, la1, lb1, false)
+    LLC_NHWC_STEP(kt + 1, 1, la1, lb1, la0, lb0, false)
+  }
+  for (; kt < nk; kt += 2) {
+    LLC_NHWC_STEP(kt, 0, la0, lb0, la1, lb1, true)
+    if (kt + 1 < nk) LLC_NHWC_STEP(kt + 1, 1, la1, lb1, la0, lb0, true)
   }
 #undef LLC_NHWC_STEP
 
