@@ -31,6 +31,14 @@ class CompiledModule:
             return out[0]
         return out
 
+    def save_plan(self, path, *args):
+        """Writes the recorded kernel plan for the extents of `args` (the module's own inputs) to `path`, with its
+        description beside it: see Torch_ExecutionEngine.save_plan.  Parameters that were lifted to graph inputs
+        stay parameters of the plan's block (in front of `args`); with weights="npy" they are part of the file."""
+        if len(args) != self.n_user:
+            raise ValueError("expected %d inputs, got %d" % (self.n_user, len(args)))
+        return self.engine.save_plan(path, *self.lifted, *args)
+
 
 def compile_module(model, example_args, dynamic_shapes=None, verbose=False, weights=None, weight_dir=None):
     """weights="npy": parameters and buffers are written to .npy files (in weight_dir, or a fresh temporary

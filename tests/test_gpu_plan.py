@@ -450,7 +450,7 @@ def test_saved_plan_with_baked_weights_runs_in_another_process(tmp_path):
         cm = compile_module(m, (x.cuda(),), weights="npy", weight_dir=str(tmp_path / "w"))
         want = cm(x.cuda()).cpu().numpy()
         path = str(tmp_path / "mlp.llcplan")
-        meta = cm.engine.save_plan(path, x.cuda())
+        meta = cm.save_plan(path, x.cuda())
     assert len(meta["inputs"]) == 1 and len(meta["outputs"]) == 1 and meta["steps"] == 2
     n_weight_bytes = sum(p.numel() * 4 for p in m.parameters())
     assert n_weight_bytes <= os.path.getsize(path) < n_weight_bytes + 8192
