@@ -421,11 +421,8 @@ template <int NW, bool MASK>
 int launch_f32(const AttnParams& p, hipStream_t s) {
   constexpr int lds = 4 * kF32Tile + 2 * kBlockKV * 4;
   auto kern = attention_f32_kernel<NW, MASK>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_allowed{0};
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)lds, lds_allowed));
   const dim3 grid((unsigned)((p.Sq + 32 * NW - 1) / (32 * NW)), (unsigned)(p.B * p.H));
   hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, p);
   return check_launch("attention_f32_kernel");

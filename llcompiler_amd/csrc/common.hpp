@@ -5,6 +5,7 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -63,6 +64,10 @@ int check_launch(const char* kernel);
 // Kernels of one stream run in order, so successive calls on a stream can share it; calls that overlap
 // on different streams of one device must not both use kernels that need it.
 int get_workspace(size_t bytes, void** out);
+
+// A kernel that takes more than 64 KB of dynamic LDS must be allowed to, once per device: `done` (one per kernel
+// instantiation, static at the call site) keeps a bit per device ordinal.
+int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done);
 
 #define LLC_TRY(expr)              \
   do {                             \

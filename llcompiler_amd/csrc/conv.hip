@@ -747,11 +747,8 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
   const bool bfull = p.F % BN == 0;
   auto kern = bfull ? conv_nhwc_kernel<T, BM, BN, WM, WN, true> : conv_nhwc_kernel<T, BM, BN, WM, WN, false>;
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[bfull]) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set[bfull] = true;
-  }
+  static std::atomic<uint32_t> lds_allowed[2];  // one per instantiation
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)lds, lds_allowed[bfull]));
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)splits, 1), dim3(64 * WM * WN), lds, s, p);
   LLC_TRY(check_launch("conv_nhwc_kernel"));
   if (splits > 1) {
@@ -784,11 +781,8 @@ int launch_cfg(const ConvParams& p0, int groups, hipStream_t s) {
   p.tiles_n = (p.ncols + BN - 1) / BN;
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;
   auto kern = conv_kernel<T, BM, BN, LA>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_allowed{0};
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)lds, lds_allowed));
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffff || groups > 65535) return set_error(LLC_ERR_TOO_LARGE, "conv: grid too large");
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1, (unsigned)groups), dim3(256), lds, s, p);

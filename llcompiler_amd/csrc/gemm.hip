@@ -436,11 +436,8 @@ int launch_dma(const GemmParams& p0, int batch, hipStream_t s) {
   p.tiles_n = p.N / 128;
   const size_t lds = NS * kDmaStage > 2 * kStageHalf ? NS * kDmaStage : 2 * kStageHalf;
   auto kern = gemm_dma_kernel<T, BMODE, NS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_allowed{0};
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)lds, lds_allowed));
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(512), lds, s, p);
   return check_launch("gemm_dma_kernel");
 }
@@ -622,11 +619,8 @@ int launch_dma2(const GemmParams& p0, int batch, hipStream_t s) {
   p.tiles_m = p.M / 128;
   p.tiles_n = p.N / 128;
   auto kern = gemm_dma2_kernel<T, BMODE>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kDma2Lds));
-    attr_set = true;
-  }
+  static std::atomic<uint32_t> lds_allowed{0};
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)kDma2Lds, lds_allowed));
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(512), kDma2Lds, s, p);
   return check_launch("gemm_dma2_kernel");
 }
@@ -640,11 +634,8 @@ int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
   // every tile complete: the unguarded instantiation (no per-access branches in the main loop)
   const bool full = p.M % BM == 0 && p.N % BN == 0 && p.K % (kRowBytes / (int)sizeof(T)) == 0;
   auto kern = full ? gemm_kernel<T, BM, BN, WM, WN, LA, LB, true> : gemm_kernel<T, BM, BN, WM, WN, LA, LB, false>;
-  static bool attr_set[2] = {false, false};  // per instantiation
-  if (!attr_set[full]) {
-    LLC_HIP_TRY(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set[full] = true;
-  }
+  static std::atomic<uint32_t> lds_allowed[2];  // one per instantiation
+  LLC_TRY(allow_dynamic_lds((const void*)kern, (int)lds, lds_allowed[full]));
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffff || batch > 65535) return set_error(LLC_ERR_TOO_LARGE, "matmul: grid too large");
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1, (unsigned)batch), dim3(64 * WM * WN), lds, s, p);

@@ -50,6 +50,16 @@ void* g_ws[kMaxDevices];
 size_t g_ws_cap[kMaxDevices];
 }  // namespace
 
+int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done) {
+  int dev = 0;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  const uint32_t bit = 1u << (dev & 31);
+  if (done.load(std::memory_order_acquire) & bit) return LLC_OK;
+  LLC_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  done.fetch_or(bit, std::memory_order_release);
+  return LLC_OK;
+}
+
 int get_workspace(size_t bytes, void** out) {
   int dev = 0;
   LLC_HIP_TRY(hipGetDevice(&dev));
