@@ -89,6 +89,17 @@ def build_cases(ops, device, only=()):
                           lambda: (_uniform((8192, 1024), dt, gen, device), torch.ones(1024, dtype=dt, device=device),
                                    torch.zeros(1024, dtype=dt, device=device), torch.empty((8192, 1024), dtype=dt, device=device)),
                           lambda x, g, b, o: ops.layer_norm(x, g, b, 1e-5, out=o, defer=True), 16)
+    # not part of the suite (config 3's hot kernel, for counter runs: bench.py --only conv_f32,conv_bf16): the 3x3
+    # convolution of a ResNet-18 body layer at batch 16, 64 -> 64 channels on 56x56, channels-last
+    for dt_name, dt, es in (("f32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+        if "conv_%s" % dt_name in cases.only:
+            cl = torch.channels_last
+            n, c, hw, f = 16, 64, 56, 64
+            cases.add("conv", dt_name, "mfma", 2.0 * n * hw * hw * f * c * 9, (n * c * hw * hw + f * c * 9 + n * f * hw * hw) * es,
+                      lambda: (_uniform((n, c, hw, hw), dt, gen, device).contiguous(memory_format=cl),
+                               (_uniform((f, c, 3, 3), dt, gen, device) * 0.05).contiguous(memory_format=cl),
+                               torch.empty((n, f, hw, hw), dtype=dt, device=device).contiguous(memory_format=cl)),
+                      lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 4)
     # not part of the suite: a plain device copy of known size, used to calibrate the profiler's
     # FETCH_SIZE / WRITE_SIZE counters (bench.py --only copy_f32)
     if "copy_f32" in cases.only:
@@ -303,7 +314,8 @@ def main():
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32+bf16 (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": WORKLOAD, "values": "U(-1,1), seed 0", "ops_per_step": len(cases)},
+        "config": {"workload": WORKLOAD if not only else "subset for profiling: " + ",".join(only), "values": "U(-1,1), seed 0",
+                   "ops_per_step": len(cases)},
         "roofline": {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
         "dominant_kernel": dominant["kernel"],
         "kernels": kernels,
