@@ -10,6 +10,8 @@ shared library is generated per model: the "compiled artefact" is the kernel pla
 """
 from typing import Any, List
 
+import os
+
 import torch
 import torch.fx
 from torch._decomp import get_decompositions
@@ -53,6 +55,28 @@ class LLCompiler:
         self.compile_count = 0
         self.engines = []
 
+    def _log_dir(self):
+        """With `log_root` set, every compiled graph leaves its IR in `<log_root>_<compile_count>`, as the reference's
+        compiler does with its IR tree (llcompiler/compiler/compiler.py:101-105, src/Compiler/Compiler.cpp:50-58): here
+        the imported LLH graph, the graph after the LLH passes and the kernel plan."""
+        if not self.log_root:
+            return ""
+        d = "%s_%d" % (self.log_root, self.compile_count)
+        os.makedirs(d, exist_ok=True)
+        return d
+
+    @staticmethod
+    def _log(log_dir, name, graph):
+        if not log_dir:
+            return
+        from ..llh.text import print_llh
+        try:
+            text = print_llh(graph)       # the reference's generic syntax, readable by the LLH text reader
+        except Exception:                 # attributes the printer has no spelling for: the graph's own listing
+            text = graph.dump()
+        with open(os.path.join(log_dir, name + ".mlir"), "w") as f:
+            f.write(text)
+
     def _process_fx(self, model: torch.fx.GraphModule, inputs: List[torch.Tensor], **kwargs):
         partition = CapabilityBasedPartitioner(model, LLCOperatorSupport(), allows_single_node_partition=True)
         return partition.partition_and_fuse()
@@ -75,7 +99,14 @@ class LLCompiler:
 
     def compiler_fx_submodule(self, model: torch.fx.GraphModule, **kwargs):
         graph = self.importer(model)
+        log_dir = self._log_dir()
+        self._log(log_dir, "0_imported", graph)
         run_llh_pipeline(graph)
+        self._log(log_dir, "1_after_llh_passes", graph)
+        if log_dir:
+            from ..llh.plan_tool import plan_text
+            with open(os.path.join(log_dir, "2_kernel_plan.txt"), "w") as f:
+                f.write(plan_text(graph))
         if self.vebose_first_ir:
             print(graph.dump())
         self.compile_count += 1

@@ -201,6 +201,28 @@ def test_import_mlp_from_fx_and_plan():
     assert names.count("add") == 2
 
 
+def test_log_root_leaves_the_ir_of_every_compiled_graph(tmp_path):
+    """log_root, as in the reference (compiler.py:101-105): one directory per compiled graph, named
+    <log_root>_<compile_count>, here with the imported LLH, the LLH after the passes (both in the generic syntax the
+    text reader takes back) and the kernel plan."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.llh.text import parse_llh
+    from llcompiler_amd.test_models import MLP, make_mlp_inputs
+    torch._dynamo.reset()
+    comp = LLCompiler(log_root=str(tmp_path / "ir"))
+    opt = torch.compile(MLP().eval(), backend=comp, fullgraph=True)
+    with torch.no_grad(), pytest.raises(RuntimeError, match="no CPU fallback"):
+        opt(*make_mlp_inputs())
+    d = tmp_path / "ir_0"
+    assert sorted(p.name for p in d.iterdir()) == ["0_imported.mlir", "1_after_llh_passes.mlir", "2_kernel_plan.txt"]
+    before = parse_llh((d / "0_imported.mlir").read_text())
+    after = parse_llh((d / "1_after_llh_passes.mlir").read_text())
+    assert before.op_names().count("matmul") == 2 and after.op_names().count("matmul") == 2
+    plan = (d / "2_kernel_plan.txt").read_text()
+    assert plan.count("matmul") == 2 and "relu" in plan
+    torch._dynamo.reset()
+
+
 def test_compiler_rejects_other_targets_and_pipelines():
     from llcompiler_amd import LLCompiler
     with pytest.raises(ValueError):
