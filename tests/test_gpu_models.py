@@ -653,6 +653,25 @@ def test_random_conv_networks_match_eager(seed, tmp_path):
     assert torch.equal(want_again, first) and torch.equal(from_file, first), what + ": the plan read back from a file differs"
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_conv_networks_in_bf16(seed):
+    """The same random convolutional networks in bf16 storage (channel counts on both sides of what the channels-last
+    16-bit kernel takes), against a float64 evaluation of the bf16-valued weights at the bf16 bar plus what torch's
+    own bf16 evaluation misses it by."""
+    from llcompiler_amd.compiler.aot import compile_module
+    net = _RandomConvNet(seed).eval().to(torch.bfloat16)
+    x = torch.randn(2, 3, 40, 36, generator=torch.Generator().manual_seed(2000 + seed)).to(torch.bfloat16)
+    with torch.no_grad():
+        want64 = copy.deepcopy(net).double()(x.double()).numpy()
+        eager = net(x).float().numpy()
+        cm = compile_module(copy.deepcopy(net).cuda(), (x.cuda(),))
+        first = cm(x.cuda())
+        second = cm(x.cuda())
+    what = "random conv net %d in bf16: %s" % (seed, " ".join(net.kinds))
+    _assert_as_close_as_eager(first.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, what)
+    assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
+
+
 @pytest.mark.parametrize("seed", range(27))
 def test_random_networks_symbolic_batch_and_sequence(seed):
     """One compiled graph with symbolic batch and sequence extents serves every binding: the same random networks,
