@@ -274,12 +274,34 @@ for _name, _targets in {
     "add": (aten.add.Tensor, aten.add.Scalar, prims.add.default),
     "sub": (aten.sub.Tensor, aten.sub.Scalar, prims.sub.default),
     "mul": (aten.mul.Tensor, aten.mul.Scalar, prims.mul.default),
-    "div": (aten.div.Tensor, aten.div.Scalar, prims.div.default),
     "max": (aten.maximum.default, prims.maximum.default),
     "min": (aten.minimum.default, prims.minimum.default),
     "pow": (aten.pow.Tensor_Scalar, aten.pow.Tensor_Tensor, prims.pow.default),
 }.items():
     TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_binary(_name))
+
+
+def _div_ok(node):
+    """True division only: the result is floating point.  prims.div of two integers truncates in torch and the
+    elementwise kernel's integer division floors, so that form stays in eager."""
+    return node.meta["val"].dtype.is_floating_point
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.div.Tensor, aten.div.Scalar, prims.div.default, check=_div_ok)
+def _div(ctx, node):
+    """llh.div on floating point operands.  Integer (or bool) operands of a true division are converted to the
+    result type first: torch computes int / int in floating point, an integer llh.div would floor."""
+    a, b = node.args[0], node.args[1]
+    dt = _out_dtype(node)
+    av = ctx.tensor_or_const(a, ctx.val(b) if isinstance(b, torch.fx.Node) else None)
+    bv = ctx.tensor_or_const(b, av)
+    if not isinstance(a, torch.fx.Node):
+        av = ctx.tensor_or_const(a, bv)
+    if av.dtype != dt:
+        av = ctx.g.constant(a, dt) if not isinstance(a, torch.fx.Node) else ctx.g.add_op("convert_to", [av], {"dtype": dt})
+    if bv.dtype != dt:
+        bv = ctx.g.constant(b, dt) if not isinstance(b, torch.fx.Node) else ctx.g.add_op("convert_to", [bv], {"dtype": dt})
+    return ctx.g.add_op("div", [av, bv])
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.rsub.Scalar, aten.rsub.Tensor)
@@ -291,7 +313,13 @@ def _rsub(ctx, node):
 
 def _unary(name):
     def tr(ctx, node):
-        return ctx.g.add_op(name, [ctx.val(node.args[0])])
+        x = ctx.val(node.args[0])
+        dt = _out_dtype(node)
+        # torch promotes the integer operand of exp / sqrt / reciprocal ... to floating point: convert first, an
+        # integer program would compute in int64
+        if dt.is_floating_point and not x.dtype.is_floating_point:
+            x = ctx.g.add_op("convert_to", [x], {"dtype": dt})
+        return ctx.g.add_op(name, [x])
     return tr
 
 
@@ -450,7 +478,11 @@ def _adaptive_avg_pool(ctx, node):
                                    check=lambda n: n.args[1] % n.args[0].meta["val"].dim() == n.args[0].meta["val"].dim() - 1)
 def _softmax(ctx, node):
     x = ctx.val(node.args[0])
-    return ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
+    y = ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
+    dt = _out_dtype(node)  # half_to_float: a 16-bit input with an fp32 result
+    if y.dtype != dt:
+        y = ctx.g.add_op("convert_to", [y], {"dtype": dt})
+    return y
 
 
 def _first_result_only(node):
@@ -527,7 +559,10 @@ def _max_pool(ctx, node):
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten.embedding.default)
 def _embedding(ctx, node):
-    return ctx.g.add_op("gather", [ctx.val(node.args[0]), ctx.val(node.args[1])])
+    idx = ctx.val(node.args[1])
+    if idx.dtype != torch.int64:  # the row gather takes int64 indices; torch also accepts int32
+        idx = ctx.g.add_op("convert_to", [idx], {"dtype": torch.int64})
+    return ctx.g.add_op("gather", [ctx.val(node.args[0]), idx])
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(operator.getitem)

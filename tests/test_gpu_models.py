@@ -206,6 +206,60 @@ def test_unsupported_nodes_fall_back_to_eager():
     assert len(comp.engines) == 2  # relu+1 before the cumsum, *2 after it
 
 
+def test_true_division_of_integer_tensors_is_floating_point():
+    """aten.div of integer operands is a true division (7 / 2 = 3.5, -7 / 2 = -3.5): the importer converts the
+    operands to the result type first; an integer llh.div would floor."""
+    class M(torch.nn.Module):
+        def forward(self, a, b):
+            return a / 2, a / b, 3 / a, (a / b) * 2.0
+
+    a = torch.tensor([[7, -7, 9, -1, 5, 6]], dtype=torch.int64)
+    b = torch.tensor([[2, 2, -4, 3, -2, 4]], dtype=torch.int64)
+    with torch.no_grad():
+        want = M()(a, b)
+        opt, _ = _compile(M())
+        got = opt(a.cuda(), b.cuda())
+    for g, w in zip(got, want):
+        assert g.dtype == w.dtype
+        assert_close(g.cpu().numpy(), w.numpy(), F32_RTOL, F32_ATOL, "int true division")
+    a32 = a.to(torch.int32)
+    with torch.no_grad():
+        opt, _ = _compile(M())
+        got = opt(a32.cuda(), b.cuda())
+        want = M()(a32, b)
+    for g, w in zip(got, want):
+        assert_close(g.cpu().numpy(), w.numpy(), F32_RTOL, F32_ATOL, "int32 / int64 true division")
+
+
+def test_softmax_half_to_float_and_int32_embedding():
+    class S(torch.nn.Module):
+        def forward(self, x):
+            return torch.softmax(x, dim=-1, dtype=torch.float32)
+
+    class E(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = torch.nn.Embedding(37, 16)
+
+        def forward(self, idx):
+            return self.emb(idx)
+
+    x = torch.randn(6, 50, generator=torch.Generator().manual_seed(3)).to(torch.float16)
+    with torch.no_grad():
+        opt, _ = _compile(S())
+        got = opt(x.cuda())
+        want = torch.softmax(x.cuda(), dim=-1, dtype=torch.float32).cpu()
+    assert got.dtype == torch.float32
+    assert_close(got.cpu().numpy(), want.numpy(), 2e-3, 1e-4, "softmax half_to_float")
+    torch.manual_seed(4)
+    e = E().eval()
+    idx = torch.randint(0, 37, (3, 7), generator=torch.Generator().manual_seed(5)).to(torch.int32)
+    with torch.no_grad():
+        opt, _ = _compile(e)
+        got = opt(idx.cuda())
+    np.testing.assert_array_equal(got.cpu().numpy(), e(idx).detach().numpy())
+
+
 def test_graph_replay_matches_per_kernel_launches():
     """With graph replay switched on, an instance replays its launch sequence as a HIP graph after two calls.
     Every replay, with other GPU

@@ -294,3 +294,21 @@ def test_prims_level_nodes_are_translated():
     from llcompiler_amd.llh.passes import run_llh_pipeline
     run_llh_pipeline(g)
     assert g.op_names() == ["reshape", "reduce_sum"]          # the identities are gone
+
+
+def test_true_division_of_integers_is_imported_as_a_floating_point_div():
+    """aten.div.Tensor / div.Scalar of integer tensors give floats in torch; the importer converts the operands to
+    the result type before llh.div (an integer llh.div would floor), and prims.div of two integers (truncating in
+    torch) is left to eager."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from llcompiler_amd.importer.fx_importer import is_supported, torch_translate_to_llh_graph
+    gm = make_fx(lambda a, b: (a / 2, a / b, 3 / a))(torch.tensor([7, -7]), torch.tensor([2, 3]))
+    g = torch_translate_to_llh_graph(gm)
+    divs = [op for op in g.ops if op.name in ("div", "recip")]  # 3 / a arrives as reciprocal(a) * 3
+    assert len(divs) == 3
+    for op in divs:
+        assert op.results[0].dtype == torch.float32
+        assert all(v.dtype == torch.float32 for v in op.operands)
+    gm = make_fx(lambda a, b: torch.ops.prims.div(a, b))(torch.tensor([7, -7]), torch.tensor([2, 3]))
+    node = [n for n in gm.graph.nodes if n.op == "call_function"][0]
+    assert node.meta["val"].dtype == torch.int64 and not is_supported(node)
