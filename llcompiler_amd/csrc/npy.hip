@@ -49,7 +49,9 @@ int parse_header(FILE* fp, const char* path, NpyInfo* info) {
   info->descr = h.substr(q0 + 1, q1 - q0 - 1);
   at = h.find("'fortran_order'");
   if (at == std::string::npos) return set_error(LLC_ERR_BAD_ARG, "npy: %s: no 'fortran_order' in the header", path);
-  info->fortran = h.compare(h.find_first_not_of(": ", at + 15), 4, "True") == 0;
+  const size_t fv = h.find_first_not_of(": ", at + 15);
+  if (fv == std::string::npos) return set_error(LLC_ERR_BAD_ARG, "npy: %s: 'fortran_order' has no value", path);
+  info->fortran = h.compare(fv, 4, "True") == 0;
   at = h.find("'shape'");
   size_t p0 = at == std::string::npos ? at : h.find('(', at);
   size_t p1 = p0 == std::string::npos ? p0 : h.find(')', p0);
@@ -118,12 +120,25 @@ extern "C" int llc_plan_load_npy(llc_plan_t* plan, const char* path, int expect_
   size_t n = 1;
   for (size_t i = rank; i-- > 0;) {
     stride_out[i] = n;
+    if (size_out[i] != 0 && n > SIZE_MAX / 16 / size_out[i]) return set_error(LLC_ERR_TOO_LARGE, "npy: %s: shape overflows", path);
     n *= size_out[i];
   }
   const size_t bytes = n * dtype_size(dtype);
-  std::vector<char> host(bytes ? bytes : 1);
   FILE* fp = fopen(path, "rb");
   if (!fp) return set_error(LLC_ERR_BAD_ARG, "npy: cannot open %s", path);
+  // the header's shape is not trusted before the file is seen to hold that much data (a damaged header must not
+  // become a huge allocation)
+  if (fseek(fp, 0, SEEK_END) != 0 || ftell(fp) < 0 || (size_t)ftell(fp) < off || (size_t)ftell(fp) - off < bytes) {
+    fclose(fp);
+    return set_error(LLC_ERR_BAD_ARG, "npy: %s holds fewer than %zu bytes of data", path, bytes);
+  }
+  std::vector<char> host;
+  try {
+    host.resize(bytes ? bytes : 1);
+  } catch (...) {
+    fclose(fp);
+    return set_error(LLC_ERR_TOO_LARGE, "npy: %s: no host memory for %zu bytes", path, bytes);
+  }
   const bool ok = fseek(fp, (long)off, SEEK_SET) == 0 && fread(host.data(), 1, bytes, fp) == bytes;
   fclose(fp);
   if (!ok) return set_error(LLC_ERR_BAD_ARG, "npy: %s holds fewer than %zu bytes of data", path, bytes);
