@@ -14,10 +14,14 @@
  *  - the caller owns every input and output buffer (Tensor.h:35: the descriptor allocates nothing).
  *  - `stream` is a hipStream_t passed as void*; NULL = the default stream.  Calls only enqueue
  *    work; the caller synchronises.
- *  - the library keeps one scratch buffer per device for kernels that split a reduction (convolutions with few
- *    output tiles, matmuls with a long K): it grows on demand, which is the only allocation an op entry
- *    point ever makes, and it is shared: such calls may follow each other on one stream, but issuing them on
- *    several streams of one device at the same time lets them overwrite each other's partial sums.
+ *  - kernels that split a reduction (convolutions with few output tiles, matmuls with a long K) keep partial
+ *    sums in scratch device memory.  A plan owns its scratch memory (sized while it is recorded, allocated by
+ *    llc_plan_end / llc_plan_load), so llc_hip_run allocates nothing and plans replayed on different streams do
+ *    not share any.  An op entry point called outside a plan uses one buffer per device that grows on demand,
+ *    which is the only allocation an op entry point ever makes (the old buffer is kept, nothing is synchronised;
+ *    refused with LLC_ERR_UNSUPPORTED while the stream is being captured): such calls may follow each other on
+ *    one stream, but issuing them on several streams of one device at the same time lets them overwrite each
+ *    other's partial sums.
  *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
  *    llc_hip_last_error() (thread local).  The reference only logs on failure
  *    (include/llcompiler/Support/Logger.h:132-134); returning a status is a deliberate tightening.
@@ -32,7 +36,7 @@
 extern "C" {
 #endif
 
-#define LLC_HIP_ABI_VERSION 1
+#define LLC_HIP_ABI_VERSION 2
 #define LLC_MAX_RANK 8
 
 /* Element type codes.  0-6 are the reference's `enum Type` (Tensor.h:25-33, and the Python map

@@ -59,11 +59,31 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 
 int check_launch(const char* kernel);
 
-// Scratch device memory for kernels that keep partial results (split-k).  One buffer per device, grown on
-// demand (the device is drained before the old buffer is released) and kept until the process ends.
-// Kernels of one stream run in order, so successive calls on a stream can share it; calls that overlap
-// on different streams of one device must not both use kernels that need it.
-int get_workspace(size_t bytes, void** out);
+// Scratch device memory for kernels that keep partial results (split reductions).  Where it comes from, in
+// this order: (1) a WorkspaceScope alive on the calling thread (a plan replaying with memory of its own, or the
+// allocation-free entry point with the library's static array): that memory is handed out and nothing is ever
+// allocated, a request beyond its capacity is an error; (2) one buffer per device, grown on demand.  Growing
+// allocates a new buffer and keeps the old one until the process ends (launches already queued, or a captured
+// graph, may still address it), never synchronises, and is refused while `stream` is being captured.
+// Kernels of one stream run in order, so successive calls on a stream can share the per-device buffer; calls
+// that overlap on different streams of one device must not both use kernels that need it (plans do not: each
+// owns its scratch memory).
+int get_workspace(size_t bytes, void** out, hipStream_t stream);
+
+struct WorkspaceScope {
+  WorkspaceScope(void* ptr, size_t capacity);
+  ~WorkspaceScope();
+  WorkspaceScope(const WorkspaceScope&) = delete;
+  WorkspaceScope& operator=(const WorkspaceScope&) = delete;
+
+ private:
+  void* prev_ptr_;
+  size_t prev_cap_;
+  bool prev_active_;
+};
+// While `high_water` is set on this thread, every get_workspace request raises *high_water to its size (a plan
+// being recorded learns how much scratch memory its steps need).  Null stops it.
+void workspace_track(size_t* high_water);
 
 // A kernel that takes more than 64 KB of dynamic LDS must be allowed to, once per device: `done` (one per kernel
 // instantiation, static at the call site) keeps a bit per device ordinal.

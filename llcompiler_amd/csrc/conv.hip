@@ -505,7 +505,7 @@ int launch_f32(const ConvParams& p0, int groups, hipStream_t s) {
   p.splits = splits;
   if (splits > 1) {
     void* ws = nullptr;
-    LLC_TRY(get_workspace((size_t)splits * p.F * p.ncols * sizeof(float), &ws));
+    LLC_TRY(get_workspace((size_t)splits * p.F * p.ncols * sizeof(float), &ws, s));
     p.partial = (char*)ws;
   }
   const size_t lds = 2 * (size_t)(BM * kRowStride + 32 * BN * 4);
@@ -741,7 +741,7 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   p.splits = splits;
   if (splits > 1) {
     void* ws = nullptr;
-    LLC_TRY(get_workspace((size_t)splits * p.ncols * p.F * sizeof(float), &ws));
+    LLC_TRY(get_workspace((size_t)splits * p.ncols * p.F * sizeof(float), &ws, s));
     p.partial = (char*)ws;
   }
   const size_t lds = 2 * (size_t)(BM + BN) * kRowStride;

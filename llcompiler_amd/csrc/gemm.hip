@@ -28,6 +28,9 @@
 // which gives each XCD's L2 a compact patch of the output (few distinct A row-panels / B
 // column-panels).
 
+#include <cstdlib>
+#include <type_traits>
+
 #include "gemm_core.hpp"
 
 namespace llc {
@@ -625,6 +628,8 @@ int launch_dma2(const GemmParams& p0, int batch, hipStream_t s) {
   return check_launch("gemm_dma2_kernel");
 }
 
+#include "gemm_wide.hpp"
+
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB>
 int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
   GemmParams p = p0;
@@ -801,7 +806,7 @@ template <typename T, int LB>
 int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
   const int64_t mn = (int64_t)p.M * p.N;
   void* ws = nullptr;
-  LLC_TRY(get_workspace((size_t)splits * mn * sizeof(float), &ws));
+  LLC_TRY(get_workspace((size_t)splits * mn * sizeof(float), &ws, s));
   GemmParams q = p;
   q.K = p.K / splits;
   q.a_sb = (int64_t)q.K * p.a_sk;
@@ -825,6 +830,40 @@ int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
   return check_launch("splitk_reduce_kernel");
 }
 
+// Column extent of the 256 x BN tile for a 16-bit product with complete tiles, 0 = keep the 128 x 128 kernels.
+// One workgroup per CU: the cost of a candidate is its number of rounds over the 256 CUs times the tile's work,
+// weighted by how well that tile shape runs (narrower tiles read more LDS and L2 bytes per MFMA).
+inline int wide_tile_n(const GemmParams& p, int batch, bool b_kvec) {
+#ifdef LLC_GEMM_TUNE
+  if (const char* e = getenv("LLC_WIDE")) {
+    const int bn = atoi(e);
+    if (bn == 0) return 0;
+    if (p.N % bn == 0 && (bn == 256 || bn == 128 || (bn == 192 && b_kvec))) return bn;
+    return 0;
+  }
+#endif
+  int best = 0;
+  double best_cost = 0.0;
+  const int cand[3] = {256, 192, 128};
+  const double weight[3] = {1.0, 1.05, 1.2};
+  for (int c = 0; c < 3; ++c) {
+    const int bn = cand[c];
+    if (p.N % bn != 0 || (bn == 192 && !b_kvec)) continue;
+    const int64_t tiles = (int64_t)(p.M / 256) * (p.N / bn) * batch;
+    if (tiles > 0x7fffffff || batch > 65535) continue;
+    const double cost = (double)((tiles + 255) / 256) * bn * weight[c];
+    if (best == 0 || cost < best_cost) {
+      best = bn;
+      best_cost = cost;
+    }
+  }
+  if (best == 0) return 0;
+  // fewer workgroups than 3/4 of the CUs: the 128 x 128 kernels fill the chip better
+  const int64_t tiles = (int64_t)(p.M / 256) * (p.N / best) * batch;
+  if (tiles < 192) return 0;
+  return best;
+}
+
 template <typename T>
 int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
@@ -838,6 +877,14 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
     if (splits > 1) return b_kvec ? launch_splitk<T, kLoadKVec>(p, splits, s) : launch_splitk<T, kLoadRVec>(p, splits, s);
   }
   if constexpr (sizeof(T) == 2) {
+    const bool dma_ok = a_kvec && (b_kvec || b_rvec) && p.K % 64 == 0 && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 &&
+                        p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) && (!p.residual || al16(p.residual));
+    if (dma_ok && p.M % 256 == 0 && p.K >= 128) {
+      const int bn = wide_tile_n(p, batch, b_kvec);
+      if (bn == 256) return b_kvec ? launch_wide<T, kBKMajor, 256>(p, batch, s) : launch_wide<T, kBNMajor, 256>(p, batch, s);
+      if (bn == 192) return launch_wide<T, kBKMajor, 192>(p, batch, s);
+      if (bn == 128) return b_kvec ? launch_wide<T, kBKMajor, 128>(p, batch, s) : launch_wide<T, kBNMajor, 128>(p, batch, s);
+    }
     const int64_t tiles = (int64_t)(p.M / 128) * (p.N / 128) * batch;
     if (a_kvec && (b_kvec || b_rvec) && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 64 == 0 && (p.K >= 256 || tiles >= 512) &&
         tiles >= 128 && tiles <= 0x7fffffff && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 && p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) &&
@@ -1015,3 +1062,12 @@ int llc_impl_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const ll
   }
   return LLC_OK;
 }
+
+#ifdef LLC_GEMM_TUNE
+// tuning builds only: shader clocks and 100 MHz ticks of the longest workgroup since the last call
+extern "C" void llc_dbg_read(unsigned long long* out) {
+  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(llc::llc_dbg_clk), 16);
+  unsigned long long z[2] = {0, 0};
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(llc::llc_dbg_clk), z, 16);
+}
+#endif

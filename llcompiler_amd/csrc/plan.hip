@@ -110,6 +110,10 @@ struct llc_plan {
   std::vector<int64_t> symbols;
   std::vector<Overlap> overlaps;
   std::vector<char*> bound;  // per run: first element of every params tensor
+  // scratch memory of the steps that split a reduction: sized while recording (the largest request), allocated
+  // by llc_plan_end / llc_plan_load, handed to the kernels by llc_hip_run (which therefore never allocates)
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
   std::mutex mu;
 };
 
@@ -163,6 +167,7 @@ struct Recorder {
     if (!ok) {
       p->state = kBroken;
       t_rec = nullptr;
+      workspace_track(nullptr);
       return set_error(LLC_ERR_BAD_ARG, "plan: a call could not be recorded (descriptor rank or attribute count)");
     }
     p->steps.push_back(std::move(st));
@@ -174,6 +179,55 @@ struct Recorder {
 inline void rebase(Step& s, char* const* bound) {
   for (Operand& o : s.opnd)
     if (o.io >= 0) o.t.data = o.t.base = bound[o.io] + o.delta;
+}
+
+// Operand count every step code is recorded with (0: variable, the elementwise program's inputs + 1).  A plan
+// file whose step disagrees is refused: replay() indexes the operands by position.
+int operands_of(int op) {
+  switch (op) {
+    case kMatmul: case kBatchMatmul: case kConv2d: case kAttention: return 5;
+    case kLayerNorm: return 4;
+    case kGatherRows: return 3;
+    case kElementwise: return 0;
+    default: return 2;
+  }
+}
+
+// The shape of a loaded step: operand count, required operands present, integer attributes sized by the
+// operand's rank.  Returns null when it is what the recorder would have written, else what is wrong.
+const char* step_defect(const Step& s) {
+  const size_t n = s.opnd.size();
+  if (s.op == kElementwise) {
+    if (!s.prog) return "elementwise step without a program";
+    if (n < 1 || n > LLC_EW_MAX_INPUTS + 1) return "elementwise step with too many operands";
+    for (const Operand& o : s.opnd)
+      if (!o.present) return "elementwise step with an absent operand";
+    return nullptr;
+  }
+  if (s.prog) return "a program on a step that is not elementwise";
+  if (n != (size_t)operands_of(s.op)) return "operand count does not fit the step code";
+  auto need = [&](size_t i) { return s.opnd[i].present; };
+  switch (s.op) {
+    case kMatmul: case kBatchMatmul: case kConv2d:
+      if (!need(0) || !need(1) || !need(4)) return "contraction without lhs, rhs or output";
+      break;
+    case kAttention:
+      if (!need(0) || !need(1) || !need(2) || !need(4)) return "attention without q, k, v or output";
+      break;
+    case kLayerNorm:
+      if (!need(0) || !need(3)) return "layer_norm without input or output";
+      break;
+    case kGatherRows:
+      if (!need(0) || !need(1) || !need(2)) return "gather without table, indices or output";
+      break;
+    default:
+      if (!need(0) || !need(1)) return "step without input or output";
+  }
+  const size_t rank0 = s.opnd[0].t.rank;
+  if (s.op == kTranspose && s.n_ints != rank0) return "transpose: one permutation entry per dim expected";
+  if (s.op == kStrideSlice && s.n_ints != 3 * rank0) return "stride_slice: start, end and step per dim expected";
+  if (s.op == kReduce && (s.n_ints == 0 || s.n_ints > rank0)) return "reduce: axis list does not fit the operand";
+  return nullptr;
 }
 
 int replay(Step& s, void* stream) {
@@ -197,6 +251,7 @@ int replay(Step& s, void* stream) {
     case kElementwise: {
       const llc_tensor* ins[LLC_EW_MAX_INPUTS];
       const size_t n = s.opnd.size() - 1;
+      if (n > LLC_EW_MAX_INPUTS) return set_error(LLC_ERR_BAD_ARG, "plan: elementwise step with %zu inputs", n);
       for (size_t i = 0; i < n; ++i) ins[i] = o[i].ptr();
       return llc_impl_elementwise(s.prog.get(), ins, n, o[n].ptr(), stream);
     }
@@ -387,7 +442,10 @@ extern "C" int llc_plan_create(llc_plan_t** plan) {
 
 extern "C" int llc_plan_destroy(llc_plan_t* p) {
   if (!p) return LLC_OK;
-  if (t_rec == p) t_rec = nullptr;
+  if (t_rec == p) {
+    t_rec = nullptr;
+    workspace_track(nullptr);
+  }
   int status = LLC_OK;
   for (void* m : p->owned) {
     hipError_t e = hipFree(m);  // waits for the device to finish with the memory
@@ -451,6 +509,8 @@ extern "C" int llc_plan_begin(llc_plan_t* p) {
   if (p->state != kOpen) return set_error(LLC_ERR_BAD_ARG, "plan_begin: the plan has been recorded already");
   LLC_TRY(check_device(p, "plan_begin"));
   p->state = kRecording;
+  p->ws_bytes = 0;
+  workspace_track(&p->ws_bytes);
   t_rec = p;
   return LLC_OK;
 }
@@ -460,6 +520,12 @@ extern "C" int llc_plan_end(llc_plan_t* p) {
   if (p->state == kBroken) return set_error(LLC_ERR_BAD_ARG, "plan_end: recording failed earlier");
   if (t_rec != p || p->state != kRecording) return set_error(LLC_ERR_BAD_ARG, "plan_end: the plan is not recording on this thread");
   t_rec = nullptr;
+  workspace_track(nullptr);
+  if (p->ws_bytes) {
+    p->state = kBroken;  // until the scratch memory is there
+    LLC_HIP_TRY(hipMalloc(&p->ws, p->ws_bytes));
+    p->owned.push_back(p->ws);
+  }
   p->state = kReady;
   p->bound.assign(p->io.size(), nullptr);
   return LLC_OK;
@@ -509,6 +575,7 @@ extern "C" int llc_hip_run(llc_plan_t* p, void* const* params, void* stream) {
     if (p->bound[ov.second] - p->bound[ov.first] != ov.diff)
       return set_error(LLC_ERR_LAYOUT, "run: tensors %d and %d shared memory when the plan was recorded and do not now", ov.first,
                        ov.second);
+  WorkspaceScope scratch(p->ws, p->ws_bytes);  // the steps use the plan's own scratch memory: nothing is allocated here
   for (Step& s : p->steps) {
     rebase(s, p->bound.data());
     LLC_TRY(replay(s, stream));
@@ -705,6 +772,7 @@ extern "C" int llc_plan_save(llc_plan_t* p, const char* path) {
   for (int64_t v : p->symbols) w.i64(v);
   w.u64(p->overlaps.size());
   for (const Overlap& ov : p->overlaps) w.i64(ov.first), w.i64(ov.second), w.i64(ov.diff);
+  w.u64(p->ws_bytes);
   w.u64(regions.size());
   std::vector<char> host;
   for (const Region& g : regions) {
@@ -805,6 +873,12 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
     if (!r.ok || ov.first < 0 || ov.second < 0 || (uint64_t)ov.first >= n_io || (uint64_t)ov.second >= n_io) return bad("malformed overlap entry");
     p->overlaps.push_back(ov);
   }
+  const uint64_t ws_bytes = r.u64();
+  if (!r.ok || ws_bytes > ((uint64_t)1 << 36)) return bad("malformed scratch size");
+  if (ws_bytes) {
+    LLC_TRY(llc_plan_alloc(p, (size_t)ws_bytes, &p->ws));
+    p->ws_bytes = (size_t)ws_bytes;
+  }
   const uint64_t n_reg = r.u64();
   if (!r.ok || n_reg > (1u << 24)) return bad("truncated region list");
   std::vector<std::pair<char*, size_t>> regions;
@@ -876,6 +950,8 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
     }
   }
   if (!r.ok) return bad("truncated file");
+  for (const Step& s : p->steps)
+    if (const char* why = step_defect(s)) return bad(why);
   p->state = kReady;
   p->bound.assign(p->io.size(), nullptr);
   *out = guard.release();

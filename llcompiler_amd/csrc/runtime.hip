@@ -60,22 +60,50 @@ int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done
   return LLC_OK;
 }
 
-int get_workspace(size_t bytes, void** out) {
+namespace {
+thread_local void* t_ws_ptr = nullptr;
+thread_local size_t t_ws_cap = 0;
+thread_local bool t_ws_active = false;
+thread_local size_t* t_ws_high_water = nullptr;
+}  // namespace
+
+WorkspaceScope::WorkspaceScope(void* ptr, size_t capacity) : prev_ptr_(t_ws_ptr), prev_cap_(t_ws_cap), prev_active_(t_ws_active) {
+  t_ws_ptr = ptr;
+  t_ws_cap = capacity;
+  t_ws_active = true;
+}
+WorkspaceScope::~WorkspaceScope() {
+  t_ws_ptr = prev_ptr_;
+  t_ws_cap = prev_cap_;
+  t_ws_active = prev_active_;
+}
+void workspace_track(size_t* high_water) { t_ws_high_water = high_water; }
+
+int get_workspace(size_t bytes, void** out, hipStream_t stream) {
+  if (t_ws_high_water && bytes > *t_ws_high_water) *t_ws_high_water = bytes;
+  if (t_ws_active) {
+    if (bytes > t_ws_cap)
+      return set_error(LLC_ERR_TOO_LARGE, "this call needs %zu bytes of scratch memory, %zu are provided and nothing may be allocated here",
+                       bytes, t_ws_cap);
+    *out = t_ws_ptr;
+    return LLC_OK;
+  }
   int dev = 0;
   LLC_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "workspace: device %d", dev);
   static std::mutex mu;  // host threads may launch at the same time; the buffer itself is shared per device
   std::lock_guard<std::mutex> lock(mu);
   if (bytes > g_ws_cap[dev]) {
-    if (g_ws[dev]) {
-      LLC_HIP_TRY(hipDeviceSynchronize());
-      LLC_HIP_TRY(hipFree(g_ws[dev]));
-      g_ws[dev] = nullptr;
-      g_ws_cap[dev] = 0;
-    }
-    const size_t cap = ((bytes + bytes / 2) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
-    LLC_HIP_TRY(hipMalloc(&g_ws[dev], cap));
-    g_ws_cap[dev] = cap;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return set_error(LLC_ERR_UNSUPPORTED, "this call needs %zu bytes of scratch memory and the stream is being captured: run it once "
+                       "outside the capture, or record it into a plan", bytes);
+    // the old buffer stays allocated: queued launches and captured graphs may still address it
+    const size_t cap_bytes = ((bytes + bytes / 2) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    void* fresh = nullptr;
+    LLC_HIP_TRY(hipMalloc(&fresh, cap_bytes));
+    g_ws[dev] = fresh;
+    g_ws_cap[dev] = cap_bytes;
   }
   *out = g_ws[dev];
   return LLC_OK;
