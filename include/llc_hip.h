@@ -21,7 +21,7 @@
  *    which is the only allocation an op entry point ever makes (the old buffer is kept, nothing is synchronised;
  *    refused with LLC_ERR_UNSUPPORTED while the stream is being captured): such calls may follow each other on
  *    one stream, but issuing them on several streams of one device at the same time lets them overwrite each
- *    other's partial sums.
+ *    other's partial sums.  llc_hip_matmul_static never allocates (see there).
  *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
  *    llc_hip_last_error() (thread local).  The reference only logs on failure
  *    (include/llcompiler/Support/Logger.h:132-134); returning a status is a deliberate tightening.
@@ -110,6 +110,18 @@ typedef struct llc_epilogue {
  * of the sum is fixed, so results are the same bits on every run. */
 int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                    void* stream);
+
+/* llc_hip_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels
+ * and the same bits as llc_hip_matmul; the partial sums of a split reduction go to a 32 MiB array that is part of
+ * the library's code object (each GPU the library runs on holds it until the process ends) instead of the
+ * per-device buffer that llc_hip_matmul grows on demand.  The call never allocates or frees; a product whose
+ * partial sums need more than 32 MiB is refused with LLC_ERR_TOO_LARGE (use llc_hip_matmul or a plan).  Every call
+ * on a GPU shares that GPU's array (nothing in it has to start at zero: partial sums are written before they are
+ * read): calls that overlap on different streams of one GPU race, like llc_hip_matmul's.  The call is not recorded
+ * into a plan (a plan owns its scratch memory anyway). */
+int llc_hip_matmul_static(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+                          void* stream);
 
 /* llh.batch_matmul (LLHOps.td:446-452; LLHToHLO.cpp:363-382: batch dims {0}/{0}, contracting lhs
  * dim 2 with rhs dim 1): rank 3.  The two inner dims of each operand may be a transposed view.

@@ -71,6 +71,7 @@ class LlcEwProgram(ctypes.Structure):
 # every symbol include/llc_hip.h declares
 EXPORTS = [
     "llc_hip_abi_version", "llc_hip_init", "llc_hip_last_error", "llc_hip_status_string", "llc_hip_matmul",
+    "llc_hip_matmul_static",
     "llc_hip_batch_matmul", "llc_hip_conv2d", "llc_hip_elementwise", "llc_hip_reduce", "llc_hip_softmax",
     "llc_hip_layer_norm", "llc_hip_max_pool", "llc_hip_global_avg_pool", "llc_hip_transpose",
     "llc_hip_stride_slice", "llc_hip_broadcast_to", "llc_hip_copy", "llc_hip_gather_rows", "llc_hip_convert",
@@ -109,6 +110,7 @@ def lib():
         vp = ctypes.c_void_p
         i64p = P(ctypes.c_int64)
         L.llc_hip_matmul.argtypes = [T, T, P(LlcEpilogue), T, vp]
+        L.llc_hip_matmul_static.argtypes = [T, T, P(LlcEpilogue), T, vp]
         L.llc_hip_batch_matmul.argtypes = [T, T, P(LlcEpilogue), T, vp]
         L.llc_hip_conv2d.argtypes = [T, T, P(LlcConvAttrs), P(LlcEpilogue), T, vp]
         L.llc_hip_elementwise.argtypes = [P(LlcEwProgram), P(T), ctypes.c_size_t, T, vp]

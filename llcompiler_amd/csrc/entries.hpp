@@ -26,3 +26,5 @@ int llc_impl_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_ten
 int llc_impl_convert(const llc_tensor* x, llc_tensor* out, void* stream);
 int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask, float scale,
                        llc_tensor* out, void* stream);
+// Looks up, for the current device, the address of the scratch array behind llc_hip_matmul_static (gemm.hip).
+int llc_impl_static_scratch_setup(void);

@@ -29,6 +29,7 @@
 // column-panels).
 
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "gemm_core.hpp"
@@ -1061,6 +1062,51 @@ int llc_impl_batch_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const ll
     LLC_TRY(gemm_dispatch(a.dtype, q, cnt, s));
   }
   return LLC_OK;
+}
+
+// ---- llc_hip_matmul for callers that may not allocate -------------------------------------------------------
+// The split reductions keep their partial sums in `scratch`, device memory that is part of the library's
+// code object (every GPU the library runs on holds its own copy from load to process end), instead of the
+// per-device buffer that llc_hip_matmul grows with hipMalloc.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kScratchDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kScratchDevices];  // device address of `scratch` on each device, null until asked for
+
+// `scratch` names a host-side stand-in, not a device address: the address on the current device comes from
+// hipGetSymbolAddress, once per device, and is what every kernel and copy is given afterwards.
+int static_scratch(void** out) {
+  int dev = -1;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kScratchDevices) return set_error(LLC_ERR_BAD_ARG, "matmul_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    LLC_HIP_TRY(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return set_error(LLC_ERR_HIP, "matmul_static: the scratch array has no address on device %d", dev);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return LLC_OK;
+}
+}  // namespace
+
+// called by llc_hip_init with the device current
+int llc_impl_static_scratch_setup(void) {
+  void* ptr = nullptr;
+  return static_scratch(&ptr);
+}
+
+extern "C" int llc_hip_matmul_static(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
+                                     void* stream) {
+  void* ptr = nullptr;
+  LLC_TRY(static_scratch(&ptr));
+  // while this scope lives, get_workspace hands out `ptr` and refuses what does not fit; nothing allocates
+  WorkspaceScope scope(ptr, kStaticScratchBytes);
+  return llc_impl_matmul(lhs, rhs, epi, out, stream);
 }
 
 #ifdef LLC_GEMM_TUNE

@@ -142,7 +142,8 @@ extern "C" int llc_hip_init(int device) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return set_error(LLC_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device,
                      prop.gcnArchName);
-  return LLC_OK;
+  // the scratch array of the allocation-free entry point has an address of its own on every device
+  return llc_impl_static_scratch_setup();
 }
 
 extern "C" int llc_hip_unpack_params(void* const* params, size_t n_tensors, const size_t* ranks, const size_t* types,

@@ -75,6 +75,15 @@ def matmul(a, b, epilogue=None, out=None, defer=False):
                    defer)
 
 
+def matmul_static(a, b, out, epilogue=None, defer=False):
+    """llc_hip_matmul_static: the same product through the entry point that allocates nothing (split reductions
+    keep their partial sums in the library's static device array).  `out` is the caller's, as in the C-ABI."""
+    dev = _dev(a)
+    ra, rb, ro = C.tensor_ref(a), C.tensor_ref(b), C.tensor_ref(out)
+    return _launch(C.lib().llc_hip_matmul_static, (ra.ptr, rb.ptr, _epi(epilogue), ro.ptr), (ra, rb, ro, epilogue), out,
+                   dev, defer)
+
+
 def batch_matmul(a, b, epilogue=None, out=None, defer=False):
     dev = _dev(a)
     if out is None:
