@@ -2,53 +2,10 @@
 // Included by gemm.hip inside namespace llc::{anonymous} (uses GemmParams and the LDS-DMA helpers defined there).
 //
 // Why a second tile shape: a 128x128 tile needs 64 B/clk/CU of operands from L2 at the full MFMA rate and
-// 192 B/clk of LDS traffic, both above what a CU gets; a 256x256 tile halves the first and, with 64x128 wave
-// tiles, brings the second to 128 B/clk.
-//
-// Eight waves, two per SIMD, in two groups of four (waves w and w+4 share a SIMD).  A wave owns a
-// 64 x BN/2 accumulator tile (group g = column half g, wave w of the group = row quarter w).  The groups
-// run the same program half a step apart ("ping-pong"): per half k-tile (two MFMA k-steps) a wave first
-// spends a MEMORY phase (issue its share of the next k-tile's direct-to-LDS loads, read the fragments
-// of this half tile into registers, wait for them), then a COMPUTE phase (TM*TN*2 MFMAs at raised priority).
-// Every phase ends at a workgroup barrier and group 1 enters the loop one barrier late, so in every barrier
-// interval one wave of each SIMD issues MFMAs back to back while the other one issues the memory
-// instructions.  Fragments need no double buffer (they are read in one phase and consumed in the next).
-//
-// LDS: NS stages of one k-tile each (A [256 m][128 B of k], then B as [BN n][128 B of k] or, row-major B,
-// [64 k][2 BN B of n]), swizzled like the 128x128 kernels and filled by global_load_lds_dwordx4.  Stage of
-// tile t-1 is reloaded with tile t+NS-1 in the first memory phase of tile t (every wave has read it by
-// then: group 1's last read of tile t-1 ended one barrier earlier).  A wave waits for its own loads of tile
-// t+1 before the barrier that ends the last phase of tile t (vmcnt counts in order, so the loads of later
-// tiles may stay in flight).
-//
-// MFMA operands are swapped (C^T = B^T A^T per fragment pair): a lane then holds, per accumulator quad,
-// four consecutive columns of ONE row, so the fused epilogue act(alpha acc + bias + residual) packs 8-byte
-// groups, stages them in a wave-private LDS tile and stores row-major 16 bytes per lane.
+// 192 B/clk of LDS traffic, both above what a CU gets; a 256x256 tile halves the first and, with 128x128 wave
+// tiles, brings the second to 96 B/clk.
 
-template <int BN, int NS>
-struct WideGeom {
-  static constexpr int BM = 256;
-  static constexpr int TM = 2, TN = BN / 64;          // 32x32 fragments per wave tile (64 x BN/2)
-  static constexpr int WTN = BN / 2;
-  static constexpr int kBOff = BM * 128;
-  static constexpr int kStage = (BM + BN) * 128;
-  static constexpr int kLoadsB = BN / 64;             // 1 KB slices per wave and tile: 4 of A, BN/64 of B
-  static constexpr int kLoads = 4 + kLoadsB;
-  static constexpr int kOutPitch = WTN * 2 + 16;      // bytes per row of a wave's 16-bit staging tile
-  static constexpr int kOutWave = 64 * kOutPitch;
-  static constexpr int kLds = NS * kStage > 8 * kOutWave ? NS * kStage : 8 * kOutWave;
-};
-
-#if defined(LLC_WIDE_ABL) && (LLC_WIDE_ABL & 4)
-#define LLC_WAIT_VM_LOOP(VM)
-#else
-#define LLC_WAIT_VM_LOOP(VM) LLC_WAIT_VM(VM)
-#endif
 #define LLC_WAIT_VM(VM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (7 << 4) | (15 << 8) | (((VM) >> 4) << 14))
-#define LLC_PHASE_END()                \
-  __builtin_amdgcn_sched_barrier(0);   \
-  __builtin_amdgcn_s_barrier();        \
-  __builtin_amdgcn_sched_barrier(0)
 
 #ifdef LLC_GEMM_TUNE
 __device__ unsigned long long llc_dbg_clk[2];  // longest workgroup: shader clocks, 100 MHz ticks
@@ -63,12 +20,68 @@ __device__ unsigned long long llc_dbg_clk[2];  // longest workgroup: shader cloc
 #define LLC_DBG_T1()
 #endif
 
-template <typename T, int BMODE, int BN, int NS>
-__global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmParams p) {
+// ---------------------------------------------------------------------------------------------
+// FOUR waves, one per SIMD, each owning a 128 x BN/2 accumulator tile (up to 256 accumulator registers per
+// lane, which the compiler keeps in the accumulation half of the register file).  With one wave per SIMD
+// nothing else can issue while that wave waits, so the instruction stream is ordered by hand: a k-step
+// (TM x TN MFMAs) is cut into slots of one MFMA, each followed by at most one fragment read of the NEXT k-step
+// and at most one direct-to-LDS load of a later k-tile, and slots are fenced (sched_barrier) so that the
+// compiler keeps that order; in-order issue then hides the memory instructions behind the 32 clocks an MFMA
+// occupies the matrix pipe.  (A variant with eight waves in two groups that alternate between a memory phase
+// and an MFMA phase, one barrier per phase, was measured at 0.43 of peak on 8192^3 against 0.49 here: its
+// 64 x 128 wave tiles read half as much again from LDS per MFMA and every phase pays a barrier.)
+//
+// LDS: two stages; A tiles at [0, 64 KB), B tiles behind them, so that the stage and the fragment row block
+// are immediate offsets of the LDS reads and a lane needs four address registers per operand (its row's
+// swizzled chunk for each k-step).  Stage of tile t is free once every wave has read its last fragments:
+// the barrier sits in front of the last k-step's MFMAs, the loads of tile t+2 go out behind it (first in that
+// k-step, the rest in the first k-steps of tile t+1) and have a whole k-tile of MFMAs to land.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+template <int TM, int TN>
+struct MmaOrder {
+  int i[TM * TN], j[TM * TN];
+  // growing squares: (0,0); (0,1) (1,0) (1,1); ... so that fragments are needed in the order A0 B0 A1 B1 ...
+  constexpr MmaOrder() : i{}, j{} {
+    int n = 0;
+    for (int d = 0; d < (TM > TN ? TM : TN); ++d) {
+      if (d < TN)
+        for (int a = 0; a < d && a < TM; ++a) { i[n] = a; j[n] = d; ++n; }
+      if (d < TM)
+        for (int b = 0; b <= d && b < TN; ++b) { i[n] = d; j[n] = b; ++n; }
+    }
+  }
+};
+
+template <int TM, int TN>
+constexpr MmaOrder<TM, TN> kMmaOrder{};
+
+template <int BN>
+struct WideGeom {
+  static constexpr int TM = 4, TN = BN / 64, WTN = BN / 2;
+  static constexpr int kAStage = 256 * 128, kBStage = BN * 128, kB0 = 2 * kAStage;
+  static constexpr int kLoadsA = 8, kLoadsB = BN / 32, kLoads = kLoadsA + kLoadsB;  // 1 KB slices per wave and k-tile
+  static constexpr int NG = TM * TN / 2;  // MFMA slots of a k-step that may carry a direct-to-LDS load (every other one)
+  static constexpr int NR = TM + TN;      // fragment reads per k-step
+  // direct-to-LDS loads of a tile by the k-step they are issued in: the last k-step of the tile two ahead of it,
+  // then k-steps 0 and 1 of the tile before it
+  static constexpr int kD3 = NG < 6 ? NG : 6, kD0 = (kLoads - kD3 + 1) / 2, kD1 = kLoads - kD3 - kD0;
+  static_assert(kD1 >= 0 && kD1 <= NG && kD0 <= NG, "load schedule");
+  static constexpr int kOutPitch = WTN * 2 + 16, kOutWave = 128 * kOutPitch;
+  static constexpr int kLds = 2 * (kAStage + kBStage) > 4 * kOutWave ? 2 * (kAStage + kBStage) : 4 * kOutWave;
+};
+
+template <typename T, int BMODE, int BN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_wide_kernel(const GemmParams p) {
   static_assert(sizeof(T) == 2, "16-bit operands");
-  static_assert(NS == 2 || NS == 3, "two or three LDS stages");
   static_assert(BMODE == kBKMajor || BN != 192, "row-major B: the chunk swizzle needs 16 or 32 chunks per row");
-  using G = WideGeom<BN, NS>;
+  using G = WideGeom<BN>;
   constexpr int TM = G::TM, TN = G::TN;
   extern __shared__ __align__(16) char smem[];
   LLC_DBG_T0();
@@ -77,75 +90,75 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmParams p) {
   const int m0 = tile_m * 256, n0 = tile_n * BN;
   const int z = blockIdx.z;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
-  const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
-  const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
+  const char* A = (const char*)((const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1 + (int64_t)m0 * p.a_sm);
+  const char* B = (const char*)((const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1 +
+                                (BMODE == kBKMajor ? (int64_t)n0 * p.b_sn : (int64_t)n0));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
-  const int grp = wave >> 2, wm = wave & 3, wn = grp;
+  const int wm = wave >> 1, wn = wave & 1;
   const int li = lane % 32, lh = lane / 32;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
-  // ---- this wave's direct-to-LDS loads: slices wave + 8 j of the A tile (8 rows each), then of the B tile ----
-  const char* ga[4];
-  const char* gb[G::kLoadsB];
-  int64_t b_step;
+  // ---- direct-to-LDS loads.  Load d < 8 of a tile is A slice wave + 4 d (rows 8 wave + lane / 8 + 32 d), the others
+  //      B slices the same way: a uniform base per load plus one of two lane offsets (the row swizzle alternates
+  //      with d).  Offsets are bytes. ----
+  const int64_t a_row_bytes = p.a_sm * 2, b_row_bytes = (BMODE == kBKMajor ? p.b_sn : p.b_sk) * 2;
+  uint32_t la_off[2], lb_off[2];
+  {
+    const int row0 = wave * 8 + lane / 8;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = (wave + 8 * j) * 8 + lane / 8;
-    ga[j] = (const char*)(A + (int64_t)(m0 + row) * p.a_sm + (((lane % 8) ^ lds_swz(row)) << 3));
+    for (int par = 0; par < 2; ++par) {
+      la_off[par] = (uint32_t)(row0 * a_row_bytes) + ((((lane % 8) ^ lds_swz(row0) ^ (4 * par)) & 7) << 4);
+      if constexpr (BMODE == kBKMajor) lb_off[par] = (uint32_t)(row0 * b_row_bytes) + ((((lane % 8) ^ lds_swz(row0) ^ (4 * par)) & 7) << 4);
+    }
+    if constexpr (BMODE != kBKMajor) {
+      constexpr int RPS = 1024 / (2 * BN);  // k rows per slice
+      const int krow0 = RPS * wave + lane / (64 / RPS), slot = lane % (64 / RPS);
+      lb_off[0] = lb_off[1] = (uint32_t)(krow0 * b_row_bytes) + ((slot ^ ((krow0 & 3) << 2)) << 4);
+    }
   }
-#pragma unroll
-  for (int j = 0; j < G::kLoadsB; ++j) {
-    if constexpr (BMODE == kBKMajor) {
-      const int row = (wave + 8 * j) * 8 + lane / 8;
-      gb[j] = (const char*)(B + (int64_t)(n0 + row) * p.b_sn + (((lane % 8) ^ lds_swz(row)) << 3));
+  // load d of k-tile kt into `stage`: a uniform 64-bit base (scalar registers) plus the lane's 32-bit offset.  The
+  // empty asm keeps the compiler from folding base and offset into sixteen loop-invariant 64-bit lane pointers.
+  auto dma = [&](auto d_tag, int kt, int stage) {
+    constexpr int D = decltype(d_tag)::value;
+    if constexpr (D < G::kLoadsA) {
+      uint32_t off = la_off[D & 1];
+      asm volatile("" : "+v"(off));
+      const char* g = A + (int64_t)(32 * D) * a_row_bytes + (int64_t)kt * 128;
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(g + off), LLC_LPTR(smem + stage * G::kAStage + (wave + 4 * D) * 1024), 16, 0, 0);
     } else {
-      const int byte = (wave + 8 * j) * 1024 + lane * 16;
-      const int krow = byte / (2 * BN), slot = (byte % (2 * BN)) / 16;
-      gb[j] = (const char*)(B + (int64_t)krow * p.b_sk + n0 + ((slot ^ ((krow & 3) << 2)) << 3));
-    }
-  }
-  if constexpr (BMODE == kBKMajor) b_step = 128;
-  else b_step = 64 * p.b_sk * 2;
-  auto issue = [&](int stage) {
-    char* base = smem + stage * G::kStage;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      __builtin_amdgcn_global_load_lds(LLC_GPTR(ga[j]), LLC_LPTR(base + (wave + 8 * j) * 1024), 16, 0, 0);
-      ga[j] += 128;
-    }
-#pragma unroll
-    for (int j = 0; j < G::kLoadsB; ++j) {
-      __builtin_amdgcn_global_load_lds(LLC_GPTR(gb[j]), LLC_LPTR(base + G::kBOff + (wave + 8 * j) * 1024), 16, 0, 0);
-      gb[j] += b_step;
+      constexpr int DB = D - G::kLoadsA;
+      uint32_t off = lb_off[BMODE == kBKMajor ? (DB & 1) : 0];
+      asm volatile("" : "+v"(off));
+      const char* g;
+      if constexpr (BMODE == kBKMajor) g = B + (int64_t)(32 * DB) * b_row_bytes + (int64_t)kt * 128;
+      else g = B + ((int64_t)(4 * DB * (1024 / (2 * BN))) + (int64_t)kt * 64) * b_row_bytes;
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(g + off), LLC_LPTR(smem + G::kB0 + stage * G::kBStage + (wave + 4 * DB) * 1024), 16, 0, 0);
     }
   };
 
-  // ---- fragment addresses.  k-major tiles: row r, 16-byte chunk c at r * 128 + ((c ^ swz(r)) << 4); lane half lh
-  //      of k-step s takes chunk 2 s + lh: off = base + (x ^ (s << 5)) with x = (lh ^ swz) << 4. ----
-  int a_base[TM], a_x[TM], b_base[TN], b_x[TN];
+  // ---- fragment addresses: ua[c] / ub[c] = this lane's row with k chunk pair c; fragment (k-step s, row block i) reads
+  //      ua[s ^ 2 (i & 1)] + 4096 i + stage (the row swizzle of block i differs from block 0's by 4 (i & 1)) ----
+  uint32_t ua[4], ub[4];
+  {
+    const int ra = wm * 128 + li, va = lh ^ lds_swz(ra);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int r = wm * 64 + i * 32 + li;
-    a_base[i] = r * 128;
-    a_x[i] = (lh ^ lds_swz(r)) << 4;
-  }
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
+    for (int c = 0; c < 4; ++c) ua[c] = ra * 128 + (((va ^ (2 * c)) & 7) << 4);
     if constexpr (BMODE == kBKMajor) {
-      const int r = wn * G::WTN + j * 32 + li;
-      b_base[j] = G::kBOff + r * 128;
-      b_x[j] = (lh ^ lds_swz(r)) << 4;
+      const int rb = wn * G::WTN + li, vb = lh ^ lds_swz(rb);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) ub[c] = G::kB0 + rb * 128 + (((vb ^ (2 * c)) & 7) << 4);
     } else {
-      // transposing read: lane = 16 g + 4 jj + q reads 8 bytes: k row 16 s + 8 (g >> 1) + 4 u + jj, n chunk
-      // (16 (g & 1) + 4 q) / 8 of the fragment's 32 columns; slot = chunk ^ (jj << 2)
+      // transposing read of fragment j: lane = 16 g + 4 jj + q reads 8 bytes of k row 16 s + 8 (g >> 1) + 4 u + jj at
+      // n chunk (16 (g & 1) + 4 q) / 8 of the fragment's 32 columns, stored at slot chunk ^ (jj << 2)
       const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
-      const int nchunk = (wn * G::WTN + j * 32) / 8 + 2 * (g & 1) + (q >> 1);
-      b_base[j] = G::kBOff + (8 * (g >> 1) + jj) * (2 * BN) + ((nchunk ^ (jj << 2)) << 4) + (q & 1) * 8;
-      b_x[j] = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int nchunk = (wn * G::WTN + j * 32) / 8 + 2 * (g & 1) + (q >> 1);
+        ub[j] = G::kB0 + (8 * (g >> 1) + jj) * (2 * BN) + ((nchunk ^ (jj << 2)) << 4) + (q & 1) * 8;
+      }
     }
   }
 
-  f32x16_t acc[TM][TN];  // register r of lane (li, lh): row li of A fragment i, column 8 (r / 4) + 4 lh + r % 4 of B fragment j
+  f32x16_t acc[TM][TN];  // register r of lane (li, lh): row li of A block i, column 8 (r / 4) + 4 lh + r % 4 of B block j
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -153,118 +166,121 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   u32x4_t fa[2][TM], fb[2][TN];
-  uint2 tb[2][TN][2];
+  uint2 tb[2][TN][2];  // row-major B: the two transposing reads of each B fragment
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
-  // fragments of half tile h of `stage` into registers
-#define LLC_WIDE_READ(STAGE, H)                                                                                \
-  {                                                                                                            \
-    const int sb_ = (STAGE) * G::kStage;                                                                       \
-    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                                         \
-      const int s_ = 2 * (H) + s2;                                                                             \
-      _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                           \
-          fa[s2][i] = *(const u32x4_t*)(smem + sb_ + a_base[i] + (a_x[i] ^ (s_ << 5)));                        \
-      _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                                         \
-        if constexpr (BMODE == kBKMajor) {                                                                     \
-          fb[s2][j] = *(const u32x4_t*)(smem + sb_ + b_base[j] + (b_x[j] ^ (s_ << 5)));                        \
-        } else {                                                                                               \
-          _Pragma("unroll") for (int u = 0; u < 2; ++u)                                                        \
-              tb[s2][j][u] = lds_read_tr16(lds0 + sb_ + b_base[j] + (16 * s_ + 4 * u) * (2 * BN));            \
-        }                                                                                                      \
-      }                                                                                                        \
-    }                                                                                                          \
-  }
-  // after the wait: results of the (untracked) transposing reads become the B fragments
-#define LLC_WIDE_TIE()                                                                                         \
-  if constexpr (BMODE != kBKMajor) {                                                                           \
-    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) _Pragma("unroll") for (int j = 0; j < TN; ++j) {          \
-      asm volatile("" : "+v"(tb[s2][j][0]), "+v"(tb[s2][j][1]));                                               \
-      fb[s2][j] = u32x4_t{tb[s2][j][0].x, tb[s2][j][0].y, tb[s2][j][1].x, tb[s2][j][1].y};                     \
-    }                                                                                                          \
-  }
-#define LLC_WIDE_MMA()                                                                                         \
-  _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) _Pragma("unroll") for (int i = 0; i < TM; ++i)              \
-      _Pragma("unroll") for (int j = 0; j < TN; ++j) mfma_step<T>(fb[s2][j], fa[s2][i], acc[i][j]);
-
-  const int nk = p.K / 64;
-#pragma unroll
-  for (int x = 0; x < NS - 1; ++x)
-    if (x < nk) issue(x);
-  // tile 0 complete; with three stages tile 1 may still be in flight
-  if (NS == 3 && nk >= 2) LLC_WAIT_VM(G::kLoads);
-  else LLC_WAIT_VM(0);
-  LLC_PHASE_END();
-  if (grp == 1) { LLC_PHASE_END(); }  // group 1 runs one phase behind group 0
-
-  auto main_loop = [&](auto grp_tag) {
-    constexpr int GRP = decltype(grp_tag)::value;
-    int st = 0;  // t % NS
-    for (int t = 0; t < nk; ++t) {
-      // ---- memory phase, first half of tile t ----
-#if defined(LLC_WIDE_ABL) && (LLC_WIDE_ABL & 1)
-      if (t + NS - 1 < nk && t < 0) {
-#else
-      if (t + NS - 1 < nk) {
-#endif
-        int dst = st + NS - 1;
-        if (dst >= NS) dst -= NS;
-        issue(dst);
-      }
-#if defined(LLC_WIDE_ABL) && (LLC_WIDE_ABL & 2)
-      if (t < 1)
-#endif
-      LLC_WIDE_READ(st, 0)
-      LLC_WAIT_LGKM0();
-      LLC_WIDE_TIE()
-      LLC_PHASE_END();
-      // ---- compute phase ----
-      __builtin_amdgcn_s_setprio(1);
-      LLC_WIDE_MMA()
-      __builtin_amdgcn_s_setprio(0);
-      LLC_PHASE_END();
-      // ---- memory phase, second half ----
-#if defined(LLC_WIDE_ABL) && (LLC_WIDE_ABL & 2)
-      if (t < 1)
-#endif
-      LLC_WIDE_READ(st, 1)
-      LLC_WAIT_LGKM0();
-      LLC_WIDE_TIE()
-      if constexpr (GRP == 1) {
-        // tile t+1 must be complete before the next barrier; the loads of tile t+2 (NS = 3) may still fly
-        if (NS >= 3 && t + 2 < nk) { LLC_WAIT_VM_LOOP(G::kLoads); }
-        else { LLC_WAIT_VM_LOOP(0); }
-      }
-      LLC_PHASE_END();
-      // ---- compute phase ----
-      __builtin_amdgcn_s_setprio(1);
-      LLC_WIDE_MMA()
-      __builtin_amdgcn_s_setprio(0);
-      if constexpr (GRP == 0) {
-        if (NS >= 3 && t + 2 < nk) { LLC_WAIT_VM_LOOP(G::kLoads); }
-        else { LLC_WAIT_VM_LOOP(0); }
-      }
-      LLC_PHASE_END();
-      st = st + 1 == NS ? 0 : st + 1;
+  // read item R (A0 B0 A1 B1 ... in the order the MFMAs need them) of k-step S of `STAGE` into fragment set SET
+  auto read_item = [&](auto r_tag, auto s_tag, auto stage_tag, auto set_tag) {
+    constexpr int R = decltype(r_tag)::value, S = decltype(s_tag)::value, ST = decltype(stage_tag)::value, SET = decltype(set_tag)::value;
+    // item R: blocks alternate A, B while both remain
+    constexpr int both = 2 * (TM < TN ? TM : TN);
+    constexpr bool is_a = R < both ? (R % 2 == 0) : (TM > TN);
+    constexpr int blk = R < both ? R / 2 : (R - both) + (TM < TN ? TM : TN);
+    if constexpr (is_a) {
+      fa[SET][blk] = *(const u32x4_t*)(smem + (ua[S ^ (2 * (blk & 1))] + blk * 4096 + ST * G::kAStage));
+    } else if constexpr (BMODE == kBKMajor) {
+      fb[SET][blk] = *(const u32x4_t*)(smem + (ub[S ^ (2 * (blk & 1))] + blk * 4096 + ST * G::kBStage));
+    } else {
+      // inline asm: the compiler would order a transposing read it knows about behind every direct-to-LDS load in
+      // flight (vmcnt(0)).  Its result is used only behind the s_waitcnt at the top of the k-step that consumes it.
+      uint2& t0 = tb[SET][blk][0];  // asm operands inside a generic lambda must be locals
+      uint2& t1 = tb[SET][blk][1];
+      const uint32_t addr = lds0 + ub[blk];
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(t0) : "v"(addr), "n"((16 * S) * (2 * BN) + ST * G::kBStage));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(t1) : "v"(addr), "n"((16 * S + 4) * (2 * BN) + ST * G::kBStage));
     }
   };
-  if (grp == 0) {
-    main_loop(std::integral_constant<int, 0>{});
-    LLC_PHASE_END();  // pairs with group 1's last compute phase
-  } else {
-    main_loop(std::integral_constant<int, 1>{});
-  }
-#undef LLC_WIDE_READ
-#undef LLC_WIDE_TIE
-#undef LLC_WIDE_MMA
 
-  // ---- epilogue.  Every wave is past the last barrier: no fragment read and no load is outstanding, the
-  //      stages are free.  Each wave stages its 64 x WTN tile in LDS of its own (no barrier needed). ----
+  const int nk = p.K / 64;
+  // One k-step: S of tile t (stage ST).  The fragments of the next k-step are read here (behind the last tile that is
+  // the other stage's stale data, read and never used).  The loads scheduled in this k-step belong to tile t+1 (S < 3) or
+  // t+2 (S == 3); CHECK: that tile may not exist, look before loading.
+  auto step = [&](auto stage_tag, auto s_tag, auto check_tag, int t) {
+    constexpr int ST = decltype(stage_tag)::value, S = decltype(s_tag)::value;
+    constexpr bool CHECK = decltype(check_tag)::value;
+    constexpr int CUR = S & 1, NXT = CUR ^ 1;
+    constexpr int RST = S == 3 ? (ST ^ 1) : ST, RS = (S + 1) & 3;
+    if constexpr (S == 3) {
+      // every fragment of this tile is in registers (this wave's), tile t+1 has landed (this wave's loads)
+      __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (BMODE != kBKMajor) {
+      // the transposing reads of this k-step's B fragments were issued at least four MFMAs ago
+      LLC_WAIT_LGKM0();
+      static_for<TN>([&](auto j_tag) {
+        constexpr int J = decltype(j_tag)::value;
+        uint2& t0 = tb[CUR][J][0];
+        uint2& t1 = tb[CUR][J][1];
+        asm volatile("" : "+v"(t0), "+v"(t1));
+        fb[CUR][J] = u32x4_t{t0.x, t0.y, t1.x, t1.y};
+      });
+    }
+    constexpr int dlo = S == 3 ? 0 : (S == 0 ? G::kD3 : G::kD3 + G::kD0);
+    constexpr int dcnt = S == 3 ? G::kD3 : (S == 0 ? G::kD0 : (S == 1 ? G::kD1 : 0));
+    const int kt = S == 3 ? t + 2 : t + 1;
+    const bool load = !CHECK || kt < nk;
+    // one MFMA per slot; behind it at most one memory instruction of either kind: fragment reads of the next k-step in
+    // the odd slots, direct-to-LDS loads in the even ones (what does not fit that pattern shares a slot)
+    constexpr int NS1 = TM * TN;                                       // MFMA slots
+    constexpr int NRS = BMODE == kBKMajor ? NS1 : NS1 - 4;             // slots that may carry reads (asm reads: not the last four)
+    static_for<NS1>([&](auto q_tag) {
+      constexpr int Q = decltype(q_tag)::value;
+      constexpr int i0 = kMmaOrder<TM, TN>.i[Q], j0 = kMmaOrder<TM, TN>.j[Q];
+      mfma_step<T>(fb[CUR][j0], fa[CUR][i0], acc[i0][j0]);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (Q < NRS) {
+        constexpr int lo = Q * G::NR / NRS, hi = (Q + 1) * G::NR / NRS;
+        static_for<hi - lo>([&](auto r_tag) {
+          read_item(std::integral_constant<int, lo + decltype(r_tag)::value>{}, std::integral_constant<int, RS>{},
+                    std::integral_constant<int, RST>{}, std::integral_constant<int, NXT>{});
+        });
+      }
+      if constexpr (!(Q & 1) && (Q / 2) < dcnt) {
+        if (load) dma(std::integral_constant<int, dlo + Q / 2>{}, kt, S == 3 ? ST : (ST ^ 1));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto tile = [&](auto stage_tag, auto check_tag, int t) {
+    step(stage_tag, std::integral_constant<int, 0>{}, check_tag, t);
+    step(stage_tag, std::integral_constant<int, 1>{}, check_tag, t);
+    step(stage_tag, std::integral_constant<int, 2>{}, check_tag, t);
+    step(stage_tag, std::integral_constant<int, 3>{}, check_tag, t);
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+
+  // ---- prologue: tile 0 whole, the first loads of tile 1; fragments of the first k-step ----
+  static_for<G::kLoads>([&](auto d_tag) { dma(d_tag, 0, 0); });
+  static_for<G::kD3>([&](auto d_tag) { dma(d_tag, 1, 1); });
+  LLC_WAIT_VM(G::kD3);
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  static_for<G::NR>([&](auto r_tag) { read_item(r_tag, S0{}, S0{}, S0{}); });
+
+  // tiles in pairs (the stage is a compile-time constant) while the loads they schedule all exist, then one by one
+  int t = 0;
+  for (; t + 3 < nk; t += 2) {
+    tile(S0{}, std::false_type{}, t);
+    tile(S1{}, std::false_type{}, t + 1);
+  }
+  // two or three tiles are left, the first of them at stage 0
+  tile(S0{}, std::true_type{}, t);
+  tile(S1{}, std::true_type{}, t + 1);
+  if (t + 2 < nk) tile(S0{}, std::true_type{}, t + 2);
+
+  // ---- epilogue.  The last barrier (in front of the last k-step) has seen every wave's last fragment read and
+  //      last load complete: the stages are free.  Each wave stages its 128 x WTN tile in LDS of its own. ----
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
   const T* bias = p.bias ? (const T*)p.bias + (int64_t)z0 * p.bias_sb : nullptr;
   char* wst = smem + wave * G::kOutWave;
-  const int ncol0 = n0 + wn * G::WTN;
-  // one instantiation per (activation, residual) so that the per-element code has no branches
+  const int ncol0 = n0 + wn * G::WTN, mrow0 = m0 + wm * 128;
   auto stage_out = [&](auto act_tag, auto res_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     constexpr bool RES = decltype(res_tag)::value;
@@ -279,7 +295,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmParams p) {
         for (int i = 0; i < TM; ++i) {
           const int row = i * 32 + li;
           uint2 rq = {0, 0};
-          if constexpr (RES) rq = *(const uint2*)(res + (int64_t)(m0 + wm * 64 + row) * p.c_sm + ncol0 + col);
+          if constexpr (RES) rq = *(const uint2*)(res + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + col);
           uint32_t o[2];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -308,25 +324,24 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemmParams p) {
   else with_res(std::integral_constant<int, LLC_ACT_NONE>{});
   constexpr int kChunks = G::WTN / 8;  // 16-byte chunks per row of the wave tile
 #pragma unroll
-  for (int it = 0; it < kChunks; ++it) {
+  for (int it = 0; it < 2 * kChunks; ++it) {
     const int idx = it * 64 + lane;
     const int row = idx / kChunks, ch = idx % kChunks;
     const u32x4_t v = *(const u32x4_t*)(wst + row * G::kOutPitch + ch * 16);
-    *(u32x4_t*)(C + (int64_t)(m0 + wm * 64 + row) * p.c_sm + ncol0 + ch * 8) = v;
+    *(u32x4_t*)(C + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + ch * 8) = v;
   }
   LLC_DBG_T1();
 }
 
 template <typename T, int BMODE, int BN>
 int launch_wide(const GemmParams& p0, int batch, hipStream_t s) {
-  constexpr int NS = BN == 128 ? 3 : 2;
-  using G = WideGeom<BN, NS>;
+  using G = WideGeom<BN>;
   GemmParams p = p0;
   p.tiles_m = p.M / 256;
   p.tiles_n = p.N / BN;
-  auto kern = gemm_wide_kernel<T, BMODE, BN, NS>;
+  auto kern = gemm_wide_kernel<T, BMODE, BN>;
   static std::atomic<uint32_t> lds_allowed{0};
   LLC_TRY(allow_dynamic_lds((const void*)kern, G::kLds, lds_allowed));
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(512), G::kLds, s, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(256), G::kLds, s, p);
   return check_launch("gemm_wide_kernel");
 }

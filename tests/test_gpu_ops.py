@@ -455,6 +455,50 @@ def test_matmul_16bit_complete_tiles(ops, oracle, M, N, K):
         assert_close_bf16(host(ops.matmul(da, bt.t(), epi)), bf16_round(w), "NT epilogue " + act)
 
 
+@pytest.mark.parametrize("M,N,K", [(3584, 3584, 128), (3584, 3584, 192), (3584, 2688, 256), (2048, 3200, 320),
+                                   (3584, 3584, 448)])
+def test_matmul_16bit_wide_tiles(ops, oracle, M, N, K):
+    """Shapes that take the 256 x BN tile kernel (complete tiles, at least 192 of them): BN = 256, 192 (N = 2688 =
+    14 x 192) and 128 (N = 3200 = 25 x 128); reductions of 2, 3, 4, 5 and 7 k-tiles (the pipeline's prologue, paired
+    main loop and two- or three-tile tail); row-major and transposed-view rhs, bf16 and f16, every fused epilogue."""
+    r = rng(M + 3 * N + 7 * K)
+    a = bf16_round(r.uniform(-1, 1, (M, K)))
+    b = bf16_round(r.uniform(-1, 1, (K, N)))
+    base = oracle.matmul(a, b, "mkn")
+    want = bf16_round(base)
+    da = dev(a, torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(da, dev(b, torch.bfloat16))), want, "NN bf16")
+    bt = dev(np.ascontiguousarray(b.T), torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(da, bt.t())), want, "NT bf16")
+    assert_close_bf16(host(ops.matmul(dev(a, torch.float16), dev(b, torch.float16))), base, "NN f16")
+    bth = dev(np.ascontiguousarray(b.T), torch.float16)
+    assert_close_bf16(host(ops.matmul(dev(a, torch.float16), bth.t())), base, "NT f16")
+    bias = bf16_round(r.standard_normal(N))
+    res = bf16_round(r.standard_normal((M, N)))
+    for act, alpha, with_res in [("none", 1.0, True), ("relu", 0.5, False), ("gelu", 0.125, True)]:
+        w = base * np.float32(alpha) + bias[None, :]
+        if with_res:
+            w = w + res
+        if act != "none":
+            w = oracle.unary(act, w)
+        epi = ops.Epilogue(alpha=alpha, bias=dev(bias, torch.bfloat16), residual=dev(res, torch.bfloat16) if with_res else None, act=act)
+        assert_close_bf16(host(ops.matmul(da, dev(b, torch.bfloat16), epi)), bf16_round(w), "NN epilogue " + act)
+        assert_close_bf16(host(ops.matmul(da, bt.t(), epi)), bf16_round(w), "NT epilogue " + act)
+
+
+def test_batch_matmul_16bit_wide_tiles(ops, oracle):
+    """Batches of complete 256-row tiles: the batch index rides in the grid's z dimension of the wide-tile kernel."""
+    r = rng(77)
+    B, M, N, K = 4, 1792, 1792, 192
+    a = bf16_round(r.uniform(-1, 1, (B, M, K)))
+    b = bf16_round(r.uniform(-1, 1, (B, K, N)))
+    want = bf16_round(oracle.batch_matmul(a, b, "mkn"))
+    got = ops.batch_matmul(dev(a, torch.bfloat16), dev(b, torch.bfloat16))
+    assert_close_bf16(host(got), want, "wide batch_matmul NN")
+    bt = dev(np.ascontiguousarray(b.transpose(0, 2, 1)), torch.bfloat16)
+    assert_close_bf16(host(ops.batch_matmul(dev(a, torch.bfloat16), bt.transpose(1, 2))), want, "wide batch_matmul NT")
+
+
 def _attention_oracle(oracle, q, k, v, mask, scale, rnd):
     """The unfused op group on the CPU oracle: batch_matmul, scale, mask add, softmax over the keys, the
     probabilities rounded to the storage type (the fused kernel feeds them to the matrix cores in it), batch_matmul."""
