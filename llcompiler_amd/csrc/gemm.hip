@@ -882,13 +882,6 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
                         p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) && (!p.residual || al16(p.residual));
     if (dma_ok && p.M % 256 == 0 && p.K >= 128) {
       const int bn = wide_tile_n(p, batch, b_kvec);
-#ifdef LLC_GEMM_TUNE
-      if (getenv("LLC_WIDE_REGS")) {
-        if (bn == 256) return b_kvec ? launch_wide<T, kBKMajor, 256, kStageRegs>(p, batch, s) : launch_wide<T, kBNMajor, 256, kStageRegs>(p, batch, s);
-        if (bn == 192) return launch_wide<T, kBKMajor, 192, kStageRegs>(p, batch, s);
-        if (bn == 128) return b_kvec ? launch_wide<T, kBKMajor, 128, kStageRegs>(p, batch, s) : launch_wide<T, kBNMajor, 128, kStageRegs>(p, batch, s);
-      }
-#endif
       if (bn == 256) return b_kvec ? launch_wide<T, kBKMajor, 256>(p, batch, s) : launch_wide<T, kBNMajor, 256>(p, batch, s);
       if (bn == 192) return launch_wide<T, kBKMajor, 192>(p, batch, s);
       if (bn == 128) return b_kvec ? launch_wide<T, kBKMajor, 128>(p, batch, s) : launch_wide<T, kBNMajor, 128>(p, batch, s);

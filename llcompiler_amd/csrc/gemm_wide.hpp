@@ -77,9 +77,7 @@ struct WideGeom {
   static constexpr int kLds = 2 * (kAStage + kBStage) > 4 * kOutWave ? 2 * (kAStage + kBStage) : 4 * kOutWave;
 };
 
-enum { kStageDma = 0, kStageRegs = 1 };
-
-template <typename T, int BMODE, int BN, int STG>
+template <typename T, int BMODE, int BN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_wide_kernel(const GemmParams p) {
   static_assert(sizeof(T) == 2, "16-bit operands");
   static_assert(BMODE == kBKMajor || BN != 192, "row-major B: the chunk swizzle needs 16 or 32 chunks per row");
@@ -135,33 +133,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       else g = B + ((int64_t)(4 * DB * (1024 / (2 * BN))) + (int64_t)kt * 64) * b_row_bytes;
       __builtin_amdgcn_global_load_lds(LLC_GPTR(g + off), LLC_LPTR(smem + G::kB0 + stage * G::kBStage + (wave + 4 * DB) * 1024), 16, 0, 0);
     }
-  };
-
-  // Register staging (STG == kStageRegs): the same 1 KB slices come through registers instead, slice d of a tile in
-  // stg[d]: loaded two tiles ahead, written to its LDS stage three k-steps after the load was issued.  That
-  // gives a load a k-tile and a half to arrive without an LDS stage being reserved for it, and lets the loads go
-  // out at an even rate (one per four MFMAs) instead of in the burst that the two-stage window of the direct-to-LDS
-  // form forces.
-  u32x4_t stg[STG == kStageRegs ? G::kLoads : 1];
-  const uint32_t sa_off = (uint32_t)(wave * 1024 + lane * 16), sb_off = (uint32_t)(G::kB0 + wave * 1024 + lane * 16);
-  auto gload = [&](auto d_tag, int kt) {
-    constexpr int D = decltype(d_tag)::value;
-    if constexpr (D < G::kLoadsA) {
-      uint32_t off = la_off[D & 1];
-      asm volatile("" : "+v"(off));
-      stg[D] = *(const u32x4_t*)(A + (int64_t)(32 * D) * a_row_bytes + (int64_t)kt * 128 + off);
-    } else {
-      constexpr int DB = D - G::kLoadsA;
-      uint32_t off = lb_off[BMODE == kBKMajor ? (DB & 1) : 0];
-      asm volatile("" : "+v"(off));
-      if constexpr (BMODE == kBKMajor) stg[D] = *(const u32x4_t*)(B + (int64_t)(32 * DB) * b_row_bytes + (int64_t)kt * 128 + off);
-      else stg[D] = *(const u32x4_t*)(B + ((int64_t)(4 * DB * (1024 / (2 * BN))) + (int64_t)kt * 64) * b_row_bytes + off);
-    }
-  };
-  auto lstore = [&](auto d_tag, int stage) {
-    constexpr int D = decltype(d_tag)::value;
-    if constexpr (D < G::kLoadsA) *(u32x4_t*)(smem + (sa_off + stage * G::kAStage + 4 * D * 1024)) = stg[D];
-    else *(u32x4_t*)(smem + (sb_off + stage * G::kBStage + 4 * (D - G::kLoadsA) * 1024)) = stg[D];
   };
 
   // ---- fragment addresses: ua[c] / ub[c] = this lane's row with k chunk pair c; fragment (k-step s, row block i) reads
@@ -230,10 +201,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     constexpr int CUR = S & 1, NXT = CUR ^ 1;
     constexpr int RST = S == 3 ? (ST ^ 1) : ST, RS = (S + 1) & 3;
     if constexpr (S == 3) {
-      // every fragment of this tile is in registers (this wave's), tile t+1 is in LDS (this wave's share: its
-      // direct-to-LDS loads have landed, or its LDS stores are done)
-      if constexpr (STG == kStageDma) __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));
-      else LLC_WAIT_LGKM0();
+      // every fragment of this tile is in registers (this wave's), tile t+1 has landed (this wave's loads)
+      __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
@@ -269,29 +238,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     std::integral_constant<int, RST>{}, std::integral_constant<int, NXT>{});
         });
       }
-      if constexpr (STG == kStageDma) {
-        if constexpr (!(Q & 1) && (Q / 2) < dcnt) {
-          if (load) dma(std::integral_constant<int, dlo + Q / 2>{}, kt, S == 3 ? ST : (ST ^ 1));
-        }
-      } else {
-        // slice d is loaded (for tile t+2) in slot d NT / kLoads of the tile's NT = 4 NS1 slots and written to LDS
-        // 3 NS1 slots later: in this tile's last k-step if it was loaded in the first one, else in tile t+1
-        constexpr int GS = S * NS1 + Q, NT = 4 * NS1;
-        static_for<G::kLoads>([&](auto d_tag) {
-          constexpr int D = decltype(d_tag)::value, LS = D * NT / G::kLoads;
-          if constexpr (S == 3 && LS == Q) {
-            if (!CHECK || t + 2 < nk) lstore(d_tag, ST);
-          }
-          if constexpr (S < 3 && LS == GS + NS1) {
-            if (!CHECK || t + 1 < nk) lstore(d_tag, ST ^ 1);
-          }
-        });
-        static_for<G::kLoads>([&](auto d_tag) {
-          constexpr int D = decltype(d_tag)::value, LS = D * NT / G::kLoads;
-          if constexpr (LS == GS) {
-            if (!CHECK || t + 2 < nk) gload(d_tag, t + 2);
-          }
-        });
+      if constexpr (!(Q & 1) && (Q / 2) < dcnt) {
+        if (load) dma(std::integral_constant<int, dlo + Q / 2>{}, kt, S == 3 ? ST : (ST ^ 1));
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -306,21 +254,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   using S1 = std::integral_constant<int, 1>;
 
   // ---- prologue: tile 0 whole, the first loads of tile 1; fragments of the first k-step ----
-  if constexpr (STG == kStageDma) {
-    static_for<G::kLoads>([&](auto d_tag) { dma(d_tag, 0, 0); });
-    static_for<G::kD3>([&](auto d_tag) { dma(d_tag, 1, 1); });
-    LLC_WAIT_VM(G::kD3);
-  } else {
-    // tile 0 into stage 0; tile 1 into the registers, and the slices that the steady state writes in the last
-    // k-step of the tile before into stage 1 (the others are written during tile 0)
-    static_for<G::kLoads>([&](auto d_tag) { gload(d_tag, 0); });
-    static_for<G::kLoads>([&](auto d_tag) { lstore(d_tag, 0); });
-    static_for<G::kLoads>([&](auto d_tag) { gload(d_tag, 1); });
-    static_for<G::kLoads>([&](auto d_tag) {
-      if constexpr (decltype(d_tag)::value * 4 * TM * TN / G::kLoads < TM * TN) lstore(d_tag, 1);
-    });
-    LLC_WAIT_LGKM0();
-  }
+  static_for<G::kLoads>([&](auto d_tag) { dma(d_tag, 0, 0); });
+  static_for<G::kD3>([&](auto d_tag) { dma(d_tag, 1, 1); });
+  LLC_WAIT_VM(G::kD3);
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
@@ -397,13 +333,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   LLC_DBG_T1();
 }
 
-template <typename T, int BMODE, int BN, int STG = kStageDma>
+template <typename T, int BMODE, int BN>
 int launch_wide(const GemmParams& p0, int batch, hipStream_t s) {
   using G = WideGeom<BN>;
   GemmParams p = p0;
   p.tiles_m = p.M / 256;
   p.tiles_n = p.N / BN;
-  auto kern = gemm_wide_kernel<T, BMODE, BN, STG>;
+  auto kern = gemm_wide_kernel<T, BMODE, BN>;
   static std::atomic<uint32_t> lds_allowed{0};
   LLC_TRY(allow_dynamic_lds((const void*)kern, G::kLds, lds_allowed));
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(256), G::kLds, s, p);
