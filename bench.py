@@ -6,8 +6,10 @@ layernorm; fp32 and bf16) run through the C-ABI kernel library on one MI355X.
 
 A step is one pass over all ten ops with their inputs already resident in HBM.  Prints ONE JSON
 line: whole-suite latency per pass, the roofline of the kernel that dominates the pass (and of
-every other kernel under "kernels"), the end-to-end latencies of the four model configurations
-("model_latency_ms"), and the CPU oracle timed on a bounded sample of the same workload on this host.
+every other kernel under "kernels"), contraction shapes outside the suite ("extra_kernels"), the end-to-end latencies
+of the four model configurations with percentiles and achieved TFLOP/s ("model_configs"; medians also under
+"model_latency_ms"), and the CPU stand-ins timed on this host in the same run ("cpu_baseline": the C oracle on a
+bounded sample and torch CPU eager, for the suite and for every model configuration).
 """
 import argparse
 import json
@@ -110,6 +112,45 @@ def build_cases(ops, device, only=()):
     return cases
 
 
+def build_extra_cases(ops, device):
+    """Contractions outside the suite that the model configurations are made of, reported under "extra_kernels" (not
+    part of `value`): the bf16 matmul at 4096^3, the feed-forward products of the encoder block at batch 32 with their
+    fused epilogues (Linear weights [N,K] consumed as transposed views), and the convolution classes of ResNet-18 at
+    batch 16 (3x3 body layers channels-last in fp32 and bf16, the 7x7 stride-2 stem in NCHW)."""
+    gen = torch.Generator().manual_seed(1)
+    cases = _Cases([])
+    bf = torch.bfloat16
+    n = 4096
+    cases.add("matmul_4096", "bf16", "mfma", 2.0 * n * n * n, 3 * n * n * 2,
+              lambda: (_uniform((n, n), bf, gen, device), _uniform((n, n), bf, gen, device), torch.empty((n, n), dtype=bf, device=device)),
+              lambda a, b, o: ops.matmul(a, b, out=o, defer=True), 1)
+
+    def linear(name, M, N, K, act, with_res):
+        def make():
+            return (_uniform((M, K), bf, gen, device), _uniform((N, K), bf, gen, device) * 0.05, _uniform((N,), bf, gen, device),
+                    _uniform((M, N), bf, gen, device) if with_res else None, torch.empty((M, N), dtype=bf, device=device))
+        cases.add(name, "bf16", "mfma", 2.0 * M * N * K, (M * K + N * K + M * N * (2 if with_res else 1) + N) * 2, make,
+                  lambda x, w, b, r, o: ops.matmul(x, w.t(), ops.Epilogue(bias=b, residual=r, act=act), out=o, defer=True), 1)
+
+    linear("encoder_ffn1_16384x3072x768_gelu", 16384, 3072, 768, "gelu", False)
+    linear("encoder_ffn2_16384x768x3072_residual", 16384, 768, 3072, "none", True)
+    linear("encoder_proj_16384x768x768_residual", 16384, 768, 768, "none", True)
+    cl = torch.channels_last
+    for dt_name, dt, es in (("f32", torch.float32, 4), ("bf16", bf, 2)):
+        for c, hw in ((64, 56), (128, 28), (256, 14), (512, 7)):
+            cases.add("conv3x3_%dch_%dx%d" % (c, hw, hw), dt_name, "mfma", 2.0 * 16 * hw * hw * c * c * 9,
+                      (16 * c * hw * hw * 2 + c * c * 9) * es,
+                      lambda c=c, hw=hw, dt=dt: (_uniform((16, c, hw, hw), dt, gen, device).contiguous(memory_format=cl),
+                                                 (_uniform((c, c, 3, 3), dt, gen, device) * 0.05).contiguous(memory_format=cl),
+                                                 torch.empty((16, c, hw, hw), dtype=dt, device=device).contiguous(memory_format=cl)),
+                      lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 2)
+    cases.add("conv7x7_stem_3to64_224", "f32", "mfma", 2.0 * 16 * 112 * 112 * 64 * 147, (16 * 3 * 224 * 224 + 64 * 147 + 16 * 64 * 112 * 112) * 4,
+              lambda: (_uniform((16, 3, 224, 224), torch.float32, gen, device), _uniform((64, 3, 7, 7), torch.float32, gen, device) * 0.05,
+                       torch.empty((16, 64, 112, 112), dtype=torch.float32, device=device)),
+              lambda x, w, o: ops.conv2d(x, w, pad=(3, 3, 3, 3), stride=(2, 2), out=o, defer=True), 2)
+    return cases
+
+
 def time_gpu(fn, steps, warmup):
     """Average milliseconds per call of fn(i), HIP events on the stream the kernels are launched on."""
     for i in range(warmup):
@@ -141,15 +182,29 @@ def launch_spread_us(fn, n=100):
     return {"p10": round(times[n // 10], 2), "median": round(times[n // 2], 2), "p90": round(times[(9 * n) // 10], 2)}
 
 
-# HBM bytes per launch (reads + writes) of each case's kernel, from two rocprofv3 counter runs over this
-# same workload (FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000, the factors a plain copy of known
-# size gives): profiles/single_op_suite_hbm_counters.md holds the commands and the table.  Counters cannot
-# be read from inside a timed run, so these are carried as measured constants of the kernels as committed.
-MEASURED_TRAFFIC_BYTES = {
-    "matmul_f32": 117661870, "matmul_bf16": 58942540, "batch_matmul_f32": 59096383, "batch_matmul_bf16": 29560277,
-    "add_relu_f32": 805396346, "add_relu_bf16": 402856019, "softmax_f32": 134281219, "softmax_bf16": 67171380,
-    "layernorm_f32": 67250632, "layernorm_bf16": 33666897, "copy_f32": 536870912,
-}
+def measured_traffic():
+    """HBM bytes per launch (reads + writes) of each case's kernel, read from the table in
+    profiles/single_op_suite_hbm_counters.md: two rocprofv3 counter runs over this same workload (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what a plain copy of known size reads; the file holds the commands).  Counters
+    cannot be read from inside a timed run; a case the table does not list reports null."""
+    path = os.path.join(ROOT, "profiles", "single_op_suite_hbm_counters.md")
+    table = {}
+    try:
+        for line in open(path):
+            parts = line.split()
+            # case name first, then the kernel's name, then five numbers: read, write, total, algorithmic MB, ratio
+            if len(parts) >= 7 and parts[0].count("_") >= 1:
+                try:
+                    nums = [float(x) for x in parts[-5:]]
+                except ValueError:
+                    continue
+                table[parts[0]] = int(round(nums[2] * 1e6))
+    except OSError:
+        pass
+    return table
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic()
 
 
 def roofline_of(case, ms):
@@ -218,58 +273,140 @@ def cpu_baseline():
 
 MODELS = ("mlp", "resnet18", "encoder", "bert")
 
+# algorithmic flops per forward pass of each configuration (multiply-adds counted as two): the contractions only
+FLOP_MLP = 2.0 * 4 * (784 * 512 + 512 * 10)
+FLOP_RESNET18_B16 = 58.0e9 + 16.4e6
+FLOP_ENCODER_PER_SAMPLE = 8.05e9
 
-def model_latencies(which=MODELS):
-    """End-to-end latency per batch of the other four configurations (whole compiled graphs through the
-    executor, inputs resident on the GPU, synchronised wall clock over repeated calls): an MLP, ResNet-18
-    with folded batch norm, a bf16 encoder block compiled once with a symbolic batch, and a 12-layer BERT-base
-    shaped encoder compiled once with a symbolic sequence length.  Reported next to the suite, not part of
-    `value`.  `which` selects a subset (for profiling one model's kernels at a time)."""
+
+def flop_bert(seq, batch=8, layers=12, hidden=768):
+    return layers * batch * seq * (14.16e6 + 4.0 * seq * hidden)
+
+
+def _call_times_ms(f, n, warmup):
+    """Per-call device time of f(): one HIP event pair per call on the stream the kernels are launched on (torch's
+    current stream), calls issued back to back, host dispatch included in what the device sees."""
+    for _ in range(warmup):
+        f()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    evs[0].record()
+    for i in range(n):
+        f()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    return sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(n))
+
+
+def _stats(times, flops, dtype_name):
+    n = len(times)
+    med = times[n // 2]
+    tf = flops / (med * 1e-3) / 1e12
+    return {"median_ms": round(med, 4), "p10_ms": round(times[n // 10], 4), "p90_ms": round(times[(9 * n) // 10], 4), "calls": n,
+            "gflop": round(flops / 1e9, 3), "achieved_tflops": round(tf, 2), "peak_tflops": PEAK_MFMA_TFLOPS[dtype_name],
+            "frac_of_peak": round(tf / PEAK_MFMA_TFLOPS[dtype_name], 4), "dtype": dtype_name}
+
+
+def model_latencies(which=MODELS, calls=100):
+    """End-to-end latency per batch of the other four configurations (whole compiled graphs through the executor,
+    inputs resident on the GPU): an MLP, ResNet-18 with folded batch norm, a bf16 encoder block compiled once with a
+    symbolic batch, and a 12-layer BERT-base shaped encoder compiled once with a symbolic sequence length.  Median, p10
+    and p90 over `calls` event-timed calls each, and the achieved TFLOP/s against the peak of the type the contractions
+    run in.  Reported next to the suite, not part of `value`.  `which` selects a subset."""
     import warnings
     from llcompiler_amd.compiler.aot import compile_module
     from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18Folded, make_bert_inputs,
                                             make_encoder_inputs, make_mlp_inputs, make_resnet_inputs)
     warnings.filterwarnings("ignore")
-
-    def timed(f, n, w):
-        for _ in range(w):
-            f()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(n):
-            f()
-        torch.cuda.synchronize()
-        return round((time.perf_counter() - t0) * 1e3 / n, 4)
-
     res = {}
     with torch.no_grad():
         if "mlp" in which:
             x = make_mlp_inputs()[0].cuda()
             cm = compile_module(MLP().cuda(), (x,))
-            res["mlp_f32_batch4_ms"] = timed(lambda: cm(x), 200, 20)
+            res["mlp_f32_batch4"] = _stats(_call_times_ms(lambda: cm(x), max(calls, 200), 20), FLOP_MLP, "f32")
         if "resnet18" in which:
             xs = make_resnet_inputs(16, 224)[0].cuda()
             cr = compile_module(ResNet18Folded().cuda(), (xs,))
-            res["resnet18_f32_batch16_ms"] = timed(lambda: cr(xs), 20, 3)
+            res["resnet18_f32_batch16"] = _stats(_call_times_ms(lambda: cr(xs), calls, 3), FLOP_RESNET18_B16, "f32")
             # the same network in bf16 storage (not one of the five configurations: its convolutions run on the
             # bf16 matrix instructions, which the fp32 configuration cannot show)
             xh = xs.to(torch.bfloat16)
             ch = compile_module(ResNet18Folded().to(torch.bfloat16).cuda(), (xh,))
-            res["resnet18_bf16_batch16_ms"] = timed(lambda: ch(xh), 20, 3)
+            res["resnet18_bf16_batch16"] = _stats(_call_times_ms(lambda: ch(xh), calls, 3), FLOP_RESNET18_B16, "bf16")
         if "encoder" in which:
             xe = make_encoder_inputs(8, 512)[0].to(torch.bfloat16).cuda()
             ce = compile_module(EncoderBlock().to(torch.bfloat16).cuda(), (xe,),
                                 dynamic_shapes=({0: torch.export.Dim("batch")},))
             for b in (1, 8, 32):
                 xb = make_encoder_inputs(b, 512, seed=b)[0].to(torch.bfloat16).cuda()
-                res["encoder_block_bf16_seq512_batch%d_ms" % b] = timed(lambda: ce(xb), 50, 5)
+                res["encoder_block_bf16_seq512_batch%d" % b] = _stats(_call_times_ms(lambda: ce(xb), calls, 5),
+                                                                      FLOP_ENCODER_PER_SAMPLE * b, "bf16")
         if "bert" in which:
             cb = compile_module(BertEncoder().cuda(), tuple(t.cuda() for t in make_bert_inputs(8, 128)),
                                 dynamic_shapes=({1: torch.export.Dim("seq")}, {3: torch.export.Dim("seq")}))
             for sl in (128, 256, 512):
                 xi, mi = (t.cuda() for t in make_bert_inputs(8, sl, seed=sl))
-                res["bert_base_f32_batch8_seq%d_ms" % sl] = timed(lambda: cb(xi, mi), 10, 2)
+                res["bert_base_f32_batch8_seq%d" % sl] = _stats(_call_times_ms(lambda: cb(xi, mi), calls, 2), flop_bert(sl), "f32")
     return res
+
+
+def cpu_model_baselines(which=MODELS):
+    """The two CPU stand-ins for the model configurations, on this host: torch eager on all host threads, one timed
+    forward pass each after one warm-up pass (what the reference asserts equality with and falls back to), and the
+    C oracle (one thread, the reference's generated loop nests restated) on a sample whose rate is extrapolated by
+    flops to the whole pass."""
+    import warnings
+    from oracle import ref
+    from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18Folded, make_bert_inputs,
+                                            make_encoder_inputs, make_mlp_inputs, make_resnet_inputs)
+    warnings.filterwarnings("ignore")
+
+    def once(f):
+        f()
+        t0 = time.perf_counter()
+        f()
+        return round((time.perf_counter() - t0) * 1e3, 2)
+
+    eager, port = {}, {}
+    r = np.random.default_rng(1)
+    # oracle rates on samples: a Linear layer of the transformer configurations, one 3x3 body convolution and the stem
+    # of one image of the ResNet
+    a = r.uniform(-1, 1, (256, 768)).astype(np.float32)
+    w = r.uniform(-1, 1, (768, 768)).astype(np.float32)
+    t0 = time.perf_counter()
+    ref.matmul(a, w, "mnk")
+    linear_rate = 2.0 * 256 * 768 * 768 / (time.perf_counter() - t0)
+    xc = r.standard_normal((1, 64, 56, 56)).astype(np.float32)
+    wc = r.standard_normal((64, 64, 3, 3)).astype(np.float32)
+    t0 = time.perf_counter()
+    ref.conv2d(xc, wc, None, (1, 1, 1, 1))
+    conv_rate = 2.0 * 56 * 56 * 64 * 64 * 9 / (time.perf_counter() - t0)
+    sample = ("C oracle, 1 thread: a [256,768]x[768,768] matmul (%.2f GFLOP/s) stands for the Linear layers and attention "
+              "products, a 64->64 3x3 convolution of one 56x56 image (%.2f GFLOP/s) for the convolutions; each pass is its "
+              "flops divided by that rate" % (linear_rate / 1e9, conv_rate / 1e9))
+    with torch.no_grad():
+        if "mlp" in which:
+            m, x = MLP().eval(), make_mlp_inputs()[0]
+            eager["mlp_f32_batch4"] = once(lambda: m(x))
+            port["mlp_f32_batch4"] = round(FLOP_MLP / linear_rate * 1e3, 3)
+        if "resnet18" in which:
+            m, x = ResNet18Folded().eval(), make_resnet_inputs(16, 224)[0]
+            eager["resnet18_f32_batch16"] = once(lambda: m(x))
+            port["resnet18_f32_batch16"] = round(FLOP_RESNET18_B16 / conv_rate * 1e3, 1)
+        if "encoder" in which:
+            m = EncoderBlock().to(torch.bfloat16).eval()
+            for b in (1, 8, 32):
+                x = make_encoder_inputs(b, 512, seed=b)[0].to(torch.bfloat16)
+                eager["encoder_block_bf16_seq512_batch%d" % b] = once(lambda: m(x))
+                port["encoder_block_bf16_seq512_batch%d" % b] = round(FLOP_ENCODER_PER_SAMPLE * b / linear_rate * 1e3, 1)
+        if "bert" in which:
+            m = BertEncoder().eval()
+            for sl in (128, 256, 512):
+                xi, mi = make_bert_inputs(8, sl, seed=sl)
+                eager["bert_base_f32_batch8_seq%d" % sl] = once(lambda: m(xi, mi))
+                port["bert_base_f32_batch8_seq%d" % sl] = round(flop_bert(sl) / linear_rate * 1e3, 1)
+    return {"torch_cpu_eager_ms": eager, "threads": torch.get_num_threads(), "c_oracle_extrapolated_ms": port, "cores": 1,
+            "sample": sample}
 
 
 def main():
@@ -279,6 +416,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-models", action="store_true", help="skip the end-to-end latencies of the model configurations")
+    ap.add_argument("--no-extra", action="store_true", help="skip the contraction rows outside the suite (extra_kernels)")
     ap.add_argument("--models", default="", help="comma-separated subset of %s whose end-to-end latencies to "
                     "measure (default: all of them, or none when --only is given)" % ",".join(MODELS))
     ap.add_argument("--only", default="", help="comma-separated kernel names (e.g. matmul_bf16,softmax_f32): run just "
@@ -320,13 +458,25 @@ def main():
         "dominant_kernel": dominant["kernel"],
         "kernels": kernels,
     }
+    if not only and not args.no_extra:
+        extra = build_extra_cases(ops, device)
+        out["extra_kernels"] = [roofline_of(c, time_gpu(c.run, 50, 10)) for c in extra]
+        del extra
+        torch.cuda.empty_cache()
     if not args.no_models and models:
         try:
-            out["model_latency_ms"] = model_latencies(models)
+            configs = model_latencies(models)
+            out["model_configs"] = configs
+            out["model_latency_ms"] = {k + "_ms": v["median_ms"] for k, v in configs.items()}
         except Exception as e:  # the suite's line is still worth printing
             out["model_latency_ms"] = {"error": "%s: %s" % (type(e).__name__, e)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        if not args.no_models and models:
+            try:
+                out["cpu_baseline"]["model_configs"] = cpu_model_baselines(models)
+            except Exception as e:
+                out["cpu_baseline"]["model_configs"] = {"error": "%s: %s" % (type(e).__name__, e)}
     print(json.dumps(out))
 
 
