@@ -373,6 +373,119 @@ def test_plan_file_round_trip(oracle, tmp_path):
             except C.LlcHipError:
                 refused += 1
     assert refused > 100, refused
+    # an operand count that does not fit the step code (replay indexes the operands by position) is refused: the two
+    # matmul steps carry five operand records each, behind an empty attribute block (no integers, zeroed convolution
+    # and pooling attributes, no program), which is what locates the count in the file
+    marker = bytes(8 * (1 + 11 + 11 + 1)) + (5).to_bytes(8, "little")
+    counts = []
+    at = good.find(marker, size - 1400)
+    while at >= 0:
+        counts.append(at + len(marker) - 8)
+        at = good.find(marker, at + 1)
+    assert len(counts) == 2, counts
+    for pos in counts:
+        for n_op in (1, 2, 4, 6, 13):
+            bad = tmp_path / "bad_count.llcplan"
+            bad.write_bytes(good[:pos] + n_op.to_bytes(8, "little") + good[pos + 8:])
+            with pytest.raises(C.LlcHipError):
+                Plan.load(bad)
+
+
+def test_execution_and_tensor_have_the_reference_binding_surface(oracle, tmp_path):
+    """`Execution.load / run / run_with_symbols` and `Tensor(data, base, type, offset, size, stride)` as the
+    reference binds them (src/Pybind/Entrance.cpp:70-92,113-119), over a plan file: called the way
+    llcompiler/executor/engine.py:34-78 calls them."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.execution import Execution, Tensor
+    from llcompiler_amd.executor.plan_runner import Plan
+    C.init(0)
+    rng = np.random.default_rng(21)
+    M, K, H, N = 24, 40, 64, 8
+    w1 = rng.standard_normal((K, H), dtype=np.float32) * 0.1
+    b1 = rng.standard_normal((H,), dtype=np.float32)
+    w2 = rng.standard_normal((H, N), dtype=np.float32) * 0.1
+    x = torch.from_numpy(rng.standard_normal((M, K), dtype=np.float32)).cuda()
+    out = torch.empty((M, N), device="cuda")
+    plan = Plan()
+    plan.expect_symbols([M])
+    _record_two_layer(plan, x, out, w1, b1, w2, H)
+    path = tmp_path / "sym.llcplan"
+    plan.save(path)
+    del plan
+
+    def trans_to_tensor(*args):  # the reference's own conversion (engine.py:34-54), storage offset 0
+        return [Tensor(a.data_ptr(), a.data_ptr() + a.storage_offset(), C.FLOAT32, a.storage_offset(), a.shape, a.stride())
+                for a in args]
+
+    ex = Execution()
+    with pytest.raises(RuntimeError):
+        ex.run(trans_to_tensor(x), trans_to_tensor(out))          # nothing loaded yet
+    ex.load(str(path))
+    xs = rng.standard_normal((M, K), dtype=np.float32)
+    x2, out2 = torch.from_numpy(xs).cuda(), torch.zeros((M, N), device="cuda")
+    ex.run_with_symbols([M], trans_to_tensor(x2), trans_to_tensor(out2))
+    torch.cuda.synchronize()
+    want = oracle.matmul(oracle.unary("relu", oracle.matmul(xs, w1) + b1), w2)
+    assert_close(out2.cpu().numpy(), want, F32_RTOL, F32_ATOL, "Execution.run_with_symbols")
+    with pytest.raises(C.LlcHipError):
+        ex.run_with_symbols([M + 1], trans_to_tensor(x2), trans_to_tensor(out2))   # not the binding it was recorded for
+    with pytest.raises(C.LlcHipError):
+        ex.run(trans_to_tensor(x2), trans_to_tensor(out2))                         # the plan expects its symbol values
+    with pytest.raises(ValueError):
+        ex.run_with_symbols([M], trans_to_tensor(x2, x2), trans_to_tensor(out2))
+    # a second object with the same file is independent of the first (no process-wide binding)
+    ex2 = Execution()
+    ex2.load(str(path))
+    out3 = torch.zeros((M, N), device="cuda")
+    ex2.run_with_symbols([M], trans_to_tensor(x2), trans_to_tensor(out3))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out3.cpu().numpy(), out2.cpu().numpy())
+
+
+def test_two_plans_with_split_reductions_run_on_two_streams_at_once():
+    """Each plan owns the scratch memory of its split reductions: two plans replayed at the same time on two streams
+    give, bit for bit, what each gives alone (with one scratch buffer per device they overwrote each other's partial
+    sums)."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    L = C.lib()
+    M, N, K = 1024, 768, 3072                       # few output tiles, long reduction: split into chunks
+    gen = torch.Generator().manual_seed(5)
+    plans, blocks, outs = [], [], []
+    for _ in range(2):
+        a = (torch.rand(M, K, generator=gen) * 2 - 1).cuda()
+        w = (torch.rand(N, K, generator=gen) * 2 - 1).cuda()
+        out = torch.empty((M, N), device="cuda")
+        plan = Plan()
+        plan.declare_io(a, False)
+        plan.declare_io(w, False)
+        plan.declare_io(out, True)
+        ra, rw, ro = C.tensor_ref(a), C.tensor_ref(w.t()), C.tensor_ref(out)
+        with plan.recording():
+            C.check(L.llc_hip_matmul(ra.ptr, rw.ptr, None, ro.ptr, _stream()))
+        plans.append(plan)
+        blocks.append(ParamBlock([a, w, out]))
+        outs.append(out)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    alone = []
+    for plan, block, out, st in zip(plans, blocks, outs, streams):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        plan.run(block, st.cuda_stream)
+        torch.cuda.synchronize()
+        alone.append(out.clone())
+        assert not torch.isnan(out).any()
+    for out in outs:
+        out.fill_(float("nan"))
+    torch.cuda.synchronize()
+    for _ in range(10):
+        for plan, block, st in zip(plans, blocks, streams):
+            plan.run(block, st.cuda_stream)
+    torch.cuda.synchronize()
+    for out, want in zip(outs, alone):
+        np.testing.assert_array_equal(out.cpu().numpy(), want.cpu().numpy())
 
 
 @pytest.mark.parametrize("which", ["encoder_bf16", "resnet"])
