@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import (BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_close, assert_close_bf16, assert_close_f32,
+from tests.util import (BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_as_close_as_eager, assert_close, assert_close_bf16, assert_close_f32,
                         bf16_round, dev, host, rng)
 
 pytestmark = pytest.mark.gpu
@@ -33,9 +33,15 @@ def test_matmul_2048_f32(ops, oracle):
     # ones that cancel to ~0).  So: the stated tolerance must hold for all but 1 in 10^4 outputs, and
     # every output must be within 1e-4 of the output scale.
     strict_bad = int((err > F32_ATOL + F32_RTOL * np.abs(want)).sum())
-    assert strict_bad <= want.size // 10000, "%d outputs outside rtol 1e-4 / atol 1e-5" % strict_bad
+    assert strict_bad <= 150, "%d outputs outside rtol 1e-4 / atol 1e-5" % strict_bad
     scale = float(np.sqrt((want ** 2).mean()))
     assert err.max() <= F32_ATOL + F32_RTOL * scale, "max abs error %g at output scale %g" % (err.max(), scale)
+    # and against the float64 product: the kernel's rounding noise is no worse than the oracle's own (both sum 2048
+    # fp32 products per output, in nearly the same order), in the mean and at the worst output
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    e_kernel, e_oracle = np.abs(got - exact), np.abs(want - exact)
+    assert np.sqrt((e_kernel ** 2).mean()) <= 1.25 * np.sqrt((e_oracle ** 2).mean()), "rms error against fp64 worse than the oracle's"
+    assert e_kernel.max() <= 1.25 * e_oracle.max(), "max error against fp64 %g, the oracle's %g" % (e_kernel.max(), e_oracle.max())
     # aggregate check that no tile was dropped or duplicated: (A B) v == A (B v)
     v = _uniform((2048,), 3).astype(np.float64)
     np.testing.assert_allclose(got @ v, a.astype(np.float64) @ (b.astype(np.float64) @ v), rtol=1e-4, atol=1e-2)
@@ -86,4 +92,9 @@ def test_layernorm_full(ops, oracle):
                      "layernorm f32 gamma=1 beta=0")
     xb, gb, bb = bf16_round(x), bf16_round(g), bf16_round(b)
     got = host(ops.layer_norm(dev(xb, torch.bfloat16), dev(gb, torch.bfloat16), dev(bb, torch.bfloat16), 1e-5))
-    assert_close(got, bf16_round(oracle.layernorm_lastdim(xb, gb, bb, 1e-5)), BF16_RTOL, 2e-2, "layernorm bf16")
+    # bf16 outputs near zero (beta - gamma x_hat cancelling) have no meaningful relative error: the bar is the stated
+    # tolerance plus what the oracle's own result, rounded to bf16, misses the float64 evaluation by
+    x64, g64, b64 = xb.astype(np.float64), gb.astype(np.float64), bb.astype(np.float64)
+    mu = x64.mean(-1, keepdims=True)
+    exact = (x64 - mu) / np.sqrt(((x64 - mu) ** 2).mean(-1, keepdims=True) + 1e-5) * g64 + b64
+    assert_as_close_as_eager(got, bf16_round(oracle.layernorm_lastdim(xb, gb, bb, 1e-5)), exact, BF16_RTOL, BF16_ATOL, "layernorm bf16")
