@@ -13,8 +13,9 @@
  *
  * Layouts: dense row-major, extents as int64.  NCHW activations, FCHW weights.
  *
- * Pinning (which independent check holds each function in place) is listed in oracle/README.md
- * and exercised by tests/test_oracle_*.py.
+ * Pinning: tests/test_oracle_pins.py holds every function here against an independent check (the
+ * reference's own golden values, closed forms, float64 library routines, brute force on tiny inputs);
+ * the docstring of each test there names the function it pins and the mistake it would catch.
  */
 #include <math.h>
 #include <stdint.h>

@@ -97,6 +97,84 @@ def test_config5_bert_f32_symbolic_seq():
     assert len(cm.engine.instances) == 3
 
 
+def _oracle_linear(oracle, x2d, lin):
+    w, b = lin.weight.detach().numpy(), lin.bias.detach().numpy()
+    return oracle.matmul(x2d, np.ascontiguousarray(w.T), "mkn") + b[None, :]
+
+
+def _oracle_attention(oracle, attn, x, mask):
+    B, S, H = x.shape
+    nh, dh = attn.heads, attn.dh
+    x2 = x.reshape(B * S, H)
+
+    def split(t):
+        return np.ascontiguousarray(t.reshape(B, S, nh, dh).transpose(0, 2, 1, 3)).reshape(B * nh, S, dh)
+    q, k, v = (split(_oracle_linear(oracle, x2, l)) for l in (attn.q, attn.k, attn.v))
+    sc = oracle.batch_matmul(q, np.ascontiguousarray(k.transpose(0, 2, 1)), "mkn").reshape(B, nh, S, S) / np.float32(np.sqrt(dh))
+    if mask is not None:
+        sc = sc + mask
+    p = oracle.softmax_lastdim(np.ascontiguousarray(sc.reshape(-1, S), dtype=np.float32)).reshape(B * nh, S, S)
+    ctx = oracle.batch_matmul(p, v, "mkn").reshape(B, nh, S, dh).transpose(0, 2, 1, 3).reshape(B * S, H)
+    return _oracle_linear(oracle, np.ascontiguousarray(ctx), attn.o).reshape(B, S, H)
+
+
+def _oracle_layer_norm(oracle, ln, x):
+    return oracle.layernorm_lastdim(np.ascontiguousarray(x.reshape(-1, x.shape[-1])), ln.weight.detach().numpy(),
+                                    ln.bias.detach().numpy(), ln.eps).reshape(x.shape)
+
+
+def test_config3_resnet18_against_the_oracle_composition(oracle):
+    """ResNet-18 spelt with the C oracle's own primitives (direct convolution with bias, relu, max-pool, residual adds,
+    global average pool, matmul) on a size it finishes in seconds: the compiled network against the restated loop nests,
+    not only against torch eager."""
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval()
+    (x,) = make_resnet_inputs(2, 64)
+
+    def conv(mod, t):
+        c = mod.conv
+        p = c.padding[0]
+        y = oracle.conv2d(t, c.weight.detach().numpy(), c.bias.detach().numpy(), (p, p, p, p), tuple(c.stride))
+        return oracle.unary("relu", y) if mod.relu else y
+    t = conv(m.stem, x.numpy())
+    t = oracle.maxpool2d(t, (3, 3), (1, 1, 1, 1), (2, 2))
+    for blk in m.blocks:
+        idt = t if blk.down is None else conv(blk.down, t)
+        t = oracle.unary("relu", oracle.binary("add", conv(blk.c2, conv(blk.c1, t)), idt))
+    t = oracle.global_avgpool(t).reshape(2, 512)
+    want = _oracle_linear(oracle, t, m.fc)
+    with torch.no_grad():
+        opt, _ = _compile(m)
+        got = opt(x.cuda())
+    assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, "resnet18 2x3x64x64 vs the oracle composition")
+
+
+def test_config4_and_5_blocks_against_the_oracle_composition(oracle):
+    """The pre-LN encoder block (config 4's graph, in fp32) and a post-LN BERT layer with its additive padding mask
+    (config 5's graph) spelt with the oracle's matmul, batch_matmul, softmax, layernorm and elementwise primitives."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import BertEncoder, EncoderBlock, make_bert_inputs, make_encoder_inputs
+    enc = EncoderBlock().eval()
+    (x,) = make_encoder_inputs(2, 64)
+    xn = x.numpy()
+    h = xn + _oracle_attention(oracle, enc.attn, _oracle_layer_norm(oracle, enc.ln1, xn), None)
+    f = oracle.unary("gelu", _oracle_linear(oracle, _oracle_layer_norm(oracle, enc.ln2, h).reshape(-1, 768), enc.fc1))
+    want = h + _oracle_linear(oracle, f, enc.fc2).reshape(h.shape)
+    with torch.no_grad():
+        got = compile_module(copy.deepcopy(enc).cuda(), (x.cuda(),))(x.cuda())
+    assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, "encoder block vs the oracle composition")
+    bert = BertEncoder(layers=2).eval()
+    xb, mb = make_bert_inputs(2, 48)
+    t, mask = xb.numpy(), mb.numpy()
+    for layer in bert.layers:
+        t = _oracle_layer_norm(oracle, layer.ln1, t + _oracle_attention(oracle, layer.attn, t, mask))
+        f = oracle.unary("gelu", _oracle_linear(oracle, t.reshape(-1, 768), layer.fc1))
+        t = _oracle_layer_norm(oracle, layer.ln2, t + _oracle_linear(oracle, f, layer.fc2).reshape(t.shape))
+    with torch.no_grad():
+        got = compile_module(copy.deepcopy(bert).cuda(), (xb.cuda(), mb.cuda()))(xb.cuda(), mb.cuda())
+    assert_close(got.cpu().numpy(), t, F32_RTOL, F32_ATOL, "2-layer BERT stack vs the oracle composition")
+
+
 def _kernel_names(engine):
     return [[c.fn.__name__ for c in inst.calls] for inst in engine.instances.values()]
 

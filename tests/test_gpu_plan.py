@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import BF16_RTOL, F32_ATOL, F32_RTOL, assert_close
+from tests.util import BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_as_close_as_eager, assert_close
 
 pytestmark = pytest.mark.gpu
 
@@ -207,7 +207,10 @@ def test_engine_plan_replay_matches_kernel_by_kernel_launches_encoder():
     planned, direct = _run_both_ways(build, calls)
     for (x,), a, b in zip(calls, planned, direct):
         assert torch.equal(a, b)
-        assert_close(a.float().cpu().numpy(), ref(x.float().cpu()).detach().numpy(), BF16_RTOL, 2e-2, "encoder via plan")
+        xc = x.cpu()
+        with torch.no_grad():
+            assert_as_close_as_eager(a.float().cpu().numpy(), enc(xc).float().numpy(), ref.double()(xc.double()).numpy(),
+                                     BF16_RTOL, BF16_ATOL, "encoder via plan")
 
 
 def test_engine_plan_replay_matches_kernel_by_kernel_launches_resnet():
