@@ -71,9 +71,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   extern __shared__ __align__(16) char smem[];
 
   int tile_m, tile_n;
-  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int z;
+  tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int z = blockIdx.z;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
   const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
   const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
@@ -274,9 +274,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   static_assert(sizeof(T) == 2, "16-bit operands");
   extern __shared__ __align__(16) char smem[];
   int tile_m, tile_n;
-  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int z;
+  tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
   const int m0 = tile_m * 128, n0 = tile_n * 128;
-  const int z = blockIdx.z;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
   const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
   const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
@@ -468,9 +468,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   static_assert(sizeof(T) == 2, "16-bit operands");
   extern __shared__ __align__(16) char smem[];
   int tile_m, tile_n;
-  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int z;
+  tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
   const int m0 = tile_m * 128, n0 = tile_n * 128;
-  const int z = blockIdx.z;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
   const T* A = (const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1;
   const T* B = (const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1;
@@ -630,6 +630,7 @@ int launch_dma2(const GemmParams& p0, int batch, hipStream_t s) {
 }
 
 #include "gemm_wide.hpp"
+#include "gemm_sweep.hpp"
 
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB>
 int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
@@ -877,6 +878,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
     const int splits = splitk_chunks(p, kRowBytes / (int)sizeof(T));
     if (splits > 1) return b_kvec ? launch_splitk<T, kLoadKVec>(p, splits, s) : launch_splitk<T, kLoadRVec>(p, splits, s);
   }
+  if (p.K == 64 && a_kvec && b_rvec && sweep_ok<T>(p, batch)) return launch_sweep<T>(p, batch, s);
   if constexpr (sizeof(T) == 2) {
     const bool dma_ok = a_kvec && (b_kvec || b_rvec) && p.K % 64 == 0 && al16(p.C) && p.c_sb % EPV == 0 && p.c_sb1 % EPV == 0 &&
                         p.c_sm % EPV == 0 && (!p.bias || (al16(p.bias) && p.bias_sb % EPV == 0)) && (!p.residual || al16(p.residual));

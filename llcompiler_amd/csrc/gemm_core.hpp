@@ -226,10 +226,7 @@ __device__ __forceinline__ float load_as_f32(const char* p, int dtype, int64_t i
 // XCD-aware workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8
 // XCDs by the hardware, so ids are first regrouped per XCD, then walked in column-grouped order
 // (8 tile rows per group): each XCD's L2 sees a compact patch of the output.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int total = tiles_m * tiles_n;
-  int id = blockIdx.x;
-  if (total % kXcds == 0) id = (id % kXcds) * (total / kXcds) + id / kXcds;
+__device__ __forceinline__ void tile_of_id(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int G = 8;
   const int per_group = G * tiles_n;
   const int group = id / per_group;
@@ -238,6 +235,29 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm,
   const int in_group = id % per_group;
   tm = first_m + in_group % gsize;
   tn = in_group / gsize;
+}
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  int id = blockIdx.x;
+  if (total % kXcds == 0) id = (id % kXcds) * (total / kXcds) + id / kXcds;
+  tile_of_id(id, tiles_m, tiles_n, tm, tn);
+}
+// The same for a grid (tiles, 1, batch): the hardware deals workgroups to the XCDs in x-then-z order, so with a
+// tile count that is a multiple of 8 every XCD would get an eighth of EVERY batch entry and each operand panel
+// would be fetched into all eight L2s.  The (tile, batch) pairs are regrouped so that an XCD walks whole batch
+// entries, one after the other.
+__device__ __forceinline__ void tile_and_batch_of_block(int tiles_m, int tiles_n, int& tm, int& tn, int& z) {
+  if (gridDim.z == 1) {
+    z = 0;
+    tile_of_block(tiles_m, tiles_n, tm, tn);
+    return;
+  }
+  const unsigned tiles = (unsigned)(tiles_m * tiles_n);
+  const unsigned long long total = (unsigned long long)tiles * gridDim.z;
+  unsigned long long w = blockIdx.x + (unsigned long long)tiles * blockIdx.z;
+  if (total % kXcds == 0) w = (w % kXcds) * (total / kXcds) + w / kXcds;
+  z = (int)(w / tiles);
+  tile_of_id((int)(w % tiles), tiles_m, tiles_n, tm, tn);
 }
 
 // MFMAs of one LDS tile pair for one wave: TM x TN fragments of 32x32, four steps of two 16-byte

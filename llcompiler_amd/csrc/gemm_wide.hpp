@@ -86,9 +86,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   extern __shared__ __align__(16) char smem[];
   LLC_DBG_T0();
   int tile_m, tile_n;
-  tile_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int z;
+  tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
   const int m0 = tile_m * 256, n0 = tile_n * BN;
-  const int z = blockIdx.z;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
   const char* A = (const char*)((const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1 + (int64_t)m0 * p.a_sm);
   const char* B = (const char*)((const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1 +

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import (assert_close_bf16, assert_close_f32, bf16_round, dev, host, rng)
+from tests.util import (assert_close, assert_close_bf16, assert_close_f32, bf16_round, dev, host, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -497,6 +497,43 @@ def test_batch_matmul_16bit_wide_tiles(ops, oracle):
     assert_close_bf16(host(got), want, "wide batch_matmul NN")
     bt = dev(np.ascontiguousarray(b.transpose(0, 2, 1)), torch.bfloat16)
     assert_close_bf16(host(ops.batch_matmul(dev(a, torch.bfloat16), bt.transpose(1, 2))), want, "wide batch_matmul NT")
+
+
+def f16_round(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def assert_close_f16(got, want, what=""):
+    # half precision keeps 11 significant bits; the absolute floor covers sums that cancel to ~0
+    assert_close(got, want, 2e-3, 4e-3, what)
+
+
+@pytest.mark.parametrize("B,M,N", [(8, 1024, 384), (2, 4096, 128), (1, 8192, 256), (32, 512, 512)])
+def test_batch_matmul_reduction_of_64_sweeps_the_columns(ops, oracle, B, M, N):
+    """K = 64 with a row-major B goes to the kernel that keeps a 64-row panel of A in registers and sweeps B's
+    columns in 256-byte tiles (odd and even tile counts, one tile, plain matmul as batch 1), in all three storage
+    types, bare and with alpha, bias, residual and an activation in the epilogue."""
+    r = rng(B * 31 + N)
+    a = r.uniform(-1, 1, (B, M, 64)).astype(np.float32)
+    b = r.uniform(-1, 1, (B, 64, N)).astype(np.float32)
+    bias = r.uniform(-0.5, 0.5, (N,)).astype(np.float32)
+    res = r.uniform(-0.5, 0.5, (B, M, N)).astype(np.float32)
+    want = oracle.batch_matmul(a, b, "mkn")
+    got = ops.batch_matmul(dev(a), dev(b)) if B > 1 else ops.matmul(dev(a[0]), dev(b[0]))[None]
+    assert_close_f32(host(got), want, "f32")
+    for act in ("relu", "gelu"):
+        w2 = oracle.unary(act, (want * np.float32(0.5) + bias[None, None, :] + res).astype(np.float32))
+        epi = ops.Epilogue(alpha=0.5, bias=dev(bias), residual=dev(res), act=act)
+        assert_close_f32(host(ops.batch_matmul(dev(a), dev(b), epi)), w2, "f32 epilogue " + act)
+    for dt, rnd, tol in ((torch.bfloat16, bf16_round, assert_close_bf16), (torch.float16, f16_round, assert_close_f16)):
+        if N % 128:
+            continue
+        ar, br, biasr, resr = rnd(a), rnd(b), rnd(bias), rnd(res)
+        w = oracle.batch_matmul(ar, br, "mkn")
+        tol(host(ops.batch_matmul(dev(ar, dt), dev(br, dt))), rnd(w), "16-bit")
+        w2 = oracle.unary("relu", (w * np.float32(0.5) + biasr[None, None, :] + resr).astype(np.float32))
+        epi = ops.Epilogue(alpha=0.5, bias=dev(biasr, dt), residual=dev(resr, dt), act="relu")
+        tol(host(ops.batch_matmul(dev(ar, dt), dev(br, dt), epi)), rnd(w2), "16-bit epilogue")
 
 
 def _attention_oracle(oracle, q, k, v, mask, scale, rnd):
