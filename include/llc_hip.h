@@ -195,7 +195,8 @@ int llc_hip_elementwise(const llc_ew_program* prog, const llc_tensor* const* inp
 
 /* llh.reduce_sum / reduce_max / reduce_min {axis} (LLHOps.td:528-553; LLHToHLO.cpp:81-171,
  * 448-464): init 0 / -inf / +inf, the result drops the reduced axes
- * (LLHinfersymbolShape.cpp:185-212).  The reduced axes must be adjacent. */
+ * (LLHinfersymbolShape.cpp:185-212).  Any set of axes: runs of adjacent reduced axes are reduced one kernel
+ * each, innermost first, partial results in scratch memory (two runs or more only). */
 typedef enum llc_reduce_kind { LLC_REDUCE_SUM = 0, LLC_REDUCE_MAX = 1, LLC_REDUCE_MIN = 2 } llc_reduce_kind;
 int llc_hip_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n_axes, llc_tensor* out,
                    void* stream);

@@ -42,6 +42,14 @@ struct AttnParams {
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr float kLog2e = 1.4426950408889634f;
+
+// An additive mask value in log2 units.  A finite value that overflows in the conversion (the most negative number
+// of the storage type, a common "minus infinity") stays finite: a row whose every key carries it then softmaxes to
+// the uniform row an unscaled evaluation gives, instead of 0 * inf.  A true -inf stays -inf (and such a row NaN).
+__device__ __forceinline__ float mask_log2(float m) {
+  const float r = m * kLog2e;
+  return (r == -INFINITY && m != -INFINITY) ? -3.4028234663852886e38f : r;
+}
 constexpr int kD = 64;
 constexpr int kBlockQ = 128, kBlockKV = 64;
 constexpr int kTileBytes = kBlockKV * 128;
@@ -111,7 +119,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         const int key = blk * kBlockKV + tid;
         const int kc = key < p.Skv ? key : p.Skv - 1;
         float mv = 0.0f;
-        if (M) mv = load_as_f32((const char*)M, Elem<T>::kDtype, kc) * kLog2e;
+        if (M) mv = mask_log2(load_as_f32((const char*)M, Elem<T>::kDtype, kc));
         ar = key < p.Skv ? mv : -INFINITY;
       }
     }
@@ -363,7 +371,7 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(const AttnParams
         if constexpr (MASK) av = *(const f32x4_t*)&addrow[s * kBlockKV + 32 * t2 + 8 * i + 4 * lh];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          float x = MASK ? fmaf(sacc[t2][4 * i + j], p.scale_log2e, av[j] * kLog2e) : sacc[t2][4 * i + j] * p.scale_log2e;
+          float x = MASK ? fmaf(sacc[t2][4 * i + j], p.scale_log2e, mask_log2(av[j])) : sacc[t2][4 * i + j] * p.scale_log2e;
           if (tail && blk * kBlockKV + 32 * t2 + 8 * i + 4 * lh + j >= p.Skv) x = -INFINITY;
           sacc[t2][4 * i + j] = x;
           mx = fmaxf(mx, x);

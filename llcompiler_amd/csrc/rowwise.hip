@@ -594,24 +594,68 @@ int llc_impl_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n
     if (ax < 0 || ax >= a.rank) return set_error(LLC_ERR_BAD_ARG, "reduce: axis %lld out of range", (long long)axes[i]);
     red[ax] = true;
   }
-  int first = -1, last = -1;
-  for (int d = 0; d < a.rank; ++d)
-    if (red[d]) {
-      if (first < 0) first = d;
-      last = d;
-    }
-  int64_t outer = 1, R = 1, inner = 1, kept = 1;
+  // Runs of adjacent dims with the same role (dims of extent 1 belong to whatever surrounds them): sizes alternate
+  // between kept and reduced.
+  int64_t run_size[LLC_MAX_RANK + 1];
+  bool run_red[LLC_MAX_RANK + 1];
+  int runs = 0;
+  int64_t kept = 1;
   for (int d = 0; d < a.rank; ++d) {
-    if (d < first) outer *= a.size[d];
-    else if (d <= last) {
-      // a kept dim of extent 1 between reduced dims does not break adjacency
-      if (!red[d] && a.size[d] != 1) return set_error(LLC_ERR_UNSUPPORTED, "reduce: reduced axes must be adjacent");
-      R *= a.size[d];
-    } else inner *= a.size[d];
     if (!red[d]) kept *= a.size[d];
+    if (a.size[d] == 1) continue;
+    if (runs > 0 && run_red[runs - 1] == red[d]) run_size[runs - 1] *= a.size[d];
+    else {
+      run_size[runs] = a.size[d];
+      run_red[runs] = red[d];
+      ++runs;
+    }
   }
   if (o.numel() != kept) return set_error(LLC_ERR_SHAPE, "reduce: output holds %lld elements, expected %lld", (long long)o.numel(), (long long)kept);
-  return reduce_3d(a, o, kind, outer, R, inner, 1.0f, as_stream(stream));
+  int n_red = 0;
+  for (int r = 0; r < runs; ++r) n_red += run_red[r] ? 1 : 0;
+  hipStream_t s = as_stream(stream);
+  if (n_red == 0) {
+    // every reduced dim has extent 1 (or an extent is 0 and there is nothing to write): the values themselves
+    if (kept == 0) return LLC_OK;
+    return reduce_3d(a, o, kind, kept, 1, 1, 1.0f, s);
+  }
+  // One kernel per reduced run, innermost first; partial results of all but the last alternate between the two
+  // halves of the scratch buffer.  (Sums are then grouped by run, maxima and minima do not care.)
+  const int es = a.dtype == LLC_FLOAT32 ? 4 : 2;
+  char* scratch = nullptr;
+  size_t half = 0;
+  if (n_red > 1) {
+    int64_t last_red = 1;
+    for (int r = runs - 1; r >= 0; --r)
+      if (run_red[r]) {
+        last_red = run_size[r];
+        break;
+      }
+    const int64_t partial = last_red ? a.numel() / last_red : 0;
+    half = ((size_t)partial * es + 255) & ~(size_t)255;
+    if (half) {
+      void* ws = nullptr;
+      LLC_TRY(get_workspace(2 * half, &ws, s));
+      scratch = (char*)ws;
+    }
+  }
+  View cur = a;
+  int left = n_red, flip = 0;
+  for (int r = runs - 1; r >= 0; --r) {
+    if (!run_red[r]) continue;
+    int64_t outer = 1, inner = 1;
+    for (int q = 0; q < r; ++q) outer *= run_size[q];
+    for (int q = r + 1; q < runs; ++q) inner *= run_size[q];
+    View dst = o;
+    if (--left > 0) {
+      dst.ptr = scratch + flip * half;
+      flip ^= 1;
+    }
+    LLC_TRY(reduce_3d(cur, dst, kind, outer, run_size[r], inner, 1.0f, s));
+    run_size[r] = 1;
+    cur = dst;
+  }
+  return LLC_OK;
 }
 
 int llc_impl_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream) {

@@ -341,10 +341,41 @@ def test_random_rowwise_and_shape_cases(ops, oracle, seed):
         np.testing.assert_array_equal(host(ops.copy(view)), view.cpu().numpy(), err_msg="copy of a strided view %s %s" % (shape, perms))
 
 
-def test_reduce_rejects_split_axes(ops):
-    from llcompiler_amd._capi import LlcHipError
-    with pytest.raises(LlcHipError, match="adjacent"):
-        ops.reduce("sum", torch.zeros(2, 3, 4, 5, device="cuda"), [0, 2])
+@pytest.mark.parametrize("shape,axes", [((2, 3, 4, 5), [0, 2]), ((6, 1, 7, 33), [0, 3]), ((4, 5, 6, 7, 8), [0, 2, 4]),
+                                        ((3, 64, 2, 70), [-1, 1]), ((5, 1, 1, 9), [1, 2]), ((8, 17, 3), [0, 1, 2]),
+                                        ])
+def test_reduce_over_split_axes(ops, oracle, shape, axes):
+    """Axis sets that are not one run of adjacent dims: the library reduces run by run, innermost first."""
+    r = rng(len(shape) * 100 + sum(shape))
+    x = r.uniform(-1, 1, shape).astype(np.float32)
+    for kind in ("sum", "max", "min"):
+        want = oracle.reduce(kind, x, axes)
+        got = ops.reduce(kind, dev(x), axes)
+        assert tuple(got.shape) == want.shape
+        if kind == "sum":
+            assert_close_f32(host(got), want, "reduce %s %s %s" % (kind, shape, axes))
+        else:
+            np.testing.assert_array_equal(host(got), want)
+    # 16-bit storage: the partial results between two runs are stored in that type too
+    norm = sorted(a % len(shape) for a in axes)
+    runs = []
+    for a in norm:
+        if runs and runs[-1][-1] == a - 1:
+            runs[-1].append(a)
+        else:
+            runs.append([a])
+    want = bf16_round(x)
+    for run in reversed(runs):
+        want = bf16_round(oracle.reduce("sum", want, run))
+    gotb = host(ops.reduce("sum", dev(bf16_round(x), torch.bfloat16), axes))
+    assert_close_bf16(gotb.reshape(-1), np.asarray(want).reshape(-1), "bf16")
+
+
+def test_reduce_over_split_axes_with_an_empty_run(ops):
+    """An empty reduced run yields the init value whatever the other runs hold."""
+    x = torch.zeros(2, 0, 3, 4, device="cuda")
+    np.testing.assert_array_equal(host(ops.reduce("sum", x, [1, 3])), np.zeros((2, 3), np.float32))
+    np.testing.assert_array_equal(host(ops.reduce("max", x, [1, 3])), np.full((2, 3), -np.inf, np.float32))
 
 
 # --------------------------------------------------------------------------- data movement (bit exact)
@@ -547,6 +578,27 @@ def _attention_oracle(oracle, q, k, v, mask, scale, rnd):
         s = s + mask[:, None, None, :]
     p = rnd(oracle.softmax_lastdim(s.reshape(-1, Skv))).reshape(B * H, Sq, Skv)
     return oracle.batch_matmul(p, v.reshape(B * H, Skv, D), "mkn").reshape(B, H, Sq, D)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_attention_with_a_fully_masked_sample(ops, oracle, dt):
+    """A batch entry whose every key carries the most negative finite number of the storage type (an all-padding
+    sequence): the unfused group adds it to the scores, which it absorbs, and softmaxes to the uniform row, so the
+    output is the mean of V; the fused kernel works in log2 units, where that value would overflow."""
+    r = rng(5)
+    B, H, S = 2, 2, 128
+    rnd = bf16_round if dt == "bf16" else (lambda a: np.asarray(a, np.float32))
+    tdt = torch.bfloat16 if dt == "bf16" else torch.float32
+    q, k, v = (rnd(r.uniform(-1, 1, (B, H, S, 64))) for _ in range(3))
+    lowest = float(torch.finfo(tdt).min)
+    mask = np.zeros((B, S), np.float32)
+    mask[0, :] = lowest
+    mask[1, S // 2:] = lowest
+    want = _attention_oracle(oracle, q, k, v, mask, 0.125, rnd)
+    assert np.isfinite(want).all()
+    np.testing.assert_allclose(want[0, 0, 0], v[0, 0].mean(axis=0), rtol=1e-4, atol=1e-5)
+    got = ops.attention(dev(q, tdt), dev(k, tdt), dev(v, tdt), dev(mask, tdt), 0.125)
+    (assert_close_bf16 if dt == "bf16" else assert_close_f32)(host(got), rnd(want), "fully masked sample " + dt)
 
 
 @pytest.mark.parametrize("B,H,Sq,Skv,masked", [(1, 1, 128, 128, False), (2, 3, 100, 200, True), (1, 2, 64, 64, False),
