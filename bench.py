@@ -182,6 +182,26 @@ def launch_spread_us(fn, n=100):
     return {"p10": round(times[n // 10], 2), "median": round(times[n // 2], 2), "p90": round(times[(9 * n) // 10], 2)}
 
 
+_COPY_FLOOR = {}
+
+
+def copy_floor_us(ops, device, nbytes):
+    """Microseconds a plain streaming kernel (one fp32 tensor in, relu, one out; 16 bytes per lane, the suite's own
+    elementwise kernel) takes to move `nbytes` in total, half read and half written, on rotating operand sets like
+    the cases themselves: what the memory system of this box delivers at that size, launch and ramp-up included.
+    The HBM-bound rows are reported against it next to the published 8 TB/s."""
+    n = max(1024, int(nbytes // 8) // 1024 * 1024)
+    if n not in _COPY_FLOOR:
+        sets = max(2, int(1.2e9 // (8 * n)))
+        prog = ops.make_program([("relu", "r0", "in0")], "r0")
+        xs = [torch.zeros(n, dtype=torch.float32, device=device) for _ in range(sets)]
+        outs = [torch.empty(n, dtype=torch.float32, device=device) for _ in range(sets)]
+        calls = [ops.elementwise(prog, [x], (n,), torch.float32, out=o, defer=True) for x, o in zip(xs, outs)]
+        _COPY_FLOOR[n] = time_gpu(lambda i: calls[i % sets].launch(), 100, 20) * 1e3
+        del xs, outs, calls
+    return _COPY_FLOOR[n]
+
+
 def measured_traffic():
     """HBM bytes per launch (reads + writes) of each case's kernel, read from the table in
     profiles/single_op_suite_hbm_counters.md: two rocprofv3 counter runs over this same workload (FETCH_SIZE and
@@ -447,6 +467,9 @@ def main():
     kernels = [roofline_of(c, time_gpu(c.run, max(args.steps, 100), max(args.warmup, 20))) for c in cases]
     for c, k in zip(cases, kernels):
         k["single_launch_us"] = launch_spread_us(c.run)
+        if c.bound == "hbm":
+            k["copy_same_bytes_us"] = round(copy_floor_us(ops, device, c.bytes), 2)
+            k["frac_of_copy"] = round(k["copy_same_bytes_us"] / (k["avg_ms"] * 1e3), 3)
     dominant = max(kernels, key=lambda k: k["avg_ms"])
     out = {
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,

@@ -40,8 +40,10 @@ class CompiledModule:
         return self.engine.save_plan(path, *self.lifted, *args)
 
 
-def compile_module(model, example_args, dynamic_shapes=None, verbose=False, weights=None, weight_dir=None):
-    """weights="npy": parameters and buffers are written to .npy files (in weight_dir, or a fresh temporary
+def compile_module(model, example_args, dynamic_shapes=None, verbose=False, weights=None, weight_dir=None,
+                   target_layout="NCHW"):
+    """target_layout: the layout convolutions are rewritten to (LLCompiler's keyword of the same name).
+    weights="npy": parameters and buffers are written to .npy files (in weight_dir, or a fresh temporary
     directory) and enter the graph as llh.weight ops, the reference importer's convention
     (llcompiler/importer/fx_translate.py:415-435); the engine uploads each file once.  By default they stay
     torch tensors and are passed to the engine with every call."""
@@ -83,7 +85,7 @@ def compile_module(model, example_args, dynamic_shapes=None, verbose=False, weig
     elif weights is not None:
         raise ValueError("weights must be None or \"npy\"")
     graph = torch_translate_to_llh_graph(gm, weight_files)
-    run_llh_pipeline(graph)
+    run_llh_pipeline(graph, target_layout)
     if verbose:
         print(graph.dump())
     return CompiledModule(Torch_ExecutionEngine(graph), lifted, n_user)

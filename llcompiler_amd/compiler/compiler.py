@@ -44,8 +44,10 @@ class LLCompiler:
             raise ValueError("target %r: this backend generates code for %s only" % (target, ", ".join(TARGETS)))
         if pipeline not in PIPELINES:
             raise ValueError("pipeline %r: only %s is available" % (pipeline, ", ".join(PIPELINES)))
-        if target_layout != "NCHW":
-            raise ValueError("target_layout %r: NCHW only" % (target_layout,))
+        # the layout convolutions are rewritten to by the layout transform (include/llcompiler/Dialect/LLH/IR/
+        # LLHEnums.td:61-75, src/Dialect/LLH/Transforms/TransformLayout.cpp:141-198)
+        if target_layout not in ("NCHW", "NHWC"):
+            raise ValueError("target_layout %r: NCHW or NHWC" % (target_layout,))
         if mode not in ("inference", "training"):
             raise ValueError("mode %r" % (mode,))
         self.mode, self.target, self.pipeline = mode, target, pipeline
@@ -101,7 +103,7 @@ class LLCompiler:
         graph = self.importer(model)
         log_dir = self._log_dir()
         self._log(log_dir, "0_imported", graph)
-        run_llh_pipeline(graph)
+        run_llh_pipeline(graph, self.target_layout)
         self._log(log_dir, "1_after_llh_passes", graph)
         if log_dir:
             from ..llh.plan_tool import plan_text

@@ -560,40 +560,75 @@ class Instance:
                         full = _concrete(st.output.shape, self.env)
                         bias = bias.view(full[0], full[3])
                         natural = full
-                cl = k == "conv" and self._channels_last_ok(st, ins, out, natural)
-                if res is not None and not cl:
-                    res = contiguous(res)
-                epi = None
-                if bias is not None or res is not None or e["act"] or e["alpha"] != 1.0:
-                    epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=res, act=e["act"] or "none")
-                o = out.view(natural)
-                if k == "matmul":
-                    call = ops.matmul(ins[0], ins[1], epi, out=o, defer=True)
-                elif k == "batch_matmul":
-                    hm = head_merge(st, natural[0], natural[1], natural[2]) if (res is None and len(natural) == 3) else None
-                    if hm is not None:
-                        # the head merge that follows, [B0,B1,M,N] -> [B0,M,B1,N], is done by the kernel's stores
-                        r1, b0, b1 = hm
-                        o = out.view(-1).view(b0, natural[1], b1, natural[2]).permute(0, 2, 1, 3)
-                        val[id(r1.output)] = o
-                        skip.add(id(r1))
-                    call = ops.batch_matmul(ins[0], ins[1], epi, out=o, defer=True)
-                elif cl:
-                    xc = to_channels_last(st.inputs[0], ins[0])
-                    wc = to_channels_last(st.inputs[1], ins[1])
-                    if res is not None:
-                        epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=to_channels_last(e["residual"], res),
-                                           act=e["act"] or "none")
-                    n_, f_, oh_, ow_ = natural
-                    out = out.view(-1).view(n_, oh_, ow_, f_).permute(0, 3, 1, 2)  # NCHW shape over NHWC memory
-                    call = ops.conv2d(xc, wc, pad=st.attrs["pad"], stride=st.attrs["stride"], dilation=st.attrs["dilation"],
-                                      group=1, epilogue=epi, out=out, defer=True)
+                if k == "conv" and st.attrs.get("layout", "NCHW") == "NHWC":
+                    # operands and result are [N,H,W,C] / [F,KH,KW,C] / [N,OH,OW,F] tensors: their NCHW-shaped views
+                    # are channels-last tensors, which is what the kernel for that memory layout takes
+                    n_, oh_, ow_, f_ = natural
+                    x4, w4 = ins[0].permute(0, 3, 1, 2), ins[1].permute(0, 3, 1, 2)
+                    r4 = res.permute(0, 3, 1, 2) if res is not None else None
+                    kernel_ok = CHANNELS_LAST and st.attrs["group"] == 1 and out.numel() and \
+                        x4.shape[1] % (128 // out.dtype.itemsize) == 0 and f_ % 4 == 0 and w4.shape[2] * w4.shape[3] <= 64
+                    if kernel_ok:
+                        xc, wc = to_channels_last(st.inputs[0], x4), to_channels_last(st.inputs[1], w4)
+                        kernel_ok = xc.data_ptr() % 16 == 0 and wc.data_ptr() % 16 == 0
+                    if kernel_ok:
+                        epi = None
+                        if bias is not None or r4 is not None or e["act"] or e["alpha"] != 1.0:
+                            epi = ops.Epilogue(alpha=e["alpha"], bias=bias, act=e["act"] or "none",
+                                               residual=to_channels_last(e["residual"], r4) if r4 is not None else None)
+                        self._launch_later(ops.conv2d(xc, wc, pad=st.attrs["pad"], stride=st.attrs["stride"],
+                                                      dilation=st.attrs["dilation"], group=1, epilogue=epi,
+                                                      out=out.view(natural).permute(0, 3, 1, 2), defer=True))
+                    elif out.numel():
+                        # shapes the channels-last kernel does not take: NCHW copies, the NCHW kernel, and a copy back
+                        epi = None
+                        if bias is not None or r4 is not None or e["act"] or e["alpha"] != 1.0:
+                            epi = ops.Epilogue(alpha=e["alpha"], bias=bias, act=e["act"] or "none",
+                                               residual=contiguous(r4) if r4 is not None else None)
+                        nbytes = out.numel() * out.dtype.itemsize
+                        buf = pool.take(nbytes)
+                        temps.append(buf)
+                        t4 = buf[:nbytes].view(out.dtype).view(n_, f_, oh_, ow_)
+                        self._launch_later(ops.conv2d(contiguous(x4), contiguous(w4), pad=st.attrs["pad"], stride=st.attrs["stride"],
+                                                      dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi,
+                                                      out=t4, defer=True))
+                        self._launch_later(ops.copy(t4.permute(0, 2, 3, 1), out=out.view(natural), defer=True))
+                    val[id(st.output)] = out
                 else:
-                    call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],
-                                      dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi, out=o, defer=True)
-                if out.numel():
-                    self._launch_later(call)
-                val[id(st.output)] = out
+                    cl = k == "conv" and self._channels_last_ok(st, ins, out, natural)
+                    if res is not None and not cl:
+                        res = contiguous(res)
+                    epi = None
+                    if bias is not None or res is not None or e["act"] or e["alpha"] != 1.0:
+                        epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=res, act=e["act"] or "none")
+                    o = out.view(natural)
+                    if k == "matmul":
+                        call = ops.matmul(ins[0], ins[1], epi, out=o, defer=True)
+                    elif k == "batch_matmul":
+                        hm = head_merge(st, natural[0], natural[1], natural[2]) if (res is None and len(natural) == 3) else None
+                        if hm is not None:
+                            # the head merge that follows, [B0,B1,M,N] -> [B0,M,B1,N], is done by the kernel's stores
+                            r1, b0, b1 = hm
+                            o = out.view(-1).view(b0, natural[1], b1, natural[2]).permute(0, 2, 1, 3)
+                            val[id(r1.output)] = o
+                            skip.add(id(r1))
+                        call = ops.batch_matmul(ins[0], ins[1], epi, out=o, defer=True)
+                    elif cl:
+                        xc = to_channels_last(st.inputs[0], ins[0])
+                        wc = to_channels_last(st.inputs[1], ins[1])
+                        if res is not None:
+                            epi = ops.Epilogue(alpha=e["alpha"], bias=bias, residual=to_channels_last(e["residual"], res),
+                                               act=e["act"] or "none")
+                        n_, f_, oh_, ow_ = natural
+                        out = out.view(-1).view(n_, oh_, ow_, f_).permute(0, 3, 1, 2)  # NCHW shape over NHWC memory
+                        call = ops.conv2d(xc, wc, pad=st.attrs["pad"], stride=st.attrs["stride"], dilation=st.attrs["dilation"],
+                                          group=1, epilogue=epi, out=out, defer=True)
+                    else:
+                        call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],
+                                          dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi, out=o, defer=True)
+                    if out.numel():
+                        self._launch_later(call)
+                    val[id(st.output)] = out
             elif k == "softmax":
                 out = new_tensor(st.output)
                 if out.numel():

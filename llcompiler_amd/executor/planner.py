@@ -98,7 +98,7 @@ class Planner:
         return root
 
     def match_epilogue(self, op):
-        channel_dim = 1 if op.name in ("conv", "conv_bias") else op.results[0].rank - 1
+        channel_dim = 1 if op.name in ("conv", "conv_bias") and op.attrs.get("layout", "NCHW") == "NCHW" else op.results[0].rank - 1
         epi = {"alpha": 1.0, "bias": None, "residual": None, "act": None}
         if op.name == "conv_bias":
             epi["bias"] = op.operands[2]
@@ -272,6 +272,7 @@ class Planner:
                 attrs = {"epilogue": epi}
                 if kind == "conv":
                     attrs.update({k: op.attrs[k] for k in ("dilation", "kernel_shape", "pad", "stride", "group")})
+                    attrs["layout"] = op.attrs.get("layout", "NCHW")
                 step = Step(kind, op.operands[:2], out, attrs)
                 step.attrs["natural_shape"] = tuple(op.results[0].shape)
                 self.absorbed.add(id(op))

@@ -59,11 +59,14 @@ def infer(name, operands, attrs):
         (b, m, k), (b2, k2, n) = shapes
         return [(b, m, n)], [dt]
     if name in ("conv", "conv_bias"):  # :214-331
-        n, c, h, w = shapes[0]
+        # layout NCHW: x [N,C,H,W], w [F,C,KH,KW]; layout NHWC: x [N,H,W,C], w [F,KH,KW,C] (LLHEnums.td:61-75)
+        nhwc = attrs.get("layout", "NCHW") == "NHWC"
+        n, h, w = (shapes[0][0], shapes[0][1], shapes[0][2]) if nhwc else (shapes[0][0], shapes[0][2], shapes[0][3])
         f = shapes[1][0]
         kh, kw = attrs["kernel_shape"]
         p, s, d = attrs["pad"], attrs["stride"], attrs["dilation"]
-        return [(n, f, window_out(h, p[0], p[2], d[0], kh, s[0]), window_out(w, p[1], p[3], d[1], kw, s[1]))], [dt]
+        oh, ow = window_out(h, p[0], p[2], d[0], kh, s[0]), window_out(w, p[1], p[3], d[1], kw, s[1])
+        return [(n, oh, ow, f) if nhwc else (n, f, oh, ow)], [dt]
     if name == "max_pool":
         n, c, h, w = shapes[0]
         kh, kw = attrs["kernel_shape"]

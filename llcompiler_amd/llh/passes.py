@@ -70,6 +70,17 @@ def canonicalize(g):
                 rep = op.operands[0]
             elif op.name == "transpose" and tuple(op.attrs["perms"]) == tuple(range(r.rank)):
                 rep = op.operands[0]
+            elif op.name == "transpose" and op.operands[0].producer is not None and op.operands[0].producer.name == "transpose":
+                # transpose(transpose(x, p), q) -> transpose(x, p o q): what the layout transform leaves between two
+                # convolutions that follow each other cancels this way
+                inner = op.operands[0].producer
+                src = inner.operands[0]
+                op.attrs = dict(op.attrs, perms=tuple(inner.attrs["perms"][q] for q in op.attrs["perms"]))
+                op.operands[0].users.remove(op)
+                op.operands[0] = src
+                src.users.append(op)
+                changed = True
+                continue
             elif op.name == "abs" and op.operands[0].producer is not None and op.operands[0].producer.name == "abs":
                 rep = op.operands[0]      # abs(abs(x)) (canonicalize.mlir fold_two_abs)
             elif op.name == "reshape" and _static(r.shape) and op.operands[0].producer is not None and \
@@ -208,11 +219,45 @@ def fuse_softmax(g):
     return g
 
 
-def run_llh_pipeline(g):
+LAYOUT_PERMS = {("NCHW", "NHWC"): (0, 2, 3, 1), ("NHWC", "NCHW"): (0, 3, 1, 2)}
+
+
+def transform_layout(g, target="NCHW"):
+    """Every convolution whose layout attribute differs from `target` becomes transpose(x), transpose(w) ->
+    conv{layout = target} -> transpose back, with the permutations of the reference's pass
+    (src/Dialect/LLH/Transforms/TransformLayout.cpp:141-198, perms :47-72; pinned by its
+    test/Dialect/LLH/transform_layout.mlir: 0,2,3,1 on both operands, 0,3,1,2 on the result).  The weight moves
+    with the same permutation (FCHW -> FHWC), as there."""
+    if target not in ("NCHW", "NHWC"):
+        raise ValueError("target layout %r (NCHW or NHWC)" % (target,))
+    for op in list(g.ops):
+        if op.name not in ("conv", "conv_bias"):
+            continue
+        layout = op.attrs.get("layout", "NCHW")
+        if layout == target:
+            continue
+        to, back = LAYOUT_PERMS[(layout, target)], LAYOUT_PERMS[(target, layout)]
+        idx = g.ops.index(op)
+        tail = g.ops[idx:]
+        del g.ops[idx:]
+        x = g.add_op("transpose", [op.operands[0]], {"perms": to})
+        w = g.add_op("transpose", [op.operands[1]], {"perms": to})
+        attrs = dict(op.attrs, layout=target, weight_layout=target)
+        y = g.add_op(op.name, [x, w] + list(op.operands[2:]), attrs)
+        z = g.add_op("transpose", [y], {"perms": back})
+        g.ops += tail
+        g.replace_all_uses(op.results[0], z)
+        g.erase(op)
+    return g
+
+
+def run_llh_pipeline(g, target_layout="NCHW"):
     """Order follows the reference's pipeline (src/Pipeline/TransformPipeline.cpp:103-128):
-    legalise/remove-redundant, decompose, canonicalise."""
+    legalise/remove-redundant, decompose, canonicalise, layout transform, canonicalise."""
     canonicalize(g)
     decompose_batch_norm(g)
     fuse_softmax(g)
+    canonicalize(g)
+    transform_layout(g, target_layout)
     canonicalize(g)
     return g

@@ -71,11 +71,13 @@ def main(argv=None):
     ap.add_argument("--func", default=None, help="function to read when the file holds several (default: the entrance)")
     ap.add_argument("--emit", choices=("plan", "llh", "both"), default="plan")
     ap.add_argument("--no-pipeline", action="store_true", help="plan the graph as written, without the LLH-level rewrites")
+    ap.add_argument("--target-layout", choices=("NCHW", "NHWC"), default="NCHW",
+                    help="layout the convolutions are rewritten to (the reference's --transform-layout option)")
     args = ap.parse_args(argv)
     text = sys.stdin.read() if args.file == "-" else open(args.file).read()
     graph = parse_llh(text, func=args.func)
     if not args.no_pipeline:
-        run_llh_pipeline(graph)
+        run_llh_pipeline(graph, args.target_layout)
     out = ""
     if args.emit in ("llh", "both"):
         out += print_llh(graph)

@@ -320,10 +320,15 @@ class _Reader:
         if name == "convert_to":
             return g.add_op("convert_to", [self.tensor(operands[0])], {"dtype": rt.dtype})
         if name in ("conv", "conv_bias"):
-            if str(attrs.get("layout", "NCHW")) != "NCHW":
-                raise NotImplementedError("llh.conv layout %s (NCHW is implemented)" % attrs["layout"])
+            layout = str(attrs.get("layout", "NCHW")).split("<")[-1].strip(">")
+            if layout not in ("NCHW", "NHWC"):
+                raise NotImplementedError("llh.conv layout %s (NCHW and NHWC are implemented)" % layout)
+            wl = str(attrs.get("weight_layout", layout)).split("<")[-1].strip(">")
+            if wl not in ({"NCHW": ("NCHW", "FCHW"), "NHWC": ("NHWC", "FHWC")}[layout]):
+                raise NotImplementedError("llh.conv weight_layout %s with layout %s" % (wl, layout))
             a = {k: tuple(attrs[k]) for k in ("dilation", "kernel_shape", "pad", "stride")}
             a["group"] = int(attrs.get("group", 1))
+            a["layout"] = layout
             return g.add_op(name, [self.tensor(o) for o in operands], a)
         if name == "max_pool":
             a = {k: tuple(attrs[k]) for k in ("dilation", "kernel_shape", "pad", "stride")}
@@ -501,7 +506,7 @@ def _attr_text(key, v, result):
     if isinstance(v, str):
         if key == "kind":
             return "#llh.Compare<%s>" % v
-        if key == "layout":
+        if key in ("layout", "weight_layout"):
             return "#llh.Layout<%s>" % v
         return '"%s"' % v
     if isinstance(v, (tuple, list)):

@@ -775,6 +775,63 @@ def test_random_conv_networks_match_eager(seed, tmp_path):
     assert torch.equal(want_again, first) and torch.equal(from_file, first), what + ": the plan read back from a file differs"
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_conv_networks_with_the_nhwc_target_layout(seed):
+    """target_layout="NHWC": every convolution is rewritten to the NHWC layout between transposes
+    (TransformLayout.cpp:141-198); channel counts the channels-last kernel takes and ones it does not, with bias,
+    residual and relu around them.  Same numbers as eager, through torch.compile and through the export entry."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.compiler.aot import compile_module
+    net = _RandomConvNet(seed).eval()
+    x = torch.randn(2, 3, 40, 36, generator=torch.Generator().manual_seed(2000 + seed))
+    with torch.no_grad():
+        want = net(x).numpy()
+        cm = compile_module(copy.deepcopy(net).cuda(), (x.cuda(),), target_layout="NHWC")
+        got = cm(x.cuda())
+        again = cm(x.cuda())
+    what = "random conv net %d, NHWC target: %s" % (seed, " ".join(net.kinds))
+    layouts = [st.attrs.get("layout") for st in cm.engine.steps if st.kind == "conv"]
+    assert layouts and all(l == "NHWC" for l in layouts), layouts
+    assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, what)
+    assert torch.equal(got, again)
+    if seed == 0:
+        torch._dynamo.reset()
+        comp = LLCompiler(mode="inference", target_layout="NHWC")
+        with torch.no_grad():
+            opt = torch.compile(copy.deepcopy(net).cuda(), backend=comp, fullgraph=True)
+            assert_close(opt(x.cuda()).cpu().numpy(), want, F32_RTOL, F32_ATOL, what + " (torch.compile)")
+        assert all(st.attrs.get("layout") == "NHWC" for eng in comp.engines for st in eng.steps if st.kind == "conv")
+
+
+def test_llh_text_conv_in_the_nhwc_layout_against_the_oracle(oracle):
+    """llh.conv {layout = NHWC} read from text and run as written (target layout NHWC: no transposes are added): the
+    oracle's NCHW loop nest on the permuted operands, permuted back.  64 channels go to the channels-last kernel,
+    3 channels through NCHW copies."""
+    from llcompiler_amd.executor.engine import Torch_ExecutionEngine
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    from llcompiler_amd.llh.text import parse_llh
+    from tests.test_llh_text_cpu import NHWC_CONV
+    r = np.random.default_rng(11)
+    for c in (64, 3):
+        text = NHWC_CONV.replace("9x9x64", "9x9x%d" % c).replace("3x3x64", "3x3x%d" % c)
+        g = parse_llh(text)
+        run_llh_pipeline(g, "NHWC")
+        assert g.op_names() == ["conv"]
+        x = r.uniform(-1, 1, (2, 9, 9, c)).astype(np.float32)
+        w = r.uniform(-1, 1, (8, 3, 3, c)).astype(np.float32)
+        want = oracle.conv2d(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), np.ascontiguousarray(w.transpose(0, 3, 1, 2)),
+                             None, (1, 1, 1, 1), (1, 1)).transpose(0, 2, 3, 1)
+        got = Torch_ExecutionEngine(g).run(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda())
+        assert tuple(got.shape) == (2, 9, 9, 8)
+        assert_close(got.cpu().numpy(), want, F32_RTOL, F32_ATOL, "NHWC conv from text, %d channels" % c)
+        # the default target turns it into an NCHW convolution between transposes: same numbers
+        g2 = parse_llh(text)
+        run_llh_pipeline(g2)
+        assert g2.op_names() == ["transpose", "transpose", "conv", "transpose"]
+        got2 = Torch_ExecutionEngine(g2).run(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda())
+        assert_close(got2.cpu().numpy(), want, F32_RTOL, F32_ATOL, "the same through the NCHW target")
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_random_conv_networks_in_bf16(seed):
     """The same random convolutional networks in bf16 storage (channel counts on both sides of what the channels-last

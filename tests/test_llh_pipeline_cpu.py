@@ -7,7 +7,7 @@ import torch
 from llcompiler_amd.executor.planner import make_plan
 from llcompiler_amd.llh.expr import Expr, ceildiv, evaluate
 from llcompiler_amd.llh.graph import Graph
-from llcompiler_amd.llh.passes import canonicalize, decompose_batch_norm, fuse_softmax, run_llh_pipeline
+from llcompiler_amd.llh.passes import canonicalize, decompose_batch_norm, fuse_softmax, run_llh_pipeline, transform_layout
 
 f32 = torch.float32
 s0, s2 = Expr.sym("s0"), Expr.sym("s2")
@@ -312,3 +312,63 @@ def test_true_division_of_integers_is_imported_as_a_floating_point_div():
     gm = make_fx(lambda a, b: torch.ops.prims.div(a, b))(torch.tensor([7, -7]), torch.tensor([2, 3]))
     node = [n for n in gm.graph.nodes if n.op == "call_function"][0]
     assert node.meta["val"].dtype == torch.int64 and not is_supported(node)
+
+
+# ---- layout transform (test/Dialect/LLH/transform_layout.mlir) ----
+CONV_ATTRS = {"dilation": (2, 2), "kernel_shape": (7, 7), "pad": (3, 3, 3, 3), "stride": (2, 2), "group": 1, "layout": "NCHW"}
+
+
+def test_infer_conv_in_the_nhwc_layout():
+    g = Graph()
+    x = g.add_input((2, 224, 200, 3), f32)
+    w = g.add_input((64, 7, 7, 3), f32)
+    y = g.add_op("conv", [x, w], dict(CONV_ATTRS, dilation=(1, 1), layout="NHWC"))
+    assert y.shape == (2, 112, 100, 64)
+
+
+def test_transform_layout_wraps_a_conv_in_the_reference_transposes():
+    """transform_layout.mlir conv_nchw_to_nhwc: transposes 0,2,3,1 on both operands, the conv, 0,3,1,2 on the result;
+    dynamic extents move with their dims."""
+    g = Graph()
+    w = g.add_input((4, 3, 7, 7), f32)
+    x = g.add_input((s0, 3, s2, s2), f32)
+    y = g.add_op("conv", [x, w], dict(CONV_ATTRS))
+    g.set_outputs([y])
+    natural = y.shape
+    transform_layout(g, "NHWC")
+    assert g.op_names() == ["transpose", "transpose", "conv", "transpose"]
+    tx, tw, conv, back = g.ops
+    assert tuple(tx.attrs["perms"]) == (0, 2, 3, 1) and tuple(tw.attrs["perms"]) == (0, 2, 3, 1)
+    assert tuple(back.attrs["perms"]) == (0, 3, 1, 2)
+    assert conv.attrs["layout"] == "NHWC" and conv.attrs["weight_layout"] == "NHWC"
+    assert tx.results[0].shape == (s0, s2, s2, 3) and tw.results[0].shape == (4, 7, 7, 3)
+    assert conv.results[0].shape == (natural[0], natural[2], natural[3], 4)
+    assert g.outputs[0] is back.results[0] and back.results[0].shape == natural
+    # a conv already in the target layout is left alone, and the other direction uses the inverse permutations
+    before = g.op_names()
+    transform_layout(g, "NHWC")
+    assert g.op_names() == before
+    transform_layout(g, "NCHW")
+    canonicalize(g)
+    assert g.op_names() == ["conv"] and g.ops[0].attrs["layout"] == "NCHW"
+
+
+def test_transposes_between_two_transformed_convs_cancel():
+    g = Graph()
+    x = g.add_input((2, 8, 16, 16), f32)
+    w1 = g.add_input((8, 8, 3, 3), f32)
+    w2 = g.add_input((8, 8, 3, 3), f32)
+    a = {"dilation": (1, 1), "kernel_shape": (3, 3), "pad": (1, 1, 1, 1), "stride": (1, 1), "group": 1, "layout": "NCHW"}
+    y = g.add_op("conv", [g.add_op("conv", [x, w1], dict(a)), w2], dict(a))
+    g.set_outputs([y])
+    run_llh_pipeline(g, "NHWC")
+    assert g.op_names() == ["transpose", "transpose", "conv", "transpose", "conv", "transpose"]
+    assert g.ops[4].operands[0] is g.ops[2].results[0]      # the second conv reads the first one's NHWC result
+
+
+def test_compiler_takes_both_layouts_and_nothing_else():
+    from llcompiler_amd import LLCompiler
+    assert LLCompiler(target_layout="NHWC").target_layout == "NHWC"
+    assert LLCompiler().target_layout == "NCHW"
+    with pytest.raises(ValueError):
+        LLCompiler(target_layout="NCWH")

@@ -58,7 +58,8 @@ def test_conv_attributes_and_symbolic_result_shape():
     g = parse_llh(CONV_AND_SHAPES, func="conv_nchw_fchw")
     (conv,) = g.ops
     assert conv.name == "conv" and [v.name for v in conv.operands] == ["arg1", "arg0"]
-    assert conv.attrs == {"dilation": (2, 2), "kernel_shape": (5, 5), "pad": (2, 2, 2, 2), "stride": (2, 2), "group": 1}
+    assert conv.attrs == {"dilation": (2, 2), "kernel_shape": (5, 5), "pad": (2, 2, 2, 2), "stride": (2, 2), "group": 1,
+                          "layout": "NCHW"}
     n, f, oh, ow = conv.results[0].shape
     assert f == 4 and isinstance(n, Expr) and isinstance(oh, Expr)
     # out = (in + 2 + 2 - 2 * (5 - 1) - 1) / 2 + 1 (src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:257-268)
@@ -150,3 +151,22 @@ def test_llh_plan_tool_prints_the_fused_plan(tmp_path, capsys):
     assert plan_tool.main([str(multi), "--func", "conv_nchw_fchw"]) == 0
     out = capsys.readouterr().out
     assert "= conv(%arg1, %arg0) : tensor<?x4x?x?xf32>" in out
+
+
+NHWC_CONV = '''func.func @main(%x: tensor<2x9x9x64xf32>, %w: tensor<8x3x3x64xf32>) -> tensor<2x9x9x8xf32> attributes {entrance} {
+  %y = "llh.conv"(%x, %w) <{dilation = array<i64: 1, 1>, group = 1 : i64, kernel_shape = array<i64: 3, 3>, layout = #llh.Layout<NHWC>, weight_layout = #llh.Layout<FHWC>, pad = array<i64: 1, 1, 1, 1>, stride = array<i64: 1, 1>}> : (tensor<2x9x9x64xf32>, tensor<8x3x3x64xf32>) -> tensor<2x9x9x8xf32>
+  return %y : tensor<2x9x9x8xf32>
+}
+'''
+
+
+def test_conv_in_the_nhwc_layout_is_read_printed_and_read_again():
+    """layout = #llh.Layout<NHWC> (include/llcompiler/Dialect/LLH/IR/LLHEnums.td:61-75): operands and result are
+    [N,H,W,C] / [F,KH,KW,C] / [N,OH,OW,F]."""
+    g = parse_llh(NHWC_CONV)
+    (conv,) = g.ops
+    assert conv.attrs["layout"] == "NHWC" and conv.results[0].shape == (2, 9, 9, 8)
+    again = parse_llh(print_llh(g))
+    assert again.ops[0].attrs["layout"] == "NHWC" and again.ops[0].results[0].shape == (2, 9, 9, 8)
+    with pytest.raises(NotImplementedError):
+        parse_llh(NHWC_CONV.replace("weight_layout = #llh.Layout<FHWC>", "weight_layout = #llh.Layout<HWCF>"))
