@@ -144,6 +144,14 @@ def build_extra_cases(ops, device):
                                                  (_uniform((c, c, 3, 3), dt, gen, device) * 0.05).contiguous(memory_format=cl),
                                                  torch.empty((16, c, hw, hw), dtype=dt, device=device).contiguous(memory_format=cl)),
                       lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 2)
+    # layers with work for the whole chip (batch 32): what the bf16 convolution reaches when it is not launch-bound
+    for c, f, hw in ((256, 256, 56), (128, 128, 56), (128, 256, 28)):
+        cases.add("conv3x3_%dto%d_%dx%d_batch32" % (c, f, hw, hw), "bf16", "mfma", 2.0 * 32 * hw * hw * c * f * 9,
+                  (32 * (c + f) * hw * hw + c * f * 9) * 2,
+                  lambda c=c, f=f, hw=hw: (_uniform((32, c, hw, hw), bf, gen, device).contiguous(memory_format=cl),
+                                           (_uniform((f, c, 3, 3), bf, gen, device) * 0.05).contiguous(memory_format=cl),
+                                           torch.empty((32, f, hw, hw), dtype=bf, device=device).contiguous(memory_format=cl)),
+                  lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 2)
     cases.add("conv7x7_stem_3to64_224", "f32", "mfma", 2.0 * 16 * 112 * 112 * 64 * 147, (16 * 3 * 224 * 224 + 64 * 147 + 16 * 64 * 112 * 112) * 4,
               lambda: (_uniform((16, 3, 224, 224), torch.float32, gen, device), _uniform((64, 3, 7, 7), torch.float32, gen, device) * 0.05,
                        torch.empty((16, 64, 112, 112), dtype=torch.float32, device=device)),

@@ -89,6 +89,21 @@ void workspace_track(size_t* high_water);
 // instantiation, static at the call site) keeps a bit per device ordinal.
 int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done);
 
+// Convolution on channels-last 16-bit tensors as an implicit GEMM on the wide-tile matmul kernel (gemm.hip):
+// out[pixel, f] = sum over (tap, c) of x[pixel's window at tap, c] * w[f, tap, c].
+struct ConvWideGeom {
+  int32_t C, H, W, OH, OW, KH, KW;
+  int32_t sh, sw, ph, pw, dh, dw;
+  int32_t ncols;                    // N * OH * OW output pixels
+  int32_t cblocks;                  // C / 64: k-tiles per tap
+  uint32_t cblocks_magic, kw_magic; // for d = cblocks, KW: floor(2^32 / d) + 1, so that n / d == (n * magic) >> 32 for
+                                    // the small n that occur; 0 when d == 1
+};
+// Runs it and returns LLC_OK (or an error); returns 1 without doing anything when the shape is not one the wide-tile
+// kernel takes (the caller then uses its own kernels).
+int conv_wide_16bit(int dtype, const char* x, const char* w, char* y, const char* bias, const char* residual, int F,
+                    const ConvWideGeom& g, float alpha, int act, hipStream_t s);
+
 #define LLC_TRY(expr)              \
   do {                             \
     int _st = (expr);              \

@@ -761,6 +761,19 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
 
 template <typename T>
 int launch_nhwc(const ConvParams& p, hipStream_t s) {
+  if constexpr (sizeof(T) == 2) {
+    // layers with work for the whole chip: the wide-tile matmul kernel with the image as its row operand
+    auto magic = [](uint32_t d) { return d == 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / d) + 1u; };
+    ConvWideGeom g{};
+    g.C = p.C, g.H = p.H, g.W = p.Wd, g.OH = p.OH, g.OW = p.OW, g.KH = p.KH, g.KW = p.KW;
+    g.sh = p.sh, g.sw = p.sw, g.ph = p.ph, g.pw = p.pw, g.dh = p.dh, g.dw = p.dw;
+    g.ncols = p.ncols;
+    g.cblocks = p.C / 64;
+    g.cblocks_magic = magic((uint32_t)(p.C / 64));
+    g.kw_magic = magic((uint32_t)p.KW);
+    const int st = conv_wide_16bit(Elem<T>::kDtype, p.X, p.W, p.Y, p.bias, p.residual, p.F, g, p.alpha, p.act, s);
+    if (st != 1) return st;
+  }
   // 128-pixel tiles when they fill the chip by themselves; else 64 x 64 tiles if those are numerous enough to need
   // no split of the reduction (a split costs a pass over the partial sums: the middle layers of a ResNet); the
   // last layers split either way and do better on the large tiles, unless their reduction is too short to split

@@ -58,6 +58,7 @@ struct GemmParams {
   int32_t act;
   int32_t tiles_m, tiles_n;
   int32_t c_f32;  // gemm_kernel only: C holds raw fp32 sums whatever T is (the chunks of a split reduction)
+  ConvWideGeom cg;  // gemm_wide_kernel<.., CONV = true> only: A is an image, its rows are gathered windows
 };
 
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB, bool FULL>
@@ -905,6 +906,44 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
 }
 
 }  // namespace
+
+int conv_wide_16bit(int dtype, const char* x, const char* w, char* y, const char* bias, const char* residual, int F,
+                    const ConvWideGeom& g, float alpha, int act, hipStream_t s) {
+#ifdef LLC_GEMM_TUNE
+  if (const char* e = getenv("LLC_CONV_WIDE"))
+    if (atoi(e) == 0) return 1;
+#endif
+  const int64_t K = (int64_t)g.KH * g.KW * g.C;
+  // (reductions shorter than 2048 are too few k-tiles per tile for one workgroup per CU: a tile's fill and drain weigh
+  // as much as its loop, and the kernels that keep two workgroups on a CU are faster; measured at batch 32:
+  // 128 -> 128 channels 3x3 on 56x56 68 us here against 61, 256 -> 256 159 against 197, 512 -> 512 on 28x28 127 against 177)
+  if ((dtype != LLC_BFLOAT16 && dtype != LLC_FLOAT16) || g.C % 64 != 0 || g.KH * g.KW > 32 || K < 2048 || F % 128 != 0) return 1;
+  // one workgroup per CU and tile: worth it only when the tiles fill at least three quarters of the chip
+  const int64_t tiles_m = (g.ncols + 255) / 256;
+  int bn = 0;
+  if (F % 256 == 0 && tiles_m * (F / 256) >= 192) bn = 256;
+  else if (tiles_m * (F / 128) >= 192) bn = 128;
+  if (bn == 0 || tiles_m * (F / bn) > 0x7fffffff) return 1;
+  GemmParams p{};
+  p.A = x;
+  p.B = w;
+  p.C = y;
+  p.bias = bias;
+  p.residual = residual;
+  p.M = g.ncols;
+  p.N = F;
+  p.K = (int32_t)K;
+  p.a_sk = 1;
+  p.b_sk = 1;
+  p.b_sn = K;
+  p.c_sm = F;
+  p.bdiv = 1;
+  p.alpha = alpha;
+  p.act = act;
+  p.cg = g;
+  if (dtype == LLC_BFLOAT16) return bn == 256 ? launch_wide<__bf16, kBKMajor, 256, true>(p, 1, s) : launch_wide<__bf16, kBKMajor, 128, true>(p, 1, s);
+  return bn == 256 ? launch_wide<_Float16, kBKMajor, 256, true>(p, 1, s) : launch_wide<_Float16, kBKMajor, 128, true>(p, 1, s);
+}
 
 namespace {
 int gemm_dispatch(int dtype, const GemmParams& p, int batch, hipStream_t s) {

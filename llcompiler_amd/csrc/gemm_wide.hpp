@@ -77,9 +77,18 @@ struct WideGeom {
   static constexpr int kLds = 2 * (kAStage + kBStage) > 4 * kOutWave ? 2 * (kAStage + kBStage) : 4 * kOutWave;
 };
 
-template <typename T, int BMODE, int BN>
+// Rows of zeros for the taps of a convolution window that fall outside the image (CONV: a lane whose tap is outside
+// loads from here instead).
+static __device__ __align__(256) unsigned char llc_zero_row[256];
+
+// CONV: A is a channels-last image [n, H, W, C] and row m of the product is output pixel m; k runs over (tap, channel)
+// in 64-channel k-tiles that lie inside one tap, so a k-tile of a row is 128 contiguous bytes of the image (or of
+// zeros).  Each lane keeps, for its 8 rows, the element offset of the window origin and one validity bit per tap,
+// computed once; a k-tile adds one scalar offset.  B is the weight [F, taps * C].
+template <typename T, int BMODE, int BN, bool CONV = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_wide_kernel(const GemmParams p) {
   static_assert(sizeof(T) == 2, "16-bit operands");
+  static_assert(!CONV || BMODE == kBKMajor, "convolution weights are k-contiguous");
   static_assert(BMODE == kBKMajor || BN != 192, "row-major B: the chunk swizzle needs 16 or 32 chunks per row");
   using G = WideGeom<BN>;
   constexpr int TM = G::TM, TN = G::TN;
@@ -90,7 +99,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
   const int m0 = tile_m * 256, n0 = tile_n * BN;
   const int z0 = z / p.bdiv, z1 = z - z0 * p.bdiv;
-  const char* A = (const char*)((const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1 + (int64_t)m0 * p.a_sm);
+  const char* A = CONV ? p.A : (const char*)((const T*)p.A + (int64_t)z0 * p.a_sb + (int64_t)z1 * p.a_sb1 + (int64_t)m0 * p.a_sm);
   const char* B = (const char*)((const T*)p.B + (int64_t)z0 * p.b_sb + (int64_t)z1 * p.b_sb1 +
                                 (BMODE == kBKMajor ? (int64_t)n0 * p.b_sn : (int64_t)n0));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -115,11 +124,50 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       lb_off[0] = lb_off[1] = (uint32_t)(krow0 * b_row_bytes) + ((slot ^ ((krow0 & 3) << 2)) << 4);
     }
   }
+  // CONV: window origin (element offset into the image, may be negative) and valid taps of this lane's row in each of
+  // its 8 A loads (rows wave * 8 + lane / 8 + 32 d of the tile)
+  int pix_off[CONV ? 8 : 1];
+  uint32_t pix_taps[CONV ? 8 : 1];
+  if constexpr (CONV) {
+    const ConvWideGeom& cg = p.cg;
+    const int ohw = cg.OH * cg.OW;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      const int m = m0 + wave * 8 + lane / 8 + 32 * d;
+      pix_off[d] = 0;
+      pix_taps[d] = 0;
+      if (m < cg.ncols) {
+        const int n = m / ohw, rem = m - n * ohw;
+        const int oh = rem / cg.OW, ow = rem - oh * cg.OW;
+        const int ih0 = oh * cg.sh - cg.ph, iw0 = ow * cg.sw - cg.pw;
+        pix_off[d] = ((n * cg.H + ih0) * cg.W + iw0) * cg.C;
+        uint32_t bits = 0;
+        for (int kh = 0; kh < cg.KH; ++kh)
+          for (int kw = 0; kw < cg.KW; ++kw) {
+            const int ih = ih0 + kh * cg.dh, iw = iw0 + kw * cg.dw;
+            if (ih >= 0 && ih < cg.H && iw >= 0 && iw < cg.W) bits |= 1u << (kh * cg.KW + kw);
+          }
+        pix_taps[d] = bits;
+      }
+    }
+  }
   // load d of k-tile kt into `stage`: a uniform 64-bit base (scalar registers) plus the lane's 32-bit offset.  The
   // empty asm keeps the compiler from folding base and offset into sixteen loop-invariant 64-bit lane pointers.
   auto dma = [&](auto d_tag, int kt, int stage) {
     constexpr int D = decltype(d_tag)::value;
-    if constexpr (D < G::kLoadsA) {
+    if constexpr (CONV && D < G::kLoadsA) {
+      const ConvWideGeom& cg = p.cg;
+      // uniform: tap and channel block of the k-tile, the tap's offset from the window origin
+      // (n / d as (n * magic) >> 32 with magic = floor(2^32 / d) + 1; magic 0 stands for d = 1)
+      const uint32_t tap = cg.cblocks_magic ? (uint32_t)(((uint64_t)(uint32_t)kt * cg.cblocks_magic) >> 32) : (uint32_t)kt;
+      const int c0 = (kt - (int)tap * cg.cblocks) * 64;
+      const uint32_t kh = cg.kw_magic ? (uint32_t)(((uint64_t)tap * cg.kw_magic) >> 32) : tap, kw = tap - kh * cg.KW;
+      const int64_t toff = (int64_t)(((int)kh * cg.dh * cg.W + (int)kw * cg.dw) * cg.C + c0) * 2;
+      const uint32_t chunk = ((((lane % 8) ^ lds_swz(wave * 8 + lane / 8) ^ (4 * (D & 1))) & 7) << 4);
+      const bool inside = (pix_taps[D] >> tap) & 1u;
+      const char* g = inside ? A + (int64_t)pix_off[D] * 2 + toff + chunk : (const char*)llc_zero_row + chunk;
+      __builtin_amdgcn_global_load_lds(LLC_GPTR(g), LLC_LPTR(smem + stage * G::kAStage + (wave + 4 * D) * 1024), 16, 0, 0);
+    } else if constexpr (D < G::kLoadsA) {
       uint32_t off = la_off[D & 1];
       asm volatile("" : "+v"(off));
       const char* g = A + (int64_t)(32 * D) * a_row_bytes + (int64_t)kt * 128;
@@ -295,7 +343,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int i = 0; i < TM; ++i) {
           const int row = i * 32 + li;
           uint2 rq = {0, 0};
-          if constexpr (RES) rq = *(const uint2*)(res + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + col);
+          if constexpr (RES) {
+            // rows past the last pixel of a convolution are computed and dropped: read their residual from the last row
+            const int rrow = (CONV && mrow0 + row >= p.M) ? p.M - 1 : mrow0 + row;
+            rq = *(const uint2*)(res + (int64_t)rrow * p.c_sm + ncol0 + col);
+          }
           uint32_t o[2];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -328,18 +380,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int idx = it * 64 + lane;
     const int row = idx / kChunks, ch = idx % kChunks;
     const u32x4_t v = *(const u32x4_t*)(wst + row * G::kOutPitch + ch * 16);
-    *(u32x4_t*)(C + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + ch * 8) = v;
+    if (!CONV || mrow0 + row < p.M) *(u32x4_t*)(C + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + ch * 8) = v;
   }
   LLC_DBG_T1();
 }
 
-template <typename T, int BMODE, int BN>
+template <typename T, int BMODE, int BN, bool CONV = false>
 int launch_wide(const GemmParams& p0, int batch, hipStream_t s) {
   using G = WideGeom<BN>;
   GemmParams p = p0;
-  p.tiles_m = p.M / 256;
+  p.tiles_m = (p.M + 255) / 256;  // whole tiles, except the last rows of a convolution
   p.tiles_n = p.N / BN;
-  auto kern = gemm_wide_kernel<T, BMODE, BN>;
+  auto kern = gemm_wide_kernel<T, BMODE, BN, CONV>;
   static std::atomic<uint32_t> lds_allowed{0};
   LLC_TRY(allow_dynamic_lds((const void*)kern, G::kLds, lds_allowed));
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch), dim3(256), G::kLds, s, p);

@@ -1021,6 +1021,43 @@ def test_conv2d_channels_last(ops, oracle, case):
                           "channels-last conv+bias+res+relu %s %s" % (dt, case))
 
 
+WIDE_CONV_CASES = [
+    # N, C, H, W, F, KH, KW, pad, stride, dil: reductions of 2048 and more, at least 192 tiles of 256 pixels x 128 (256) filters
+    (17, 256, 54, 54, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 49572 pixels: the last tile has 164 rows
+    (16, 256, 112, 112, 128, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),   # stride 2
+    (13, 128, 66, 66, 256, 4, 4, (1, 0, 2, 1), (1, 1), (2, 1)),     # 256-filter tiles, even window, dilation, asymmetric pads
+]
+
+
+@pytest.mark.parametrize("case", WIDE_CONV_CASES)
+def test_conv2d_channels_last_16bit_on_wide_tiles(ops, oracle, case):
+    """Channels-last 16-bit convolutions with work for the whole chip and a long reduction run on the wide-tile matmul
+    kernel, the image as its row operand (windows gathered by the loads, taps outside the image read as zeros).  The
+    oracle evaluates the first and the last image of the batch (samples are independent; the last one holds the
+    incomplete tile)."""
+    N, C, H, W, Fo, KH, KW, pad, s, d = case
+    r = rng(sum(case[:7]) + 3)
+    cl = torch.channels_last
+    xb = bf16_round(r.standard_normal((N, C, H, W)))
+    wb = bf16_round(r.standard_normal((Fo, C, KH, KW)) / np.sqrt(C * KH * KW))
+    bb = bf16_round(r.standard_normal(Fo))
+    pick = [0, N - 1]
+    wantb = oracle.conv2d(xb[pick], wb, None, pad=pad, stride=s, dilation=d)
+    full = (N,) + wantb.shape[1:]
+    assert (N * full[2] * full[3] + 255) // 256 * (Fo // 128) >= 192 and C * KH * KW >= 2048
+    rb = bf16_round(r.standard_normal(full))
+    wantb2 = oracle.unary("relu", (wantb * np.float32(0.5) + bb[None, :, None, None] + rb[pick]).astype(np.float32))
+    for dt in (torch.bfloat16, torch.float16):
+        tx, tw = dev(xb, dt).contiguous(memory_format=cl), dev(wb, dt).contiguous(memory_format=cl)
+        o = torch.empty(full, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        g = ops.conv2d(tx, tw, pad=pad, stride=s, dilation=d, out=o)
+        assert_close_bf16(host(g)[pick], wantb, "wide channels-last conv %s %s" % (dt, case))
+        epi = ops.Epilogue(alpha=0.5, bias=dev(bb, dt), residual=dev(rb, dt).contiguous(memory_format=cl), act="relu")
+        o2 = torch.empty(full, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        assert_close_bf16(host(ops.conv2d(tx, tw, pad=pad, stride=s, dilation=d, epilogue=epi, out=o2))[pick], wantb2,
+                          "wide channels-last conv with epilogue %s %s" % (dt, case))
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_conv_cases(ops, oracle, seed):
     """Randomly drawn convolutions: window, stride, dilation, asymmetric pads, groups, channel and filter counts on
