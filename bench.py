@@ -112,13 +112,13 @@ def build_cases(ops, device, only=()):
     return cases
 
 
-def build_extra_cases(ops, device):
+def build_extra_cases(ops, device, only=()):
     """Contractions outside the suite that the model configurations are made of, reported under "extra_kernels" (not
     part of `value`): the bf16 matmul at 4096^3, the feed-forward products of the encoder block at batch 32 with their
     fused epilogues (Linear weights [N,K] consumed as transposed views), and the convolution classes of ResNet-18 at
     batch 16 (3x3 body layers channels-last in fp32 and bf16, the 7x7 stride-2 stem in NCHW)."""
     gen = torch.Generator().manual_seed(1)
-    cases = _Cases([])
+    cases = _Cases(list(only))
     bf = torch.bfloat16
     n = 4096
     cases.add("matmul_4096", "bf16", "mfma", 2.0 * n * n * n, 3 * n * n * 2,
@@ -478,7 +478,14 @@ def main():
         if c.bound == "hbm":
             k["copy_same_bytes_us"] = round(copy_floor_us(ops, device, c.bytes), 2)
             k["frac_of_copy"] = round(k["copy_same_bytes_us"] / (k["avg_ms"] * 1e3), 3)
-    dominant = max(kernels, key=lambda k: k["avg_ms"])
+    extra_rows = []
+    if not args.no_extra:
+        # with --only, the rows outside the suite that it names (for counter runs on one of them)
+        extra = build_extra_cases(ops, device, only)
+        extra_rows = [roofline_of(c, time_gpu(c.run, 50, 10)) for c in extra]
+        del extra
+        torch.cuda.empty_cache()
+    dominant = max(kernels or extra_rows, key=lambda k: k["avg_ms"])
     out = {
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False,
@@ -489,11 +496,8 @@ def main():
         "dominant_kernel": dominant["kernel"],
         "kernels": kernels,
     }
-    if not only and not args.no_extra:
-        extra = build_extra_cases(ops, device)
-        out["extra_kernels"] = [roofline_of(c, time_gpu(c.run, 50, 10)) for c in extra]
-        del extra
-        torch.cuda.empty_cache()
+    if extra_rows:
+        out["extra_kernels"] = extra_rows
     if not args.no_models and models:
         try:
             configs = model_latencies(models)
