@@ -491,13 +491,97 @@ def _first_result_only(node):
     return all(u.op == "call_function" and u.target is operator.getitem and u.args[1] == 0 for u in node.users)
 
 
-@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm.default, check=lambda n: len(n.args[1]) == 1 and _first_result_only(n))
+def _as(ctx, v, dtype):
+    return v if v.dtype == dtype else ctx.g.add_op("convert_to", [v], {"dtype": dtype})
+
+
+def _sum_keep_last(ctx, v):
+    """Sum over the last dim, kept as an extent of 1 (what broadcasts back over the rows)."""
+    r = ctx.g.add_op("reduce_sum", [v], {"axis": (v.rank - 1,)})
+    return _reshape_to(ctx, r, tuple(v.shape[:-1]) + (1,))
+
+
+def _used_results(node):
+    return set(u.args[1] for u in node.users if u.op == "call_function" and u.target is operator.getitem)
+
+
+def _last_dim_static(node):
+    return len(node.args[1]) == 1 and isinstance(node.args[0].meta["val"].shape[-1], int)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm.default,
+                                   check=lambda n: len(n.args[1]) == 1 and (_first_result_only(n) or _last_dim_static(n)))
 def _layer_norm(ctx, node):
+    """The output is llh.layer_norm; the saved statistics a backward graph asks for (mean and 1/std of every row, kept
+    as [.., 1]) are spelt with reductions and elementwise ops in fp32, as torch computes them."""
     x, shape, w, b, eps = node.args
     ops = [ctx.val(x)] + [ctx.val(t) for t in (w, b) if t is not None]
     attrs = {"epsilon": float(eps), "axis": -1, "has_scale": w is not None, "has_bias": b is not None}
     y = ctx.g.add_op("layer_norm", ops, attrs)
-    return (y, None, None)
+    used = _used_results(node)
+    if not (used - {0}):
+        return (y, None, None)
+    g = ctx.g
+    x32 = _as(ctx, ctx.val(x), torch.float32)
+    n = float(x32.shape[-1])
+    mean = g.add_op("div", [_sum_keep_last(ctx, x32), g.constant(n, torch.float32)])
+    d = g.add_op("sub", [x32, mean])
+    var = g.add_op("div", [_sum_keep_last(ctx, g.add_op("mul", [d, d])), g.constant(n, torch.float32)])
+    rstd = g.add_op("rsqrt", [g.add_op("add", [var, g.constant(float(eps), torch.float32)])])
+    vals = node.meta["val"]
+    return (y, _as(ctx, mean, vals[1].dtype), _as(ctx, rstd, vals[2].dtype))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.native_layer_norm_backward.default,
+                                   check=lambda n: len(n.args[2]) == 1 and isinstance(n.args[1].meta["val"].shape[-1], int))
+def _layer_norm_backward(ctx, node):
+    """dx = rstd (g w - mean(g w) - xhat mean(g w xhat)), dw = sum over rows of g xhat, db = sum over rows of g, with
+    xhat = (x - mean) rstd from the saved statistics; fp32 arithmetic whatever the storage type (torch's own)."""
+    go, x, shape, mean, rstd, w, b, mask = node.args
+    g = ctx.g
+    f32 = torch.float32
+    go32, x32 = _as(ctx, ctx.val(go), f32), _as(ctx, ctx.val(x), f32)
+    mean32, rstd32 = _as(ctx, ctx.val(mean), f32), _as(ctx, ctx.val(rstd), f32)
+    n = float(x32.shape[-1])
+    xhat = g.add_op("mul", [g.add_op("sub", [x32, mean32]), rstd32])
+    vals = node.meta["val"]
+    dx = dw = db = None
+    if mask[0]:
+        gw = g.add_op("mul", [go32, _as(ctx, ctx.val(w), f32)]) if w is not None else go32
+        m1 = g.add_op("div", [_sum_keep_last(ctx, gw), g.constant(n, f32)])
+        m2 = g.add_op("div", [_sum_keep_last(ctx, g.add_op("mul", [gw, xhat])), g.constant(n, f32)])
+        inner = g.add_op("sub", [g.add_op("sub", [gw, m1]), g.add_op("mul", [xhat, m2])])
+        dx = _as(ctx, g.add_op("mul", [inner, rstd32]), vals[0].dtype)
+    rows = tuple(range(x32.rank - 1))
+    if mask[1] and w is not None:
+        dw = _as(ctx, g.add_op("reduce_sum", [g.add_op("mul", [go32, xhat])], {"axis": rows}), vals[1].dtype)
+    if mask[2] and b is not None:
+        db = _as(ctx, g.add_op("reduce_sum", [go32], {"axis": rows}), vals[2].dtype)
+    return (dx, dw, db)
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._softmax_backward_data.default,
+                                   check=lambda n: n.args[2] % n.args[0].meta["val"].dim() == n.args[0].meta["val"].dim() - 1)
+def _softmax_backward(ctx, node):
+    """dx = y (g - sum(g y)) over the last dim, in fp32."""
+    go, y = _as(ctx, ctx.val(node.args[0]), torch.float32), _as(ctx, ctx.val(node.args[1]), torch.float32)
+    g = ctx.g
+    s = _sum_keep_last(ctx, g.add_op("mul", [go, y]))
+    return _as(ctx, g.add_op("mul", [y, g.add_op("sub", [go, s])]), _out_dtype(node))
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten.gelu_backward.default, check=lambda n: n.kwargs.get("approximate", "none") == "none")
+def _gelu_backward(ctx, node):
+    """g (Phi(x) + x phi(x)): the derivative of x Phi(x), one elementwise program after fusion."""
+    g = ctx.g
+    f32 = torch.float32
+    go, x = _as(ctx, ctx.val(node.args[0]), f32), _as(ctx, ctx.val(node.args[1]), f32)
+
+    def c(v):
+        return g.constant(v, f32)
+    cdf = g.add_op("mul", [g.add_op("add", [g.add_op("erf", [g.add_op("mul", [x, c(0.7071067811865476)])]), c(1.0)]), c(0.5)])
+    pdf = g.add_op("mul", [g.add_op("exp", [g.add_op("mul", [g.add_op("mul", [x, x]), c(-0.5)])]), c(0.3989422804014327)])
+    return _as(ctx, g.add_op("mul", [go, g.add_op("add", [cdf, g.add_op("mul", [x, pdf])])]), _out_dtype(node))
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(aten._native_batch_norm_legit_no_training.default, check=_first_result_only)

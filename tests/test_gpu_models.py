@@ -486,6 +486,50 @@ def test_training_mode_with_eager_fallbacks(which):
         assert_close(p.grad.cpu().numpy(), q.grad.cpu().numpy(), 1e-4, 1e-5 * scale, "grad of %s" % name)
     kinds = [s.kind for e in comp.engines for s in e.steps]
     assert kinds.count("matmul") >= 3 and len(comp.engines) >= 2
+    if which == "encoder":
+        # layer norm (with its saved statistics), softmax and gelu have translators for their backward ops: the forward
+        # and the backward graph are one compiled partition each, nothing of the block runs in eager
+        assert len(comp.engines) == 2, len(comp.engines)
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_backward_ops_against_eager(dt):
+    """native_layer_norm (output and saved statistics), native_layer_norm_backward, _softmax_backward_data and
+    gelu_backward as compiled graphs against the ATen kernels (for bf16: at the bf16 bar plus what eager's own bf16
+    evaluation misses the float64 result by)."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from llcompiler_amd.executor.engine import Torch_ExecutionEngine
+    from llcompiler_amd.importer.fx_importer import torch_translate_to_llh_graph
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    aten = torch.ops.aten
+
+    def f(x, w, b, go, y):
+        out, mean, rstd = aten.native_layer_norm(x, [96], w, b, 1e-5)
+        dx, dw, db = aten.native_layer_norm_backward(go, x, [96], mean, rstd, w, b, [True, True, True])
+        ds = aten._softmax_backward_data(go, y, -1, x.dtype)
+        dg = aten.gelu_backward(go, x)
+        return out, mean, rstd, dx, dw, db, ds, dg
+
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 33, 96, generator=gen)
+    w, b = torch.rand(96, generator=gen) + 0.5, torch.randn(96, generator=gen)
+    go = torch.randn(5, 33, 96, generator=gen)
+    y = torch.softmax(torch.randn(5, 33, 96, generator=gen), -1)
+    args = [t.to(dt).cuda() for t in (x, w, b, go, y)]
+    gm = make_fx(f, tracing_mode="fake")(*args)
+    g = torch_translate_to_llh_graph(gm)
+    run_llh_pipeline(g)
+    got = Torch_ExecutionEngine(g).run(*args)
+    eager = f(*args)
+    want64 = f(*[t.double() for t in args])
+    names = ["out", "mean", "rstd", "dx", "dw", "db", "dsoftmax", "dgelu"]
+    for name, a, e, w64 in zip(names, got, eager, want64):
+        assert a.dtype == e.dtype and a.shape == e.shape, name
+        if dt == torch.float32:
+            scale = float(w64.abs().max())
+            assert_close(a.cpu().numpy(), w64.cpu().numpy(), 1e-4, 1e-5 * max(scale, 1.0), name)
+        else:
+            assert_as_close_as_eager(a.float().cpu().numpy(), e.float().cpu().numpy(), w64.cpu().numpy(), BF16_RTOL, BF16_ATOL, name)
 
 
 def test_projections_of_the_same_rows_run_as_one_product():

@@ -372,3 +372,35 @@ def test_compiler_takes_both_layouts_and_nothing_else():
     assert LLCompiler().target_layout == "NCHW"
     with pytest.raises(ValueError):
         LLCompiler(target_layout="NCWH")
+
+
+def test_backward_ops_of_layer_norm_softmax_and_gelu_are_imported():
+    """aten.native_layer_norm with its saved statistics, native_layer_norm_backward, _softmax_backward_data and
+    gelu_backward are spelt with reductions and elementwise ops (fp32 arithmetic), so training-mode graphs of
+    transformer blocks need no eager fallback for them."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from llcompiler_amd.importer.fx_importer import is_supported, torch_translate_to_llh_graph
+    aten = torch.ops.aten
+
+    def f(x, w, b, go, y):
+        out, mean, rstd = aten.native_layer_norm(x, [32], w, b, 1e-5)
+        dx, dw, db = aten.native_layer_norm_backward(go, x, [32], mean, rstd, w, b, [True, True, True])
+        ds = aten._softmax_backward_data(go, y, -1, torch.float32)
+        dg = aten.gelu_backward(go, x)
+        return out, dx, dw, db, ds, dg
+
+    args = [torch.zeros(4, 6, 32), torch.zeros(32), torch.zeros(32), torch.zeros(4, 6, 32), torch.zeros(4, 6, 32)]
+    gm = make_fx(f, tracing_mode="fake")(*args)
+    calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+    assert all(is_supported(n) for n in calls), [str(n.target) for n in calls if not is_supported(n)]
+    g = torch_translate_to_llh_graph(gm)
+    names = g.op_names()
+    assert names.count("layer_norm") == 1 and "rsqrt" in names and "erf" in names and "exp" in names
+    shapes = [tuple(o.shape) for o in g.outputs]
+    assert shapes == [(4, 6, 32), (4, 6, 32), (32,), (32,), (4, 6, 32), (4, 6, 32)]
+    # the statistics are [.., 1] rows and the weight gradients reduce over every row dim
+    red = [op for op in g.ops if op.name == "reduce_sum"]
+    assert any(tuple(op.attrs["axis"]) == (0, 1) for op in red) and any(tuple(op.attrs["axis"]) == (2,) for op in red)
+    run_llh_pipeline(g)
+    kinds = [s.kind for s in make_plan(g)]
+    assert "layer_norm" in kinds and kinds.count("reduce") >= 6
