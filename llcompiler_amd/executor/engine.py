@@ -50,6 +50,7 @@ CHANNELS_LAST = True
 # linear layers that read the same rows with weights that are graph inputs (q, k, v projections) run as one
 # product against a stacked copy of the weights
 FUSE_PROJECTIONS = True
+PROJ_TILE_LIMIT = 1024  # projections of the same rows are stacked while one of them has fewer 64x64 tiles than this
 
 
 def _concrete(shape, env):
@@ -428,10 +429,11 @@ class Instance:
             if x.dim() != 2:
                 return False
             m, kdim = x.shape
-            # worth it while one layer's product leaves CUs idle (under two rounds of 64x64 tiles); with more rows
-            # the separate products are as fast and their results lie denser for the attention kernel (measured
-            # on the bf16 encoder block: 17% faster at 512 rows, 1% slower at 4096, 5% slower at 16384)
-            if ((m + 63) // 64) * ((nat[1] + 63) // 64) >= 512:
+            # worth it while one layer's product leaves CUs idle or fills them unevenly; with more rows the separate
+            # products are as fast and their results lie denser for the attention kernel (measured on the bf16
+            # encoder block: 17% faster at 512 rows, 9% faster at 4096, 3% slower at 16384; BERT-base fp32 at
+            # 4096 rows 1.5% faster)
+            if ((m + 63) // 64) * ((nat[1] + 63) // 64) >= PROJ_TILE_LIMIT:
                 return False
 
             def member(s2):
