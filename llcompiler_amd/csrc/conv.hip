@@ -811,11 +811,14 @@ int launch_tiles(const ConvParams& p, int groups, hipStream_t s) {
   return launch_cfg<T, 64, 64, LA>(p, groups, s);
 }
 
+#include "conv_rows.hpp"
+
 template <typename T>
 int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
   const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
   if constexpr (sizeof(T) == 4) {
+    if (conv_rows_ok(p, groups)) return launch_conv_rows(p, s);
     if (w_vec && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
         ((uintptr_t)p.X % 4) == 0 && (int64_t)p.N * p.C * p.H * p.Wd < ((int64_t)1 << 30))  // 32-bit byte offsets
       return launch_f32(p, groups, s);

@@ -1021,6 +1021,35 @@ def test_conv2d_channels_last(ops, oracle, case):
                           "channels-last conv+bias+res+relu %s %s" % (dt, case))
 
 
+ROW_CONV_CASES = [
+    # N, C, H, W, KH, KW, pad(h_lo, w_lo, h_hi, w_hi), stride: fp32 NCHW, 64 filters, reduction <= 148, stride 2 along w
+    (4, 3, 128, 128, 7, 7, (3, 3, 3, 3), (2, 2)),     # an image network's first layer
+    (6, 3, 98, 200, 7, 7, (3, 3, 3, 3), (2, 2)),      # 100 output columns: the last pixel block is partly outside
+    (2, 4, 130, 224, 5, 7, (2, 2, 1, 3), (1, 2)),     # 4 channels, 5 x 7 window, stride 1 along h, asymmetric pads
+    (5, 2, 60, 64, 7, 5, (0, 2, 3, 2), (1, 2)),       # no padding on top, 32 output columns
+]
+
+
+@pytest.mark.parametrize("case", ROW_CONV_CASES)
+def test_conv2d_first_layer_row_kernel(ops, oracle, case):
+    """Few input channels, a large window, stride 2: the kernel that keeps the input rows under the window in LDS as
+    they lie in memory and feeds the MFMAs from them (64 filters; zeros left, right, above and below come from the
+    padding columns of the LDS rows and from a row of zeros)."""
+    N, C, H, W, KH, KW, pad, s = case
+    r = rng(sum(case[:6]) + 9)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((64, C, KH, KW)) / np.sqrt(C * KH * KW)).astype(np.float32)
+    b = r.standard_normal(64).astype(np.float32)
+    want = oracle.conv2d(x, w, None, pad=pad, stride=s)
+    assert want.shape[0] * want.shape[2] >= 256 and want.shape[3] % 4 == 0
+    assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s)), want, "first-layer conv %s" % (case,))
+    want2 = oracle.unary("relu", (oracle.conv2d(x, w, b, pad=pad, stride=s) * np.float32(1.0)).astype(np.float32))
+    epi = ops.Epilogue(bias=dev(b), act="relu")
+    assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s, epilogue=epi)), want2, "first-layer conv + bias + relu")
+    want3 = oracle.conv2d(x, w, None, pad=pad, stride=s) * np.float32(0.25)
+    assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s, epilogue=ops.Epilogue(alpha=0.25))), want3, "alpha")
+
+
 WIDE_CONV_CASES = [
     # N, C, H, W, F, KH, KW, pad, stride, dil: reductions of 2048 and more, at least 192 tiles of 256 pixels x 128 (256) filters
     (17, 256, 54, 54, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 49572 pixels: the last tile has 164 rows
