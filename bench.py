@@ -485,6 +485,8 @@ def main():
         extra_rows = [roofline_of(c, time_gpu(c.run, 50, 10)) for c in extra]
         del extra
         torch.cuda.empty_cache()
+    if not kernels and not extra_rows:
+        raise SystemExit("bench.py: --only %s selects no case (with --no-extra only the single-op suite's names count)" % args.only)
     dominant = max(kernels or extra_rows, key=lambda k: k["avg_ms"])
     out = {
         "metric": "end-to-end latency ms/batch", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
