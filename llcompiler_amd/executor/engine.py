@@ -356,7 +356,15 @@ class Instance:
                 b0, b1 = full[0], full[1]
             else:
                 four = [t for t in (qa, ka, va) if t.dim() == 4]
-                b0, b1 = (four[0].shape[0], four[0].shape[1]) if four else (nat[0], 1)
+                merge = head_merge(second, nat[0], nat[1], 64)
+                if four:
+                    b0, b1 = four[0].shape[0], four[0].shape[1]
+                elif merge is not None:
+                    # every operand already lies as [B * H, S, 64] (a batch of one): the head merge that follows
+                    # says how B * H splits
+                    b0, b1 = merge[1], merge[2]
+                else:
+                    b0, b1 = nat[0], 1
 
             def as4(t):
                 if t.dim() == 4:
