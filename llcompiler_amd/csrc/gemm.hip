@@ -632,6 +632,7 @@ int launch_dma2(const GemmParams& p0, int batch, hipStream_t s) {
 
 #include "gemm_wide.hpp"
 #include "gemm_sweep.hpp"
+#include "gemm_deep.hpp"
 
 template <typename T, int BM, int BN, int WM, int WN, int LA, int LB>
 int launch_cfg(const GemmParams& p0, int batch, hipStream_t s) {
@@ -899,6 +900,7 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
       if (two) return b_kvec ? launch_dma2<T, kBKMajor>(p, batch, s) : launch_dma2<T, kBNMajor>(p, batch, s);
       return b_kvec ? launch_dma<T, kBKMajor>(p, batch, s) : launch_dma<T, kBNMajor>(p, batch, s);
     }
+    if (dma_ok && b_kvec && deep_ok(p, batch)) return launch_deep<T>(p, batch, s);
   }
   if (a_kvec && b_kvec) return launch_tiles<T, kLoadKVec, kLoadKVec>(p, batch, s);
   if (a_kvec && b_rvec) return launch_tiles<T, kLoadKVec, kLoadRVec>(p, batch, s);

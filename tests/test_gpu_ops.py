@@ -539,6 +539,43 @@ def assert_close_f16(got, want, what=""):
     assert_close(got, want, 2e-3, 4e-3, what)
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 64, 256), (128, 192, 320), (512, 768, 768), (192, 1088, 704), (512, 2304, 512)])
+def test_matmul_16bit_small_rows_deep_ring(ops, oracle, M, N, K):
+    """A few hundred rows times a linear layer's weight [N, K] (k-contiguous): the 64 x 64 tile kernel with a ring of
+    direct-to-LDS stages.  Reductions of 4 and 5 k-tiles (shorter than the ring of 8), 12, 11 (odd) and 8; up to 256
+    tiles (8 stages, one workgroup per CU) and more (4 stages, two per CU); bf16 and f16, every fused epilogue."""
+    r = rng(5 * M + 3 * N + K)
+    a = bf16_round(r.uniform(-1, 1, (M, K)))
+    wt = bf16_round(r.uniform(-1, 1, (N, K)) * 0.25)
+    base = oracle.matmul(a, np.ascontiguousarray(wt.T), "mkn")
+    da, dw = dev(a, torch.bfloat16), dev(wt, torch.bfloat16)
+    assert_close_bf16(host(ops.matmul(da, dw.t())), bf16_round(base), "NT bf16 %s" % ((M, N, K),))
+    assert_close_f16(host(ops.matmul(dev(a, torch.float16), dev(wt, torch.float16).t())), f16_round(base), "NT f16 %s" % ((M, N, K),))
+    bias = bf16_round(r.standard_normal(N))
+    res = bf16_round(r.standard_normal((M, N)))
+    for act, alpha, with_res in [("none", 1.0, True), ("relu", 0.5, False), ("gelu", 0.125, True)]:
+        w = base * np.float32(alpha) + bias[None, :]
+        if with_res:
+            w = w + res
+        if act != "none":
+            w = oracle.unary(act, w)
+        epi = ops.Epilogue(alpha=alpha, bias=dev(bias, torch.bfloat16), residual=dev(res, torch.bfloat16) if with_res else None, act=act)
+        assert_close_bf16(host(ops.matmul(da, dw.t(), epi)), bf16_round(w), "NT epilogue %s %s" % (act, (M, N, K)))
+
+
+def test_batch_matmul_16bit_small_rows_deep_ring(ops, oracle):
+    """The same kernel over a batch (the batch index rides in the grid's z dimension), with a residual per entry."""
+    r = rng(91)
+    B, M, N, K = 5, 128, 192, 448
+    a = bf16_round(r.uniform(-1, 1, (B, M, K)))
+    wt = bf16_round(r.uniform(-1, 1, (B, N, K)) * 0.25)
+    res = bf16_round(r.standard_normal((B, M, N)))
+    base = oracle.batch_matmul(a, np.ascontiguousarray(wt.transpose(0, 2, 1)), "mkn")
+    got = ops.batch_matmul(dev(a, torch.bfloat16), dev(wt, torch.bfloat16).transpose(1, 2),
+                           ops.Epilogue(residual=dev(res, torch.bfloat16)))
+    assert_close_bf16(host(got), bf16_round(base + res), "deep ring batch_matmul NT + residual")
+
+
 @pytest.mark.parametrize("B,M,N", [(8, 1024, 384), (2, 4096, 128), (1, 8192, 256), (32, 512, 512)])
 def test_batch_matmul_reduction_of_64_sweeps_the_columns(ops, oracle, B, M, N):
     """K = 64 with a row-major B goes to the kernel that keeps a 64-row panel of A in registers and sweeps B's
