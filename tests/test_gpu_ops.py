@@ -247,7 +247,9 @@ def test_elementwise_empty_and_errors(ops):
 
 
 # --------------------------------------------------------------------------- row kernels
-@pytest.mark.parametrize("shape", [(37, 129), (64, 128), (9, 512), (5, 4096), (3, 5000), (2, 20000), (4, 12, 64, 64), (1, 1)])
+# 768 and 1536 columns: the exact-fit tiles of three and six vectors per lane (16 lanes per row from 8192 rows on)
+@pytest.mark.parametrize("shape", [(37, 129), (64, 128), (9, 512), (5, 4096), (3, 5000), (2, 20000), (4, 12, 64, 64), (1, 1),
+                                   (9, 768), (8, 1536), (8200, 768)])
 def test_softmax(ops, oracle, shape):
     r = rng(8)
     x = (r.standard_normal(shape) * 3).astype(np.float32)
@@ -269,7 +271,7 @@ def test_softmax_masked_rows(ops, oracle):
     np.testing.assert_allclose(got.sum(-1), 1.0, rtol=1e-5)
 
 
-@pytest.mark.parametrize("shape", [(19, 96), (32, 768), (8, 1024), (5, 100), (2, 9000), (3, 7, 64)])
+@pytest.mark.parametrize("shape", [(19, 96), (32, 768), (8, 1024), (5, 100), (2, 9000), (3, 7, 64), (8, 1536), (8200, 768)])
 def test_layer_norm(ops, oracle, shape):
     r = rng(9)
     x = (r.standard_normal(shape) * 2 + 1).astype(np.float32)
@@ -285,7 +287,8 @@ def test_layer_norm(ops, oracle, shape):
 
 
 @pytest.mark.parametrize("shape,axes", [((3, 4, 5, 6), [3]), ((3, 4, 5, 6), [1, 2]), ((3, 4, 5, 6), [0]), ((3, 4, 5, 6), [2, 3]),
-                                        ((3, 4, 5, 6), [0, 1, 2, 3]), ((16, 4096), [1]), ((7, 300, 9), [1]), ((2, 3000), [-1])])
+                                        ((3, 4, 5, 6), [0, 1, 2, 3]), ((16, 4096), [1]), ((7, 300, 9), [1]), ((2, 3000), [-1]),
+                                        ((8, 1536), [1])])
 def test_reduce(ops, oracle, shape, axes):
     r = rng(10)
     x = r.standard_normal(shape).astype(np.float32)
@@ -298,6 +301,19 @@ def test_reduce(ops, oracle, shape, axes):
             np.testing.assert_array_equal(host(got), want)
     neg = -np.abs(x) - 1  # init is -inf, not 0 (LLHToHLO.cpp:81-133)
     assert host(ops.reduce("max", dev(neg), axes)).max() < 0
+
+
+def test_reduce_many_rows_of_768(ops, oracle):
+    """8192 rows and more of 768 elements: 16 lanes per row, six vectors each in bf16 (three on 64 lanes in fp32).
+    Sums of positive values, so that the comparison is not one of rounding order on sums that cancel."""
+    r = rng(12)
+    x = r.uniform(0.0, 1.0, (8200, 768)).astype(np.float32)
+    assert_close_f32(host(ops.reduce("sum", dev(x), [1])), oracle.reduce("sum", x, [1]), "reduce_sum (8200, 768)")
+    for kind in ["max", "min"]:
+        np.testing.assert_array_equal(host(ops.reduce(kind, dev(x), [1])), oracle.reduce(kind, x, [1]))
+    xb = bf16_round(x)
+    np.testing.assert_array_equal(host(ops.reduce("max", dev(xb, torch.bfloat16), [1])), oracle.reduce("max", xb, [1]))
+    assert_close_bf16(host(ops.reduce("sum", dev(xb, torch.bfloat16), [1])), bf16_round(oracle.reduce("sum", xb, [1])), "reduce_sum bf16 (8200, 768)")
 
 
 @pytest.mark.parametrize("seed", range(3))
