@@ -451,7 +451,7 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
   // smallest register tile that holds a row; among equal capacities prefer 4 then 2 vectors per
   // lane (enough loads in flight per lane, rows spread over many lanes), then 3 and 6 (rows of 3 x 2^n
   // elements, a transformer's 768, fit them exactly: no masked lanes), then 8, then 1
-  const int tprs[3] = {16, 64, 256};
+  const int tprs[4] = {16, 32, 64, 256};
   const int items[6] = {4, 2, 3, 6, 8, 1};
   int best_t = 0, best_i = 0;
   int64_t best_cap = -1;
@@ -460,6 +460,7 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
       // six vectors on each of 16 lanes: few lanes per row, worth it only with rows enough to fill the chip anyway
       // (768 bf16 elements: 16384 rows 14.6 -> 13.3 us, 4096 rows 5.3 -> 5.6 us, 512 rows 3.8 -> 4.9 us)
       if (i == 6 && t == 16 && p.rows < 8192) continue;
+      if (t == 32 && i != 3) continue;  // 32 lanes: only as the exact fit of 768 16-bit elements
       int64_t cap = (int64_t)t * i * VEC;
       if (cap >= p.cols && (best_cap < 0 || cap < best_cap)) {
         best_cap = cap;
@@ -469,6 +470,7 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
     }
   if (best_cap < 0) return false;
   if (best_t == 16) launch_items<OP, VEC, 16>(p, best_i, s);
+  else if (best_t == 32) launch_items<OP, VEC, 32>(p, 3, s);
   else if (best_t == 64) launch_items<OP, VEC, 64>(p, best_i, s);
   else launch_items<OP, VEC, 256>(p, best_i, s);
   return true;
