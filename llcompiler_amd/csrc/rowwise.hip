@@ -460,7 +460,7 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
       // six vectors on each of 16 lanes: few lanes per row, worth it only with rows enough to fill the chip anyway
       // (768 bf16 elements: 16384 rows 14.6 -> 13.3 us, 4096 rows 5.3 -> 5.6 us, 512 rows 3.8 -> 4.9 us)
       if (i == 6 && t == 16 && p.rows < 8192) continue;
-      if (t == 32 && i != 3) continue;  // 32 lanes: only as the exact fit of 768 16-bit elements
+      if (t == 32 && i != 3 && i != 4) continue;  // 32 lanes: measured with three and four vectors only
       int64_t cap = (int64_t)t * i * VEC;
       if (cap >= p.cols && (best_cap < 0 || cap < best_cap)) {
         best_cap = cap;
@@ -470,7 +470,7 @@ bool launch_tpr(const RowParams& p, hipStream_t s) {
     }
   if (best_cap < 0) return false;
   if (best_t == 16) launch_items<OP, VEC, 16>(p, best_i, s);
-  else if (best_t == 32) launch_items<OP, VEC, 32>(p, 3, s);
+  else if (best_t == 32) launch_items<OP, VEC, 32>(p, best_i, s);
   else if (best_t == 64) launch_items<OP, VEC, 64>(p, best_i, s);
   else launch_items<OP, VEC, 256>(p, best_i, s);
   return true;
