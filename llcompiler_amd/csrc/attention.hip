@@ -267,6 +267,223 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   }
 }
 
+// ---- few workgroups (one sequence, a dozen heads): the keys split over the waves ----
+// With 128 queries per workgroup a batch of one leaves most CUs idle and every wave walks all the keys of its 32
+// queries, one block after the other.  Here a workgroup has 32 queries and its four waves take every fourth key block
+// each (a K / V stage of its own per wave: no barrier inside the walk), so the chain is a quarter as long and there
+// are four times the workgroups; the four partial results (running shift, row sum, O^T) meet in LDS at the end and
+// are combined like the blocks of one wave are: scaled by exp2(shift - largest shift), summed, divided by the sum.
+constexpr int kSplitLds = 8 * kTileBytes + 4 * kBlockKV * 4;
+template <typename T, bool ADD>
+__global__ __launch_bounds__(256) void attention_split_kernel(const AttnParams p) {
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  char* kt = smem + wave * kTileBytes;
+  char* vt = smem + (4 + wave) * kTileBytes;
+  float* addrow = (float*)(smem + 8 * kTileBytes) + wave * kBlockKV;
+  const int li = lane % 32, lh = lane / 32;
+  const int bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
+  const int q0 = blockIdx.x * 32;
+  const T* Q = (const T*)p.Q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const T* K = (const T*)p.K + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+  const T* V = (const T*)p.V + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+  const T* M = p.mask ? (const T*)p.mask + (int64_t)b * p.m_sb : nullptr;
+
+  u32x4_t qf[4];
+  {
+    const int qrow = q0 + li < p.Sq ? q0 + li : p.Sq - 1;
+    const T* qp = Q + (int64_t)qrow * p.q_ss + lh * 8;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const u32x4_t*)(qp + ks * 16);
+  }
+  // block loader: 512 16-byte chunks of K and of V by the 64 lanes of this wave
+  const int lc = lane % 8;
+  int koff[8], voff[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = lane / 8 + 8 * j;
+    koff[j] = row * 128 + ((lc ^ lds_swz(row)) << 4);
+    voff[j] = row * 128 + ((lc ^ ((row & 3) << 1)) << 4);
+  }
+  u32x4_t kr[8], vr[8];
+  float ar = 0.0f;
+  auto gload = [&](int blk) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      int row = blk * kBlockKV + lane / 8 + 8 * j;
+      row = row < p.Skv ? row : p.Skv - 1;
+      kr[j] = *(const u32x4_t*)(K + (int64_t)row * p.k_ss + lc * 8);
+      vr[j] = *(const u32x4_t*)(V + (int64_t)row * p.v_ss + lc * 8);
+    }
+    if constexpr (ADD) {
+      const int key = blk * kBlockKV + lane;
+      const int kc = key < p.Skv ? key : p.Skv - 1;
+      float mv = 0.0f;
+      if (M) mv = mask_log2(load_as_f32((const char*)M, Elem<T>::kDtype, kc));
+      ar = key < p.Skv ? mv : -INFINITY;
+    }
+  };
+  auto lstore = [&]() {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      *(u32x4_t*)(kt + koff[j]) = kr[j];
+      *(u32x4_t*)(vt + voff[j]) = vr[j];
+    }
+    if constexpr (ADD) addrow[lane] = ar;
+  };
+  int ka[2][4];
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int row = 32 * t2 + li;
+      ka[t2][ks] = row * 128 + (((2 * ks + lh) ^ lds_swz(row)) << 4);
+    }
+  int va[2][2];
+  {
+    const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int row = 8 * u + 4 * (g >> 1) + jj;
+        const int c = 4 * dt + 2 * (g & 1) + (q >> 1);
+        va[dt][u] = row * 128 + ((c ^ (jj << 1)) << 4) + (q & 1) * 8;
+      }
+  }
+
+  f32x16_t oacc[2];
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const int nblk = (p.Skv + kBlockKV - 1) / kBlockKV;
+  if (wave < nblk) gload(wave);
+  for (int blk = wave; blk < nblk; blk += 4) {
+    // the stage is this wave's own: its previous reads are done when these writes are issued (LDS works in order)
+    lstore();
+    if (blk + 4 < nblk) gload(blk + 4);
+    f32x16_t sacc[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[t2][r] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) mfma_step<T>(*(const u32x4_t*)(kt + ka[t2][ks]), qf[ks], sacc[t2]);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (ADD) {
+          const f32x4_t av = *(const f32x4_t*)&addrow[32 * t2 + 8 * i + 4 * lh];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sacc[t2][4 * i + j] = fmaf(sacc[t2][4 * i + j], p.scale_log2e, av[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mx = fmaxf(mx, sacc[t2][4 * i + j]);
+      }
+    if constexpr (!ADD) mx *= p.scale_log2e;
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    float m_use = m_run == -INFINITY ? 0.0f : m_run;
+    if (__any(mx > m_run + 8.0f)) {
+      const float m_max = fmaxf(m_run, mx);
+      m_use = m_max == -INFINITY ? 0.0f : m_max;
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
+      m_run = m_max;
+      l_run *= corr;
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    }
+    const float m_new = m_use;
+    float psum = 0.0f;
+    u32x4_t pb[2][2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float pv[2];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            const float x = sacc[t2][8 * t + 2 * e + w];
+            pv[w] = ADD ? __builtin_amdgcn_exp2f(x - m_new) : __builtin_amdgcn_exp2f(fmaf(x, p.scale_log2e, -m_new));
+            psum += pv[w];
+          }
+          pb[t2][t][e] = pack2<T>(pv[0], pv[1]);
+        }
+    l_run += psum;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const char* vrow = vt + (32 * t2 + 16 * t) * 128;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          const uint2 lo = lds_tr16(vrow + va[dt][0]), hi = lds_tr16(vrow + va[dt][1]);
+          mfma_step<T>(u32x4_t{lo.x, lo.y, hi.x, hi.y}, pb[t2][t], oacc[dt]);
+        }
+      }
+  }
+
+  // ---- the four partial results meet: xo[wave][register][lane] over the K / V stages, shift and row sum beside ----
+  const float l_part = l_run + __shfl_xor(l_run, 32, kWave);
+  __syncthreads();  // every wave has left its stages
+  float* xo = (float*)smem;                            // [4][32][64]
+  float* xm = (float*)(smem + 8 * kTileBytes);         // [4][32] shifts, then [4][32] sums
+#pragma unroll
+  for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) xo[((wave * 32) + dt * 16 + r) * 64 + lane] = oacc[dt][r];
+  if (lh == 0) {
+    xm[wave * 32 + li] = m_run;
+    xm[128 + wave * 32 + li] = l_part;
+  }
+  __syncthreads();
+  float mw[4], sc[4];
+  float m_ref = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    mw[w] = xm[w * 32 + li];
+    m_ref = fmaxf(m_ref, mw[w]);
+  }
+  float l_tot = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    // a wave that saw no key, or only keys masked with -inf, holds zeros against a shift of 0: it adds nothing
+    sc[w] = mw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - m_ref);
+    l_tot += xm[128 + w * 32 + li] * sc[w];
+  }
+  const float inv = 1.0f / l_tot;
+  if (q0 + li < p.Sq) {
+    // this wave writes registers 8 wave .. 8 wave + 7 of the O^T layout: d tile wave / 2, i = 2 (wave % 2) + {0, 1}
+    T* op = (T*)p.O + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)(q0 + li) * p.o_ss;
+    const int dt = wave >> 1;
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const int i = 2 * (wave & 1) + ii;
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc += xo[((w * 32) + dt * 16 + 4 * i + j) * 64 + lane] * sc[w];
+        o[j] = acc * inv;
+      }
+      uint2 wv;
+      wv.x = pack2<T>(o[0], o[1]);
+      wv.y = pack2<T>(o[2], o[3]);
+      *(uint2*)(op + 32 * dt + 8 * i + 4 * lh) = wv;
+    }
+  }
+}
+
 // ---- fp32 operands: v_mfma_f32_32x32x2_f32 takes one k per lane and instruction ----
 // Same plan as above with these differences.  K block [64 keys][256 B] and V block [64 keys][256 B] come straight
 // into LDS (global_load_lds: no staging registers; lane L of a wave load lands at byte 16 L of its 1 KB, so it
@@ -496,8 +713,22 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
     if (four) return p.mask ? launch_f32<4, true>(p, s) : launch_f32<4, false>(p, s);
     return p.mask ? launch_f32<2, true>(p, s) : launch_f32<2, false>(p, s);
   }
-  const dim3 grid((unsigned)((p.Sq + kBlockQ - 1) / kBlockQ), (unsigned)(p.B * p.H));
   const bool add = p.mask || p.Skv % kBlockKV != 0;
+  if ((int64_t)((p.Sq + kBlockQ - 1) / kBlockQ) * p.B * p.H < 128 && p.Skv > 3 * kBlockKV) {
+    // fewer workgroups of 128 queries than half the CUs, and keys enough for every wave: 32 queries per workgroup,
+    // the key blocks dealt to its four waves (12 heads, 512 x 512: one sequence 10.7 -> 6.6 us, two 10.9 -> 9.4 us;
+    // four sequences, 192 workgroups of 128 queries, are faster as they were: 11.4 against 16.6 us)
+    const dim3 g32((unsigned)((p.Sq + 31) / 32), (unsigned)(p.B * p.H));
+    auto go = [&](auto kern) {
+      static std::atomic<uint32_t> lds_allowed{0};
+      LLC_TRY(allow_dynamic_lds((const void*)kern, kSplitLds, lds_allowed));
+      hipLaunchKernelGGL(kern, g32, dim3(256), kSplitLds, s, p);
+      return check_launch("attention_split_kernel");
+    };
+    if (a.dtype == LLC_BFLOAT16) return add ? go(attention_split_kernel<__bf16, true>) : go(attention_split_kernel<__bf16, false>);
+    return add ? go(attention_split_kernel<_Float16, true>) : go(attention_split_kernel<_Float16, false>);
+  }
+  const dim3 grid((unsigned)((p.Sq + kBlockQ - 1) / kBlockQ), (unsigned)(p.B * p.H));
   if (a.dtype == LLC_BFLOAT16) {
     if (add) hipLaunchKernelGGL((attention_kernel<__bf16, true>), grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL((attention_kernel<__bf16, false>), grid, dim3(256), 0, s, p);

@@ -756,6 +756,31 @@ def test_random_bmm_attention_pool_gather_cases(ops, oracle, seed):
         np.testing.assert_array_equal(host(ops.gather_rows(dev(tb, torch.bfloat16), dev(idx))), oracle.gather_rows(tb, idx))
 
 
+@pytest.mark.parametrize("B,H,Sq,Skv", [(1, 12, 512, 512), (1, 3, 40, 257), (2, 2, 96, 320)])
+def test_attention_few_workgroups_keys_split_over_the_waves(ops, oracle, B, H, Sq, Skv):
+    """A sequence or two with a few heads: 32 queries per workgroup, every fourth key block to each of its waves, the
+    four partial results combined at the end.  An encoder block's shape at a batch of one; key counts that leave the
+    waves with two, one and one blocks (the last block one key long); a whole block of one wave masked with -inf
+    (that wave's partial result then carries no weight) and a finite padding tail."""
+    r = rng(B + 7 * H + Sq + Skv)
+    q = bf16_round(r.uniform(-1, 1, (B, H, Sq, 64)))
+    k = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+    v = bf16_round(r.uniform(-1, 1, (B, H, Skv, 64)))
+    for dt, rnd in ((torch.bfloat16, bf16_round), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+        want = _attention_oracle(oracle, q, k, v, None, 0.125, rnd)
+        got = ops.attention(dev(q, dt), dev(k, dt), dev(v, dt), None, 0.125)
+        assert_close_bf16(host(got), want, "split attention %s %s" % (dt, (B, H, Sq, Skv)))
+    mask = np.zeros((B, Skv), np.float32)
+    mask[:, 64:128] = -np.inf              # the second wave's first block
+    mask[0, Skv - Skv // 5:] = -1e4        # a padding tail
+    keep = np.ones(Skv, bool)
+    keep[64:128] = False
+    tail = bf16_round(mask[:, keep])
+    want = _attention_oracle(oracle, q, k[:, :, keep], v[:, :, keep], tail, 0.125, bf16_round)
+    got = ops.attention(dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(v, torch.bfloat16), dev(mask, torch.bfloat16), 0.125)
+    assert_close_bf16(host(got), want, "split attention, one block at -inf %s" % ((B, H, Sq, Skv),))
+
+
 def test_attention_fully_masked_leading_block_and_errors(ops, oracle):
     # -inf on the whole first block of keys: the running maximum stays -inf there and must not turn into NaN
     r = rng(5)
