@@ -126,6 +126,20 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
 
+// two fp32 values rounded to the 16-bit storage type `dtype` (LLC_BFLOAT16 or LLC_FLOAT16), `lo` in the low half of the
+// word: one v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 (round to nearest even) instead of two conversions, a shift and an or
+template <int DTYPE>
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  if constexpr (DTYPE == LLC_BFLOAT16) {
+    typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{lo, hi}, bf2_t));
+  } else {
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{lo, hi}, h2_t));
+  }
+}
+
 // erf-based GELU, 0.5 x (1 + erf(x / sqrt 2)).  erf comes from the rational approximation 7.1.26 of
 // Abramowitz & Stegun (absolute error below 1.5e-7) on the hardware reciprocal and exp2: the result stays
 // within 5e-7 of the exactly rounded one over the whole range, a fortieth of the fp32 tolerance, at a third

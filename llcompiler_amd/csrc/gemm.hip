@@ -412,7 +412,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
     if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
-    u32x4_t outv;
+    float xs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const uint16_t bb = (uint16_t)(bq[e / 2] >> (16 * (e & 1))), rb = (uint16_t)(rq[e / 2] >> (16 * (e & 1)));
@@ -422,11 +422,10 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
       if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
       if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
       else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
-      const uint32_t bits = (Elem<T>::kDtype == LLC_BFLOAT16) ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
-      if (e & 1) outv[e / 2] |= bits << 16;
-      else outv[e / 2] = bits;
+      xs[e] = x;
     }
-    *(u32x4_t*)(C + o) = outv;
+    *(u32x4_t*)(C + o) = u32x4_t{pack_pair<Elem<T>::kDtype>(xs[0], xs[1]), pack_pair<Elem<T>::kDtype>(xs[2], xs[3]),
+                                pack_pair<Elem<T>::kDtype>(xs[4], xs[5]), pack_pair<Elem<T>::kDtype>(xs[6], xs[7])};
   }
 }
 
@@ -600,7 +599,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
     if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
     if (res) rq = *(const u32x4_t*)(res + o);
-    u32x4_t outv;
+    float xs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const uint16_t bb = (uint16_t)(bq[e / 2] >> (16 * (e & 1))), rb = (uint16_t)(rq[e / 2] >> (16 * (e & 1)));
@@ -610,11 +609,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
       if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
       else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
-      const uint32_t bits = (Elem<T>::kDtype == LLC_BFLOAT16) ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
-      if (e & 1) outv[e / 2] |= bits << 16;
-      else outv[e / 2] = bits;
+      xs[e] = x;
     }
-    *(u32x4_t*)(C + o) = outv;
+    *(u32x4_t*)(C + o) = u32x4_t{pack_pair<Elem<T>::kDtype>(xs[0], xs[1]), pack_pair<Elem<T>::kDtype>(xs[2], xs[3]),
+                                pack_pair<Elem<T>::kDtype>(xs[4], xs[5]), pack_pair<Elem<T>::kDtype>(xs[6], xs[7])};
   }
 }
 

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             const int rrow = (CONV && mrow0 + row >= p.M) ? p.M - 1 : mrow0 + row;
             rq = *(const uint2*)(res + (int64_t)rrow * p.c_sm + ncol0 + col);
           }
-          uint32_t o[2];
+          float xv[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const uint32_t bw = e < 2 ? bq.x : bq.y, rw = e < 2 ? rq.x : rq.y;
@@ -359,11 +359,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if constexpr (RES) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
             if constexpr (ACT == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
             else if constexpr (ACT == LLC_ACT_GELU) x = gelu_exact(x);
-            const uint32_t bits = (Elem<T>::kDtype == LLC_BFLOAT16) ? f32_to_bf16_bits(x) : f32_to_f16_bits(x);
-            if (e & 1) o[e / 2] |= bits << 16;
-            else o[e / 2] = bits;
+            xv[e] = x;
           }
-          *(uint2*)(wst + row * G::kOutPitch + col * 2) = uint2{o[0], o[1]};
+          *(uint2*)(wst + row * G::kOutPitch + col * 2) =
+              uint2{pack_pair<Elem<T>::kDtype>(xv[0], xv[1]), pack_pair<Elem<T>::kDtype>(xv[2], xv[3])};
         }
       }
   };
