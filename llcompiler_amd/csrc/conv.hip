@@ -818,10 +818,16 @@ int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   constexpr int EPV = 16 / sizeof(T);
   const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
   if constexpr (sizeof(T) == 4) {
-    if (conv_rows_ok(p, groups)) return launch_conv_rows(p, s);
+    if (conv_rows_ok(p, groups)) return launch_conv_rows<float>(p, s);
     if (w_vec && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
         ((uintptr_t)p.X % 4) == 0 && (int64_t)p.N * p.C * p.H * p.Wd < ((int64_t)1 << 30))  // 32-bit byte offsets
       return launch_f32(p, groups, s);
+  }
+  if constexpr (sizeof(T) == 2) {
+    // an image network's first layer in 16-bit storage: the fp32 row kernel on widened copies
+    if (conv_rows_ok(p, groups) && ((uintptr_t)p.W % 16) == 0 && (int64_t)p.N * p.C * p.H * p.Wd % 8 == 0 &&
+        (!p.bias || ((uintptr_t)p.bias % 2) == 0))
+      return launch_conv_rows_16bit<T>(p, s);
   }
   if (w_vec) return launch_tiles<T, kLoadKVec>(p, groups, s);
   return launch_tiles<T, kLoadGeneric>(p, groups, s);

@@ -12,6 +12,10 @@
 // 16 filters and keeps their weights in 37 registers for the whole kernel; accumulators of a lane are 4 consecutive
 // pixels of one filter, stored as 16 bytes into NCHW.
 //
+// 16-bit tensors take the same kernel (TO = their type): the image and the filters are first copied to fp32 in scratch
+// memory (the image is 3 % of the layer's bytes), the products are the same fp32 ones the 16-bit matrix instruction
+// would form, and the result is rounded once on its way out; the gather kernel this replaces takes twice as long.
+//
 // LDS reads are inline asm with hand-placed waits: with direct-to-LDS loads in flight the compiler would put
 // s_waitcnt vmcnt(0) in front of every LDS read it knows about.
 
@@ -37,6 +41,7 @@ __device__ __forceinline__ void rows_static_for(F&& f) {
   }
 }
 
+template <typename TO>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_rows_f32_kernel(const ConvParams p) {
   extern __shared__ __align__(16) char smem[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -61,7 +66,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // pixel i of block 0 reads column 2 i + kw - pw of row (c, kh); a k past the reduction reads row 0 (times weight 0)
     kaddr[s] = lds0 + kRowsLead + (uint32_t)((c * p.KH + kh) * kRowsPitch) + (uint32_t)((2 * li + kw - p.pw) * 4);
   }
-  const float bias = p.bias ? ((const float*)p.bias)[f] : 0.0f;
+  const float bias = p.bias ? load_as_f32(p.bias, Elem<TO>::kDtype, f) : 0.0f;
   // the lead-in of both buffers and whatever the loads never write stays zero
   for (int i = threadIdx.x; i < kRowsLds / 4; i += 256) ((uint32_t*)smem)[i] = 0u;
   __builtin_amdgcn_s_waitcnt(0);  // weights and bias are here, the zeros are written
@@ -138,7 +143,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __builtin_amdgcn_sched_barrier(0);
     // ---- act(alpha acc + bias) -> y[n][f][oh][16 pb + 4 kk .. + 3] ----
     const int n = r / p.OH, oh = r - n * p.OH;
-    float* yrow = (float*)p.Y + (((int64_t)n * p.F + f) * p.OH + oh) * p.OW;
+    TO* yrow = (TO*)p.Y + (((int64_t)n * p.F + f) * p.OH + oh) * p.OW;
 #pragma unroll
     for (int b = 0; b < kRowsBlocks; ++b) {
       const int ow = 16 * b + 4 * kk;
@@ -150,12 +155,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
         o[e] = v;
       }
-      if (ow < p.OW) *(f32x4_t*)(yrow + ow) = o;
+      if (ow < p.OW) {
+        if constexpr (sizeof(TO) == 4) *(f32x4_t*)(yrow + ow) = o;
+        else *(uint2*)(yrow + ow) = uint2{pack_pair<Elem<TO>::kDtype>(o[0], o[1]), pack_pair<Elem<TO>::kDtype>(o[2], o[3])};
+      }
     }
   }
 }
 
-// Whether the row kernel takes this convolution (NCHW fp32, checked by the caller).
+// Whether the row kernel takes this convolution (NCHW, contiguous, checked by the caller).
 inline bool conv_rows_ok(const ConvParams& p, int groups) {
   if (groups != 1 || p.F != 64 || p.Kdim > 4 * kRowsSteps || p.C * p.KH > kRowsMaxRows || p.residual) return false;
   if (p.sw != 2 || p.dh != 1 || p.dw != 1) return false;
@@ -166,11 +174,55 @@ inline bool conv_rows_ok(const ConvParams& p, int groups) {
   return (int64_t)p.N * p.OH >= 256;  // rows enough for every CU
 }
 
-inline int launch_conv_rows(const ConvParams& p, hipStream_t s) {
+template <typename TO>
+int launch_conv_rows(const ConvParams& p, hipStream_t s) {
+  auto kern = conv_rows_f32_kernel<TO>;
   static std::atomic<uint32_t> lds_allowed{0};
-  LLC_TRY(allow_dynamic_lds((const void*)conv_rows_f32_kernel, kRowsLds, lds_allowed));
+  LLC_TRY(allow_dynamic_lds((const void*)kern, kRowsLds, lds_allowed));
   const int64_t total = (int64_t)p.N * p.OH;
   const unsigned wgs = (unsigned)(total < 512 ? total : 512);  // two workgroups per CU, each walking rows wgs apart
-  hipLaunchKernelGGL(conv_rows_f32_kernel, dim3(wgs), dim3(256), kRowsLds, s, p);
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), kRowsLds, s, p);
   return check_launch("conv_rows_f32_kernel");
+}
+
+// 16-bit values to fp32, 8 per lane
+template <typename T>
+__global__ __launch_bounds__(256) void widen_to_f32_kernel(const T* __restrict__ in, float* __restrict__ out, int64_t n) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i + 8 <= n) {
+    const u32x4_t v = *(const u32x4_t*)(in + i);
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) {
+        f[2 * e] = __uint_as_float(v[e] << 16);
+        f[2 * e + 1] = __uint_as_float(v[e] & 0xffff0000u);
+      } else {
+        f[2 * e] = f16_bits_to_f32((uint16_t)(v[e] & 0xffffu));
+        f[2 * e + 1] = f16_bits_to_f32((uint16_t)(v[e] >> 16));
+      }
+    }
+    *(f32x4_t*)(out + i) = f32x4_t{f[0], f[1], f[2], f[3]};
+    *(f32x4_t*)(out + i + 4) = f32x4_t{f[4], f[5], f[6], f[7]};
+  } else {
+    for (int64_t j = i; j < n; ++j) out[j] = load_as_f32((const char*)in, Elem<T>::kDtype, j);
+  }
+}
+
+// The 16-bit form: fp32 copies of the image and the filters in scratch memory, then the row kernel with a 16-bit result.
+template <typename T>
+int launch_conv_rows_16bit(const ConvParams& p, hipStream_t s) {
+  const int64_t nx = (int64_t)p.N * p.C * p.H * p.Wd, nw = (int64_t)p.F * p.Kdim;
+  const size_t xbytes = ((size_t)nx * 4 + 255) / 256 * 256;
+  void* ws = nullptr;
+  LLC_TRY(get_workspace(xbytes + (size_t)nw * 4, &ws, s));
+  float* x32 = (float*)ws;
+  float* w32 = (float*)((char*)ws + xbytes);
+  hipLaunchKernelGGL(widen_to_f32_kernel<T>, dim3((unsigned)((nx + 2047) / 2048)), dim3(256), 0, s, (const T*)p.X, x32, nx);
+  hipLaunchKernelGGL(widen_to_f32_kernel<T>, dim3((unsigned)((nw + 2047) / 2048)), dim3(256), 0, s, (const T*)p.W, w32, nw);
+  LLC_TRY(check_launch("widen_to_f32_kernel"));
+  ConvParams q = p;
+  q.X = (const char*)x32;
+  q.W = (const char*)w32;
+  return launch_conv_rows<T>(q, s);
 }

@@ -1126,6 +1126,14 @@ def test_conv2d_first_layer_row_kernel(ops, oracle, case):
     assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s, epilogue=epi)), want2, "first-layer conv + bias + relu")
     want3 = oracle.conv2d(x, w, None, pad=pad, stride=s) * np.float32(0.25)
     assert_close_f32(host(ops.conv2d(dev(x), dev(w), pad=pad, stride=s, epilogue=ops.Epilogue(alpha=0.25))), want3, "alpha")
+    # 16-bit storage: the same kernel on fp32 copies of the image and the filters, the result rounded on its way out
+    xb, wb, bb = bf16_round(x), bf16_round(w), bf16_round(b)
+    want16 = oracle.unary("relu", oracle.conv2d(xb, wb, bb, pad=pad, stride=s))
+    for dt, rnd, close in ((torch.bfloat16, bf16_round, assert_close_bf16), (torch.float16, f16_round, assert_close_f16)):
+        epi = ops.Epilogue(bias=dev(bb, dt), act="relu")
+        got = ops.conv2d(dev(xb, dt), dev(wb, dt), pad=pad, stride=s, epilogue=epi)
+        assert got.dtype == dt
+        close(host(got), rnd(want16), "first-layer conv + bias + relu %s %s" % (dt, case))
 
 
 WIDE_CONV_CASES = [
