@@ -759,6 +759,9 @@ int launch_nhwc_cfg(const ConvParams& p0, hipStream_t s) {
   return LLC_OK;
 }
 
+#include "conv_rows.hpp"
+#include "conv_patch.hpp"
+
 template <typename T>
 int launch_nhwc(const ConvParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
@@ -774,6 +777,8 @@ int launch_nhwc(const ConvParams& p, hipStream_t s) {
     const int st = conv_wide_16bit(Elem<T>::kDtype, p.X, p.W, p.Y, p.bias, p.residual, p.F, g, p.alpha, p.act, s);
     if (st != 1) return st;
   }
+  // stride-1 windows over images small enough for an LDS patch: the input is read once, not once per tap
+  if (conv_patch_ok<T>(p)) return launch_conv_patch<T>(p, s);
   // 128-pixel tiles when they fill the chip by themselves; else 64 x 64 tiles if those are numerous enough to need
   // no split of the reduction (a split costs a pass over the partial sums: the middle layers of a ResNet); the
   // last layers split either way and do better on the large tiles, unless their reduction is too short to split
@@ -810,8 +815,6 @@ int launch_tiles(const ConvParams& p, int groups, hipStream_t s) {
   if ((int64_t)((p.ncols + 127) / 128) * groups >= 128) return launch_cfg<T, 64, 128, LA>(p, groups, s);
   return launch_cfg<T, 64, 64, LA>(p, groups, s);
 }
-
-#include "conv_rows.hpp"
 
 template <typename T>
 int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {

@@ -1136,6 +1136,39 @@ def test_conv2d_first_layer_row_kernel(ops, oracle, case):
         close(host(got), rnd(want16), "first-layer conv + bias + relu %s %s" % (dt, case))
 
 
+PATCH_CONV_CASES = [
+    # N, H, W, F, KH, KW, pad(h_lo, w_lo, h_hi, w_hi): 64 channels in 16-bit storage, stride 1, at least 192 tiles
+    (16, 56, 56, 64, 3, 3, (1, 1, 1, 1)),     # a ResNet's first stage: 24 whole tiles and one of 64 pixels per image
+    (9, 30, 50, 128, 3, 3, (1, 1, 1, 1)),     # 1500 pixels per image (the last tile has 92), two filter tiles
+    (20, 33, 41, 64, 3, 2, (0, 1, 2, 0)),     # 3 x 2 window, no padding above, two rows below, none on the right
+    (12, 48, 48, 64, 5, 5, (2, 2, 2, 2)),     # 5 x 5 window: 25 taps, a patch of 7 rows of 52 pixels
+]
+
+
+@pytest.mark.parametrize("case", PATCH_CONV_CASES)
+def test_conv2d_channels_last_16bit_input_patch_in_lds(ops, oracle, case):
+    """Stride-1 windows over 64 channels in 16-bit storage: the kernel that parks the input patch of 128 output pixels
+    in LDS once and reads every tap from it at a shifted address (zeros around the image come from a row of zeros);
+    bf16 and f16, with and without bias + residual + relu."""
+    N, H, W, F, KH, KW, pad = case
+    r = rng(N + H + W + F + KH)
+    x = bf16_round(r.standard_normal((N, 64, H, W)))
+    w = bf16_round(r.standard_normal((F, 64, KH, KW)) / np.sqrt(64 * KH * KW))
+    b = bf16_round(r.standard_normal(F))
+    base = oracle.conv2d(x, w, None, pad=pad)
+    res = bf16_round(r.standard_normal(base.shape))
+    assert base.shape[0] * ((base.shape[2] * base.shape[3] + 127) // 128) * (F // 64) >= 192
+    cl = torch.channels_last
+    for dt, rnd, close in ((torch.bfloat16, bf16_round, assert_close_bf16), (torch.float16, f16_round, assert_close_f16)):
+        dx, dw = dev(x, dt).contiguous(memory_format=cl), dev(w, dt).contiguous(memory_format=cl)
+        o = torch.empty(base.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        close(host(ops.conv2d(dx, dw, pad=pad, out=o)), rnd(base), "patch conv %s %s" % (dt, case))
+        want = oracle.unary("relu", oracle.conv2d(x, w, b, pad=pad) + res)
+        epi = ops.Epilogue(bias=dev(b, dt), residual=dev(res, dt).contiguous(memory_format=cl), act="relu")
+        o2 = torch.empty(base.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        close(host(ops.conv2d(dx, dw, pad=pad, epilogue=epi, out=o2)), rnd(want), "patch conv+bias+res+relu %s %s" % (dt, case))
+
+
 WIDE_CONV_CASES = [
     # N, C, H, W, F, KH, KW, pad, stride, dil: reductions of 2048 and more, at least 192 tiles of 256 pixels x 128 (256) filters
     (17, 256, 54, 54, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 49572 pixels: the last tile has 164 rows
