@@ -17,11 +17,13 @@
  *  - kernels that split a reduction (convolutions with few output tiles, matmuls with a long K) keep partial
  *    sums in scratch device memory.  A plan owns its scratch memory (sized while it is recorded, allocated by
  *    llc_plan_end / llc_plan_load), so llc_hip_run allocates nothing and plans replayed on different streams do
- *    not share any.  An op entry point called outside a plan uses one buffer per device that grows on demand,
- *    which is the only allocation an op entry point ever makes (the old buffer is kept, nothing is synchronised;
- *    refused with LLC_ERR_UNSUPPORTED while the stream is being captured): such calls may follow each other on
- *    one stream, but issuing them on several streams of one device at the same time lets them overwrite each
- *    other's partial sums.  llc_hip_matmul_static never allocates (see there).
+ *    not share any.  An op entry point called outside a plan uses a buffer per (device, stream) that grows on
+ *    demand, which is the only allocation an op entry point ever makes (nothing is synchronised; an outgrown
+ *    buffer is kept until llc_hip_trim, since queued launches may still address it; growing is refused with
+ *    LLC_ERR_UNSUPPORTED while the stream is being captured).  Calls on one stream follow each other, calls on
+ *    different streams use different buffers: op entry points are re-entrant per stream, like plans.  Two host
+ *    threads must not issue work to the SAME stream at the same time.  llc_hip_matmul_static never allocates
+ *    (see there).
  *  - every entry returns an llc_status (0 = ok, negative = error) and leaves a message for
  *    llc_hip_last_error() (thread local).  The reference only logs on failure
  *    (include/llcompiler/Support/Logger.h:132-134); returning a status is a deliberate tightening.
@@ -84,6 +86,13 @@ int llc_hip_abi_version(void);
 int llc_hip_init(int device);
 const char* llc_hip_last_error(void);
 const char* llc_hip_status_string(int status);
+/* Scratch memory the op entry points hold on `device` outside plans: in use (one buffer per stream that needed
+ * one) and retired (outgrown, not yet freed).  Either pointer may be NULL. */
+int llc_hip_scratch_bytes(int device, size_t* live_bytes, size_t* retired_bytes);
+/* Waits for the current device to finish everything queued, then frees the retired scratch buffers and, with
+ * release_live != 0, the live ones too (the next call that needs one allocates again).  For a host that wants
+ * the memory back after a one-off large product; never called by the library itself. */
+int llc_hip_trim(int release_live);
 
 /* ---- fused epilogue of the contractions.  The reference's pipeline fuses the elementwise
  * consumers of a linalg op into it (linalg-fuse-elementwise-ops,
@@ -106,7 +115,7 @@ typedef struct llc_epilogue {
  * transposed view (stride[0] == 1), which is how llh.transpose{perms=[1,0]} of a weight
  * (llcompiler/importer/fx_op_translate/transpose.py:39-48) is consumed without a copy.
  * `epi` may be NULL.  Products with a long reduction and few output tiles sum the reduction in
- * chunks through the library's per-device scratch buffer (grown on demand by this call); the order
+ * chunks through the library's scratch buffer of this stream (grown on demand by this call); the order
  * of the sum is fixed, so results are the same bits on every run. */
 int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                    void* stream);
@@ -115,10 +124,10 @@ int llc_hip_matmul(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilo
  * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels
  * and the same bits as llc_hip_matmul; the partial sums of a split reduction go to a 32 MiB array that is part of
  * the library's code object (each GPU the library runs on holds it until the process ends) instead of the
- * per-device buffer that llc_hip_matmul grows on demand.  The call never allocates or frees; a product whose
+ * per-stream buffer that llc_hip_matmul grows on demand.  The call never allocates or frees; a product whose
  * partial sums need more than 32 MiB is refused with LLC_ERR_TOO_LARGE (use llc_hip_matmul or a plan).  Every call
  * on a GPU shares that GPU's array (nothing in it has to start at zero: partial sums are written before they are
- * read): calls that overlap on different streams of one GPU race, like llc_hip_matmul's.  The call is not recorded
+ * read): calls that overlap on different streams of one GPU race (llc_hip_matmul's do not).  The call is not recorded
  * into a plan (a plan owns its scratch memory anyway). */
 int llc_hip_matmul_static(const llc_tensor* lhs, const llc_tensor* rhs, const llc_epilogue* epi, llc_tensor* out,
                           void* stream);

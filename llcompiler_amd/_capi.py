@@ -70,7 +70,8 @@ class LlcEwProgram(ctypes.Structure):
 
 # every symbol include/llc_hip.h declares
 EXPORTS = [
-    "llc_hip_abi_version", "llc_hip_init", "llc_hip_last_error", "llc_hip_status_string", "llc_hip_matmul",
+    "llc_hip_abi_version", "llc_hip_init", "llc_hip_last_error", "llc_hip_status_string", "llc_hip_scratch_bytes",
+    "llc_hip_trim", "llc_hip_matmul",
     "llc_hip_matmul_static",
     "llc_hip_batch_matmul", "llc_hip_conv2d", "llc_hip_elementwise", "llc_hip_reduce", "llc_hip_softmax",
     "llc_hip_layer_norm", "llc_hip_max_pool", "llc_hip_global_avg_pool", "llc_hip_transpose",
@@ -127,6 +128,8 @@ def lib():
         L.llc_hip_convert.argtypes = [T, T, vp]
         L.llc_hip_attention.argtypes = [T, T, T, T, ctypes.c_float, T, vp]
         L.llc_hip_init.argtypes = [ctypes.c_int]
+        L.llc_hip_scratch_bytes.argtypes = [ctypes.c_int, P(ctypes.c_size_t), P(ctypes.c_size_t)]
+        L.llc_hip_trim.argtypes = [ctypes.c_int]
         L.llc_hip_unpack_params.argtypes = [P(vp), ctypes.c_size_t, P(ctypes.c_size_t), P(ctypes.c_size_t), T,
                                             P(i64p)]
         L.llc_plan_create.argtypes = [P(vp)]

@@ -62,13 +62,15 @@ int check_launch(const char* kernel);
 // Scratch device memory for kernels that keep partial results (split reductions).  Where it comes from, in
 // this order: (1) a WorkspaceScope alive on the calling thread (a plan replaying with memory of its own, or the
 // allocation-free entry point with the library's static array): that memory is handed out and nothing is ever
-// allocated, a request beyond its capacity is an error; (2) one buffer per device, grown on demand.  Growing
-// allocates a new buffer and keeps the old one until the process ends (launches already queued, or a captured
-// graph, may still address it), never synchronises, and is refused while `stream` is being captured.
-// Kernels of one stream run in order, so successive calls on a stream can share the per-device buffer; calls
-// that overlap on different streams of one device must not both use kernels that need it (plans do not: each
-// owns its scratch memory).
+// allocated, a request beyond its capacity is an error; (2) one buffer per (device, stream), grown on demand.
+// Growing allocates a new buffer and retires the old one (launches already queued, or a captured graph, may still
+// address it) until scratch_trim frees it after a device synchronisation; it never synchronises by itself and is
+// refused while `stream` is being captured.  Kernels of one stream run in order, so successive calls on a stream
+// share that stream's buffer; calls on different streams never share one.
 int get_workspace(size_t bytes, void** out, hipStream_t stream);
+
+int scratch_bytes(int dev, size_t* live, size_t* retired);
+int scratch_trim(int all);
 
 struct WorkspaceScope {
   WorkspaceScope(void* ptr, size_t capacity);

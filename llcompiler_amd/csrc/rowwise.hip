@@ -571,12 +571,12 @@ int reduce_3d(const View& a, const View& o, int kind, int64_t outer, int64_t R, 
   p.scale = scale;
   if (outer * inner == 0) return LLC_OK;
   if (R >= (int64_t)1 << 31) return set_error(LLC_ERR_TOO_LARGE, "reduce: %lld reduced elements", (long long)R);
-  if (inner == 1) {
+  if (!p.y || (R > 0 && !p.x)) return set_error(LLC_ERR_BAD_ARG, "reduce: null operand with %lld outputs", (long long)(outer * inner));
+  // an empty reduction stores the init value: mid_reduce_kernel does that without reading anything (the row
+  // kernels return early on empty rows and would leave the output unwritten)
+  if (inner == 1 && R > 0) {
     p.rows = outer;
     p.cols = (int32_t)R;
-    if (R == 0) {  // empty reduction: the init value
-      p.cols = 0;
-    }
     return launch_rows<kReduce>(p, s);
   }
   const int64_t n = outer * inner;
@@ -622,6 +622,12 @@ int llc_impl_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n
   int n_red = 0;
   for (int r = 0; r < runs; ++r) n_red += run_red[r] ? 1 : 0;
   hipStream_t s = as_stream(stream);
+  if (a.numel() == 0) {
+    // some extent is 0: nothing to write when it is a kept one, else every output is the init value
+    // (one launch that reads nothing; no partial results, no scratch memory)
+    if (kept == 0) return LLC_OK;
+    return reduce_3d(a, o, kind, kept, 0, 1, 1.0f, s);
+  }
   if (n_red == 0) {
     // every reduced dim has extent 1 (or an extent is 0 and there is nothing to write): the values themselves
     if (kept == 0) return LLC_OK;
@@ -633,19 +639,18 @@ int llc_impl_reduce(int kind, const llc_tensor* x, const int64_t* axes, size_t n
   char* scratch = nullptr;
   size_t half = 0;
   if (n_red > 1) {
-    int64_t last_red = 1;
-    for (int r = runs - 1; r >= 0; --r)
-      if (run_red[r]) {
-        last_red = run_size[r];
-        break;
-      }
-    const int64_t partial = last_red ? a.numel() / last_red : 0;
+    // the largest partial result is what the innermost reduced run leaves: the product of all other runs
+    int innermost = -1;
+    for (int r = runs - 1; r >= 0 && innermost < 0; --r)
+      if (run_red[r]) innermost = r;
+    int64_t partial = 1;
+    for (int r = 0; r < runs; ++r)
+      if (r != innermost) partial *= run_size[r];
     half = ((size_t)partial * es + 255) & ~(size_t)255;
-    if (half) {
-      void* ws = nullptr;
-      LLC_TRY(get_workspace(2 * half, &ws, s));
-      scratch = (char*)ws;
-    }
+    void* ws = nullptr;
+    LLC_TRY(get_workspace(2 * half, &ws, s));
+    scratch = (char*)ws;
+    if (!scratch) return set_error(LLC_ERR_HIP, "reduce: no scratch memory for %lld partial results", (long long)partial);
   }
   View cur = a;
   int left = n_red, flip = 0;

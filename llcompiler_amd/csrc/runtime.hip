@@ -3,6 +3,7 @@
 #include <cstring>
 
 #include <mutex>
+#include <vector>
 
 #include "common.hpp"
 
@@ -46,8 +47,20 @@ int check_launch(const char* kernel) {
 
 namespace {
 constexpr int kMaxDevices = 64;
-void* g_ws[kMaxDevices];
-size_t g_ws_cap[kMaxDevices];
+// Scratch buffers of op entry points called outside a plan: one per (device, stream), so that calls on different
+// streams never share partial sums.  A buffer that was outgrown moves to `retired` (launches already queued may still
+// address it) until llc_hip_trim frees it.
+struct StreamScratch {
+  hipStream_t stream;
+  void* ptr;
+  size_t cap;
+};
+struct DeviceScratch {
+  std::vector<StreamScratch> live;
+  std::vector<StreamScratch> retired;
+};
+DeviceScratch g_scratch[kMaxDevices];
+std::mutex g_scratch_mu;
 }  // namespace
 
 int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done) {
@@ -91,21 +104,57 @@ int get_workspace(size_t bytes, void** out, hipStream_t stream) {
   int dev = 0;
   LLC_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "workspace: device %d", dev);
-  static std::mutex mu;  // host threads may launch at the same time; the buffer itself is shared per device
-  std::lock_guard<std::mutex> lock(mu);
-  if (bytes > g_ws_cap[dev]) {
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  DeviceScratch& d = g_scratch[dev];
+  StreamScratch* mine = nullptr;
+  for (StreamScratch& e : d.live)
+    if (e.stream == stream) mine = &e;
+  if (!mine || bytes > mine->cap) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
       return set_error(LLC_ERR_UNSUPPORTED, "this call needs %zu bytes of scratch memory and the stream is being captured: run it once "
                        "outside the capture, or record it into a plan", bytes);
-    // the old buffer stays allocated: queued launches and captured graphs may still address it
     const size_t cap_bytes = ((bytes + bytes / 2) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
     void* fresh = nullptr;
     LLC_HIP_TRY(hipMalloc(&fresh, cap_bytes));
-    g_ws[dev] = fresh;
-    g_ws_cap[dev] = cap_bytes;
+    if (mine) {
+      d.retired.push_back(*mine);  // queued launches and captured graphs may still address it
+      mine->ptr = fresh;
+      mine->cap = cap_bytes;
+    } else {
+      d.live.push_back(StreamScratch{stream, fresh, cap_bytes});
+      mine = &d.live.back();
+    }
   }
-  *out = g_ws[dev];
+  *out = mine->ptr;
+  return LLC_OK;
+}
+
+int scratch_bytes(int dev, size_t* live, size_t* retired) {
+  if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "scratch: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  size_t a = 0, b = 0;
+  for (const StreamScratch& e : g_scratch[dev].live) a += e.cap;
+  for (const StreamScratch& e : g_scratch[dev].retired) b += e.cap;
+  if (live) *live = a;
+  if (retired) *retired = b;
+  return LLC_OK;
+}
+
+int scratch_trim(int all) {
+  int dev = 0;
+  LLC_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(LLC_ERR_BAD_ARG, "scratch: device %d", dev);
+  // nothing queued may still address what is freed
+  LLC_HIP_TRY(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  DeviceScratch& d = g_scratch[dev];
+  for (StreamScratch& e : d.retired) (void)hipFree(e.ptr);
+  d.retired.clear();
+  if (all) {
+    for (StreamScratch& e : d.live) (void)hipFree(e.ptr);
+    d.live.clear();
+  }
   return LLC_OK;
 }
 
@@ -145,6 +194,12 @@ extern "C" int llc_hip_init(int device) {
   // the scratch array of the allocation-free entry point has an address of its own on every device
   return llc_impl_static_scratch_setup();
 }
+
+extern "C" int llc_hip_scratch_bytes(int device, size_t* live_bytes, size_t* retired_bytes) {
+  return scratch_bytes(device, live_bytes, retired_bytes);
+}
+
+extern "C" int llc_hip_trim(int release_live) { return scratch_trim(release_live); }
 
 extern "C" int llc_hip_unpack_params(void* const* params, size_t n_tensors, const size_t* ranks, const size_t* types,
                                      llc_tensor* tensors_out, const int64_t** symbols_out) {

@@ -110,6 +110,7 @@ class Instance:
         self.prep_calls = []       # run before `calls` when an input listed in prep_inputs changed
         self.prep_inputs = []
         self._prep_key = None
+        self._preparing = None     # while a prepared step is built: the graph inputs its result depends on
         self.patches = []          # (TensorRef, "in"|"out", index, byte offset from that tensor's data_ptr)
         self.keep = []
         self._roots = {}           # storage data_ptr -> ("in"|"out", index, base data_ptr)
@@ -122,19 +123,24 @@ class Instance:
         self._roots.setdefault(t.untyped_storage().data_ptr(), (kind, index, t.data_ptr()))
 
     def _launch_later(self, call):
+        if self._preparing is not None:
+            # a step that computes a derived weight (batch norm folded into a convolution's filters)
+            return self._prepare_later(call, self._preparing)
         # every descriptor the call holds is checked against the per-call storages
         for item in call.keep:
             self._scan(item)
         self.calls.append(call)
 
     def _prepare_later(self, call, input_index):
-        """A call whose result depends only on graph input `input_index` (a layout copy of a weight): it runs
-        before the instance's other calls, and again only when that input's address or version counter changed."""
+        """A call whose result depends only on graph inputs that are weights (`input_index`: one index or several; a
+        layout copy of a weight, folded filters): it runs before the instance's other calls, and again only when
+        one of those inputs' address or version counter changed."""
         for item in call.keep:
             self._scan(item)
         self.prep_calls.append(call)
-        if input_index not in self.prep_inputs:
-            self.prep_inputs.append(input_index)
+        for i in ([input_index] if isinstance(input_index, int) else input_index):
+            if i not in self.prep_inputs:
+                self.prep_inputs.append(i)
 
     def _channels_last_ok(self, st, ins, out, natural):
         if not CHANNELS_LAST or out.dtype not in (torch.float32, torch.bfloat16, torch.float16) or \
@@ -207,6 +213,11 @@ class Instance:
                 self.out_buffers.append(t)
                 n_out_bufs += 1
                 return t
+            if self._preparing is not None:
+                # written ahead of every other call and read by every run: never a buffer of the reuse pool
+                t = torch.empty(shape, dtype=v.dtype, device=dev)
+                self.keep.append(t)
+                return t
             n = 1
             for d in shape:
                 n *= d
@@ -248,6 +259,17 @@ class Instance:
             return materialise(x)
 
         cl_copies = {}   # id(value) -> its channels-last copy
+        prep_deps = {}   # id(value written by a prepared step) -> indices of the graph inputs it depends on
+
+        def prep_root(v):
+            """The dependencies of `v` when it is a derived weight or a view of one, else None."""
+            seen = 0
+            while id(v) not in prep_deps and seen < 16:
+                st = producer.get(id(v))
+                if st is None or st.kind != "view":
+                    return None
+                v, seen = st.inputs[0], seen + 1
+            return prep_deps.get(id(v))
 
         def to_channels_last(v, t):
             """`t` (the tensor of value `v`, logical NCHW) as a channels-last tensor: itself if it already is, else a
@@ -260,6 +282,9 @@ class Instance:
                 n = t.numel()
                 root = self._roots.get(t.untyped_storage().data_ptr())
                 prepared = root is not None and root[0] == "in" and id(v) in input_ids
+                deps = root[1] if prepared else None
+                if not prepared and prep_root(v) is not None:
+                    prepared, deps = True, prep_root(v)  # a derived weight: its copy is made where it is made
                 if prepared:
                     # written ahead of every other call and kept: never a buffer that earlier steps have used
                     nhwc = torch.empty((t.shape[0], t.shape[2], t.shape[3], t.shape[1]), dtype=t.dtype, device=dev)
@@ -270,11 +295,18 @@ class Instance:
                     nhwc = buf[: n * t.dtype.itemsize].view(t.dtype).view(t.shape[0], t.shape[2], t.shape[3], t.shape[1])
                 call = ops.copy(t.permute(0, 2, 3, 1), out=nhwc, defer=True)
                 if prepared:
-                    self._prepare_later(call, root[1])
+                    self._prepare_later(call, deps)
                 else:
                     self._launch_later(call)
                 c = cl_copies[id(v)] = nhwc.permute(0, 3, 1, 2)
             return c
+
+        def epi_of(st):
+            """The step's epilogue with a symbol-valued scale (x / x.shape[0] folded into alpha) as this binding's number."""
+            e = st.attrs["epilogue"]
+            if isinstance(e["alpha"], Expr):
+                e = dict(e, alpha=float(evaluate(e["alpha"], self.env)))
+            return e
 
         input_ids = set(id(v) for v in g.inputs)
         consumers = {}
@@ -308,7 +340,7 @@ class Instance:
             """scores = batch_matmul(q, k^T) {alpha, mask rows} -> softmax over the keys -> batch_matmul(p, v), every
             intermediate read once and only reshaped in between: returns (softmax step, second product, the
             reshapes) or None."""
-            e = st.attrs["epilogue"]
+            e = epi_of(st)
             if e["act"] or e["residual"] is not None or e["alpha"] <= 0 or (e["bias"] is not None and not e.get("bias_rows")):
                 return None
             if st.output.dtype not in (torch.bfloat16, torch.float16, torch.float32):
@@ -333,7 +365,7 @@ class Instance:
             v, u = through_reshapes(sm.output)
             if u is None or u.kind != "batch_matmul" or u.inputs[0] is not v or u.inputs[1] is v:
                 return None
-            e2 = u.attrs["epilogue"]
+            e2 = epi_of(u)
             if e2["act"] or e2["residual"] is not None or e2["bias"] is not None or e2["alpha"] != 1.0:
                 return None
             return sm, u, between
@@ -347,7 +379,7 @@ class Instance:
             sm, second, between = grp
             if not resolve_early(second.inputs[1]):
                 return False
-            e = st.attrs["epilogue"]
+            e = epi_of(st)
             qa, ka = (batched_operand(val[id(v)]) for v in st.inputs)
             va = batched_operand(val[id(second.inputs[1])])
             nat = _concrete(st.attrs["natural_shape"], self.env)
@@ -427,7 +459,7 @@ class Instance:
             """Several linear layers over the same rows (the q, k and v projections of an attention block) run as one
             product against the stacked weights: [M,K] x [K, N1+N2+..].  The stacked weight and bias are copies made
             by the instance's preparation calls; every layer's result is a column slice of the one output."""
-            e = st.attrs["epilogue"]
+            e = epi_of(st)
             if e["residual"] is not None or e.get("bias_rows") or id(st.output) in out_ids:
                 return False
             nat = _concrete(st.attrs["natural_shape"], self.env)
@@ -446,7 +478,9 @@ class Instance:
 
             def member(s2):
                 """(weight as [N,K], its input index, bias, its input index) when s2 can join, else None."""
-                e2 = s2.attrs["epilogue"]
+                if s2.kind != "matmul":
+                    return None
+                e2 = epi_of(s2)
                 if s2.kind != "matmul" or id(s2) in skip or id(s2.output) in out_ids or s2.output.dtype != st.output.dtype:
                     return None
                 if e2["residual"] is not None or e2.get("bias_rows") or e2["act"] != e["act"] or e2["alpha"] != e["alpha"] or \
@@ -520,6 +554,16 @@ class Instance:
             k = st.kind
             if id(st) in skip:
                 continue
+            self._preparing = None
+            if isinstance(st.attrs, dict) and st.attrs.get("prepared") and k in ("ew", "view") and id(st.output) not in out_ids:
+                deps = set()
+                for v in st.inputs:
+                    if id(v) in input_ids:
+                        deps.add(g.inputs.index(v))
+                    else:
+                        deps.update(prep_root(v) or ())
+                self._preparing = sorted(deps)
+                prep_deps[id(st.output)] = self._preparing
             if k == "matmul" and FUSE_PROJECTIONS and fused_projections(st, si):
                 for buf in temps:
                     pool.give(buf)
@@ -543,6 +587,8 @@ class Instance:
                     self.keep.append(temps.pop())
             elif k == "constant":
                 shape, v = _concrete(st.output.shape, self.env), st.attrs["value"]
+                if isinstance(v, Expr):  # llh.scalar_cast of a symbol's value: this binding's number
+                    v = evaluate(v, self.env)
                 if isinstance(v, (list, tuple)):  # a dense constant spelt element by element (LLH text)
                     c = torch.tensor(v, dtype=st.output.dtype).reshape(shape).to(dev)
                 else:
@@ -553,12 +599,15 @@ class Instance:
                 val[id(st.output)] = self.weights.get(st.attrs["weight_file"], _concrete(st.output.shape, self.env), st.output.dtype)
             elif k == "ew":
                 out = new_tensor(st.output)
-                prog = ops.make_program(st.attrs["insts"], st.attrs["result"], st.attrs["integer"])
+                insts = st.attrs["insts"]
+                if any(isinstance(x, Expr) for ins in insts for x in ins):
+                    insts = [tuple(float(evaluate(x, self.env)) if isinstance(x, Expr) else x for x in ins) for ins in insts]
+                prog = ops.make_program(insts, st.attrs["result"], st.attrs["integer"])
                 if out.numel():
                     self._launch_later(ops.elementwise(prog, ins, tuple(out.shape), out.dtype, out=out, defer=True))
                 val[id(st.output)] = out
             elif k in ("matmul", "batch_matmul", "conv"):
-                e = st.attrs["epilogue"]
+                e = epi_of(st)
                 out = new_tensor(st.output)
                 natural = _concrete(st.attrs["natural_shape"], self.env)
                 bias = materialise(val[id(e["bias"])]) if e["bias"] is not None else None
@@ -683,6 +732,7 @@ class Instance:
             del temps[:]
             for rid in [r for r in owner if last_use.get(r, si) <= si]:
                 pool.give(owner.pop(rid))
+        self._preparing = None
         # graph outputs
         self.output_plan = []
         for o in g.outputs:

@@ -14,6 +14,7 @@ A plan is a list of Steps over graph Values:
 """
 import torch
 
+from ..llh.expr import Expr
 from ..llh.graph import BINARY_OPS, ELEMENTWISE_OPS, UNARY_OPS, VIEW_OPS, Value
 
 MAX_INPUTS, MAX_REGS, MAX_INSTS = 6, 4, 24
@@ -28,18 +29,22 @@ class Step:
 
     def __repr__(self):
         extra = ""
+        if self.attrs.get("prepared"):
+            extra = " (prepared)"
         if self.kind == "ew":
-            extra = " [%s]" % " ".join(i[0] for i in self.attrs["insts"])
+            extra += " [%s]" % " ".join(i[0] for i in self.attrs["insts"])
         elif self.kind in ("matmul", "batch_matmul", "conv"):
             e = self.attrs["epilogue"]
             parts = [k for k in ("bias", "residual") if e.get(k) is not None]
-            if e.get("alpha", 1.0) != 1.0:
+            if isinstance(e.get("alpha", 1.0), Expr):
+                parts.append("alpha=%r" % (e["alpha"],))
+            elif e.get("alpha", 1.0) != 1.0:
                 parts.append("alpha=%g" % e["alpha"])
             if e.get("act"):
                 parts.append(e["act"])
             extra = " {%s}" % ",".join(parts) if parts else ""
         elif self.kind == "view":
-            extra = " " + self.attrs["op"]
+            extra += " " + self.attrs["op"]
         return "%s%s(%s) -> %%%s" % (self.kind, extra, ", ".join("%" + v.name for v in self.inputs), self.output.name)
 
 
@@ -122,7 +127,8 @@ class Planner:
                 c = _scalar_const(other)
                 if c is None or (u.name == "div" and u.operands[0] is not v) or tuple(u.results[0].shape) != tuple(v.shape):
                     break
-                epi["alpha"] = epi["alpha"] * float(c) if u.name == "mul" else epi["alpha"] / float(c)
+                c = c if isinstance(c, Expr) else float(c)  # (a symbol-valued scale stays an expression)
+                epi["alpha"] = epi["alpha"] * c if u.name == "mul" else epi["alpha"] / c
                 absorbed.append(u)
                 v = u.results[0]
                 continue
@@ -192,6 +198,8 @@ class Planner:
             if id(o) in produced:
                 return "r%d" % reg_of[id(o)]
             c = _scalar_const(o) if id(o) != keep_as_input else None
+            if isinstance(c, Expr):
+                return c  # a symbol-valued immediate: the engine puts in the number per binding
             if c is not None:
                 return float(c) if not isinstance(c, bool) else float(int(c))
             if id(o) not in in_index:
@@ -249,6 +257,8 @@ class Planner:
                     continue
                 if tuple(o.shape) != out_shape or self._ew_class(p) != cls:
                     continue
+                if (p in self.g.prepared) != (op in self.g.prepared):
+                    continue  # derived weights are computed once per instance, the rest on every call
                 cand = members + [m for m in group[id(p)] if m not in members]
                 try:
                     self.build_program(cand + [op])
@@ -289,10 +299,14 @@ class Planner:
             r = op.results[0]
             if op.name in ELEMENTWISE_OPS:
                 prog, inputs = self.build_program(groups[id(op)])
+                if all(m in g.prepared for m in groups[id(op)]):
+                    prog["prepared"] = True
                 self.steps.append(Step("ew", inputs, r, prog))
             elif op.name in VIEW_OPS:
                 self.steps.append(Step("view", op.operands[:1], r, dict(op.attrs, op=op.name)))
-            elif op.name == "constant":
+                if op in g.prepared:
+                    self.steps[-1].attrs["prepared"] = True
+            elif op.name in ("constant", "scalar_cast"):
                 self.steps.append(Step("constant", [], r, {"value": op.attrs["value"]}))
             elif op.name == "weight":
                 self.steps.append(Step("weight", [], r, {"weight_file": op.attrs["weight_file"]}))

@@ -13,6 +13,7 @@ import operator
 
 import torch
 
+from ..llh import expr as sym
 from ..llh.expr import Expr, from_sympy
 from ..llh.graph import Graph, Value
 
@@ -57,16 +58,30 @@ class Ctx:
     def val(self, a):
         return self.env[a] if isinstance(a, torch.fx.Node) else a
 
+    def like(self, a):
+        """The tensor value of `a` when it is one (the operand whose element type a scalar beside it takes)."""
+        v = self.env.get(a) if isinstance(a, torch.fx.Node) else None
+        return v if isinstance(v, Value) else None
+
     def tensor_or_const(self, a, like):
-        """Python scalars become tensor<1xT> constants of the other operand's element type."""
+        """Python scalars become tensor<1xT> constants of the other operand's element type.  A symbolic scalar (an
+        extent, or arithmetic on extents) becomes llh.scalar_cast of its value followed by llh.convert_to that
+        type, as in the reference's importer (llcompiler/importer/fx_translate.py:309-323)."""
         if isinstance(a, torch.fx.Node):
             v = self.env[a]
             if isinstance(v, Value):
                 return v
-            raise NotImplementedError("symbolic scalar operand %s" % a)
+            if v is None:
+                raise NotImplementedError("scalar operand %s has no value" % a)
+            a = v
         dt = like.dtype if like is not None else torch.float32
-        if isinstance(a, float) and not dt.is_floating_point:
+        real = sym.is_float(a)
+        if real and not dt.is_floating_point:
             dt = torch.float32
+        if isinstance(a, Expr):
+            own = torch.float32 if real else torch.int64
+            c = self.g.add_op("scalar_cast", [], {"value": a}, shapes=[(1,)], dtypes=[own], const=a)
+            return c if own == dt else self.g.add_op("convert_to", [c], {"dtype": dt})
         return self.g.constant(a, dt)
 
 
@@ -234,6 +249,10 @@ def _slice(ctx, node):
     start = args[2] or 0
     end = size if args[3] is None else args[3]
     step = 1 if args[4] is None else args[4]
+    if isinstance(start, torch.fx.Node):
+        start = ctx.env[start]
+    if isinstance(end, torch.fx.Node):
+        end = ctx.env[end]
     if isinstance(size, int):
         if start < 0:
             start += size
@@ -255,9 +274,9 @@ def _slice(ctx, node):
 def _binary(name):
     def tr(ctx, node):
         a, b = node.args[0], node.args[1]
-        av = ctx.tensor_or_const(a, ctx.val(b) if isinstance(b, torch.fx.Node) else None)
+        av = ctx.tensor_or_const(a, ctx.like(b))
         bv = ctx.tensor_or_const(b, av)
-        if not isinstance(a, torch.fx.Node):
+        if ctx.like(a) is None:
             av = ctx.tensor_or_const(a, bv)
         alpha = node.kwargs.get("alpha", 1)
         if alpha != 1:
@@ -270,6 +289,8 @@ def _binary(name):
     return tr
 
 
+_SCALAR_OPERAND_TARGETS = set()  # translators that accept a symbol-valued scalar where a tensor or number may stand
+
 for _name, _targets in {
     "add": (aten.add.Tensor, aten.add.Scalar, prims.add.default),
     "sub": (aten.sub.Tensor, aten.sub.Scalar, prims.sub.default),
@@ -279,6 +300,8 @@ for _name, _targets in {
     "pow": (aten.pow.Tensor_Scalar, aten.pow.Tensor_Tensor, prims.pow.default),
 }.items():
     TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_binary(_name))
+    _SCALAR_OPERAND_TARGETS.update(_targets)
+_SCALAR_OPERAND_TARGETS.update((aten.div.Tensor, aten.div.Scalar, prims.div.default, aten.rsub.Scalar, aten.rsub.Tensor))
 
 
 def _div_ok(node):
@@ -293,14 +316,15 @@ def _div(ctx, node):
     result type first: torch computes int / int in floating point, an integer llh.div would floor."""
     a, b = node.args[0], node.args[1]
     dt = _out_dtype(node)
-    av = ctx.tensor_or_const(a, ctx.val(b) if isinstance(b, torch.fx.Node) else None)
+    av = ctx.tensor_or_const(a, ctx.like(b))
     bv = ctx.tensor_or_const(b, av)
-    if not isinstance(a, torch.fx.Node):
+    if ctx.like(a) is None:
         av = ctx.tensor_or_const(a, bv)
     if av.dtype != dt:
         av = ctx.g.constant(a, dt) if not isinstance(a, torch.fx.Node) else ctx.g.add_op("convert_to", [av], {"dtype": dt})
     if bv.dtype != dt:
         bv = ctx.g.constant(b, dt) if not isinstance(b, torch.fx.Node) else ctx.g.add_op("convert_to", [bv], {"dtype": dt})
+
     return ctx.g.add_op("div", [av, bv])
 
 
@@ -352,13 +376,15 @@ for _kind, _targets in {
     "LE": (aten.le.Tensor, aten.le.Scalar, prims.le.default), "LT": (aten.lt.Tensor, aten.lt.Scalar, prims.lt.default),
 }.items():
     TORCH_FUNCTION_TRANSLATE_REGISTER(*_targets)(_compare(_kind))
+    _SCALAR_OPERAND_TARGETS.update(_targets)
+_SCALAR_OPERAND_TARGETS.update((prims.where.default, aten.where.self))
 
 
 @TORCH_FUNCTION_TRANSLATE_REGISTER(prims.where.default, aten.where.self)
 def _where(ctx, node):
     pred = ctx.val(node.args[0])
     t, f = node.args[1], node.args[2]
-    like = ctx.val(t) if isinstance(t, torch.fx.Node) else (ctx.val(f) if isinstance(f, torch.fx.Node) else None)
+    like = ctx.like(t) if ctx.like(t) is not None else ctx.like(f)
     tv = ctx.tensor_or_const(t, like)
     fv = ctx.tensor_or_const(f, tv)
     out = ctx.g.add_op("where", [pred, tv, fv])
@@ -371,6 +397,8 @@ def _where(ctx, node):
 def _fill_value_ok(node):
     if node.target in (aten.full.default, aten.full_like.default):
         return isinstance(node.args[1], (int, float, bool))
+    if node.target is aten.scalar_tensor.default:
+        return isinstance(node.args[0], (int, float, bool))
     return True
 
 
@@ -655,13 +683,62 @@ def _getitem(ctx, node):
     return src[node.args[1]]
 
 
-# symbolic integer arithmetic feeds shapes only; extents are taken from each node's fake value
+# Arithmetic on symbolic scalars (the reference translates the same targets to scalar llh ops,
+# fx_op_translate/binary_ops.py:39-76, unary_ops.py:79, lowered at src/Conversion/LLHToArith/LLHToArith.cpp:112-144).
+# Shapes take their extents from each node's fake value; the value of the node itself is kept as an expression
+# for the places where it is an operand of a tensor op.
 _SYMBOLIC_TARGETS = {aten.sym_size.int, aten.sym_numel.default, operator.mul, operator.add, operator.sub,
                      operator.floordiv, operator.truediv, operator.neg, operator.pow}
 if hasattr(torch, "_sym_sqrt"):
     _SYMBOLIC_TARGETS.add(torch._sym_sqrt)
 if hasattr(torch, "sym_float"):
     _SYMBOLIC_TARGETS.add(torch.sym_float)
+_SYMBOLIC_BINARY = {operator.mul: operator.mul, operator.add: operator.add, operator.sub: operator.sub,
+                    operator.floordiv: operator.floordiv, operator.truediv: operator.truediv, operator.pow: operator.pow}
+
+
+def _symbolic_value(ctx, node):
+    """The value of a symbolic scalar node: a number, or an expression over the graph's symbols."""
+    def arg(a):
+        if isinstance(a, torch.fx.Node):
+            v = ctx.env[a]
+            if v is None or isinstance(v, (Value, tuple)):
+                raise NotImplementedError("scalar arithmetic on %s" % a)
+            return v
+        return a
+    t = node.target
+    if t is aten.sym_size.int:
+        x = ctx.val(node.args[0])
+        return x.shape[node.args[1] % x.rank]
+    if t is aten.sym_numel.default:
+        return sym.product(ctx.val(node.args[0]).shape)
+    if t in _SYMBOLIC_BINARY:
+        return _SYMBOLIC_BINARY[t](arg(node.args[0]), arg(node.args[1]))
+    if t is operator.neg:
+        return -arg(node.args[0])
+    if t is getattr(torch, "_sym_sqrt", None):
+        return sym.sqrt(arg(node.args[0]))
+    if t is getattr(torch, "sym_float", None):
+        return sym.to_float(arg(node.args[0]))
+    raise NotImplementedError("symbolic scalar target %s" % (t,))
+
+
+def _symbolic_scalar(a):
+    return isinstance(a, torch.fx.Node) and isinstance(a.meta.get("val", a.meta.get("example_value")),
+                                                      (torch.SymInt, torch.SymFloat, torch.SymBool, int, float))
+
+
+def _symbolic_ok(a):
+    """Whether the scalar node `a` is arithmetic the importer can keep as an expression."""
+    if not isinstance(a, torch.fx.Node):
+        return isinstance(a, (int, float)) and not isinstance(a, bool)
+    if a.op == "placeholder":
+        return isinstance(a.meta.get("val", a.meta.get("example_value")), (torch.SymInt, int))
+    if a.op != "call_function" or a.target not in _SYMBOLIC_TARGETS:
+        return False
+    if a.target in (aten.sym_size.int, aten.sym_numel.default):
+        return True
+    return all(_symbolic_ok(x) for x in a.args)
 
 
 def is_supported(node):
@@ -673,6 +750,11 @@ def is_supported(node):
         register_inductor_prims()
     if node.target not in TORCH_FUNCTION_TRANSLATE:
         return False
+    # a symbol-valued scalar as a direct operand (x / x.shape[0]): only the translators that build their operands
+    # with tensor_or_const take one, and only when its arithmetic can be kept as an expression
+    for a in node.args:
+        if _symbolic_scalar(a) and not (node.target in _SCALAR_OPERAND_TARGETS and _symbolic_ok(a)):
+            return False
     chk = _SUPPORT_CHECKS.get(node.target)
     try:
         return True if chk is None else bool(chk(node))
@@ -704,7 +786,7 @@ def torch_translate_to_llh_graph(gm, weight_files=None):
                 e = dim_of(val)
                 name = e.args[0] if isinstance(e, Expr) and e.kind == "sym" else str(e)
                 g.add_symbol_arg(name)
-                ctx.env[node] = None
+                ctx.env[node] = e
             elif val is None:
                 g.arg_kinds.append(("none", None))
                 ctx.env[node] = None
@@ -712,7 +794,10 @@ def torch_translate_to_llh_graph(gm, weight_files=None):
                 raise TypeError("Unsupported type: %s" % type(val))
         elif node.op == "call_function":
             if node.target in _SYMBOLIC_TARGETS:
-                ctx.env[node] = None
+                try:
+                    ctx.env[node] = _symbolic_value(ctx, node)
+                except (NotImplementedError, TypeError, ZeroDivisionError):
+                    ctx.env[node] = None  # still good for shapes, which come from the fake values
                 continue
             tr = TORCH_FUNCTION_TRANSLATE.get(node.target)
             if tr is None:
@@ -728,7 +813,7 @@ def torch_translate_to_llh_graph(gm, weight_files=None):
                     res.append(None)
                 elif isinstance(o, torch.fx.Node):
                     v = ctx.env[o]
-                    if v is None:  # a symbolic int result
+                    if v is None or isinstance(v, (Expr, int, float)):  # a symbolic int result
                         res.append(dim_of(o.meta["val"]))
                     else:
                         res.append(v)

@@ -6,8 +6,18 @@ and the executor evaluates it with the symbol values bound at call time.  The no
 ones the reference's run-time evaluator handles (llcompiler/executor/out_put_call.py:21-48: Add,
 Mul, FloorDiv, Pow, Symbol, Number) plus CeilDiv (the affine maps of
 src/Dialect/LLH/IR/LLHinfersymbolShape.cpp:281-288), Sub, Max and Min.
+
+A symbol may also be a scalar OPERAND of a tensor op (`x / x.shape[0]`, `scores / sqrt(d)`): the reference casts
+the i64 value to a one-element tensor with llh.scalar_cast (include/llcompiler/Dialect/LLH/IR/LLHOps.td:120-127,
+lowered to a fill at src/Conversion/LLHToLinalg/LLHToLinalg.cpp:67-88) after computing it with scalar arithmetic
+(src/Conversion/LLHToArith/LLHToArith.cpp:112-144).  For that use the trees also carry real-valued nodes:
+TrueDiv, Sqrt, Float, Neg and Pow with any exponent; `is_float` tells the two kinds of tree apart and `evaluate`
+returns a Python float for them.
 """
+import math
 from functools import reduce as _reduce
+
+_NUM = (int, float)
 
 
 class Expr:
@@ -33,6 +43,11 @@ class Expr:
     def __rmul__(self, o): return self._bin("mul", o, True)
     def __floordiv__(self, o): return self._bin("floordiv", o)
     def __rfloordiv__(self, o): return self._bin("floordiv", o, True)
+    def __truediv__(self, o): return self._bin("truediv", o)
+    def __rtruediv__(self, o): return self._bin("truediv", o, True)
+    def __pow__(self, o): return self._bin("pow", o)
+    def __rpow__(self, o): return self._bin("pow", o, True)
+    def __neg__(self): return simplify(Expr("neg", (self,)))
 
     def __eq__(self, other):
         if isinstance(other, Expr):
@@ -45,7 +60,7 @@ class Expr:
     def __repr__(self):
         if self.kind == "sym":
             return self.args[0]
-        op = {"add": "+", "sub": "-", "mul": "*", "floordiv": "//"}.get(self.kind)
+        op = {"add": "+", "sub": "-", "mul": "*", "floordiv": "//", "truediv": "/"}.get(self.kind)
         if op:
             return "(%r %s %r)" % (self.args[0], op, self.args[1])
         return "%s(%s)" % (self.kind, ", ".join(repr(a) for a in self.args))
@@ -72,11 +87,34 @@ def emax(a, b):
     return a if a == b else Expr("max", (a, b))
 
 
+def sqrt(a):
+    """torch._sym_sqrt of a symbolic value."""
+    return math.sqrt(a) if isinstance(a, _NUM) else Expr("sqrt", (a,))
+
+
+def to_float(a):
+    """torch.sym_float of a symbolic value."""
+    return float(a) if isinstance(a, _NUM) else Expr("float", (a,))
+
+
+def is_float(e):
+    """Whether the value of `e` is a real number rather than an integer."""
+    if isinstance(e, float):
+        return True
+    if not isinstance(e, Expr) or e.kind == "sym":
+        return False
+    if e.kind in ("truediv", "sqrt", "float"):
+        return True
+    if e.kind == "pow" and not (isinstance(e.args[1], int) and e.args[1] >= 0):
+        return True
+    return any(is_float(a) for a in e.args)
+
+
 def simplify(e):
     if not isinstance(e, Expr) or e.kind == "sym":
         return e
     a = [simplify(x) for x in e.args]
-    if all(isinstance(x, int) for x in a):
+    if all(isinstance(x, _NUM) for x in a):
         return evaluate(Expr(e.kind, a), {})
     k = e.kind
     if k == "add":
@@ -96,8 +134,9 @@ def simplify(e):
 
 
 def evaluate(e, env):
-    """Integer value of `e` with symbols bound by `env` (name -> int)."""
-    if isinstance(e, int):
+    """Value of `e` with symbols bound by `env` (name -> int): an int for extents, a float for the real-valued
+    trees of scalar operands."""
+    if isinstance(e, _NUM):
         return e
     k, a = e.kind, e.args
     if k == "sym":
@@ -106,9 +145,12 @@ def evaluate(e, env):
         except KeyError:
             raise KeyError("symbol %s is not bound by any input of this call" % a[0])
     x = evaluate(a[0], env)
-    if k == "pow":
-        return x ** int(a[1])
+    if k == "sqrt": return math.sqrt(x)
+    if k == "float": return float(x)
+    if k == "neg": return -x
     y = evaluate(a[1], env)
+    if k == "pow": return x ** y
+    if k == "truediv": return x / y
     if k == "add": return x + y
     if k == "sub": return x - y
     if k == "mul": return x * y

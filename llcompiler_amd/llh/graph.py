@@ -81,6 +81,7 @@ class Graph:
         self.outputs = []         # Values, Exprs/ints (symbolic int results) or None
         self.symbol_sources = {}  # symbol name -> (input index, dim): llh.torch_symbolic_int -> llh.dim(arg, k)
         self.single_output = False
+        self.prepared = set()     # ops that compute derived weights (batch norm folded into filters): run per instance, not per call
         self._n = 0
 
     # ---- construction ----

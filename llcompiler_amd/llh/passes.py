@@ -6,17 +6,24 @@ src/Dialect/LLH/Transforms passes and canonicalisers, on the Python graph:
                          folded (the reference does): the product is NaN where x is NaN or infinite
   decompose_batch_norm   batch_norm_inference -> add, sqrt, reshape, broadcast_to x4, sub, mul, div, add
                          (DecomposeOps.cpp:110-148; op order pinned by test/Dialect/LLH/decompose_ops.mlir:10-20)
+  fold_batch_norm        conv / conv_bias -> batch_norm_inference whose parameters are weights  ==>  conv_bias on
+                         w * scale / sqrt(var + eps) and (b - mean) * scale / sqrt(var + eps) + bias: the same
+                         affine map as the decomposition (DecomposeOps.cpp:139-144) applied to the filters instead
+                         of to every output element; the folded filters are computed by ops marked as prepared
   fuse_softmax           reduce_max -> sub -> exp -> reduce_sum -> div  ==>  softmax
                          (the group ATen _softmax decomposes to, torch_compile_config.py:24)
 """
 import torch
 
+from .expr import Expr, is_float
 from .graph import BINARY_OPS, Value
 
 
 def _is_const(v, value=None):
     if not isinstance(v, Value) or v.const is None:
         return False
+    if isinstance(v.const, Expr):
+        return value is None
     return value is None or float(v.const) == float(value)
 
 
@@ -31,6 +38,8 @@ def _splat(v):
     """The value every element of v has when v is a constant filled with one number (seen through reshape and
     broadcast_to), else None."""
     v = _through_broadcast(v)
+    if isinstance(v.const, Expr):
+        return None  # a symbol-valued scalar: known per binding only
     if v.const is not None:
         return float(v.const)
     if v.producer is not None and v.producer.name == "constant" and not isinstance(v.producer.attrs.get("value"), (list, tuple)):
@@ -53,6 +62,18 @@ def canonicalize(g):
                 rep = op.operands[0]
             elif op.name == "convert_to" and op.attrs["dtype"] == op.operands[0].dtype:
                 rep = op.operands[0]
+            elif op.name == "convert_to" and op.operands[0].producer is not None and \
+                    op.operands[0].producer.name == "scalar_cast" and \
+                    (op.attrs["dtype"].is_floating_point or not is_float(op.operands[0].const)):
+                # llh.convert_to of llh.scalar_cast (what the importer writes for a symbol-valued operand,
+                # fx_translate.py:309-323): the cast produces the wanted element type directly
+                src = op.operands[0].producer
+                idx = g.ops.index(op)
+                tail = g.ops[idx:]
+                del g.ops[idx:]
+                rep = g.add_op("scalar_cast", [], dict(src.attrs), shapes=[tuple(r.shape)], dtypes=[op.attrs["dtype"]],
+                               const=src.attrs["value"])
+                g.ops += tail
             elif op.name in ("reshape", "broadcast_to") and tuple(op.operands[0].shape) == tuple(r.shape):
                 rep = op.operands[0]
             elif op.name == "reshape" and op.operands[0].producer is not None and op.operands[0].producer.name == "reshape":
@@ -173,6 +194,74 @@ def decompose_batch_norm(g):
     return g
 
 
+def _weight_like(v, depth=0):
+    """A graph input, an llh.weight / llh.constant, or a view of one: a value that does not depend on activations
+    computed by the graph (parameters and buffers of the module)."""
+    if v.producer is None:
+        return True
+    if v.producer.name in ("weight", "constant"):
+        return True
+    if v.producer.name in ("reshape", "broadcast_to", "transpose", "identity") and depth < 8:
+        return _weight_like(v.producer.operands[0], depth + 1)
+    return False
+
+
+def fold_batch_norm(g):
+    """Eval-mode batch norm behind a convolution becomes part of the convolution's filters and bias.
+
+    batch_norm_inference(conv(x, w[, b]), scale, bias, mean, var) = conv_bias(x, w', b') with
+        k = scale / sqrt(var + eps),  w'[f, ...] = w[f, ...] * k[f],  b' = (b - mean) * k + bias,
+    which is DecomposeOps.cpp:139-144's scale * (y - mean) / sqrt(var + eps) + bias with the per-filter factor moved
+    through the sum.  Done when the convolution's result has no other reader and the filters and all four
+    batch-norm parameters are weights (graph inputs, llh.weight, constants): the ops that compute w' and b' are
+    marked in `g.prepared`, which tells the planner and the engine to run them when a plan instance is made
+    (and again when a parameter's address or version changes), not on every call."""
+    prepared = getattr(g, "prepared", None)
+    if prepared is None:
+        prepared = g.prepared = set()
+    outputs = set(id(o) for o in g.outputs if isinstance(o, Value))
+    for op in list(g.ops):
+        if op.name != "batch_norm_inference" or op not in g.ops:
+            continue
+        y, scale, bias, mean, var = op.operands
+        conv = y.producer
+        if conv is None or conv.name not in ("conv", "conv_bias") or len(y.users) != 1 or id(y) in outputs:
+            continue
+        feature = op.attrs.get("feature_index", 1) % y.rank
+        if feature != (y.rank - 1 if conv.attrs.get("layout", "NCHW") == "NHWC" else 1):
+            continue
+        w = conv.operands[1]
+        b = conv.operands[2] if conv.name == "conv_bias" else None
+        params = [w, scale, bias, mean, var] + ([b] if b is not None else [])
+        if not all(_weight_like(p) and p.is_static() for p in params):
+            continue
+        if any(p.dtype != w.dtype for p in params) or not w.dtype.is_floating_point:
+            continue
+        idx = g.ops.index(conv)
+        tail = g.ops[idx:]
+        del g.ops[idx:]
+        first_new = len(g.ops)
+        f = w.shape[0]
+        eps = g.constant(op.attrs["epsilon"], var.dtype)
+        k = g.add_op("div", [scale, g.add_op("sqrt", [g.add_op("add", [var, eps])])])
+        per_filter = (f,) + (1,) * (w.rank - 1)
+        kw = g.add_op("reshape", [k], {"shape": per_filter}, shapes=[per_filter], dtypes=[k.dtype])
+        kw = g.add_op("broadcast_to", [kw], {"shape": tuple(w.shape), "cast_dims": tuple(range(w.rank))})
+        w2 = g.add_op("mul", [w, kw])
+        shifted = g.add_op("sub", [b, mean]) if b is not None else g.add_op("neg", [mean])
+        b2 = g.add_op("add", [g.add_op("mul", [shifted, k]), bias])
+        for new in g.ops[first_new:]:
+            prepared.add(new)
+        z = g.add_op("conv_bias", [conv.operands[0], w2, b2], dict(conv.attrs))
+        g.ops += [t for t in tail if t is not conv and t is not op]
+        g.replace_all_uses(op.results[0], z)
+        for dead in (op, conv):
+            for o in dead.operands:
+                if dead in o.users:
+                    o.users.remove(dead)
+    return g
+
+
 def _strip_keepdim(v, full_shape):
     """v is (reduce result) possibly followed by reshape (keepdim) and broadcast_to back to full_shape."""
     chain = []
@@ -253,8 +342,10 @@ def transform_layout(g, target="NCHW"):
 
 def run_llh_pipeline(g, target_layout="NCHW"):
     """Order follows the reference's pipeline (src/Pipeline/TransformPipeline.cpp:103-128):
-    legalise/remove-redundant, decompose, canonicalise, layout transform, canonicalise."""
+    legalise/remove-redundant, decompose, canonicalise, layout transform, canonicalise.  Batch norms that follow a
+    convolution are folded into it before the decomposition sees them."""
     canonicalize(g)
+    fold_batch_norm(g)
     decompose_batch_norm(g)
     fuse_softmax(g)
     canonicalize(g)

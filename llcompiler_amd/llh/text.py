@@ -303,6 +303,14 @@ class _Reader:
             if name == "div" and not isinstance(b, Expr) and b == 0:
                 raise NotImplementedError("llh.div of scalars by the constant 0")
             return {"add": lambda: a + b, "sub": lambda: a - b, "mul": lambda: a * b, "div": lambda: a // b}[name]()
+        if name == "scalar_cast":
+            # an i64 (or float) scalar as a one-element tensor (LLHOps.td:120-127): a constant when the scalar is a
+            # number, else a value that every binding of the symbols fills in
+            v = self.scalar(operands[0])
+            shape = tuple(rt.shape) if len(rt.shape) else (1,)
+            if isinstance(v, Expr):
+                return g.add_op("scalar_cast", [], {"value": v}, shapes=[shape], dtypes=[rt.dtype], const=v)
+            return g.add_op("constant", [], {"value": v}, shapes=[shape], dtypes=[rt.dtype], const=v)
         if name == "print":
             self.printed.append(self.tensor(operands[0]))
             return None
@@ -520,15 +528,45 @@ def _attr_text(key, v, result):
     raise NotImplementedError("attribute %s = %r" % (key, v))
 
 
+_SCALAR_OP_NAMES = {"add": "add", "sub": "sub", "mul": "mul", "floordiv": "div"}
+
+
+def _print_scalar(e, g, lines, counter):
+    """Writes the i64 arithmetic that computes the symbolic value `e` (llh.dim of the argument that carries a
+    symbol, llh.torch_symbolic_int for a symbol passed as an int argument, llh.constant, scalar add/sub/mul/div)
+    and returns the SSA name of the result."""
+    counter[0] += 1
+    name = "e%d" % counter[0]
+    if isinstance(e, int):
+        lines.append('  %%%s = "llh.constant"() <{value = %d : i64}> : () -> i64' % (name, e))
+    elif e.kind == "sym" and e.args[0] in g.symbol_sources:
+        i, k = g.symbol_sources[e.args[0]]
+        c = _print_scalar(k, g, lines, counter)
+        lines.append('  %%%s = "llh.dim"(%%%s, %%%s) : (%s, i64) -> i64' % (name, g.inputs[i].name, c, _type_str(g.inputs[i])))
+    elif e.kind == "sym":
+        lines.append('  %%%s = "llh.torch_symbolic_int"() <{sym_name = "%s"}> : () -> i64' % (name, e.args[0]))
+    elif e.kind in _SCALAR_OP_NAMES:
+        a, b = (_print_scalar(x, g, lines, counter) for x in e.args)
+        lines.append('  %%%s = "llh.%s"(%%%s, %%%s) : (i64, i64) -> i64' % (name, _SCALAR_OP_NAMES[e.kind], a, b))
+    else:
+        raise NotImplementedError("scalar expression %r has no spelling in llh scalar ops" % (e,))
+    return name
+
+
 def print_llh(g):
     """The graph in generic op syntax; `parse_llh(print_llh(g))` gives an equivalent graph when every attribute is
     static (symbolic reshape / broadcast targets are printed as llh.dim arithmetic only for plain symbols)."""
     lines = []
+    counter = [0]
     args = ["%%%s: %s" % (v.name, _type_str(v)) for v in g.inputs]
     outs = [o for o in g.outputs if isinstance(o, Value)]
     lines.append("func.func @main(%s) -> (%s) attributes {entrance} {" % (", ".join(args), ", ".join(_type_str(o) for o in outs)))
     for op in g.ops:
         r = op.results[0]
+        if op.name == "scalar_cast":
+            src = _print_scalar(op.attrs["value"], g, lines, counter)
+            lines.append('  %%%s = "llh.scalar_cast"(%%%s) : (i64) -> %s' % (r.name, src, _type_str(r)))
+            continue
         if op.name == "constant":
             val = op.attrs["value"]
             body = "[%s]" % ", ".join(repr(x) for x in val) if isinstance(val, list) else repr(float(val) if r.dtype.is_floating_point else int(val))

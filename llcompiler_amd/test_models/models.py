@@ -92,6 +92,70 @@ class ResNet18Folded(nn.Module):
         return self.fc(x)
 
 
+class _ConvBN(nn.Module):
+    """Conv without bias followed by BatchNorm2d (the torchvision unit), optional ReLU."""
+
+    def __init__(self, cin, cout, k, stride, pad, relu=True):
+        super().__init__()
+        self.conv = nn.Conv2d(cin, cout, k, stride, pad, bias=False)
+        self.bn = nn.BatchNorm2d(cout)
+        self.relu = relu
+
+    def forward(self, x):
+        y = self.bn(self.conv(x))
+        return F.relu(y) if self.relu else y
+
+
+class _BasicBlockBN(nn.Module):
+    def __init__(self, cin, cout, stride):
+        super().__init__()
+        self.c1 = _ConvBN(cin, cout, 3, stride, 1, relu=True)
+        self.c2 = _ConvBN(cout, cout, 3, 1, 1, relu=False)
+        self.down = _ConvBN(cin, cout, 1, stride, 0, relu=False) if (stride != 1 or cin != cout) else None
+
+    def forward(self, x):
+        idt = x if self.down is None else self.down(x)
+        return F.relu(self.c2(self.c1(x)) + idt)
+
+
+class ResNet18BN(nn.Module):
+    """The same network as ResNet18Folded the way torchvision spells it: every convolution has no bias and is
+    followed by a BatchNorm2d.  In eval mode the compiler folds each batch norm into its convolution when the plan
+    is made.  The affine parameters and the running statistics are seeded random values (variances in [0.5, 1.5]),
+    so the fold is not the identity."""
+
+    def __init__(self, num_classes=1000, seed=0):
+        super().__init__()
+        self.stem = _ConvBN(3, 64, 7, 2, 3)
+        chans = [64, 128, 256, 512]
+        blocks, cin = [], 64
+        for i, c in enumerate(chans):
+            blocks += [_BasicBlockBN(cin, c, 1 if i == 0 else 2), _BasicBlockBN(c, c, 1)]
+            cin = c
+        self.blocks = nn.Sequential(*blocks)
+        self.fc = nn.Linear(512, num_classes)
+        gen = torch.Generator().manual_seed(seed)
+        for m in self.modules():
+            if isinstance(m, nn.Conv2d):
+                fan_out = m.out_channels * m.kernel_size[0] * m.kernel_size[1]
+                m.weight.data = torch.randn(m.weight.shape, generator=gen) * math.sqrt(2.0 / fan_out)
+            elif isinstance(m, nn.BatchNorm2d):
+                m.weight.data = 0.75 + 0.5 * torch.rand(m.weight.shape, generator=gen)
+                m.bias.data = torch.randn(m.bias.shape, generator=gen) * 0.05
+                m.running_mean.copy_(torch.randn(m.running_mean.shape, generator=gen) * 0.1)
+                m.running_var.copy_(0.5 + torch.rand(m.running_var.shape, generator=gen))
+            elif isinstance(m, nn.Linear):
+                m.weight.data = torch.randn(m.weight.shape, generator=gen) * 0.02
+                m.bias.data.zero_()
+
+    def forward(self, x):
+        x = self.stem(x)
+        x = F.max_pool2d(x, 3, 2, 1)
+        x = self.blocks(x)
+        x = F.adaptive_avg_pool2d(x, 1).flatten(1)
+        return self.fc(x)
+
+
 def make_resnet_inputs(batch=16, size=224, seed=1):
     return (torch.randn(batch, 3, size, size, generator=torch.Generator().manual_seed(seed)),)
 

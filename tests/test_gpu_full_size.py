@@ -33,6 +33,8 @@ def test_matmul_2048_f32(ops, oracle):
     # ones that cancel to ~0).  So: the stated tolerance must hold for all but 1 in 10^4 outputs, and
     # every output must be within 1e-4 of the output scale.
     strict_bad = int((err > F32_ATOL + F32_RTOL * np.abs(want)).sum())
+    print("matmul 2048^3 f32: %d of %d outputs outside rtol 1e-4 / atol 1e-5 of the oracle (max abs error %.3g)"
+          % (strict_bad, err.size, err.max()))
     assert strict_bad <= 150, "%d outputs outside rtol 1e-4 / atol 1e-5" % strict_bad
     scale = float(np.sqrt((want ** 2).mean()))
     assert err.max() <= F32_ATOL + F32_RTOL * scale, "max abs error %g at output scale %g" % (err.max(), scale)

@@ -1010,3 +1010,139 @@ def test_reference_op_tests_in_their_four_modes(name, shapes, modes):
             scale = max(1.0, float(want.detach().abs().nan_to_num(0.0, 0.0, 0.0).max()))
             assert_close(got.detach().cpu().numpy(), want.detach().numpy(), F32_RTOL, F32_ATOL * scale, what)
         assert comp.compile_count >= 1, what
+
+
+# ---- eval-mode batch norm folded into the convolution it follows, when the plan is made ----
+def test_resnet18_with_batch_norms_plans_to_twenty_convolutions(oracle):
+    """A ResNet-18 spelt like torchvision's (Conv2d without bias -> BatchNorm2d, randomised running statistics) in
+    eval mode: every batch norm becomes part of its convolution's filters and bias (DecomposeOps.cpp:139-144 moved
+    through the sum), computed by preparation calls; a call launches 20 convolutions, two pools and one matmul.
+    Checked against the oracle composition on filters folded by the oracle's own fold, against torch eager (the
+    unfolded batch norm), and again after the statistics were written in place."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import ResNet18BN, make_resnet_inputs
+    m = ResNet18BN().eval()
+    (x,) = make_resnet_inputs(2, 64)
+
+    def conv(mod, t):
+        c, bn = mod.conv, mod.bn
+        w, b = oracle.fold_bn_into_conv(c.weight.detach().numpy(), None, bn.weight.detach().numpy(), bn.bias.detach().numpy(),
+                                        bn.running_mean.numpy(), bn.running_var.numpy(), bn.eps)
+        p = c.padding[0]
+        y = oracle.conv2d(t, w, b, (p, p, p, p), tuple(c.stride))
+        return oracle.unary("relu", y) if mod.relu else y
+
+    def composition():
+        t = conv(m.stem, x.numpy())
+        t = oracle.maxpool2d(t, (3, 3), (1, 1, 1, 1), (2, 2))
+        for blk in m.blocks:
+            idt = t if blk.down is None else conv(blk.down, t)
+            t = oracle.unary("relu", oracle.binary("add", conv(blk.c2, conv(blk.c1, t)), idt))
+        return _oracle_linear(oracle, oracle.global_avgpool(t).reshape(2, 512), m.fc)
+
+    with torch.no_grad():
+        mg = copy.deepcopy(m).cuda()
+        cm = compile_module(mg, (x.cuda(),))
+        per_call = [s.kind for s in cm.engine.steps if not s.attrs.get("prepared") and s.kind not in ("view", "constant")]
+        assert per_call.count("conv") == 20 and per_call.count("ew") == 0 and sorted(set(per_call)) == ["avg_pool", "conv", "matmul", "max_pool"]
+        got = cm(x.cuda())
+        assert_close(got.cpu().numpy(), composition(), F32_RTOL, F32_ATOL, "resnet18 with batch norms vs the oracle composition")
+        assert_close(got.cpu().numpy(), m(x).numpy(), F32_RTOL, F32_ATOL, "resnet18 with batch norms vs torch eager")
+        inst = list(cm.engine.instances.values())[0]
+        assert len(inst.calls) == 23 + 1   # + the layout copy behind the max-pool
+        assert torch.equal(cm(x.cuda()), got)
+        # statistics and filters written in place: the folded filters follow
+        for mod, ref in zip(mg.modules(), m.modules()):
+            if isinstance(mod, torch.nn.BatchNorm2d):
+                for t in (mod.running_var, ref.running_var):
+                    t.mul_(1.25)
+                for t in (mod.running_mean, ref.running_mean):
+                    t.add_(0.05)
+        mg.stem.conv.weight.mul_(0.5)
+        m.stem.conv.weight.mul_(0.5)
+        assert_close(cm(x.cuda()).cpu().numpy(), composition(), F32_RTOL, F32_ATOL, "after writing statistics and filters in place")
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_conv_batch_norm_units_through_the_backend(dt):
+    """Conv -> BatchNorm2d -> ReLU (+ residual) through the torch.compile backend, with and without a convolution bias,
+    in both storage types: one convolution kernel per unit."""
+    from tests.util import assert_as_close_as_eager
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.c1 = torch.nn.Conv2d(64, 64, 3, 1, 1, bias=True)
+            self.b1 = torch.nn.BatchNorm2d(64)
+            self.c2 = torch.nn.Conv2d(64, 64, 3, 1, 1, bias=False)
+            self.b2 = torch.nn.BatchNorm2d(64)
+
+        def forward(self, x):
+            y = torch.relu(self.b1(self.c1(x)))
+            return torch.relu(self.b2(self.c2(y)) + x)
+
+    torch.manual_seed(3)
+    m = Net().eval()
+    for bn in (m.b1, m.b2):
+        bn.weight.data.uniform_(0.5, 1.5)
+        bn.bias.data.normal_(0, 0.1)
+        bn.running_mean.normal_(0, 0.1)
+        bn.running_var.uniform_(0.5, 1.5)
+    m = m.to(dt)
+    x = torch.randn(2, 64, 20, 20).to(dt)
+    with torch.no_grad():
+        want64 = copy.deepcopy(m).double()(x.double()).numpy()
+        eager = m(x).float().numpy()
+        opt, comp = _compile(m)
+        got = opt(x.cuda())
+    kinds = [s.kind for e in comp.engines for s in e.steps if not s.attrs.get("prepared") and s.kind not in ("view", "constant")]
+    assert kinds == ["conv", "conv"]
+    if dt == torch.float32:
+        assert_close(got.cpu().numpy(), eager, F32_RTOL, F32_ATOL, "conv-bn units fp32")
+    else:
+        assert_as_close_as_eager(got.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, "conv-bn units bf16")
+
+
+# ---- a symbol's value as an operand of a tensor op (llh.scalar_cast) ----
+class _SymbolOperands(torch.nn.Module):
+    def forward(self, x):
+        n = x.shape[0]
+        return x / n + x.sum(0) * n, (x - n) * (n // 2 + 1)
+
+
+class _ScaledScores(torch.nn.Module):
+    def forward(self, q, k):
+        return (q @ k.transpose(-1, -2)) / torch._sym_sqrt(q.shape[-1])
+
+
+def test_symbol_valued_scalar_operands_through_both_entries():
+    """x / x.shape[0], x.sum(0) * x.shape[0] and scores / sqrt(q.shape[-1]) with dynamic extents: the reference casts
+    the i64 symbol to a one-element tensor (llh.scalar_cast, LLHOps.td:120-127; Operationlegalization.cpp and
+    LLHToLinalg.cpp:67-88 legalise and lower it).  Here the value is an immediate of the elementwise program, or the
+    scale of the product's epilogue, filled in per binding: one engine, three bindings each, against eager."""
+    from torch.export import Dim
+    from llcompiler_amd.compiler.aot import compile_module
+    gen = torch.Generator().manual_seed(5)
+    m = _SymbolOperands().eval()
+    cm = compile_module(m, (torch.randn(4, 8).cuda(),), dynamic_shapes=({0: Dim("b", min=2, max=64)},))
+    kinds = [s.kind for s in cm.engine.steps if s.kind not in ("view", "constant")]
+    assert kinds.count("ew") == 3 and kinds.count("reduce") == 1
+    for n in (3, 8, 33):
+        x = torch.randn(n, 8, generator=gen)
+        for got, want in zip(cm(x.cuda()), m(x)):
+            assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "symbol operands, %d rows" % n)
+    assert len(cm.engine.instances) == 3
+    s = _ScaledScores().eval()
+    d = Dim("d", min=2, max=128)
+    cs = compile_module(s, (torch.randn(3, 4, 8).cuda(), torch.randn(3, 4, 8).cuda()), dynamic_shapes=({2: d}, {2: d}))
+    assert [st.kind for st in cs.engine.steps if st.kind not in ("view", "constant")] == ["batch_matmul"]   # the scale is the epilogue's alpha
+    for dim in (8, 20, 64):
+        q, k = torch.randn(3, 4, dim, generator=gen), torch.randn(3, 4, dim, generator=gen)
+        assert_close(cs(q.cuda(), k.cuda()).cpu().numpy(), s(q, k).numpy(), F32_RTOL, F32_ATOL, "scaled scores, dim %d" % dim)
+    # the torch.compile backend: dynamo hands the extent over as a SymInt argument
+    opt, comp = _compile(m, dynamic=True)
+    for n in (5, 9, 17):
+        x = torch.randn(n, 8, generator=gen)
+        for got, want in zip(opt(x.cuda()), m(x)):
+            assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "symbol operands through the backend, %d rows" % n)
+    assert len(comp.engines) == 1

@@ -392,6 +392,16 @@ def test_reduce_over_split_axes_with_an_empty_run(ops):
     x = torch.zeros(2, 0, 3, 4, device="cuda")
     np.testing.assert_array_equal(host(ops.reduce("sum", x, [1, 3])), np.zeros((2, 3), np.float32))
     np.testing.assert_array_equal(host(ops.reduce("max", x, [1, 3])), np.full((2, 3), -np.inf, np.float32))
+    # the empty run innermost, a non-empty reduced run further out: still the init value in every output
+    y = torch.zeros(2, 3, 4, 0, device="cuda")
+    np.testing.assert_array_equal(host(ops.reduce("sum", y, [1, 3])), np.zeros((2, 4), np.float32))
+    np.testing.assert_array_equal(host(ops.reduce("min", y, [1, 3])), np.full((2, 4), np.inf, np.float32))
+    # one empty run over the last dim: the output is written, not left as allocated
+    z = torch.zeros(5, 0, device="cuda")
+    np.testing.assert_array_equal(host(ops.reduce("sum", z, [1])), np.zeros(5, np.float32))
+    np.testing.assert_array_equal(host(ops.reduce("max", z, [1])), np.full(5, -np.inf, np.float32))
+    np.testing.assert_array_equal(host(ops.reduce("max", torch.zeros(5, 0, 3, device="cuda"), [1])),
+                                  np.full((5, 3), -np.inf, np.float32))
 
 
 # --------------------------------------------------------------------------- data movement (bit exact)

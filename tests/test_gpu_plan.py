@@ -491,6 +491,54 @@ def test_two_plans_with_split_reductions_run_on_two_streams_at_once():
         np.testing.assert_array_equal(out.cpu().numpy(), want.cpu().numpy())
 
 
+def test_op_calls_with_split_reductions_run_on_two_streams_at_once():
+    """Op entry points called outside a plan keep the partial sums of a split reduction in a scratch buffer per
+    (device, stream): the same product issued on two streams at the same time gives, bit for bit, what each call
+    gives alone.  llc_hip_scratch_bytes sees one live buffer per stream; llc_hip_trim hands the memory back."""
+    import ctypes
+    from llcompiler_amd import _capi as C
+    C.init(0)
+    L = C.lib()
+    M, N, K = 1024, 768, 3072
+    gen = torch.Generator().manual_seed(6)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    sets = []
+    for _ in range(2):
+        a = (torch.rand(M, K, generator=gen) * 2 - 1).cuda()
+        w = (torch.rand(N, K, generator=gen) * 2 - 1).cuda()
+        out = torch.empty((M, N), device="cuda")
+        sets.append((C.tensor_ref(a), C.tensor_ref(w.t()), C.tensor_ref(out), out))
+    torch.cuda.synchronize()
+    alone = []
+    for (ra, rw, ro, out), st in zip(sets, streams):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        C.check(L.llc_hip_matmul(ra.ptr, rw.ptr, None, ro.ptr, ctypes.c_void_p(st.cuda_stream)))
+        torch.cuda.synchronize()
+        assert not torch.isnan(out).any()
+        alone.append(out.clone())
+    live, retired = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    C.check(L.llc_hip_scratch_bytes(0, ctypes.byref(live), ctypes.byref(retired)))
+    assert live.value >= 2 * 2 * M * N * 4      # each stream holds its own buffer of at least two chunks of partial sums
+    for *_, out in sets:
+        out.fill_(float("nan"))
+    torch.cuda.synchronize()
+    for _ in range(10):
+        for (ra, rw, ro, out), st in zip(sets, streams):
+            C.check(L.llc_hip_matmul(ra.ptr, rw.ptr, None, ro.ptr, ctypes.c_void_p(st.cuda_stream)))
+    torch.cuda.synchronize()
+    for (*_, out), want in zip(sets, alone):
+        np.testing.assert_array_equal(out.cpu().numpy(), want.cpu().numpy())
+    C.check(L.llc_hip_trim(1))
+    C.check(L.llc_hip_scratch_bytes(0, ctypes.byref(live), ctypes.byref(retired)))
+    assert live.value == 0 and retired.value == 0
+    # and the next call allocates again
+    ra, rw, ro, out = sets[0]
+    C.check(L.llc_hip_matmul(ra.ptr, rw.ptr, None, ro.ptr, ctypes.c_void_p(streams[0].cuda_stream)))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), alone[0].cpu().numpy())
+
+
 @pytest.mark.parametrize("which", ["encoder_bf16", "resnet"])
 def test_engine_plans_survive_a_file(which, tmp_path):
     """The plan an engine instance records (fused attention, stacked projections, channels-last convolutions with

@@ -404,3 +404,142 @@ def test_backward_ops_of_layer_norm_softmax_and_gelu_are_imported():
     run_llh_pipeline(g)
     kinds = [s.kind for s in make_plan(g)]
     assert "layer_norm" in kinds and kinds.count("reduce") >= 6
+
+
+# ---- batch norm folded into the convolution it follows (the affine map of DecomposeOps.cpp:139-144 on the filters) ----
+def _conv_bn_graph(with_conv_bias=False, second_reader=False, layout="NCHW"):
+    g = Graph()
+    x = g.add_input((2, 8, 16, 16) if layout == "NCHW" else (2, 16, 16, 8), f32, "x")
+    w = g.add_input((8, 8, 3, 3) if layout == "NCHW" else (8, 3, 3, 8), f32, "w")
+    params = [g.add_input((8,), f32, n) for n in ("scale", "bias", "mean", "var")]
+    attrs = {"dilation": (1, 1), "kernel_shape": (3, 3), "pad": (1, 1, 1, 1), "stride": (1, 1), "group": 1, "layout": layout}
+    if with_conv_bias:
+        y = g.add_op("conv_bias", [x, w, g.add_input((8,), f32, "b")], attrs)
+    else:
+        y = g.add_op("conv", [x, w], attrs)
+    z = g.add_op("batch_norm_inference", [y] + params, {"epsilon": 1e-5, "momentum": 0.1,
+                                                         "feature_index": 1 if layout == "NCHW" else 3})
+    r = g.add_op("relu", [z])
+    g.set_outputs([r, y] if second_reader else [r])
+    return g
+
+
+@pytest.mark.parametrize("with_conv_bias", [False, True])
+def test_batch_norm_behind_a_convolution_folds_into_its_filters(with_conv_bias):
+    g = run_llh_pipeline(_conv_bn_graph(with_conv_bias))
+    assert "batch_norm_inference" not in g.op_names()
+    assert g.op_names().count("conv_bias") == 1 and "conv" not in g.op_names()
+    steps = make_plan(g)
+    per_call = [s for s in steps if not s.attrs.get("prepared") and s.kind not in ("view", "constant")]
+    # every call launches ONE kernel: the convolution with the folded bias and the relu in its epilogue
+    assert [s.kind for s in per_call] == ["conv"]
+    assert per_call[0].attrs["epilogue"]["act"] == "relu" and per_call[0].attrs["epilogue"]["bias"] is not None
+    prepared = [s for s in steps if s.attrs.get("prepared") and s.kind == "ew"]
+    progs = [[i[0] for i in s.attrs["insts"]] for s in prepared]
+    assert ["add", "sqrt", "div"] in progs and ["mul"] in progs
+    assert (["sub", "mul", "add"] if with_conv_bias else ["neg", "mul", "add"]) in progs
+    # every operand of the prepared programs is a graph input or another prepared value, never the activation
+    for s in prepared:
+        assert all(v.name != "x" for v in s.inputs)
+
+
+def test_batch_norm_is_not_folded_when_the_convolution_has_another_reader_or_the_statistics_are_computed():
+    g = run_llh_pipeline(_conv_bn_graph(second_reader=True))
+    assert "conv" in g.op_names() and "conv_bias" not in g.op_names()
+    assert [s.kind for s in make_plan(g) if s.kind not in ("view", "constant")] == ["conv", "ew", "ew"]
+    # statistics that the graph computes (not weights) stay with the decomposition
+    g2 = Graph()
+    x = g2.add_input((2, 8, 16, 16), f32, "x")
+    w = g2.add_input((8, 8, 3, 3), f32, "w")
+    v = g2.add_input((8,), f32, "v")
+    var = g2.add_op("exp", [v])
+    y = g2.add_op("conv", [x, w], {"dilation": (1, 1), "kernel_shape": (3, 3), "pad": (1, 1, 1, 1), "stride": (1, 1), "group": 1})
+    z = g2.add_op("batch_norm_inference", [y, v, v, v, var], {"epsilon": 1e-5, "momentum": 0.1, "feature_index": 1})
+    g2.set_outputs([z])
+    run_llh_pipeline(g2)
+    assert "conv_bias" not in g2.op_names() and not g2.prepared
+
+
+def test_batch_norm_fold_in_the_channels_last_layout():
+    g = run_llh_pipeline(_conv_bn_graph(layout="NHWC"), target_layout="NHWC")
+    per_call = [s for s in make_plan(g) if not s.attrs.get("prepared") and s.kind not in ("view", "constant")]
+    assert [s.kind for s in per_call] == ["conv"] and per_call[0].attrs["layout"] == "NHWC"
+
+
+# ---- a symbol's value as an operand of a tensor op: llh.scalar_cast (LLHOps.td:120-127; the importer writes
+#      scalar_cast + convert_to, fx_translate.py:309-323) ----
+def test_scalar_cast_of_a_symbol_becomes_an_immediate_of_the_program():
+    from llcompiler_amd.llh.text import parse_llh, print_llh
+    text = '''func.func @main(%arg0: tensor<?x4xf32> {func.input_symbol_0 = "s0"}) -> tensor<?x4xf32> attributes {entrance} {
+      %0 = "llh.constant"() <{value = 0 : i64}> : () -> i64
+      %1 = "llh.dim"(%arg0, %0) : (tensor<?x4xf32>, i64) -> i64
+      %c = "llh.constant"() <{value = 2 : i64}> : () -> i64
+      %2 = "llh.mul"(%1, %c) : (i64, i64) -> i64
+      %3 = "llh.scalar_cast"(%2) : (i64) -> tensor<1xi64>
+      %4 = "llh.convert_to"(%3) : (tensor<1xi64>) -> tensor<1xf32>
+      %5 = "llh.div"(%arg0, %4) : (tensor<?x4xf32>, tensor<1xf32>) -> tensor<?x4xf32>
+      return %5 : tensor<?x4xf32>
+    }'''
+    g = run_llh_pipeline(parse_llh(text))
+    assert g.op_names() == ["scalar_cast", "div"]           # the convert folded into the cast
+    cast = g.ops[0]
+    assert cast.results[0].dtype == f32 and evaluate(cast.attrs["value"], {"s0": 5}) == 10
+    ew = [s for s in make_plan(g) if s.kind == "ew"]
+    assert len(ew) == 1 and [v.name for v in ew[0].inputs] == ["arg0"]
+    (op, dst, a, b), = ew[0].attrs["insts"]
+    assert op == "div" and a == "in0" and isinstance(b, Expr) and evaluate(b, {"s0": 3}) == 6
+    # and it survives a trip through the printer
+    again = run_llh_pipeline(parse_llh(print_llh(g)))
+    (name,) = again.symbols()  # (the printer writes no symbol names: the reader makes one up for the dynamic extent)
+    assert again.op_names() == ["scalar_cast", "div"] and evaluate(again.ops[0].attrs["value"], {name: 7}) == 14
+
+
+def test_real_valued_symbol_expressions():
+    from llcompiler_amd.llh.expr import is_float, sqrt, to_float
+    e = 1.0 / sqrt(to_float(s0))
+    assert is_float(e) and not is_float(s0 * 2 + 1) and is_float(s0 / 4) and not is_float(s0 // 4)
+    assert evaluate(e, {"s0": 64}) == 0.125 and evaluate(s0 ** 2, {"s0": 3}) == 9 and evaluate(-(s0 / 4), {"s0": 2}) == -0.5
+    assert sqrt(16) == 4.0 and to_float(3) == 3.0
+
+
+def test_symbol_valued_operands_import_as_scalar_casts():
+    """x / x.shape[0] + x.sum(0) * x.shape[0] with a dynamic batch: the importer keeps the extent as an expression,
+    writes llh.scalar_cast for it (fx_translate.py:309-323 writes scalar_cast + convert_to) and the planner makes it an
+    immediate; scores / sqrt(q.shape[-1]) becomes the product's epilogue scale.  Nodes whose scalar arithmetic cannot
+    be kept are reported unsupported, so that the partitioner leaves them to eager instead of failing at import."""
+    from torch.export import Dim
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.importer.fx_importer import is_supported
+
+    class M(torch.nn.Module):
+        def forward(self, x):
+            return x / x.shape[0] + x.sum(0) * x.shape[0]
+
+    class S(torch.nn.Module):
+        def forward(self, q, k):
+            return (q @ k.transpose(-1, -2)) / torch._sym_sqrt(q.shape[-1])
+
+    cm = compile_module(M(), (torch.randn(4, 8),), dynamic_shapes=({0: Dim("b", min=2, max=64)},))
+    g = cm.engine.graph
+    casts = [op for op in g.ops if op.name == "scalar_cast"]
+    assert len(casts) == 2 and all(c.results[0].dtype == f32 for c in casts)
+    (name,) = g.symbols()
+    assert all(evaluate(c.attrs["value"], {name: 12}) == 12 for c in casts)
+    ew = [s for s in cm.engine.steps if s.kind == "ew"]
+    assert sorted(i[0] for s in ew for i in s.attrs["insts"]) == ["add", "div", "mul"]
+    d = Dim("d", min=2, max=64)
+    cs = compile_module(S(), (torch.randn(3, 4, 8), torch.randn(3, 4, 8)), dynamic_shapes=({2: d}, {2: d}))
+    (bmm,) = [s for s in cs.engine.steps if s.kind == "batch_matmul"]
+    alpha = bmm.attrs["epilogue"]["alpha"]
+    (name,) = cs.engine.graph.symbols()
+    assert isinstance(alpha, Expr) and evaluate(alpha, {name: 64}) == 0.125
+    # is_supported: a symbolic operand on a translator that has no place for one is refused up front
+    gm = torch.export.export(M(), (torch.randn(4, 8),), dynamic_shapes=({0: Dim("b", min=2, max=64)},)).run_decompositions().graph_module
+    calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+    assert all(is_supported(n) for n in calls)
+    sym_node = next(n for n in calls if n.target is torch.ops.aten.sym_size.int)
+    fake = next(n for n in calls if n.target is torch.ops.aten.sum.dim_IntList)
+    saved = fake.args
+    fake.args = (saved[0], sym_node)          # a reduction over a symbol-valued axis: no translator takes that
+    assert not is_supported(fake)
+    fake.args = saved
