@@ -20,7 +20,8 @@
  *    not share any.  An op entry point called outside a plan uses a buffer per (device, stream) that grows on
  *    demand, which is the only allocation an op entry point ever makes (nothing is synchronised; an outgrown
  *    buffer is kept until llc_hip_trim, since queued launches may still address it; growing is refused with
- *    LLC_ERR_UNSUPPORTED while the stream is being captured).  Calls on one stream follow each other, calls on
+ *    LLC_ERR_UNSUPPORTED while the stream is being captured: run the call once on that stream ahead of the
+ *    capture, and keep the stream to the graph).  Calls on one stream follow each other, calls on
  *    different streams use different buffers: op entry points are re-entrant per stream, like plans.  Two host
  *    threads must not issue work to the SAME stream at the same time.  llc_hip_matmul_static never allocates
  *    (see there).

@@ -112,7 +112,7 @@ int get_workspace(size_t bytes, void** out, hipStream_t stream) {
   if (!mine || bytes > mine->cap) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
-      return set_error(LLC_ERR_UNSUPPORTED, "this call needs %zu bytes of scratch memory and the stream is being captured: run it once "
+      return set_error(LLC_ERR_UNSUPPORTED, "this call needs %zu bytes of scratch memory and the stream is being captured: run it once on this stream "
                        "outside the capture, or record it into a plan", bytes);
     const size_t cap_bytes = ((bytes + bytes / 2) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
     void* fresh = nullptr;

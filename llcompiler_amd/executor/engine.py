@@ -903,12 +903,21 @@ class Instance:
             self._patch(g_in_ptrs, [t.data_ptr() for t in g_outs])
             side = torch.cuda.Stream(device=dev)
             side.wait_stream(torch.cuda.current_stream(dev))
+            # One run on the capture stream ahead of the capture: the library keeps scratch memory per stream and
+            # cannot allocate while a stream is being captured.  The graph then addresses that stream's buffer, so the
+            # stream stays with the instance and nothing else is ever issued to it.
+            with torch.cuda.stream(side):
+                sh = C.current_stream(dev)
+                for c in self.calls:
+                    c.launch(sh)
+            side.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
                 sh = C.current_stream(dev)
                 for c in self.calls:
                     c.launch(sh)
             self._graph, self._g_staging, self._g_outs, self._g_in_ptrs = graph, staging, g_outs, g_in_ptrs
+            self._g_stream = side
         except Exception:  # capture is an optimisation: fall back to per-kernel launches for this instance
             self._graph_failed = True
             self._graph = None

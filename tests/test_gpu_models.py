@@ -891,7 +891,9 @@ def test_random_conv_networks_in_bf16(seed):
         first = cm(x.cuda())
         second = cm(x.cuda())
     what = "random conv net %d in bf16: %s" % (seed, " ".join(net.kinds))
-    _assert_as_close_as_eager(first.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, what)
+    # (a batch norm folded into bf16 filters rounds them once more: see assert_as_close_as_eager)
+    _assert_as_close_as_eager(first.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, what,
+                              rms_factor=3.0 if "conv_bn" in net.kinds else 1.5)
     assert torch.equal(first, second), what + ": the recorded plan differs from the recording run"
 
 
@@ -1049,7 +1051,9 @@ def test_resnet18_with_batch_norms_plans_to_twenty_convolutions(oracle):
         assert_close(got.cpu().numpy(), composition(), F32_RTOL, F32_ATOL, "resnet18 with batch norms vs the oracle composition")
         assert_close(got.cpu().numpy(), m(x).numpy(), F32_RTOL, F32_ATOL, "resnet18 with batch norms vs torch eager")
         inst = list(cm.engine.instances.values())[0]
-        assert len(inst.calls) == 23 + 1   # + the layout copy behind the max-pool
+        names = [c.fn.__name__ for c in inst.calls]
+        # + the layout copies behind the max-pool (to channels-last) and in front of the average pool (back)
+        assert len(names) == 23 + 2 and names.count("llc_hip_conv2d") == 20 and names.count("llc_hip_elementwise") == 0, names
         assert torch.equal(cm(x.cuda()), got)
         # statistics and filters written in place: the folded filters follow
         for mod, ref in zip(mg.modules(), m.modules()):
@@ -1100,7 +1104,7 @@ def test_conv_batch_norm_units_through_the_backend(dt):
     if dt == torch.float32:
         assert_close(got.cpu().numpy(), eager, F32_RTOL, F32_ATOL, "conv-bn units fp32")
     else:
-        assert_as_close_as_eager(got.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, "conv-bn units bf16")
+        assert_as_close_as_eager(got.float().cpu().numpy(), eager, want64, BF16_RTOL, BF16_ATOL, "conv-bn units bf16", rms_factor=3.0)
 
 
 # ---- a symbol's value as an operand of a tensor op (llh.scalar_cast) ----

@@ -53,15 +53,20 @@ def assert_close_bf16(got, want, what=""):
     assert_close(got, want, BF16_RTOL, BF16_ATOL, what)
 
 
-def assert_as_close_as_eager(got, eager, want64, rtol, atol, what):
+def assert_as_close_as_eager(got, eager, want64, rtol, atol, what, rms_factor=1.5):
     """`got` against the float64 evaluation `want64`, measured by what a reference evaluation in the same storage
     type (`eager`: torch's own kernels, or the oracle rounded to the storage type) achieves on the same graph.  A fixed
     absolute floor is either too loose for well-conditioned outputs or too tight where the graph amplifies rounding
     (a layer norm over nearly constant rows, outputs that cancel to ~0), so three things are asked instead:
       * every element within the stated tolerance plus four times the reference's own WORST error (a bound on outliers),
-      * no more elements outside the plain stated tolerance than twice the reference's own count (+ 1e-5 of all):
-        an error on a few small outputs cannot hide inside the first bar's global slack,
-      * an rms error of at most 1.5 times the reference's (the bulk of the elements is as accurate as the reference's).
+      * no more elements outside the plain stated tolerance than twice the reference's own count (+ 1e-4 of all, at
+        least 3): an error on more than a few small outputs cannot hide inside the first bar's global slack,
+      * an rms error of at most `rms_factor` (1.5) times the reference's, unless it is under a quarter of the rms of
+        the plain tolerance itself (the bulk of the elements is as accurate as the reference's, or far inside the
+        stated tolerance: fp32 sums in another order than torch's pairwise ones are legitimately a few times noisier
+        at the 1e-9 level).  Networks in 16-bit storage whose batch norms are folded into their filters pass 3: the folded
+        filters are rounded to the storage type once more (every filter carries a relative error of 2^-9, which the
+        unfolded evaluation does not have), the price of one kernel per convolution unit.
     Returns the measured margins: the fractions of elements outside the plain bar (with atol, and with rtol alone)
     for `got` and for the reference, so that a test can print them."""
     got, eager, want64 = (np.asarray(t, dtype=np.float64) for t in (got, eager, want64))
@@ -75,10 +80,12 @@ def assert_as_close_as_eager(got, eager, want64, rtol, atol, what):
         raise AssertionError("%s: %d of %d elements outside rtol=%g atol=%g + 4 x the reference's own error %.3g; worst at %s: "
                              "got %r want %r" % (what, int(bad.sum()), bad.size, rtol, atol, noise, i, got[i], want64[i]))
     n_out, n_ref = int((err > plain).sum()), int((ref_err > plain).sum())
-    assert n_out <= 2 * n_ref + max(1, int(1e-5 * err.size)), \
+    assert n_out <= 2 * n_ref + max(3, int(1e-4 * err.size)), \
         "%s: %d elements outside rtol=%g atol=%g, the reference evaluation has %d" % (what, n_out, rtol, atol, n_ref)
     rms, ref_rms = float(np.sqrt((err ** 2).mean())), float(np.sqrt((ref_err ** 2).mean()))
-    assert rms <= 1.5 * ref_rms + 1e-12, "%s: rms error %.3g, the reference evaluation's %.3g" % (what, rms, ref_rms)
+    plain_rms = float(np.sqrt((plain ** 2).mean()))
+    assert rms <= max(rms_factor * ref_rms, 0.25 * plain_rms) + 1e-12, \
+        "%s: rms error %.3g, the reference evaluation's %.3g, the tolerance's rms %.3g" % (what, rms, ref_rms, plain_rms)
     rel_only = rtol * np.abs(want64)
     stats = {"n": int(err.size), "outside_plain": n_out / err.size, "outside_plain_reference": n_ref / err.size,
              "outside_rtol_only": float((err > rel_only).mean()), "outside_rtol_only_reference": float((ref_err > rel_only).mean()),
