@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LLC_HIP_ABI_VERSION 2
+#define LLC_HIP_ABI_VERSION 3
 #define LLC_MAX_RANK 8
 
 /* Element type codes.  0-6 are the reference's `enum Type` (Tensor.h:25-33, and the Python map
@@ -339,8 +339,10 @@ int64_t llc_plan_num_steps(const llc_plan_t* plan);
 /* Number of slots llc_hip_run reads from `params`: 1 + 5 per declared tensor. */
 int64_t llc_plan_num_params(const llc_plan_t* plan);
 /* Replays the plan.  `params` has the layout described above llc_hip_unpack_params; base/data are device
- * pointers.  Extents must equal the declared ones and strides too (LLC_ERR_SHAPE / LLC_ERR_LAYOUT
- * otherwise: the caller then picks or records the plan for that binding). */
+ * pointers.  Extents must equal the declared ones, strides too, and every tensor must lie at the same address
+ * modulo 16 as when the plan was recorded (the kernels and the scratch memory of a plan are chosen for that
+ * alignment) (LLC_ERR_SHAPE / LLC_ERR_LAYOUT otherwise: the caller then picks or records the plan for that
+ * binding). */
 int llc_hip_run(llc_plan_t* plan, void* const* params, void* stream);
 /* Plans on disk.  The reference's compile step leaves a shared object with the weights baked in
  * (src/Compiler/Compiler.cpp:306-330: the object is named after a hash of the module text) that a later process

@@ -89,6 +89,9 @@ struct Io {
   char* lo = nullptr;  // address range the tensor occupied while the plan was recorded
   char* hi = nullptr;
   bool output = false;
+  // address of the first element modulo 16 while the plan was recorded: kernels were chosen for that alignment
+  // (16-byte vector and direct-to-LDS paths, split reductions), so a run must bind the same class
+  unsigned align16 = 0;
 };
 
 struct Overlap {
@@ -482,6 +485,7 @@ extern "C" int llc_plan_declare_io(llc_plan_t* p, int is_output, const llc_tenso
   io.output = is_output != 0;
   io.lo = (char*)io.like.t.data;
   io.hi = io.lo ? io.lo + io.like.span_bytes() : nullptr;
+  io.align16 = (unsigned)((uintptr_t)io.lo % 16);
   p->io.push_back(std::move(io));
   Io& mine = p->io.back();
   mine.like.t.size = mine.like.t.stride = nullptr;  // the arrays moved with the copy; only like.size/.stride are read
@@ -570,6 +574,10 @@ extern "C" int llc_hip_run(llc_plan_t* p, void* const* params, void* stream) {
     }
     if (!data && !empty) return set_error(LLC_ERR_BAD_ARG, "run: tensor %zu has a null data pointer", k);
     p->bound[k] = data ? data + *off * dtype_size(like.t.type) : nullptr;
+    if (p->bound[k] && (uintptr_t)p->bound[k] % 16 != p->io[k].align16)
+      return set_error(LLC_ERR_LAYOUT, "run: tensor %zu lies at an address that is %u modulo 16, the plan was recorded with %u "
+                       "(its kernels and scratch memory were chosen for that alignment)", k,
+                       (unsigned)((uintptr_t)p->bound[k] % 16), p->io[k].align16);
   }
   for (const Overlap& ov : p->overlaps)
     if (p->bound[ov.second] - p->bound[ov.first] != ov.diff)
@@ -766,7 +774,7 @@ extern "C" int llc_plan_save(llc_plan_t* p, const char* path) {
   w.u64(p->n_inputs);
   for (const Io& io : p->io) {
     write_operand_shape(w, io.like);
-    w.u64(io.output ? 1 : 0);
+    w.u64((io.output ? 1u : 0u) | ((uint64_t)io.align16 << 8));
   }
   w.u64(p->symbols.size());
   for (int64_t v : p->symbols) w.i64(v);
@@ -859,7 +867,9 @@ extern "C" int llc_plan_load(const char* path, llc_plan_t** out) {
   for (Io& io : p->io) {
     if (!read_operand_shape(r, io.like) || !io.like.present) return bad("malformed tensor declaration");
     io.like.t.size = io.like.t.stride = nullptr;  // as after llc_plan_declare_io: only like.size / like.stride are read
-    io.output = r.u64() != 0;
+    const uint64_t flags = r.u64();
+    io.output = (flags & 1) != 0;
+    io.align16 = (unsigned)((flags >> 8) & 15);
   }
   const uint64_t n_sym = r.u64();
   if (!r.ok || n_sym > (1u << 20)) return bad("truncated symbol list");

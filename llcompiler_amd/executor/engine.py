@@ -863,7 +863,16 @@ class Instance:
             n_in = len(in_ptrs)
             for k, t in enumerate(outs):
                 blk.set_pointer(n_in + k, t.data_ptr())
-            self._plan.run(blk, stream)
+            try:
+                self._plan.run(blk, stream)
+            except C.LlcHipError as err:
+                if err.status != C.ERR_LAYOUT:
+                    raise
+                # an input at another address modulo 16 than when the plan was recorded (a view with a storage offset):
+                # the recorded kernel choices do not apply; the per-kernel entry points choose again for these addresses
+                self._patch(in_ptrs, [t.data_ptr() for t in outs])
+                for c in self.calls:
+                    c.launch(stream)
             return self._results(outs)
         self._patch(in_ptrs, [t.data_ptr() for t in outs])
         if USE_PLAN and not USE_GRAPHS:

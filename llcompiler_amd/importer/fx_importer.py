@@ -506,11 +506,12 @@ def _adaptive_avg_pool(ctx, node):
                                    check=lambda n: n.args[1] % n.args[0].meta["val"].dim() == n.args[0].meta["val"].dim() - 1)
 def _softmax(ctx, node):
     x = ctx.val(node.args[0])
-    y = ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
     dt = _out_dtype(node)  # half_to_float: a 16-bit input with an fp32 result
-    if y.dtype != dt:
-        y = ctx.g.add_op("convert_to", [y], {"dtype": dt})
-    return y
+    if x.dtype != dt:
+        # torch computes and returns fp32 probabilities from the 16-bit input: widen first, so that they are not
+        # rounded to the storage type on the way
+        x = ctx.g.add_op("convert_to", [x], {"dtype": dt})
+    return ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
 
 
 def _first_result_only(node):

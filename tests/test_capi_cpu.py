@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     L = ctypes.CDLL(C.LIB_PATH)
     for name in declared_symbols():
         assert hasattr(L, name), name
-    assert L.llc_hip_abi_version() == 2
+    assert L.llc_hip_abi_version() == 3
 
 
 def test_status_strings_and_null_argument_errors():

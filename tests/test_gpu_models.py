@@ -175,6 +175,55 @@ def test_config4_and_5_blocks_against_the_oracle_composition(oracle):
     assert_close(got.cpu().numpy(), t, F32_RTOL, F32_ATOL, "2-layer BERT stack vs the oracle composition")
 
 
+def test_config4_encoder_block_bf16_against_the_oracle_composition(oracle):
+    """Config 4's graph in its own storage type, held against the C oracle: the pre-LN encoder block spelt with the
+    oracle's primitives on bf16-valued weights and inputs, every op computed in fp32 and its result rounded to bf16
+    where the unfused graph has an op boundary (layer norm, each linear + bias, the scaled scores, the probabilities,
+    the context, each residual add, the GELU).  The yardstick is the float64 evaluation of the same bf16-valued module;
+    the compiled block must be as close to it as that oracle composition is, at the stated rtol 2e-2 (comparator of
+    record: llcompiler/test_models/utility.py:18-28).  The printed line gives the fraction of outputs outside the plain
+    bars."""
+    from tests.util import bf16_round as r16
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    enc = EncoderBlock().eval().to(torch.bfloat16)
+    (x,) = make_encoder_inputs(2, 64, dtype=torch.bfloat16)
+    encf = copy.deepcopy(enc).float()       # the same bf16-valued weights as fp32 arrays for the oracle
+    B, S, H = x.shape
+    nh, dh = enc.attn.heads, enc.attn.dh
+
+    def linear(t2d, lin):
+        return r16(r16(oracle.matmul(t2d, np.ascontiguousarray(lin.weight.detach().numpy().T), "mkn")) + lin.bias.detach().numpy()[None, :])
+
+    def layer_norm(ln, t):
+        return r16(_oracle_layer_norm(oracle, ln, t))
+
+    def attention(attn, t):
+        t2 = t.reshape(B * S, H)
+
+        def split(u):
+            return np.ascontiguousarray(u.reshape(B, S, nh, dh).transpose(0, 2, 1, 3)).reshape(B * nh, S, dh)
+        q, k, v = (split(linear(t2, l)) for l in (attn.q, attn.k, attn.v))
+        sc = r16(r16(oracle.batch_matmul(q, np.ascontiguousarray(k.transpose(0, 2, 1)), "mkn")) / np.float32(np.sqrt(dh)))
+        p = r16(oracle.softmax_lastdim(np.ascontiguousarray(sc.reshape(-1, S), dtype=np.float32))).reshape(B * nh, S, S)
+        ctx = r16(oracle.batch_matmul(p, v, "mkn")).reshape(B, nh, S, dh).transpose(0, 2, 1, 3).reshape(B * S, H)
+        return linear(np.ascontiguousarray(ctx), attn.o).reshape(B, S, H)
+
+    xn = x.float().numpy()
+    h = r16(xn + attention(encf.attn, layer_norm(encf.ln1, xn)))
+    f = r16(oracle.unary("gelu", linear(layer_norm(encf.ln2, h).reshape(-1, H), encf.fc1)))
+    composed = r16(h + linear(f, encf.fc2).reshape(h.shape))
+    with torch.no_grad():
+        want64 = copy.deepcopy(enc).double()(x.double()).numpy()
+        got = compile_module(copy.deepcopy(enc).cuda(), (x.cuda(),))(x.cuda())
+    assert got.dtype == torch.bfloat16
+    stats = assert_as_close_as_eager(got.float().cpu().numpy(), composed, want64, BF16_RTOL, 0.0,
+                                     "encoder block bf16 (B=2, S=64) vs the oracle composition, rtol 2e-2 alone")
+    # outputs near zero miss a purely relative bar in any bf16 evaluation (the oracle composition on 4.6 % of them, the
+    # compiled block on 3.5 %): the compiled block must not miss it more often than the composition does
+    assert stats["outside_rtol_only"] <= 1.25 * stats["outside_rtol_only_reference"] + 1e-3
+
+
 def _kernel_names(engine):
     return [[c.fn.__name__ for c in inst.calls] for inst in engine.instances.values()]
 
@@ -332,7 +381,8 @@ def test_softmax_half_to_float_and_int32_embedding():
         got = opt(x.cuda())
         want = torch.softmax(x.cuda(), dim=-1, dtype=torch.float32).cpu()
     assert got.dtype == torch.float32
-    assert_close(got.cpu().numpy(), want.numpy(), 2e-3, 1e-4, "softmax half_to_float")
+    # (the input is widened before the softmax, so the probabilities carry fp32 error, not the storage type's)
+    assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "softmax half_to_float")
     torch.manual_seed(4)
     e = E().eval()
     idx = torch.randint(0, 37, (3, 7), generator=torch.Generator().manual_seed(5)).to(torch.int32)

@@ -491,6 +491,58 @@ def test_two_plans_with_split_reductions_run_on_two_streams_at_once():
         np.testing.assert_array_equal(out.cpu().numpy(), want.cpu().numpy())
 
 
+def test_a_plan_refuses_tensors_at_another_alignment_and_the_engine_relaunches_kernel_by_kernel():
+    """Kernels and scratch memory of a plan are chosen for the 16-byte alignment class of the tensors it was recorded
+    with (a misaligned operand takes no split reduction and needs no scratch memory; an aligned one does): llc_hip_run
+    refuses a tensor at another address modulo 16 with LLC_ERR_LAYOUT, and the engine then launches that call's kernels
+    one by one, which choose again."""
+    from llcompiler_amd import _capi as C
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.executor.plan_runner import ParamBlock, Plan
+    C.init(0)
+    L = C.lib()
+    M, N, K = 512, 768, 3072
+    gen = torch.Generator().manual_seed(7)
+    w = (torch.rand(N, K, generator=gen) * 2 - 1).cuda()
+    base = (torch.rand(M * K + 8, generator=gen) * 2 - 1).cuda()
+    odd = base[1:1 + M * K].view(M, K)         # 4 bytes past a 16-byte boundary
+    even = base[4:4 + M * K].view(M, K)
+    assert odd.data_ptr() % 16 == 4 and even.data_ptr() % 16 == 0
+    out = torch.empty((M, N), device="cuda")
+    plan = Plan()
+    for t, is_out in ((odd, False), (w, False), (out, True)):
+        plan.declare_io(t, is_out)
+    with plan.recording():
+        C.check(L.llc_hip_matmul(C.tensor_ref(odd).ptr, C.tensor_ref(w.t()).ptr, None, C.tensor_ref(out).ptr, _stream()))
+    torch.cuda.synchronize()
+    want_odd = out.clone()
+    with pytest.raises(C.LlcHipError) as err:
+        plan.run(ParamBlock([even, w, out]), _stream())
+    assert err.value.status == C.ERR_LAYOUT and "modulo 16" in str(err.value)
+    out.fill_(float("nan"))
+    plan.run(ParamBlock([odd, w, out]), _stream())
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), want_odd.cpu().numpy())
+
+    class Lin(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = torch.nn.Linear(K, N, bias=False)
+
+        def forward(self, x):
+            return self.fc(x)
+
+    m = Lin().eval().cuda()
+    with torch.no_grad():
+        cm = compile_module(m, (even,))
+        first = cm(even)
+        assert torch.equal(cm(even), first)                      # the recorded plan
+        got_odd = cm(odd)                                        # same shape and strides, another alignment class
+        assert len(cm.engine.instances) == 1
+        torch.testing.assert_close(got_odd, m(odd), rtol=1e-4, atol=1e-4)
+        assert torch.equal(cm(even), first)
+
+
 def test_op_calls_with_split_reductions_run_on_two_streams_at_once():
     """Op entry points called outside a plan keep the partial sums of a split reduction in a scratch buffer per
     (device, stream): the same product issued on two streams at the same time gives, bit for bit, what each call

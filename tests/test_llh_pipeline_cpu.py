@@ -543,3 +543,19 @@ def test_symbol_valued_operands_import_as_scalar_casts():
     fake.args = (saved[0], sym_node)          # a reduction over a symbol-valued axis: no translator takes that
     assert not is_supported(fake)
     fake.args = saved
+
+
+def test_softmax_half_to_float_widens_before_the_softmax():
+    """aten._softmax(x, -1, half_to_float=True) on a 16-bit input returns fp32 probabilities computed in fp32: the
+    convert sits in front of llh.softmax, not behind it."""
+    from llcompiler_amd.compiler.aot import compile_module
+
+    class S(torch.nn.Module):
+        def forward(self, x):
+            return torch.softmax(x, dim=-1, dtype=torch.float32)
+
+    g = compile_module(S(), (torch.randn(4, 16).to(torch.float16),)).engine.graph
+    names = g.op_names()
+    assert names.index("convert_to") < names.index("softmax")
+    sm = next(op for op in g.ops if op.name == "softmax")
+    assert sm.operands[0].dtype == f32 and sm.results[0].dtype == f32
