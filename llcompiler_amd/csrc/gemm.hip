@@ -421,7 +421,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
       else x += f16_bits_to_f32(bb);
       if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
       if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
-      else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
+      else if (p.act == LLC_ACT_GELU) x = gelu_for<T>(x);
       xs[e] = x;
     }
     *(u32x4_t*)(C + o) = u32x4_t{pack_pair<Elem<T>::kDtype>(xs[0], xs[1]), pack_pair<Elem<T>::kDtype>(xs[2], xs[3]),
@@ -608,7 +608,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       else x += f16_bits_to_f32(bb);
       if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
       if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
-      else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
+      else if (p.act == LLC_ACT_GELU) x = gelu_for<T>(x);
       xs[e] = x;
     }
     *(u32x4_t*)(C + o) = u32x4_t{pack_pair<Elem<T>::kDtype>(xs[0], xs[1]), pack_pair<Elem<T>::kDtype>(xs[2], xs[3]),
@@ -836,14 +836,6 @@ int launch_splitk(const GemmParams& p, int splits, hipStream_t s) {
 // One workgroup per CU: the cost of a candidate is its number of rounds over the 256 CUs times the tile's work,
 // weighted by how well that tile shape runs (narrower tiles read more LDS and L2 bytes per MFMA).
 inline int wide_tile_n(const GemmParams& p, int batch, bool b_kvec) {
-#ifdef LLC_GEMM_TUNE
-  if (const char* e = getenv("LLC_WIDE")) {
-    const int bn = atoi(e);
-    if (bn == 0) return 0;
-    if (p.N % bn == 0 && (bn == 256 || bn == 128 || (bn == 192 && b_kvec))) return bn;
-    return 0;
-  }
-#endif
   int best = 0;
   double best_cost = 0.0;
   const int cand[3] = {256, 192, 128};
@@ -909,10 +901,6 @@ int launch_loaders(const GemmParams& p, int batch, hipStream_t s) {
 
 int conv_wide_16bit(int dtype, const char* x, const char* w, char* y, const char* bias, const char* residual, int F,
                     const ConvWideGeom& g, float alpha, int act, hipStream_t s) {
-#ifdef LLC_GEMM_TUNE
-  if (const char* e = getenv("LLC_CONV_WIDE"))
-    if (atoi(e) == 0) return 1;
-#endif
   const int64_t K = (int64_t)g.KH * g.KW * g.C;
   // (reductions shorter than 2048 are too few k-tiles per tile for one workgroup per CU: a tile's fill and drain weigh
   // as much as its loop, and the kernels that keep two workgroups on a CU are faster; measured at batch 32:
@@ -1150,11 +1138,3 @@ extern "C" int llc_hip_matmul_static(const llc_tensor* lhs, const llc_tensor* rh
   return llc_impl_matmul(lhs, rhs, epi, out, stream);
 }
 
-#ifdef LLC_GEMM_TUNE
-// tuning builds only: shader clocks and 100 MHz ticks of the longest workgroup since the last call
-extern "C" void llc_dbg_read(unsigned long long* out) {
-  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(llc::llc_dbg_clk), 16);
-  unsigned long long z[2] = {0, 0};
-  (void)hipMemcpyToSymbol(HIP_SYMBOL(llc::llc_dbg_clk), z, 16);
-}
-#endif

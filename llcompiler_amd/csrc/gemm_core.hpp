@@ -311,7 +311,7 @@ __device__ __forceinline__ void epilogue_store(T* C, int64_t o, float acc, float
   float v = acc * alpha + bias;
   if (res) v += load_as_f32(res, dt, o);
   if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
-  else if (act == LLC_ACT_GELU) v = gelu_exact(v);
+  else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
   if constexpr (dt == LLC_FLOAT32) C[o] = v;
   else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o] = f32_to_bf16_bits(v);
   else ((uint16_t*)C)[o] = f32_to_f16_bits(v);

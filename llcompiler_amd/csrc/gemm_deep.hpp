@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void gemm_deep_kernel(const GemmParams p) {
       else x += f16_bits_to_f32(bb);
       if (res) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
       if (p.act == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
-      else if (p.act == LLC_ACT_GELU) x = gelu_exact(x);
+      else if (p.act == LLC_ACT_GELU) x = gelu_for<T>(x);
       xs[e] = x;
     }
     *(u32x4_t*)(C + o) = u32x4_t{pack_pair<Elem<T>::kDtype>(xs[0], xs[1]), pack_pair<Elem<T>::kDtype>(xs[2], xs[3]),

@@ -73,7 +73,6 @@ __global__ __launch_bounds__(256) void bmm_sweep_kernel(const GemmParams p, int 
   using G = SweepGeom<T>;
   constexpr int ES = G::kES, NB = G::NB;
   extern __shared__ __align__(16) char smem[];
-  LLC_DBG_T0();
   int panel, range, z;
   tile_and_batch_of_block(p.tiles_m, p.tiles_n, panel, range, z);
   const int m0 = panel * 64;
@@ -286,7 +285,7 @@ __global__ __launch_bounds__(256) void bmm_sweep_kernel(const GemmParams p, int 
 #pragma unroll
       for (int j = 0; j < NB; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = gelu_exact(acc[j][r]);
+        for (int r = 0; r < 16; ++r) acc[j][r] = gelu_for<T>(acc[j][r]);
     }
     // through the wave's own LDS tile, so that a store instruction writes whole 128-byte lines (straight from the
     // accumulators it would write 32 bytes of each of 32 rows: four times the line accesses, which is what the
@@ -335,7 +334,6 @@ __global__ __launch_bounds__(256) void bmm_sweep_kernel(const GemmParams p, int 
     tile(S1{}, it + 1);
   }
   if (it < nt) tile(S0{}, it);
-  LLC_DBG_T1();
 }
 
 // Whether the sweep kernel takes this product; the caller has checked operand alignment (a_kvec, b_rvec).
@@ -363,12 +361,6 @@ int launch_sweep(const GemmParams& p0, int batch, hipStream_t s) {
   const int64_t places = 256 * 3;
   int ranges = 1;
   while ((int64_t)(p.M / 64) * batch * ranges * 2 <= places && (nt / ranges) % 2 == 0) ranges *= 2;
-#ifdef LLC_GEMM_TUNE
-  if (const char* e = getenv("LLC_SWEEP_RANGES")) {
-    const int r = atoi(e);
-    if (r > 0 && nt % r == 0) ranges = r;
-  }
-#endif
   p.tiles_m = p.M / 64;
   p.tiles_n = ranges;
   const int64_t wgs = (int64_t)p.tiles_m * ranges;

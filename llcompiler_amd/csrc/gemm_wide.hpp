@@ -7,18 +7,6 @@
 
 #define LLC_WAIT_VM(VM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (7 << 4) | (15 << 8) | (((VM) >> 4) << 14))
 
-#ifdef LLC_GEMM_TUNE
-__device__ unsigned long long llc_dbg_clk[2];  // longest workgroup: shader clocks, 100 MHz ticks
-#define LLC_DBG_T0() const long long dbg_c0 = clock64(), dbg_w0 = wall_clock64()
-#define LLC_DBG_T1()                                                                   \
-  if (threadIdx.x == 0) {                                                              \
-    atomicMax(&llc_dbg_clk[0], (unsigned long long)(clock64() - dbg_c0));              \
-    atomicMax(&llc_dbg_clk[1], (unsigned long long)(wall_clock64() - dbg_w0));         \
-  }
-#else
-#define LLC_DBG_T0()
-#define LLC_DBG_T1()
-#endif
 
 // ---------------------------------------------------------------------------------------------
 // FOUR waves, one per SIMD, each owning a 128 x BN/2 accumulator tile (up to 256 accumulator registers per
@@ -93,7 +81,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   using G = WideGeom<BN>;
   constexpr int TM = G::TM, TN = G::TN;
   extern __shared__ __align__(16) char smem[];
-  LLC_DBG_T0();
   int tile_m, tile_n;
   int z;
   tile_and_batch_of_block(p.tiles_m, p.tiles_n, tile_m, tile_n, z);
@@ -329,42 +316,76 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const T* bias = p.bias ? (const T*)p.bias + (int64_t)z0 * p.bias_sb : nullptr;
   char* wst = smem + wave * G::kOutWave;
   const int ncol0 = n0 + wn * G::WTN, mrow0 = m0 + wm * 128;
+  // Row block by row block: for one block of 32 rows a lane's sixteen residual loads (8 bytes each) cover, together
+  // with the other lanes', 32 rows x 512 contiguous bytes, so every 128-byte line that is fetched is used whole
+  // while it is still in the CU's cache (walking the row blocks inside each column group instead cycles through
+  // 128 rows x 16 bytes and fetches every line eight times); the next block's loads are requested before this
+  // block's arithmetic.
   auto stage_out = [&](auto act_tag, auto res_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     constexpr bool RES = decltype(res_tag)::value;
+    uint2 bq[TN][4];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int col = j * 32 + 8 * q + 4 * lh;  // first of 4 consecutive columns, inside the wave tile
-        uint2 bq = {0, 0};
-        if (bias) bq = *(const uint2*)(bias + ncol0 + col);
+        bq[j][q] = uint2{0, 0};
+        if (bias) bq[j][q] = *(const uint2*)(bias + ncol0 + j * 32 + 8 * q + 4 * lh);
+      }
+    uint2 rq[2][TN][4];
+    auto load_res = [&](int i, int buf) {
+      if constexpr (RES) {
+        // rows past the last pixel of a convolution are computed and dropped: read their residual from the last row
+        const int row = i * 32 + li;
+        const int rrow = (CONV && mrow0 + row >= p.M) ? p.M - 1 : mrow0 + row;
+        const T* rp = res + (int64_t)rrow * p.c_sm + ncol0 + 4 * lh;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int row = i * 32 + li;
-          uint2 rq = {0, 0};
-          if constexpr (RES) {
-            // rows past the last pixel of a convolution are computed and dropped: read their residual from the last row
-            const int rrow = (CONV && mrow0 + row >= p.M) ? p.M - 1 : mrow0 + row;
-            rq = *(const uint2*)(res + (int64_t)rrow * p.c_sm + ncol0 + col);
-          }
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) rq[buf][j][q] = *(const uint2*)(rp + j * 32 + 8 * q);
+      }
+    };
+    load_res(0, 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      if (i + 1 < TM) load_res(i + 1, (i + 1) & 1);
+      const int row = i * 32 + li;
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int col = j * 32 + 8 * q + 4 * lh;  // first of 4 consecutive columns, inside the wave tile
+          const uint2 bw2 = bq[j][q];
+          uint2 rw2 = {0, 0};
+          if constexpr (RES) rw2 = rq[i & 1][j][q];
           float xv[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const uint32_t bw = e < 2 ? bq.x : bq.y, rw = e < 2 ? rq.x : rq.y;
+            const uint32_t bw = e < 2 ? bw2.x : bw2.y, rw = e < 2 ? rw2.x : rw2.y;
             const uint16_t bb = (uint16_t)(bw >> (16 * (e & 1))), rb = (uint16_t)(rw >> (16 * (e & 1)));
             float x = acc[i][j][4 * q + e] * p.alpha;
             if constexpr (Elem<T>::kDtype == LLC_BFLOAT16) x += bf16_bits_to_f32(bb);
             else x += f16_bits_to_f32(bb);
             if constexpr (RES) x += (Elem<T>::kDtype == LLC_BFLOAT16) ? bf16_bits_to_f32(rb) : f16_bits_to_f32(rb);
             if constexpr (ACT == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
-            else if constexpr (ACT == LLC_ACT_GELU) x = gelu_exact(x);
+            else if constexpr (ACT == LLC_ACT_GELU) x = gelu_for<T>(x);
             xv[e] = x;
           }
           *(uint2*)(wst + row * G::kOutPitch + col * 2) =
               uint2{pack_pair<Elem<T>::kDtype>(xv[0], xv[1]), pack_pair<Elem<T>::kDtype>(xv[2], xv[3])};
         }
+      // this block of 32 rows goes out now, as 16-byte pieces of whole rows: its stores drain while the next block's
+      // arithmetic runs (the stores of a whole tile issued together at the end cost 10 us of a 93 us product)
+      constexpr int kChunks = G::WTN / 8;   // 16-byte chunks per row of the wave tile
+      constexpr int kIts = kChunks / 2;     // 64 lanes cover 64 / kChunks rows: kIts steps per 32 rows
+#pragma unroll
+      for (int it = 0; it < kIts; ++it) {
+        const int idx = (i * kIts + it) * 64 + lane;
+        const int orow = idx / kChunks, ch = idx % kChunks;
+        const u32x4_t v = *(const u32x4_t*)(wst + orow * G::kOutPitch + ch * 16);
+        if (!CONV || mrow0 + orow < p.M) *(u32x4_t*)(C + (int64_t)(mrow0 + orow) * p.c_sm + ncol0 + ch * 8) = v;
       }
+    }
   };
   auto with_res = [&](auto act_tag) {
     if (res) stage_out(act_tag, std::true_type{});
@@ -373,15 +394,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   if (p.act == LLC_ACT_GELU) with_res(std::integral_constant<int, LLC_ACT_GELU>{});
   else if (p.act == LLC_ACT_RELU) with_res(std::integral_constant<int, LLC_ACT_RELU>{});
   else with_res(std::integral_constant<int, LLC_ACT_NONE>{});
-  constexpr int kChunks = G::WTN / 8;  // 16-byte chunks per row of the wave tile
-#pragma unroll
-  for (int it = 0; it < 2 * kChunks; ++it) {
-    const int idx = it * 64 + lane;
-    const int row = idx / kChunks, ch = idx % kChunks;
-    const u32x4_t v = *(const u32x4_t*)(wst + row * G::kOutPitch + ch * 16);
-    if (!CONV || mrow0 + row < p.M) *(u32x4_t*)(C + (int64_t)(mrow0 + row) * p.c_sm + ncol0 + ch * 8) = v;
-  }
-  LLC_DBG_T1();
 }
 
 template <typename T, int BMODE, int BN, bool CONV = false>

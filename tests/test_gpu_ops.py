@@ -850,6 +850,46 @@ def test_batch_matmul_16bit_complete_tiles(ops, oracle):
     assert_close_bf16(host(ops.batch_matmul(dev(a, torch.bfloat16), bt.transpose(1, 2))), want, "bmm bf16 NT")
 
 
+def _gelu_16bit_restated(x):
+    """The GELU that the epilogues of the 16-bit products apply, restated in numpy fp32: x / (1 + 2^(-x p(x^2)))."""
+    f = np.float32
+    x = x.astype(f)
+    u = x * x
+    p = f(2.2971660592200047) + u * (f(0.1095363857595901) + u * (f(-0.0014344055324419125) + u * f(1.327634682739151e-05)))
+    with np.errstate(over="ignore"):
+        e = np.exp2((-x * p).astype(f)).astype(f)
+    return (x / (f(1) + e)).astype(f)
+
+
+def test_gelu_of_the_16bit_epilogues_against_the_oracle(ops, oracle):
+    """The epilogues of the 16-bit products replace the erf form of GELU by a cheaper one (their results are rounded to
+    bf16 / f16 anyway).  Its formula in fp32, against the oracle's erf form on 65536 points of [-8, 8): absolute error
+    below 2.5e-4, relative error below 1.5e-3 on [-5, 5].  Then the kernels themselves: a product spelt so that output
+    (i, j) is gelu(r_i + c_j) with r_i + c_j exact in fp32, against the oracle's gelu rounded to the storage type, at
+    the stated tolerance and at one unit of the storage type's precision."""
+    r_vals = (np.arange(256, dtype=np.float32) - 128) / 16          # -8 .. 8 in steps of 1/16: exact in bf16 and f16
+    c_vals = np.arange(256, dtype=np.float32) / 4096                # 0 .. 1/16 in steps of 2^-12: exact in both
+    x = (r_vals[:, None] + c_vals[None, :]).astype(np.float32)
+    want = oracle.unary("gelu", x)
+    formula = _gelu_16bit_restated(x)
+    err = np.abs(formula.astype(np.float64) - want.astype(np.float64))
+    inside = np.abs(x) <= 5
+    rel = err[inside] / np.maximum(np.abs(want[inside]).astype(np.float64), 1e-30)
+    print("16-bit epilogue GELU, formula in fp32 vs the oracle: max abs error %.3g, max relative error on [-5, 5] %.3g"
+          % (err.max(), rel[np.abs(x[inside]) > 1e-3].max()))
+    assert err.max() <= 2.5e-4 and rel[np.abs(x[inside]) > 1e-3].max() <= 1.5e-3
+    a = np.zeros((256, 64), np.float32)
+    a[:, 0] = r_vals
+    b = np.zeros((64, 256), np.float32)
+    b[0, :] = 1.0
+    for dt, unit in ((torch.bfloat16, 2.0 ** -8), (torch.float16, 2.0 ** -9)):
+        got = host(ops.matmul(dev(a, dt), dev(b, dt), ops.Epilogue(bias=dev(c_vals, dt), act="gelu")))
+        rounded = host(dev(want, dt))
+        assert_close_bf16(got, rounded, "gelu epilogue %s" % dt)
+        off = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert (off <= unit * np.abs(want) + 2.5e-4).all(), "gelu epilogue %s: %g" % (dt, (off - unit * np.abs(want)).max())
+
+
 def test_matmul_epilogue(ops, oracle):
     r = rng(21)
     M, N, K = 70, 136, 200
