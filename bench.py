@@ -50,6 +50,17 @@ class Case:
         self.calls[i % self.sets].launch()
 
 
+class _Sequence:
+    """Several prepared calls launched one after the other: a group of kernels timed as one case."""
+
+    def __init__(self, calls):
+        self.calls = calls
+
+    def launch(self, stream=None):
+        for c in self.calls:
+            c.launch(stream)
+
+
 class _Cases(list):
     """Collects the suite; with a filter only the named cases are built (their operands allocated)."""
 
@@ -152,6 +163,34 @@ def build_extra_cases(ops, device, only=()):
                                            (_uniform((f, c, 3, 3), bf, gen, device) * 0.05).contiguous(memory_format=cl),
                                            torch.empty((32, f, hw, hw), dtype=bf, device=device).contiguous(memory_format=cl)),
                   lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 2)
+    # The fallbacks: shapes the fast paths do not take.  Convolutions whose channel count is no multiple of 128 bytes'
+    # worth of values, or that are grouped, run in NCHW on conv_f32_kernel (fp32) / conv_kernel (16-bit, element-wise
+    # gather); attention layers whose head dim is not 64 keep their three kernels (scores with the scale in the
+    # epilogue, softmax, probabilities x values), the [B H, S, S] scores going through HBM.
+    for dt_name, dt, es in (("f32", torch.float32, 4), ("bf16", bf, 2)):
+        cases.add("conv3x3_48ch_56x56_nchw", dt_name, "mfma", 2.0 * 16 * 56 * 56 * 48 * 48 * 9, (16 * 48 * 56 * 56 * 2 + 48 * 48 * 9) * es,
+                  lambda dt=dt: (_uniform((16, 48, 56, 56), dt, gen, device), _uniform((48, 48, 3, 3), dt, gen, device) * 0.05,
+                                 torch.empty((16, 48, 56, 56), dtype=dt, device=device)),
+                  lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), out=o, defer=True), 2)
+        cases.add("conv3x3_128ch_groups32_28x28_nchw", dt_name, "mfma", 2.0 * 16 * 28 * 28 * 128 * 4 * 9, (16 * 128 * 28 * 28 * 2 + 128 * 4 * 9) * es,
+                  lambda dt=dt: (_uniform((16, 128, 28, 28), dt, gen, device), _uniform((128, 4, 3, 3), dt, gen, device) * 0.05,
+                                 torch.empty((16, 128, 28, 28), dtype=dt, device=device)),
+                  lambda x, w, o: ops.conv2d(x, w, pad=(1, 1, 1, 1), group=32, out=o, defer=True), 2)
+    for hd in (32, 128):
+        bh, sq = 8 * 12, 512
+
+        def make_attn(hd=hd):
+            q, k, v = (_uniform((bh, sq, hd), bf, gen, device) for _ in range(3))
+            return (q, k, v, torch.empty((bh, sq, sq), dtype=bf, device=device), torch.empty((bh, sq, sq), dtype=bf, device=device),
+                    torch.empty((bh, sq, hd), dtype=bf, device=device))
+
+        def run_attn(q, k, v, sc, pr, o, hd=hd):
+            return _Sequence([ops.batch_matmul(q, k.transpose(1, 2), ops.Epilogue(alpha=hd ** -0.5), out=sc, defer=True),
+                              ops.softmax(sc, out=pr, defer=True), ops.batch_matmul(pr, v, out=o, defer=True)])
+        # algorithmic bytes: q, k, v in and the result out, once (what a fused kernel moves); the three kernels move the
+        # scores four more times
+        cases.add("attention_unfused_headdim%d_batch8_seq512" % hd, "bf16", "mfma", 4.0 * bh * sq * sq * hd, 4 * bh * sq * hd * 2,
+                  make_attn, run_attn, 2)
     cases.add("conv7x7_stem_3to64_224", "f32", "mfma", 2.0 * 16 * 112 * 112 * 64 * 147, (16 * 3 * 224 * 224 + 64 * 147 + 16 * 64 * 112 * 112) * 4,
               lambda: (_uniform((16, 3, 224, 224), torch.float32, gen, device), _uniform((64, 3, 7, 7), torch.float32, gen, device) * 0.05,
                        torch.empty((16, 64, 112, 112), dtype=torch.float32, device=device)),
@@ -312,18 +351,29 @@ def flop_bert(seq, batch=8, layers=12, hidden=768):
 
 
 def _call_times_ms(f, n, warmup):
-    """Per-call device time of f(): one HIP event pair per call on the stream the kernels are launched on (torch's
-    current stream), calls issued back to back, host dispatch included in what the device sees."""
+    """Time per call of f(), calls issued back to back, host dispatch included in what the device sees: HIP events on
+    the stream the kernels are launched on (torch's current stream) around GROUPS of calls, each group's time divided
+    by its size.  Recording an event costs 4 us of host time on this platform, which a call of 10 us (the MLP: two
+    kernels, host-bound) would be charged with if every call had an event pair of its own; groups are sized so that one
+    lasts about 200 us (one call per group from 0.2 ms per call upwards)."""
     for _ in range(warmup):
         f()
     torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(5):
+        f()
+    b.record()
+    torch.cuda.synchronize()
+    group = max(1, min(32, int(0.2 / max(a.elapsed_time(b) / 5, 1e-4))))
     evs = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
     evs[0].record()
     for i in range(n):
-        f()
+        for _ in range(group):
+            f()
         evs[i + 1].record()
     torch.cuda.synchronize()
-    return sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(n))
+    return sorted(evs[i].elapsed_time(evs[i + 1]) / group for i in range(n))
 
 
 def _stats(times, flops, dtype_name):
@@ -343,7 +393,7 @@ def model_latencies(which=MODELS, calls=100):
     run in.  Reported next to the suite, not part of `value`.  `which` selects a subset."""
     import warnings
     from llcompiler_amd.compiler.aot import compile_module
-    from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18Folded, make_bert_inputs,
+    from llcompiler_amd.test_models import (MLP, BertEncoder, EncoderBlock, ResNet18BN, ResNet18Folded, make_bert_inputs,
                                             make_encoder_inputs, make_mlp_inputs, make_resnet_inputs)
     warnings.filterwarnings("ignore")
     res = {}
@@ -356,6 +406,10 @@ def model_latencies(which=MODELS, calls=100):
             xs = make_resnet_inputs(16, 224)[0].cuda()
             cr = compile_module(ResNet18Folded().cuda(), (xs,))
             res["resnet18_f32_batch16"] = _stats(_call_times_ms(lambda: cr(xs), calls, 3), FLOP_RESNET18_B16, "f32")
+            # the network as torchvision spells it (Conv2d without bias -> BatchNorm2d, eval mode, randomised statistics):
+            # the batch norms are folded into the filters when the plan is made, a call launches the same kernels
+            cn = compile_module(ResNet18BN().cuda(), (xs,))
+            res["resnet18_batchnorm_f32_batch16"] = _stats(_call_times_ms(lambda: cn(xs), calls, 3), FLOP_RESNET18_B16, "f32")
             # the same network in bf16 storage (not one of the five configurations: its convolutions run on the
             # bf16 matrix instructions, which the fp32 configuration cannot show)
             xh = xs.to(torch.bfloat16)
@@ -500,6 +554,14 @@ def main():
     }
     if extra_rows:
         out["extra_kernels"] = extra_rows
+    # `roofline` describes the kernel that takes the largest share of the pass (the fp32 matmul, measured against the
+    # fp32 matrix peak).  The rows the throughput targets are written for, side by side: contractions on the bf16
+    # matrix instructions against 2.5 PFLOP/s (target 0.50) and the bandwidth-bound kernels against 8 TB/s (target 0.70).
+    rows = kernels + extra_rows
+    out["target_rows"] = {
+        "mfma_bf16_frac_of_2500_tflops": {k["kernel"]: k["frac"] for k in rows if k["bound"] == "mfma" and k["kernel"].endswith("bf16")},
+        "hbm_frac_of_8000_gbs": {k["kernel"]: k["frac"] for k in rows if k["bound"] == "hbm"},
+    }
     if not args.no_models and models:
         try:
             configs = model_latencies(models)
