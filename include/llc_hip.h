@@ -158,7 +158,10 @@ typedef struct llc_conv_attrs {
  * Layout travels in the strides, as in torch: either every tensor (x, w, out, epilogue residual) is contiguous
  * NCHW / FCHW, or every one is channels-last (NHWC in memory: strides (H W C, 1, W C, C) under the same
  * logical shape), which takes a kernel of its own (group 1, C a multiple of 128 bytes' worth of values: 32 fp32,
- * 64 bf16 / f16; F % 4 == 0, at most 64 taps; LLC_ERR_UNSUPPORTED otherwise).  Mixed layouts are refused (LLC_ERR_LAYOUT). */
+ * 64 bf16 / f16; F % 4 == 0, at most 64 taps; LLC_ERR_UNSUPPORTED otherwise).  One mixed form is taken: contiguous x
+ * and w with a channels-last out, for an image network's first layer, whose result the channels-last layers behind it
+ * read (64 filters, stride 2 along w, C * KH at most 21 (24 for the 16-bit types) input rows under a window, rows of
+ * at most 224 values, no residual; LLC_ERR_UNSUPPORTED otherwise).  Other mixed layouts are refused (LLC_ERR_LAYOUT). */
 int llc_hip_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_attrs* attrs, const llc_epilogue* epi,
                    llc_tensor* out, void* stream);
 
@@ -223,7 +226,8 @@ int llc_hip_layer_norm(const llc_tensor* x, const llc_tensor* scale, const llc_t
 
 /* llh.max_pool (LLHOps.td:495-507; LLHToHLO.cpp:295-339), NCHW, ceil_mode false.
  * init_zero = 1 reproduces the reference's reduce_window init value 0 (LLHToHLO.cpp:313-314);
- * init_zero = 0 is torch's -inf padding. */
+ * init_zero = 0 is torch's -inf padding.  x and out are both contiguous or both channels-last (strides as for
+ * llc_hip_conv2d; C a multiple of 16 bytes' worth of values then, LLC_ERR_UNSUPPORTED otherwise). */
 typedef struct llc_pool_attrs {
   int64_t dilation[2];
   int64_t kernel_shape[2];
@@ -234,7 +238,7 @@ typedef struct llc_pool_attrs {
 int llc_hip_max_pool(const llc_tensor* x, const llc_pool_attrs* attrs, llc_tensor* out, void* stream);
 
 /* llh.adaptive_average_pool{out_size=(1,1)} (LLHOps.td:337-339; shape rule
- * LLHinfersymbolShape.cpp:587-613): [N,C,H,W] -> [N,C] (or [N,C,1,1]). */
+ * LLHinfersymbolShape.cpp:587-613): [N,C,H,W] -> [N,C] (or [N,C,1,1]); x contiguous or channels-last. */
 int llc_hip_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream);
 
 /* ---- data movement, bit exact for every element size (1, 2, 4, 8 bytes) ---- */

@@ -37,6 +37,7 @@ struct ConvParams {
   int32_t OWp;     // fp32 kernel: output row length padded to a multiple of 4 (ncols counts padded pixels)
   int32_t splits;  // split-k factor (fp32 kernel)
   char* partial;   // [splits][F][ncols] fp32 partial sums when splits > 1
+  int32_t y_nhwc;  // NCHW operands with a channels-last result (the first-layer kernels only)
 };
 
 // Gathers this lane's run of k for one pixel column of the im2col matrix.
@@ -822,15 +823,18 @@ int launch_loaders(const ConvParams& p, int groups, hipStream_t s) {
   const bool w_vec = p.Kdim % EPV == 0 && ((uintptr_t)p.W % 16) == 0;
   if constexpr (sizeof(T) == 4) {
     if (conv_rows_ok(p, groups)) return launch_conv_rows<float>(p, s);
+    if (p.y_nhwc) return set_error(LLC_ERR_UNSUPPORTED, "conv: no kernel for NCHW operands with a channels-last result of this shape");
     if (w_vec && ((uintptr_t)p.Y % 16) == 0 && (!p.residual || ((uintptr_t)p.residual % 16) == 0) &&
         ((uintptr_t)p.X % 4) == 0 && (int64_t)p.N * p.C * p.H * p.Wd < ((int64_t)1 << 30))  // 32-bit byte offsets
       return launch_f32(p, groups, s);
   }
   if constexpr (sizeof(T) == 2) {
-    // an image network's first layer in 16-bit storage: the fp32 row kernel on widened copies
+    // an image network's first layer in 16-bit storage: the 16-bit row kernel, or the fp32 one on widened copies
+    if (conv_rows_16bit_ok(p, groups)) return launch_conv_rows_16bit_mfma<T>(p, s);
     if (conv_rows_ok(p, groups) && ((uintptr_t)p.W % 16) == 0 && (int64_t)p.N * p.C * p.H * p.Wd % 8 == 0 &&
         (!p.bias || ((uintptr_t)p.bias % 2) == 0))
       return launch_conv_rows_16bit<T>(p, s);
+    if (p.y_nhwc) return set_error(LLC_ERR_UNSUPPORTED, "conv: no kernel for NCHW operands with a channels-last result of this shape");
   }
   if (w_vec) return launch_tiles<T, kLoadKVec>(p, groups, s);
   return launch_tiles<T, kLoadGeneric>(p, groups, s);
@@ -859,7 +863,9 @@ int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_att
            (v.size[0] == 1 || v.stride[0] == H * W * C);
   };
   const bool nhwc = !(a.contiguous() && k.contiguous() && o.contiguous()) && channels_last(a) && channels_last(k) && channels_last(o);
-  if (!nhwc && (!a.contiguous() || !k.contiguous() || !o.contiguous()))
+  // a first layer that hands its result to channels-last layers: NCHW operands, channels-last result
+  const bool y_nhwc = !nhwc && a.contiguous() && k.contiguous() && !o.contiguous() && channels_last(o);
+  if (!nhwc && !y_nhwc && (!a.contiguous() || !k.contiguous() || !o.contiguous()))
     return set_error(LLC_ERR_LAYOUT, "conv: tensors must all be contiguous (NCHW) or all channels-last");
   const int64_t group = at->group;
   for (int i = 0; i < 2; ++i)
@@ -905,6 +911,7 @@ int llc_impl_conv2d(const llc_tensor* x, const llc_tensor* w, const llc_conv_att
   p.ncols = (int)(a.size[0] * OH * OW);
   p.alpha = 1.0f;
   p.act = LLC_ACT_NONE;
+  p.y_nhwc = y_nhwc ? 1 : 0;
   if (epi) {
     p.alpha = epi->alpha;
     if (epi->act < LLC_ACT_NONE || epi->act > LLC_ACT_GELU) return set_error(LLC_ERR_BAD_ARG, "conv: activation %d", epi->act);

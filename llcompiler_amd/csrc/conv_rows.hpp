@@ -26,6 +26,7 @@ constexpr int kRowsMaxRows = 21;         // C * KH
 constexpr int kRowsBuf = kRowsLead + kRowsMaxRows * kRowsPitch;
 constexpr int kRowsBlocks = 7;           // pixel blocks of 16 per output row: OW <= 112
 constexpr int kRowsLds = 2 * kRowsBuf;
+constexpr int kRowsLdsAll = kRowsLds + 256;  // and the bias of the channels-last form
 
 static __device__ __align__(256) unsigned char llc_conv_zero_row[256];
 
@@ -41,7 +42,7 @@ __device__ __forceinline__ void rows_static_for(F&& f) {
   }
 }
 
-template <typename TO>
+template <typename TO, bool NHWC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_rows_f32_kernel(const ConvParams p) {
   extern __shared__ __align__(16) char smem[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -59,18 +60,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int s = 0; s < kRowsSteps; ++s) {
     const int k = 4 * s + kk;
     const bool in = k < p.Kdim;
-    bw[s] = in ? ((const float*)p.W)[(int64_t)f * p.Kdim + k] : 0.0f;
     const int kc = in ? k : 0;
+    // every load is issued, from an index inside the filter: a load under a test would be a branch with its own wait
+    const float wv = ((const float*)p.W)[(int64_t)f * p.Kdim + kc];
+    bw[s] = in ? wv : 0.0f;
     const int c = kc / (p.KH * p.KW), rem = kc - c * (p.KH * p.KW);
     const int kh = rem / p.KW, kw = rem - kh * p.KW;
     // pixel i of block 0 reads column 2 i + kw - pw of row (c, kh); a k past the reduction reads row 0 (times weight 0)
     kaddr[s] = lds0 + kRowsLead + (uint32_t)((c * p.KH + kh) * kRowsPitch) + (uint32_t)((2 * li + kw - p.pw) * 4);
   }
-  const float bias = p.bias ? load_as_f32(p.bias, Elem<TO>::kDtype, f) : 0.0f;
+  // channels-last results: the operands trade places, so a lane's four accumulators of a block are filters
+  // 16 wave + 4 kk .. + 3 of pixel li, 16 bytes of that pixel's 256
+  // (their bias waits in LDS behind the row buffers: four more registers would not fit)
+  float tie_b = (p.bias && !NHWC) ? load_as_f32(p.bias, Elem<TO>::kDtype, f) : 0.0f;
+  if (NHWC && threadIdx.x < 64) ((float*)(smem + kRowsLds))[threadIdx.x] = p.bias ? load_as_f32(p.bias, Elem<TO>::kDtype, threadIdx.x) : 0.0f;
   // the lead-in of both buffers and whatever the loads never write stays zero
   for (int i = threadIdx.x; i < kRowsLds / 4; i += 256) ((uint32_t*)smem)[i] = 0u;
   __builtin_amdgcn_s_waitcnt(0);  // weights and bias are here, the zeros are written
-  float tie_b = bias;
   asm volatile("" : "+v"(tie_b));
 #pragma unroll
   for (int s = 0; s < kRowsSteps; ++s) asm volatile("" : "+v"(bw[s]));
@@ -130,7 +136,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int s = 0; s < CNT; ++s) asm volatile("" : "+v"(av[U & 1][s]));
         if constexpr (U + 1 < 2 * kRowsBlocks) read_half(std::integral_constant<int, U + 1>{}, buf_tag);
 #pragma unroll
-        for (int s = 0; s < CNT; ++s) acc[PB] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[U & 1][s], bw[S0 + s], acc[PB], 0, 0, 0);
+        for (int s = 0; s < CNT; ++s) {
+          if constexpr (NHWC) acc[PB] = __builtin_amdgcn_mfma_f32_16x16x4f32(bw[S0 + s], av[U & 1][s], acc[PB], 0, 0, 0);
+          else acc[PB] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[U & 1][s], bw[S0 + s], acc[PB], 0, 0, 0);
+        }
       });
     };
     if (buf == 0) row(std::integral_constant<int, 0>{});
@@ -141,23 +150,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8) | (0 << 14));  // vmcnt(0)
     __builtin_amdgcn_sched_barrier(0);
-    // ---- act(alpha acc + bias) -> y[n][f][oh][16 pb + 4 kk .. + 3] ----
+    // ---- act(alpha acc + bias) -> y[n][f][oh][16 pb + 4 kk .. + 3], or y[n][oh][16 pb + li][16 wave + 4 kk .. + 3] ----
     const int n = r / p.OH, oh = r - n * p.OH;
-    TO* yrow = (TO*)p.Y + (((int64_t)n * p.F + f) * p.OH + oh) * p.OW;
+    TO* yrow = NHWC ? (TO*)p.Y + ((int64_t)r * p.OW) * p.F + 16 * wave + 4 * kk
+                    : (TO*)p.Y + (((int64_t)n * p.F + f) * p.OH + oh) * p.OW;
+    f32x4_t b4 = {tie_b, tie_b, tie_b, tie_b};
+    if constexpr (NHWC) b4 = *(const f32x4_t*)(smem + kRowsLds + (16 * wave + 4 * kk) * 4);
 #pragma unroll
     for (int b = 0; b < kRowsBlocks; ++b) {
-      const int ow = 16 * b + 4 * kk;
+      const int ow = NHWC ? 16 * b + li : 16 * b + 4 * kk;
       f32x4_t o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float v = acc[b][e] * p.alpha + tie_b;
+        float v = acc[b][e] * p.alpha + b4[e];
         if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
         else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
         o[e] = v;
       }
       if (ow < p.OW) {
-        if constexpr (sizeof(TO) == 4) *(f32x4_t*)(yrow + ow) = o;
-        else *(uint2*)(yrow + ow) = uint2{pack_pair<Elem<TO>::kDtype>(o[0], o[1]), pack_pair<Elem<TO>::kDtype>(o[2], o[3])};
+        TO* dst = NHWC ? yrow + (int64_t)ow * p.F : yrow + ow;
+        if constexpr (sizeof(TO) == 4) *(f32x4_t*)dst = o;
+        else *(uint2*)dst = uint2{pack_pair<Elem<TO>::kDtype>(o[0], o[1]), pack_pair<Elem<TO>::kDtype>(o[2], o[3])};
       }
     }
   }
@@ -174,15 +187,19 @@ inline bool conv_rows_ok(const ConvParams& p, int groups) {
   return (int64_t)p.N * p.OH >= 256;  // rows enough for every CU
 }
 
-template <typename TO>
-int launch_conv_rows(const ConvParams& p, hipStream_t s) {
-  auto kern = conv_rows_f32_kernel<TO>;
+template <typename TO, bool NHWC>
+int launch_conv_rows_as(const ConvParams& p, hipStream_t s) {
+  auto kern = conv_rows_f32_kernel<TO, NHWC>;
   static std::atomic<uint32_t> lds_allowed{0};
-  LLC_TRY(allow_dynamic_lds((const void*)kern, kRowsLds, lds_allowed));
+  LLC_TRY(allow_dynamic_lds((const void*)kern, kRowsLdsAll, lds_allowed));
   const int64_t total = (int64_t)p.N * p.OH;
   const unsigned wgs = (unsigned)(total < 512 ? total : 512);  // two workgroups per CU, each walking rows wgs apart
-  hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), kRowsLds, s, p);
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), kRowsLdsAll, s, p);
   return check_launch("conv_rows_f32_kernel");
+}
+template <typename TO>
+int launch_conv_rows(const ConvParams& p, hipStream_t s) {
+  return p.y_nhwc ? launch_conv_rows_as<TO, true>(p, s) : launch_conv_rows_as<TO, false>(p, s);
 }
 
 // 16-bit values to fp32, 8 per lane
@@ -225,4 +242,278 @@ int launch_conv_rows_16bit(const ConvParams& p, hipStream_t s) {
   q.X = (const char*)x32;
   q.W = (const char*)w32;
   return launch_conv_rows<T>(q, s);
+}
+
+// ---- the same layer in 16-bit storage, on the 16-bit matrix instruction ----
+//
+// v_mfma_f32_16x16x32 takes eight consecutive k per lane.  With k ordered (channel, window row, window column) those
+// eight are the window columns of one (channel, window row): 16 consecutive bytes of that input row in LDS, starting at
+// column 2 pixel - pad.  The start has to be a whole dword, so for an odd pad the run begins one column early and the
+// filters carry a zero in front (a 7-wide window with pad 3 fills the eight slots exactly); columns of the run outside
+// the window are also cleared in the pixel operand, so that an Inf or NaN next to a window does not reach its sum.  A
+// k-step is four (channel, window row) pairs, one per quarter wave, and there are always six k-steps: pairs past the
+// last are rows of LDS nothing is loaded into.  Each wave owns pixel blocks wave and wave + 4 of the output row and all 64 filters (96 registers of
+// filters, read once through LDS), so the pixel operand is read once per block.  Input rows arrive two per wave
+// instruction (a row slot is 512 bytes: 256 values).  The matrix instructions of a row take a fraction of a memory
+// round trip, so the rows of the next three iterations are in flight (a ring of four row buffers); every wave issues
+// the same three loads per row, also for rows past the end (they fetch zeros), which is what lets the wait in front
+// of a row be a count: all but the loads of the two rows behind it.
+constexpr int kRows16Slots = 24;
+constexpr int kRows16Pitch = 512;
+constexpr int kRows16Lead = 128;
+constexpr int kRows16Buf = kRows16Lead + kRows16Slots * kRows16Pitch;
+constexpr int kRows16Ring = 4;            // row buffers: the rows three iterations ahead are in flight
+constexpr int kRows16Loads = kRows16Slots / 8;  // direct-to-LDS loads per wave and row (two slots each, four waves)
+constexpr int kRows16Lds = kRows16Ring * kRows16Buf;
+static_assert(64 * kRows16Slots * 16 <= kRows16Lds, "the filters pass through the row buffers");
+
+typedef uint32_t rows_u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void rows16_read(rows_u32x2_t& lo, rows_u32x2_t& hi, uint32_t addr) {
+  asm volatile("ds_read2_b32 %0, %2 offset1:1\n\tds_read2_b32 %1, %2 offset0:2 offset1:3" : "=&v"(lo), "=&v"(hi) : "v"(addr));
+}
+
+template <typename T, bool NHWC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_rows_16bit_kernel(const ConvParams p) {
+  constexpr int DT = Elem<T>::kDtype;
+  extern __shared__ __align__(16) char smem[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int li = lane % 16, g = lane / 16;
+  const int nrows = p.C * p.KH, shift = p.pw & 1;
+
+  // ---- once: the filters as [64][24] runs of eight (zeros where the run leaves the window or the reduction) ----
+#pragma unroll
+  for (int v0 = 0; v0 < 64 * kRows16Slots; v0 += 256) {
+    const int v = v0 + threadIdx.x;
+    const int f = v / kRows16Slots, r = v - f * kRows16Slots;
+    uint32_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kw = j - shift;
+      const bool in = r < nrows && kw >= 0 && kw < p.KW;
+      // every load is issued, from an index inside the filters: a load under a test would be a branch with its own wait
+      const uint32_t wv = ((const uint16_t*)p.W)[in ? (int64_t)f * p.Kdim + r * p.KW + kw : 0];
+      e[j] = in ? wv : 0u;
+    }
+    ((u32x4_t*)smem)[v] = u32x4_t{e[0] | e[1] << 16, e[2] | e[3] << 16, e[4] | e[5] << 16, e[6] | e[7] << 16};
+  }
+  __syncthreads();
+  // filter operand of group fg, k-step s.  Channels-last results: the filters are the rows of the product, row li of
+  // group fg is filter 16 (li / 4) + 4 fg + li % 4, which leaves a lane with 16 consecutive filters of one pixel.
+  u32x4_t w[4][6];
+#pragma unroll
+  for (int fg = 0; fg < 4; ++fg) {
+    const int fl = NHWC ? 16 * (li / 4) + 4 * fg + (li % 4) : 16 * fg + li;
+#pragma unroll
+    for (int s = 0; s < 6; ++s) w[fg][s] = ((const u32x4_t*)smem)[fl * kRows16Slots + 4 * s + g];
+  }
+  float bias[NHWC ? 16 : 4];
+#pragma unroll
+  for (int e = 0; e < (NHWC ? 16 : 4); ++e) bias[e] = 0.0f;
+  if (p.bias) {  // one test around all the loads: they are in flight together
+#pragma unroll
+    for (int e = 0; e < (NHWC ? 16 : 4); ++e) bias[e] = load_as_f32(p.bias, DT, NHWC ? 16 * g + e : 16 * e + li);
+  }
+  // which halves of the run's four dwords lie inside the window
+  uint32_t km[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int k0 = 2 * d - shift, k1 = 2 * d + 1 - shift;
+    km[d] = ((k0 >= 0 && k0 < p.KW) ? 0x0000ffffu : 0u) | ((k1 >= 0 && k1 < p.KW) ? 0xffff0000u : 0u);
+  }
+  __syncthreads();
+  // the lead-in of both buffers, the rows past the reduction and whatever the loads never write stay zero
+  for (int i = threadIdx.x; i < kRows16Lds / 16; i += 256) ((u32x4_t*)smem)[i] = u32x4_t{0u, 0u, 0u, 0u};
+  __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+  for (int fg = 0; fg < 4; ++fg)
+#pragma unroll
+    for (int s = 0; s < 6; ++s) asm volatile("" : "+v"(w[fg][s]));
+#pragma unroll
+  for (int e = 0; e < (NHWC ? 16 : 4); ++e) asm volatile("" : "+v"(bias[e]));
+  __syncthreads();
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  // pixel li of block 0, k-step 0: row slot g, column 2 li - pad - shift
+  const uint32_t lane_addr = lds0 + kRows16Lead + (uint32_t)(g * kRows16Pitch) + (uint32_t)((2 * li - p.pw - shift) * 2);
+
+  // ---- input rows of output row `r` into buffer `buf`: two patch rows per wave instruction, three instructions per
+  //      wave whatever the row (slots past the reduction and rows past the end fetch zeros) ----
+  const int total = p.N * p.OH;
+  const int hl = lane / 32, l32 = lane % 32;
+  auto fetch = [&](int r, int buf) {
+    const int n = r / p.OH, oh = r - n * p.OH;
+    const int ih0 = oh * p.sh - p.ph;
+#pragma unroll
+    for (int j = 0; j < kRows16Loads; ++j) {
+      const int q = wave + 4 * j;
+      const int pr = 2 * q + hl;
+      const int c = pr / p.KH, kh = pr - c * p.KH;
+      const int ih = ih0 + kh;
+      const bool in = r < total && pr < nrows && ih >= 0 && ih < p.H && 8 * l32 < p.Wd;
+      const char* src = in ? p.X + ((((int64_t)n * p.C + c) * p.H + ih) * p.Wd) * 2 + l32 * 16
+                           : (const char*)llc_conv_zero_row + (lane % 16) * 16;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(smem + buf * kRows16Buf + kRows16Lead + 2 * q * kRows16Pitch),
+                                       16, 0, 0);
+    }
+  };
+  const int nblk = (p.OW + 15) / 16;
+  auto mma = [&](f32x4_t (&a)[4], const rows_u32x2_t (&lo)[6], const rows_u32x2_t (&hi)[6]) {
+#pragma unroll
+    for (int s = 0; s < 6; ++s) {
+      const u32x4_t px = u32x4_t{lo[s][0] & km[0], lo[s][1] & km[1], hi[s][0] & km[2], hi[s][1] & km[3]};
+#pragma unroll
+      for (int fg = 0; fg < 4; ++fg) {
+        if constexpr (DT == LLC_BFLOAT16) {
+          if constexpr (NHWC)
+            a[fg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[fg][s]), __builtin_bit_cast(bf16x8_t, px), a[fg], 0, 0, 0);
+          else
+            a[fg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, px), __builtin_bit_cast(bf16x8_t, w[fg][s]), a[fg], 0, 0, 0);
+        } else {
+          if constexpr (NHWC)
+            a[fg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, w[fg][s]), __builtin_bit_cast(f16x8_t, px), a[fg], 0, 0, 0);
+          else
+            a[fg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, px), __builtin_bit_cast(f16x8_t, w[fg][s]), a[fg], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  int r = blockIdx.x;
+#pragma unroll
+  for (int d = 0; d < kRows16Ring - 1; ++d) fetch(r + d * (int)gridDim.x, d);
+  int buf = 0;
+  const bool two = wave + 4 < nblk;  // this wave's second pixel block exists
+  // Vector memory operations leave the counter in the order they were issued.  Behind the loads of a row this wave has
+  // issued the loads of the next two rows and the stores of the last two rows it finished (of fewer at the start):
+  // the row is here when no more than those are still counted.  A block's stores are always issued (a block has at
+  // least one pixel inside the row), 2 per block channels-last and 4 otherwise.
+  const int row_stores = (two ? 2 : 1) * (NHWC ? 2 : 4);
+  int done = 0;  // rows this wave has stored, up to 2
+  for (; r < total; r += gridDim.x, buf = buf + 1 == kRows16Ring ? 0 : buf + 1) {
+    __builtin_amdgcn_sched_barrier(0);
+    switch (2 * kRows16Loads + done * row_stores) {
+      case 6: __builtin_amdgcn_s_waitcnt(6 | (7 << 4) | (15 << 8)); break;
+      case 8: __builtin_amdgcn_s_waitcnt(8 | (7 << 4) | (15 << 8)); break;
+      case 10: __builtin_amdgcn_s_waitcnt(10 | (7 << 4) | (15 << 8)); break;
+      case 14: __builtin_amdgcn_s_waitcnt(14 | (7 << 4) | (15 << 8)); break;
+      case 22: __builtin_amdgcn_s_waitcnt((22 & 15) | (7 << 4) | (15 << 8) | ((22 >> 4) << 14)); break;
+      default: __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8)); break;
+    }
+    done = done < 2 ? done + 1 : 2;
+    // past the barrier every wave's loads of the row are here, and every wave has read the previous row for the last time
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    f32x4_t acc[2][4];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int fg = 0; fg < 4; ++fg) acc[b][fg] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t row_addr = lane_addr + (uint32_t)(buf * kRows16Buf) + (uint32_t)(wave * 64);
+    rows_u32x2_t lo0[6], hi0[6], lo1[6], hi1[6];
+#pragma unroll
+    for (int s = 0; s < 6; ++s) rows16_read(lo0[s], hi0[s], row_addr + (uint32_t)(s * 4 * kRows16Pitch));
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+#pragma unroll
+    for (int s = 0; s < 6; ++s) asm volatile("" : "+v"(lo0[s]), "+v"(hi0[s]));
+    // the second block's operand is on its way under the matrix instructions of the first
+    if (two) {
+#pragma unroll
+      for (int s = 0; s < 6; ++s) rows16_read(lo1[s], hi1[s], row_addr + (uint32_t)(4 * 64 + s * 4 * kRows16Pitch));
+    }
+    mma(acc[0], lo0, hi0);
+    if (two) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+#pragma unroll
+      for (int s = 0; s < 6; ++s) asm volatile("" : "+v"(lo1[s]), "+v"(hi1[s]));
+      mma(acc[1], lo1, hi1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const int n = r / p.OH, oh = r - n * p.OH;
+    // one test of the activation per row, not one per element
+    auto finish = [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int pb = wave + 4 * b;
+      if (pb >= nblk) continue;
+      if constexpr (NHWC) {
+        // lane: pixel 16 pb + li, filters 16 g .. 16 g + 15 (group fg, element e is filter 16 g + 4 fg + e)
+        const int ow = 16 * pb + li;
+        uint32_t o[8];
+#pragma unroll
+        for (int fg = 0; fg < 4; ++fg) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = acc[b][fg][e] * p.alpha + bias[4 * fg + e];
+            if constexpr (ACT == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
+            else if constexpr (ACT == LLC_ACT_GELU) x = gelu_for<T>(x);
+            v[e] = x;
+          }
+          o[2 * fg] = pack_pair<DT>(v[0], v[1]);
+          o[2 * fg + 1] = pack_pair<DT>(v[2], v[3]);
+        }
+        if (ow < p.OW) {
+          T* dst = (T*)p.Y + ((int64_t)r * p.OW + ow) * p.F + 16 * g;
+          *(u32x4_t*)dst = u32x4_t{o[0], o[1], o[2], o[3]};
+          *(u32x4_t*)(dst + 8) = u32x4_t{o[4], o[5], o[6], o[7]};
+        }
+      } else {
+        // lane: filter 16 fg + li, pixels 16 pb + 4 g .. + 3
+        const int ow = 16 * pb + 4 * g;
+#pragma unroll
+        for (int fg = 0; fg < 4; ++fg) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = acc[b][fg][e] * p.alpha + bias[fg];
+            if constexpr (ACT == LLC_ACT_RELU) x = x < 0.0f ? 0.0f : x;
+            else if constexpr (ACT == LLC_ACT_GELU) x = gelu_for<T>(x);
+            v[e] = x;
+          }
+          if (ow < p.OW)
+            *(uint2*)((T*)p.Y + (((int64_t)n * p.F + 16 * fg + li) * p.OH + oh) * p.OW + ow) =
+                uint2{pack_pair<DT>(v[0], v[1]), pack_pair<DT>(v[2], v[3])};
+        }
+      }
+    }
+    };
+    if (p.act == LLC_ACT_RELU) finish(std::integral_constant<int, LLC_ACT_RELU>{});
+    else if (p.act == LLC_ACT_GELU) finish(std::integral_constant<int, LLC_ACT_GELU>{});
+    else finish(std::integral_constant<int, LLC_ACT_NONE>{});
+    // into the buffer of the previous row, which every wave has left (the barrier above)
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(r + (kRows16Ring - 1) * (int)gridDim.x, buf == 0 ? kRows16Ring - 1 : buf - 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8) | (0 << 14));  // the loads past the end have landed
+}
+
+// Whether the 16-bit row kernel takes this convolution (NCHW input, contiguous, checked by the caller).
+inline bool conv_rows_16bit_ok(const ConvParams& p, int groups) {
+  const int shift = p.pw & 1;
+  if (groups != 1 || p.F != 64 || p.C * p.KH > kRows16Slots || p.KW + shift > 8 || p.residual) return false;
+  if (p.sw != 2 || p.dh != 1 || p.dw != 1) return false;
+  // a row and its right-hand zeros fit a 256-value slot whose tail is also the next row's left-hand padding
+  if (p.Wd % 8 != 0 || p.Wd > 256 - (p.pw + shift) || (p.pw + shift) * 2 > kRows16Lead) return false;
+  if (p.OW % 4 != 0 || p.OW > 128 || 2 * (16 * ((p.OW + 15) / 16) - 1) - p.pw - shift + 7 > 255) return false;
+  if (((uintptr_t)p.X % 16) != 0 || ((uintptr_t)p.Y % 16) != 0 || ((uintptr_t)p.W % 2) != 0 ||
+      (p.bias && ((uintptr_t)p.bias % 2) != 0))
+    return false;
+  return (int64_t)p.N * p.OH >= 256;  // rows enough for every CU
+}
+
+template <typename T, bool NHWC>
+int launch_conv_rows_16bit_mfma_as(const ConvParams& p, hipStream_t s) {
+  auto kern = conv_rows_16bit_kernel<T, NHWC>;
+  const int64_t total = (int64_t)p.N * p.OH;
+  const unsigned wgs = (unsigned)(total < 512 ? total : 512);
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), kRows16Lds, s, p);
+  return check_launch("conv_rows_16bit_kernel");
+}
+template <typename T>
+int launch_conv_rows_16bit_mfma(const ConvParams& p, hipStream_t s) {
+  return p.y_nhwc ? launch_conv_rows_16bit_mfma_as<T, true>(p, s) : launch_conv_rows_16bit_mfma_as<T, false>(p, s);
 }

@@ -431,6 +431,46 @@ __global__ __launch_bounds__(256) void mid_reduce_kernel(const RowParams p, int6
   store_row_vec<1>(p.y, p.dtype, o, one);
 }
 
+// The same reduction when the outputs are too few to fill the chip with one lane each (a global average pool over a
+// channels-last tensor: 16 x 512 outputs of 49 values): 64 consecutive outputs per workgroup, the reduced range dealt
+// to its four waves (wave w takes k = w, w + 4, ...), four loads in flight per lane, the four partial results combined
+// in wave order.
+__global__ __launch_bounds__(256) void mid_reduce_split_kernel(const RowParams p, int64_t outer, int64_t R, int64_t inner) {
+  __shared__ float part[4][64];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int64_t chunks = (inner + 63) / 64;
+  const int64_t b = blockIdx.x / chunks, i = (blockIdx.x % chunks) * 64 + lane;
+  const float init = p.kind == LLC_REDUCE_SUM ? 0.0f : (p.kind == LLC_REDUCE_MAX ? -INFINITY : INFINITY);
+  auto combine = [&](float a, float v) {
+    return p.kind == LLC_REDUCE_SUM ? a + v : (p.kind == LLC_REDUCE_MAX ? nmax(a, v) : nmin(a, v));
+  };
+  float r = init;
+  if (i < inner) {
+    const int64_t base = b * R * inner + i;
+    int64_t k = wave;
+    for (; k + 12 < R; k += 16) {
+      float v[4][1];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) load_row_vec<1>(p.x, p.dtype, base + (k + 4 * u) * inner, v[u]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) r = combine(r, v[u][0]);
+    }
+    for (; k < R; k += 4) {
+      float v[1];
+      load_row_vec<1>(p.x, p.dtype, base + k * inner, v);
+      r = combine(r, v[0]);
+    }
+  }
+  part[wave][lane] = r;
+  __syncthreads();
+  if (wave == 0 && i < inner) {
+    r = combine(combine(part[0][lane], part[1][lane]), combine(part[2][lane], part[3][lane]));
+    if (p.kind == LLC_REDUCE_SUM) r *= p.scale;
+    float one[1] = {r};
+    store_row_vec<1>(p.y, p.dtype, b * inner + i, one);
+  }
+}
+
 template <int OP, int VEC, int TPR>
 void launch_items(const RowParams& p, int items, hipStream_t s) {
   const int rpb = 256 / TPR;
@@ -581,6 +621,11 @@ int reduce_3d(const View& a, const View& o, int kind, int64_t outer, int64_t R, 
   }
   const int64_t n = outer * inner;
   if ((n + 255) / 256 > 0x7fffffff) return set_error(LLC_ERR_TOO_LARGE, "reduce: too many outputs");
+  if (R >= 8 && n < 512 * 256) {  // under two workgroups per CU at one lane per output
+    const int64_t blocks = outer * ((inner + 63) / 64);
+    hipLaunchKernelGGL(mid_reduce_split_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, outer, R, inner);
+    return check_launch("mid_reduce_split_kernel");
+  }
   hipLaunchKernelGGL(mid_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, outer, R, inner);
   return check_launch("mid_reduce_kernel");
 }
@@ -678,9 +723,15 @@ int llc_impl_global_avg_pool(const llc_tensor* x, llc_tensor* out, void* stream)
   LLC_TRY(row_dtype_ok(a, "global_avg_pool"));
   if (a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "global_avg_pool: input and output types differ");
   if (a.rank != 4) return set_error(LLC_ERR_SHAPE, "global_avg_pool: NCHW input expected");
-  if (!a.contiguous() || !o.contiguous()) return set_error(LLC_ERR_LAYOUT, "global_avg_pool: contiguous tensors expected");
+  // a channels-last input ([N][H W][C] in memory) is a reduction over the middle of three runs
+  const int64_t C = a.size[1], H = a.size[2], W = a.size[3];
+  const bool nhwc = !a.contiguous() && (C == 1 || a.stride[1] == 1) && (W == 1 || a.stride[3] == C) &&
+                    (H == 1 || a.stride[2] == W * C) && (a.size[0] == 1 || a.stride[0] == H * W * C);
+  if ((!a.contiguous() && !nhwc) || !o.contiguous())
+    return set_error(LLC_ERR_LAYOUT, "global_avg_pool: a contiguous or channels-last input and a contiguous output expected");
   const int64_t nc = a.size[0] * a.size[1], hw = a.size[2] * a.size[3];
   if (o.numel() != nc) return set_error(LLC_ERR_SHAPE, "global_avg_pool: output holds %lld elements, expected %lld", (long long)o.numel(), (long long)nc);
   if (hw == 0) return set_error(LLC_ERR_SHAPE, "global_avg_pool: empty window");
+  if (nhwc) return reduce_3d(a, o, LLC_REDUCE_SUM, a.size[0], hw, C, 1.0f / (float)hw, as_stream(stream));
   return reduce_3d(a, o, LLC_REDUCE_SUM, nc, hw, 1, 1.0f / (float)hw, as_stream(stream));
 }

@@ -90,6 +90,12 @@ class _Pool:
         self.free.setdefault(buf.numel(), []).append(buf)
 
 
+def _is_channels_last(t):
+    """A 4-D tensor that is NHWC in memory and not also NCHW-contiguous."""
+    return isinstance(t, torch.Tensor) and t.dim() == 4 and not t.is_contiguous() and \
+        t.is_contiguous(memory_format=torch.channels_last)
+
+
 class _LazyReshape:
     """A reshape that is not a view of its source (e.g. the head split [B,S,H,D] -> permute -> [B*H,S,D]): the
     copy is made only if a consumer needs the reshaped tensor; batch_matmul reads the 4-D source in place."""
@@ -151,6 +157,26 @@ class Instance:
             return False
         return x.shape[1] % (128 // out.dtype.itemsize) == 0 and w.shape[0] % 4 == 0 and w.shape[2] * w.shape[3] <= 64 and \
             x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+
+    def _first_layer_channels_last_ok(self, st, x, w, out, natural, res):
+        """Whether the NCHW convolution `st` (an image network's first layer: few channels, 64 filters, stride 2) may
+        write its result channels-last, for the channels-last layers after it: the shapes the row kernels of
+        llc_hip_conv2d take with NCHW operands and a channels-last result."""
+        if not CHANNELS_LAST or res is not None or st.attrs["group"] != 1 or len(natural) != 4 or \
+                tuple(natural) != tuple(out.shape) or x.dim() != 4 or w.dim() != 4:
+            return False
+        a = st.attrs
+        (n, c, h, wd), (f, _, kh, kw), (oh, ow) = x.shape, w.shape, natural[2:]
+        pw, es = a["pad"][1], out.dtype.itemsize
+        if f != 64 or tuple(a["dilation"]) != (1, 1) or a["stride"][1] != 2 or n * oh < 256 or ow % 4 or \
+                x.data_ptr() % 16 or w.data_ptr() % 16:
+            return False
+        if es == 4:
+            return out.dtype == torch.float32 and c * kh * kw <= 148 and c * kh <= 21 and wd % 4 == 0 and wd <= 224 and \
+                pw <= min(256 - wd, 32) and ow <= 112 and 2 * 111 + kw - 1 - pw <= 255
+        shift = pw & 1
+        return out.dtype in (torch.bfloat16, torch.float16) and c * kh <= 24 and kw + shift <= 8 and wd % 8 == 0 and \
+            wd <= 256 - (pw + shift) and pw + shift <= 64 and ow <= 128 and 2 * (16 * ((ow + 15) // 16) - 1) - pw - shift + 7 <= 255
 
     def _scan(self, item):
         if isinstance(item, C.TensorRef):
@@ -655,6 +681,7 @@ class Instance:
                     val[id(st.output)] = out
                 else:
                     cl = k == "conv" and self._channels_last_ok(st, ins, out, natural)
+                    first = k == "conv" and not cl and self._first_layer_channels_last_ok(st, ins[0], ins[1], out, natural, res)
                     if res is not None and not cl:
                         res = contiguous(res)
                     epi = None
@@ -683,6 +710,9 @@ class Instance:
                         call = ops.conv2d(xc, wc, pad=st.attrs["pad"], stride=st.attrs["stride"], dilation=st.attrs["dilation"],
                                           group=1, epilogue=epi, out=out, defer=True)
                     else:
+                        if first:
+                            n_, f_, oh_, ow_ = natural
+                            out = o = out.view(-1).view(n_, oh_, ow_, f_).permute(0, 3, 1, 2)  # NCHW shape over NHWC memory
                         call = ops.conv2d(contiguous(ins[0]), contiguous(ins[1]), pad=st.attrs["pad"], stride=st.attrs["stride"],
                                           dilation=st.attrs["dilation"], group=st.attrs["group"], epilogue=epi, out=o, defer=True)
                     if out.numel():
@@ -710,14 +740,22 @@ class Instance:
             elif k == "max_pool":
                 out = new_tensor(st.output)
                 a = st.attrs
+                x = ins[0]
+                if _is_channels_last(x) and x.shape[1] % (16 // x.dtype.itemsize) == 0 and x.data_ptr() % 16 == 0 and out.dim() == 4:
+                    # a channels-last input gives a channels-last result: NCHW shape over NHWC memory
+                    n_, c_, oh_, ow_ = out.shape
+                    out = out.view(-1).view(n_, oh_, ow_, c_).permute(0, 3, 1, 2)
+                else:
+                    x = contiguous(x)
                 if out.numel():
-                    self._launch_later(ops.max_pool(contiguous(ins[0]), a["kernel_shape"], pad=a["pad"], stride=a["stride"],
+                    self._launch_later(ops.max_pool(x, a["kernel_shape"], pad=a["pad"], stride=a["stride"],
                                                     dilation=a["dilation"], init_zero=False, out=out, defer=True))
                 val[id(st.output)] = out
             elif k == "avg_pool":
                 out = new_tensor(st.output)
+                x = ins[0] if _is_channels_last(ins[0]) else contiguous(ins[0])
                 if out.numel():
-                    self._launch_later(ops.global_avg_pool(contiguous(ins[0]), out=out, defer=True))
+                    self._launch_later(ops.global_avg_pool(x, out=out, defer=True))
                 val[id(st.output)] = out
             elif k == "gather":
                 out = new_tensor(st.output)

@@ -659,6 +659,31 @@ def test_resnet18_in_bf16_runs_channels_last():
         assert torch.equal(cm(x.cuda()), got)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_resnet18_stays_channels_last_from_the_stem_on(dtype):
+    """At batch 16 the stem is a first-layer-kernel shape: it writes its result channels-last, the max-pool and the
+    global average pool read and write that layout, and no layout copy of an activation is left in the call list."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval().to(dtype)
+    (x,) = make_resnet_inputs(16, 64)
+    x = x.to(dtype)
+    with torch.no_grad():
+        eager = m(x)
+        cm = compile_module(copy.deepcopy(m).cuda(), (x.cuda(),))
+        got = cm(x.cuda())
+        inst = list(cm.engine.instances.values())[0]
+        names = [c.fn.__name__ for c in inst.calls]
+        assert names.count("llc_hip_copy") == 0 and names.count("llc_hip_conv2d") == 20 and len(names) == 23, names
+        if dtype == torch.float32:
+            assert_close(got.cpu().numpy(), eager.numpy(), F32_RTOL, F32_ATOL, "resnet18 16x3x64x64")
+        else:
+            want64 = copy.deepcopy(m).double()(x.double())
+            _assert_as_close_as_eager(got.float().cpu().numpy(), eager.float().numpy(), want64.numpy(), BF16_RTOL, BF16_ATOL,
+                                      "resnet18 bf16 16x3x64x64")
+        assert torch.equal(cm(x.cuda()), got)
+
+
 def _plan_file_round_trip(cm, args, path):
     """Saves the plan of the (single) instance of an export-compiled module, loads it back and runs it on the
     tensors the engine passes for `args`; returns the outputs of that run."""
@@ -1102,8 +1127,8 @@ def test_resnet18_with_batch_norms_plans_to_twenty_convolutions(oracle):
         assert_close(got.cpu().numpy(), m(x).numpy(), F32_RTOL, F32_ATOL, "resnet18 with batch norms vs torch eager")
         inst = list(cm.engine.instances.values())[0]
         names = [c.fn.__name__ for c in inst.calls]
-        # + the layout copies behind the max-pool (to channels-last) and in front of the average pool (back)
-        assert len(names) == 23 + 2 and names.count("llc_hip_conv2d") == 20 and names.count("llc_hip_elementwise") == 0, names
+        # + the layout copy behind the max-pool (to channels-last; at this batch the stem is no first-layer-kernel shape)
+        assert len(names) == 23 + 1 and names.count("llc_hip_conv2d") == 20 and names.count("llc_hip_elementwise") == 0, names
         assert torch.equal(cm(x.cuda()), got)
         # statistics and filters written in place: the folded filters follow
         for mod, ref in zip(mg.modules(), m.modules()):

@@ -288,7 +288,7 @@ def test_layer_norm(ops, oracle, shape):
 
 @pytest.mark.parametrize("shape,axes", [((3, 4, 5, 6), [3]), ((3, 4, 5, 6), [1, 2]), ((3, 4, 5, 6), [0]), ((3, 4, 5, 6), [2, 3]),
                                         ((3, 4, 5, 6), [0, 1, 2, 3]), ((16, 4096), [1]), ((7, 300, 9), [1]), ((2, 3000), [-1]),
-                                        ((8, 1536), [1])])
+                                        ((8, 1536), [1]), ((5, 49, 130), [1]), ((16, 49, 512), [1]), ((40, 9, 4096), [1])])
 def test_reduce(ops, oracle, shape, axes):
     r = rng(10)
     x = r.standard_normal(shape).astype(np.float32)
@@ -1186,6 +1186,54 @@ def test_conv2d_first_layer_row_kernel(ops, oracle, case):
         close(host(got), rnd(want16), "first-layer conv + bias + relu %s %s" % (dt, case))
 
 
+@pytest.mark.parametrize("case", ROW_CONV_CASES)
+def test_conv2d_first_layer_channels_last_result(ops, oracle, case):
+    """The first-layer kernels with NCHW operands and a channels-last result (what the channels-last layers after
+    them read), fp32 and 16-bit, with bias + relu; other shapes in that combination are refused."""
+    N, C, H, W, KH, KW, pad, s = case
+    r = rng(sum(case[:6]) + 10)
+    x = bf16_round(r.standard_normal((N, C, H, W)))
+    w = bf16_round(r.standard_normal((64, C, KH, KW)) / np.sqrt(C * KH * KW))
+    b = bf16_round(r.standard_normal(64))
+    plain = oracle.conv2d(x, w, None, pad=pad, stride=s)
+    want = oracle.unary("relu", oracle.conv2d(x, w, b, pad=pad, stride=s))
+    cl = torch.channels_last
+    for dt, rnd, close in ((torch.float32, lambda v: v, assert_close_f32), (torch.bfloat16, bf16_round, assert_close_bf16),
+                           (torch.float16, f16_round, assert_close_f16)):
+        o = torch.empty(want.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        got = ops.conv2d(dev(x, dt), dev(w, dt), pad=pad, stride=s, out=o)
+        assert got.is_contiguous(memory_format=cl) and not got.is_contiguous()
+        close(host(got), rnd(plain), "first-layer conv, channels-last result %s %s" % (dt, case))
+        o2 = torch.empty(want.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+        got = ops.conv2d(dev(x, dt), dev(w, dt), pad=pad, stride=s, epilogue=ops.Epilogue(bias=dev(b, dt), act="relu"), out=o2)
+        close(host(got), rnd(want), "first-layer conv + bias + relu, channels-last result %s %s" % (dt, case))
+    # stride 1 along w is no first-layer shape: NCHW operands with a channels-last result have no kernel there
+    o = torch.empty((N, 64, H, W), device="cuda").contiguous(memory_format=cl)
+    with pytest.raises(RuntimeError):
+        ops.conv2d(dev(x), dev(w), pad=(KH // 2, KW // 2, KH // 2, KW // 2), stride=(1, 1), out=o)
+
+
+def test_conv2d_first_layer_16bit_infinite_pixel_stays_in_its_windows(ops, oracle):
+    """The 16-bit first-layer kernel reads eight window columns per matrix-instruction operand for a 7-wide window
+    (the eighth against a zero filter value): an infinite pixel in that extra column must not reach the sum."""
+    r = rng(77)
+    x = bf16_round(r.standard_normal((4, 3, 128, 128)))
+    x[1, 2, 40, 51] = np.inf
+    x[2, 0, 0, 0] = -np.inf
+    w = bf16_round(r.standard_normal((64, 3, 7, 7)) / np.sqrt(147))
+    pad, s = (3, 3, 3, 3), (2, 2)
+    want = bf16_round(oracle.conv2d(x, w, None, pad=pad, stride=s))
+    for out_cl in (False, True):
+        o = torch.empty(want.shape, device="cuda", dtype=torch.bfloat16)
+        if out_cl:
+            o = o.contiguous(memory_format=torch.channels_last)
+        got = host(ops.conv2d(dev(x, torch.bfloat16), dev(w, torch.bfloat16), pad=pad, stride=s, out=o))
+        fin = np.isfinite(want)
+        assert 0 < (~fin).sum() < want.size // 100
+        np.testing.assert_array_equal(np.isfinite(got), fin)
+        assert_close_bf16(got[fin], want[fin], "finite outputs beside an infinite pixel")
+
+
 PATCH_CONV_CASES = [
     # N, H, W, F, KH, KW, pad(h_lo, w_lo, h_hi, w_hi): 64 channels in 16-bit storage, stride 1, at least 192 tiles
     (16, 56, 56, 64, 3, 3, (1, 1, 1, 1)),     # a ResNet's first stage: 24 whole tiles and one of 64 pixels per image
@@ -1344,3 +1392,36 @@ def test_max_pool_and_avg_pool(ops, oracle):
             np.testing.assert_array_equal(host(got), oracle.maxpool2d(x, k, pad=pad, stride=s, dilation=d, init_zero=iz))
     y = r.standard_normal((4, 6, 7, 7)).astype(np.float32)
     assert_close_f32(host(ops.global_avg_pool(dev(y))), oracle.global_avgpool(y))
+
+
+def test_max_pool_and_avg_pool_channels_last(ops, oracle):
+    """Channels-last tensors (NHWC in memory under NCHW shapes): the pooling kernels read and write them as they lie.
+    The maximum is one of the inputs, so 16-bit results are exact too."""
+    r = rng(33)
+    cl = torch.channels_last
+    for C in (8, 64, 72):
+        x = bf16_round(r.standard_normal((3, C, 21, 26)))
+        x[0, 1, 3, 4] = np.nan
+        for k, p, s, d in [((3, 3), (1, 1), (2, 2), (1, 1)), ((2, 2), (0, 0), (2, 2), (1, 1)), ((5, 5), (2, 2), (1, 1), (2, 2)),
+                           ((2, 3), (1, 0), (2, 1), (2, 1))]:
+            pad = (p[0], p[1], p[0], p[1])
+            for iz in (False, True):
+                want = oracle.maxpool2d(x, k, pad=pad, stride=s, dilation=d, init_zero=iz)
+                for dt in (torch.float32, torch.bfloat16, torch.float16):
+                    xs = x if dt != torch.float16 else f16_round(x)
+                    ws = want if dt != torch.float16 else oracle.maxpool2d(xs, k, pad=pad, stride=s, dilation=d, init_zero=iz)
+                    o = torch.empty(want.shape, device="cuda", dtype=dt).contiguous(memory_format=cl)
+                    got = ops.max_pool(dev(xs, dt).contiguous(memory_format=cl), k, pad=pad, stride=s, dilation=d, init_zero=iz, out=o)
+                    assert got.is_contiguous(memory_format=cl)
+                    np.testing.assert_array_equal(host(got), ws)
+    # channel counts without 16-byte runs are refused, and so are mixed layouts
+    x = dev(r.standard_normal((2, 6, 9, 9)).astype(np.float32)).contiguous(memory_format=cl)
+    with pytest.raises(RuntimeError):
+        ops.max_pool(x, (3, 3), out=torch.empty((2, 6, 7, 7), device="cuda").contiguous(memory_format=cl))
+    with pytest.raises(RuntimeError):
+        ops.max_pool(x, (3, 3), out=torch.empty((2, 6, 7, 7), device="cuda"))
+    y = r.standard_normal((16, 512, 7, 7)).astype(np.float32)
+    assert_close_f32(host(ops.global_avg_pool(dev(y).contiguous(memory_format=cl))), oracle.global_avgpool(y))
+    yb = bf16_round(y)
+    got = ops.global_avg_pool(dev(yb, torch.bfloat16).contiguous(memory_format=cl))
+    assert_close_bf16(host(got), bf16_round(oracle.global_avgpool(yb)), "channels-last average pool bf16")
