@@ -195,6 +195,12 @@ def build_extra_cases(ops, device, only=()):
               lambda: (_uniform((16, 3, 224, 224), torch.float32, gen, device), _uniform((64, 3, 7, 7), torch.float32, gen, device) * 0.05,
                        torch.empty((16, 64, 112, 112), dtype=torch.float32, device=device)),
               lambda x, w, o: ops.conv2d(x, w, pad=(3, 3, 3, 3), stride=(2, 2), out=o, defer=True), 2)
+    # the same layer as the bf16 network runs it: NCHW operands, the result channels-last for the layers behind it
+    cases.add("conv7x7_stem_3to64_224_channels_last_result", "bf16", "mfma", 2.0 * 16 * 112 * 112 * 64 * 147,
+              (16 * 3 * 224 * 224 + 64 * 147 + 16 * 64 * 112 * 112) * 2,
+              lambda: (_uniform((16, 3, 224, 224), bf, gen, device), _uniform((64, 3, 7, 7), bf, gen, device) * 0.05,
+                       torch.empty((16, 64, 112, 112), dtype=bf, device=device).contiguous(memory_format=torch.channels_last)),
+              lambda x, w, o: ops.conv2d(x, w, pad=(3, 3, 3, 3), stride=(2, 2), out=o, defer=True), 2)
     return cases
 
 
