@@ -191,6 +191,12 @@ def build_extra_cases(ops, device, only=()):
         # scores four more times
         cases.add("attention_unfused_headdim%d_batch8_seq512" % hd, "bf16", "mfma", 4.0 * bh * sq * sq * hd, 4 * bh * sq * hd * 2,
                   make_attn, run_attn, 2)
+    # the fused kernel at the head dims it takes (the same operands as [B, H, S, D])
+    for hd in (32, 64, 128):
+        cases.add("attention_headdim%d_batch8_seq512" % hd, "bf16", "mfma", 4.0 * 96 * 512 * 512 * hd, 4 * 96 * 512 * hd * 2,
+                  lambda hd=hd: tuple(_uniform((8, 12, 512, hd), bf, gen, device) for _ in range(3)) +
+                  (torch.empty((8, 12, 512, hd), dtype=bf, device=device),),
+                  lambda q, k, v, o, hd=hd: ops.attention(q, k, v, None, hd ** -0.5, out=o, defer=True), 2)
     cases.add("conv7x7_stem_3to64_224", "f32", "mfma", 2.0 * 16 * 112 * 112 * 64 * 147, (16 * 3 * 224 * 224 + 64 * 147 + 16 * 64 * 112 * 112) * 4,
               lambda: (_uniform((16, 3, 224, 224), torch.float32, gen, device), _uniform((64, 3, 7, 7), torch.float32, gen, device) * 0.05,
                        torch.empty((16, 64, 112, 112), dtype=torch.float32, device=device)),

@@ -263,10 +263,11 @@ int llc_hip_gather_rows(const llc_tensor* table, const llc_tensor* idx, llc_tens
  * scaling mul/div and the mask add (LLHOps.td:357-393), the softmax chain (amax, sub, exp, sum, div;
  * llcompiler/compiler/torch_compile_config.py:24) and the llh.batch_matmul with v.  The reference lowers each
  * of these to its own loop nest; the fused form never writes the [B, H, Sq, Skv] scores.
- * q, out: [B, H, Sq, 64]; k, v: [B, H, Skv, 64]; f32, bf16 or f16 (f32 operands run on the fp32 MFMA and keep
+ * q, out: [B, H, Sq, D]; k, v: [B, H, Skv, D] with head dim D = 64, or 32 or 128 in the 16-bit types
+ * (LLC_ERR_UNSUPPORTED otherwise); f32, bf16 or f16 (f32 operands run on the fp32 MFMA and keep
  * fp32 probabilities; 16-bit operands round the probabilities to the storage type before the second
  * product, as the unfused group does); the last dim contiguous, the other strides
- * free (multiples of 8 elements), so head-split views of [B, S, H*64] activations are read and written in
+ * free (multiples of 8 elements), so head-split views of [B, S, H*D] activations are read and written in
  * place.  mask: NULL or [B, Skv] of the same type, added to every head and query row.  scale > 0. */
 int llc_hip_attention(const llc_tensor* q, const llc_tensor* k, const llc_tensor* v, const llc_tensor* mask, float scale,
                       llc_tensor* out, void* stream);

@@ -72,11 +72,29 @@ __device__ __forceinline__ uint2 lds_tr16(const char* p) {
 }
 
 // ADD: scores get the additive LDS row (a mask, and -inf for keys past Skv).  Without it Skv is a multiple of 64.
-template <typename T, bool ADD>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void attention_kernel(const AttnParams p) {
-  __shared__ __align__(16) char kt[2][kTileBytes];
-  __shared__ __align__(16) char vt[2][kTileBytes];
-  __shared__ __align__(16) float addrow[2][kBlockKV];
+// D: head dim, 32, 64 or 128.  A K or V block is [64 keys][D values]: 128-byte rows as described above for D = 64; for
+// D = 128 two such tiles side by side (d 0..63, then d 64..127: a k-step of S^T or a d tile of O^T lies in one of
+// them); for D = 32 the same tile with half of every row used (four chunks, swizzled among themselves).
+template <int D>
+struct AttnGeom {
+  static_assert(D == 32 || D == 64 || D == 128, "head dims 32, 64 and 128");
+  static constexpr int KS = D / 16;                    // 16-d steps of S^T
+  static constexpr int DT = D / 32;                    // 32-d tiles of O^T
+  static constexpr int NH = D == 128 ? 2 : 1;          // 64-d tiles side by side
+  static constexpr int CH = D == 32 ? 4 : 8;           // 16-byte chunks in use per 128-byte row
+  static constexpr int kStage = NH * kTileBytes;       // one K (or V) block
+  static constexpr int kLoads = 64 * (D / 8) / 256;    // 16-byte chunks per lane, tensor and block
+  static constexpr int kLds = 4 * kStage + 2 * kBlockKV * 4;
+};
+
+template <typename T, bool ADD, int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 3, D == 128 ? 2 : 3))) void attention_kernel(const AttnParams p) {
+  using G = AttnGeom<D>;
+  constexpr int KS = G::KS, DT = G::DT, CH = G::CH;
+  extern __shared__ __align__(16) char smem[];
+  char* kt0 = smem;                                        // [2][G::kStage]
+  char* vt0 = smem + 2 * G::kStage;                        // [2][G::kStage]
+  float* addrow = (float*)(smem + 4 * G::kStage);          // [2][kBlockKV]
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
   const int li = lane % 32, lh = lane / 32;
   const int bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
@@ -87,32 +105,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   const T* M = p.mask ? (const T*)p.mask + (int64_t)b * p.m_sb : nullptr;
 
   // this lane's query row as the column operand of S^T: 8 consecutive d per 16-d step
-  u32x4_t qf[4];
+  u32x4_t qf[KS];
   {
     const int qrow = q0 + li < p.Sq ? q0 + li : p.Sq - 1;
     const T* qp = Q + (int64_t)qrow * p.q_ss + lh * 8;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const u32x4_t*)(qp + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4_t*)(qp + ks * 16);
   }
 
-  // block loader: 512 16-byte chunks of K and of V by 256 lanes
-  int lrow[2], koff[2], voff[2];
-  const int lc = tid % 8;
+  // block loader: 64 D / 8 16-byte chunks of K and of V by 256 lanes
+  int lrow[G::kLoads], lcol[G::kLoads], koff[G::kLoads], voff[G::kLoads];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    lrow[j] = (tid + 256 * j) / 8;
-    koff[j] = lrow[j] * 128 + ((lc ^ lds_swz(lrow[j])) << 4);
-    voff[j] = lrow[j] * 128 + ((lc ^ ((lrow[j] & 3) << 1)) << 4);
+  for (int j = 0; j < G::kLoads; ++j) {
+    const int id = tid + 256 * j;
+    lrow[j] = id / (D / 8);
+    lcol[j] = id % (D / 8);
+    const int half = lcol[j] / 8, lc = lcol[j] % 8;
+    koff[j] = half * kTileBytes + lrow[j] * 128 + ((lc ^ (lds_swz(lrow[j]) & (CH - 1))) << 4);
+    voff[j] = half * kTileBytes + lrow[j] * 128 + ((lc ^ (((lrow[j] & 3) << 1) & (CH - 1))) << 4);
   }
-  u32x4_t kr[2], vr[2];
+  u32x4_t kr[G::kLoads], vr[G::kLoads];
   float ar = 0.0f;
   auto gload = [&](int blk) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < G::kLoads; ++j) {
       int row = blk * kBlockKV + lrow[j];
       row = row < p.Skv ? row : p.Skv - 1;
-      kr[j] = *(const u32x4_t*)(K + (int64_t)row * p.k_ss + lc * 8);
-      vr[j] = *(const u32x4_t*)(V + (int64_t)row * p.v_ss + lc * 8);
+      kr[j] = *(const u32x4_t*)(K + (int64_t)row * p.k_ss + lcol[j] * 8);
+      vr[j] = *(const u32x4_t*)(V + (int64_t)row * p.v_ss + lcol[j] * 8);
     }
     if constexpr (ADD) {
       if (tid < kBlockKV) {
@@ -126,41 +146,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   };
   auto lstore = [&](int s) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      *(u32x4_t*)(kt[s] + koff[j]) = kr[j];
-      *(u32x4_t*)(vt[s] + voff[j]) = vr[j];
+    for (int j = 0; j < G::kLoads; ++j) {
+      *(u32x4_t*)(kt0 + s * G::kStage + koff[j]) = kr[j];
+      *(u32x4_t*)(vt0 + s * G::kStage + voff[j]) = vr[j];
     }
     if constexpr (ADD) {
-      if (tid < kBlockKV) addrow[s][tid] = ar;
+      if (tid < kBlockKV) addrow[s * kBlockKV + tid] = ar;
     }
   };
 
   // fragment addresses inside a stage
-  int ka[2][4];  // K rows 32 T + li, chunk 2 ks + lh
+  int ka[2][KS];  // K rows 32 T + li, chunk 2 ks + lh of the 64-d tile the k-step lies in
 #pragma unroll
   for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
       const int row = 32 * t2 + li;
-      ka[t2][ks] = row * 128 + (((2 * ks + lh) ^ lds_swz(row)) << 4);
+      ka[t2][ks] = (ks / 4) * kTileBytes + row * 128 + (((2 * (ks % 4) + lh) ^ (lds_swz(row) & (CH - 1))) << 4);
     }
   // V: a 16-lane group reads a 4 (keys) x 16 (d) patch; lane = 16 g + 4 jj + q addresses key row jj, d chunk q
-  int va[2][2];  // [d tile][which run of four keys]
+  int va[DT][2];  // [d tile][which run of four keys]
   {
     const int g = lane / 16, jj = (lane / 4) % 4, q = lane % 4;
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int row = 8 * u + 4 * (g >> 1) + jj;
-        const int c = 4 * dt + 2 * (g & 1) + (q >> 1);
-        va[dt][u] = row * 128 + ((c ^ (jj << 1)) << 4) + (q & 1) * 8;
+        const int c = 4 * (dt % 2) + 2 * (g & 1) + (q >> 1);
+        va[dt][u] = (dt / 2) * kTileBytes + row * 128 + ((c ^ ((jj << 1) & (CH - 1))) << 4) + (q & 1) * 8;
       }
   }
 
-  f32x16_t oacc[2];
+  f32x16_t oacc[DT];
 #pragma unroll
-  for (int dt = 0; dt < 2; ++dt)
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
@@ -172,8 +192,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   for (int blk = 0; blk < nblk; ++blk) {
     const int s = blk & 1;
     if (blk + 1 < nblk) gload(blk + 1);
-    const char* kb = kt[s];
-    const char* vb = vt[s];
+    const char* kb = kt0 + s * G::kStage;
+    const char* vb = vt0 + s * G::kStage;
 
     // S^T = K Q^T for 64 keys x 32 queries
     f32x16_t sacc[2];
@@ -182,7 +202,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[t2][r] = 0.0f;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) mfma_step<T>(*(const u32x4_t*)(kb + ka[t2][ks]), qf[ks], sacc[t2]);
+      for (int ks = 0; ks < KS; ++ks) mfma_step<T>(*(const u32x4_t*)(kb + ka[t2][ks]), qf[ks], sacc[t2]);
     }
     // x = scores in log2 units; accumulator register 4 i + j of tile T is key 32 T + 8 i + 4 lh + j
     float mx = -INFINITY;
@@ -191,7 +211,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if constexpr (ADD) {
-          const f32x4_t av = *(const f32x4_t*)&addrow[s][32 * t2 + 8 * i + 4 * lh];
+          const f32x4_t av = *(const f32x4_t*)&addrow[s * kBlockKV + 32 * t2 + 8 * i + 4 * lh];
 #pragma unroll
           for (int j = 0; j < 4; ++j) sacc[t2][4 * i + j] = fmaf(sacc[t2][4 * i + j], p.scale_log2e, av[j]);
         }
@@ -212,7 +232,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       m_run = m_max;
       l_run *= corr;
 #pragma unroll
-      for (int dt = 0; dt < 2; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
     }
@@ -242,7 +262,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       for (int t = 0; t < 2; ++t) {
         const char* vrow = vb + (32 * t2 + 16 * t) * 128;
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) {
+        for (int dt = 0; dt < DT; ++dt) {
           const uint2 lo = lds_tr16(vrow + va[dt][0]), hi = lds_tr16(vrow + va[dt][1]);
           mfma_step<T>(u32x4_t{lo.x, lo.y, hi.x, hi.y}, pb[t2][t], oacc[dt]);
         }
@@ -256,7 +276,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   if (q0 + li < p.Sq) {
     T* op = (T*)p.O + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)(q0 + li) * p.o_ss;
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         uint2 w;
@@ -656,7 +676,10 @@ int launch_f32(const AttnParams& p, hipStream_t s) {
 int view4(const llc_tensor* t, const char* what, View* v) {
   LLC_TRY(make_view(t, what, v));
   if (v->rank != 4) return set_error(LLC_ERR_SHAPE, "%s: rank 4 expected, [B, H, S, D]", what);
-  if (v->size[3] != kD) return set_error(LLC_ERR_UNSUPPORTED, "%s: head dim %lld (64 is implemented)", what, (long long)v->size[3]);
+  const bool wide = v->dtype == LLC_BFLOAT16 || v->dtype == LLC_FLOAT16;
+  if (v->size[3] != kD && !(wide && (v->size[3] == 32 || v->size[3] == 128)))
+    return set_error(LLC_ERR_UNSUPPORTED, "%s: head dim %lld (64, and 32 or 128 in the 16-bit types, are implemented)", what,
+                     (long long)v->size[3]);
   if (v->stride[3] != 1 || v->stride[0] % 8 || v->stride[1] % 8 || v->stride[2] % 8 || ((uintptr_t)v->ptr % 16))
     return set_error(LLC_ERR_LAYOUT, "%s: the head dim must be contiguous and every row 16-byte aligned", what);
   return LLC_OK;
@@ -675,6 +698,8 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
   LLC_TRY(view4(v, "attention v", &c));
   LLC_TRY(view4(out, "attention out", &o));
   if (a.dtype != b.dtype || a.dtype != c.dtype || a.dtype != o.dtype) return set_error(LLC_ERR_DTYPE, "attention: operand types differ");
+  if (a.size[3] != b.size[3] || a.size[3] != c.size[3] || a.size[3] != o.size[3]) return set_error(LLC_ERR_SHAPE, "attention: head dims differ");
+  const int hd = (int)a.size[3];
   if (a.dtype != LLC_BFLOAT16 && a.dtype != LLC_FLOAT16 && a.dtype != LLC_FLOAT32)
     return set_error(LLC_ERR_DTYPE, "attention: f32, bf16 or f16 operands (type %d given)", a.dtype);
   for (int d = 0; d < 2; ++d)
@@ -714,7 +739,7 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
     return p.mask ? launch_f32<2, true>(p, s) : launch_f32<2, false>(p, s);
   }
   const bool add = p.mask || p.Skv % kBlockKV != 0;
-  if ((int64_t)((p.Sq + kBlockQ - 1) / kBlockQ) * p.B * p.H < 128 && p.Skv > 3 * kBlockKV) {
+  if (hd == kD && (int64_t)((p.Sq + kBlockQ - 1) / kBlockQ) * p.B * p.H < 128 && p.Skv > 3 * kBlockKV) {
     // fewer workgroups of 128 queries than half the CUs, and keys enough for every wave: 32 queries per workgroup,
     // the key blocks dealt to its four waves (12 heads, 512 x 512: one sequence 10.7 -> 6.6 us, two 10.9 -> 9.4 us;
     // four sequences, 192 workgroups of 128 queries, are faster as they were: 11.4 against 16.6 us)
@@ -729,12 +754,26 @@ int llc_impl_attention(const llc_tensor* q, const llc_tensor* k, const llc_tenso
     return add ? go(attention_split_kernel<_Float16, true>) : go(attention_split_kernel<_Float16, false>);
   }
   const dim3 grid((unsigned)((p.Sq + kBlockQ - 1) / kBlockQ), (unsigned)(p.B * p.H));
-  if (a.dtype == LLC_BFLOAT16) {
-    if (add) hipLaunchKernelGGL((attention_kernel<__bf16, true>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((attention_kernel<__bf16, false>), grid, dim3(256), 0, s, p);
-  } else {
-    if (add) hipLaunchKernelGGL((attention_kernel<_Float16, true>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((attention_kernel<_Float16, false>), grid, dim3(256), 0, s, p);
+  auto run = [&](auto kern, int lds, std::atomic<uint32_t>& allowed) {
+    LLC_TRY(allow_dynamic_lds((const void*)kern, lds, allowed));
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p);
+    return (int)LLC_OK;
+  };
+#define LLC_ATTN_LAUNCH(TT, DD)                                                                          \
+  {                                                                                                      \
+    static std::atomic<uint32_t> allowed[2];                                                             \
+    LLC_TRY(add ? run(attention_kernel<TT, true, DD>, AttnGeom<DD>::kLds, allowed[1])                    \
+                : run(attention_kernel<TT, false, DD>, AttnGeom<DD>::kLds, allowed[0]));                 \
   }
+  if (a.dtype == LLC_BFLOAT16) {
+    if (hd == 32) LLC_ATTN_LAUNCH(__bf16, 32)
+    else if (hd == 64) LLC_ATTN_LAUNCH(__bf16, 64)
+    else LLC_ATTN_LAUNCH(__bf16, 128)
+  } else {
+    if (hd == 32) LLC_ATTN_LAUNCH(_Float16, 32)
+    else if (hd == 64) LLC_ATTN_LAUNCH(_Float16, 64)
+    else LLC_ATTN_LAUNCH(_Float16, 128)
+  }
+#undef LLC_ATTN_LAUNCH
   return check_launch("attention_kernel");
 }

@@ -41,7 +41,8 @@ MIN_CALLS_FOR_GRAPH = 2
 # reference's packed parameter block and make one call into the library, which replays the launches.  With
 # False every run launches kernel by kernel from Python (same kernels, same arguments).
 USE_PLAN = True
-# batch_matmul -> softmax -> batch_matmul groups of attention layers with head dim 64 become one fused kernel
+# batch_matmul -> softmax -> batch_matmul groups of attention layers with head dim 64 (32 and 128 too in the 16-bit
+# types) become one fused kernel
 FUSE_ATTENTION = True
 # convolutions whose channel count is a multiple of 128 bytes' worth of values (32 fp32, 64 bf16 / f16) run on
 # channels-last (NHWC) copies of their operands: the kernel for that layout needs no gather arithmetic.  Results keep the layout as strided views (logical shape NCHW), so a chain of
@@ -397,8 +398,9 @@ class Instance:
             return sm, u, between
 
         def fused_attention(st):
-            """Emits one attention call for the group that starts at `st` when the operands allow it (head dim 64,
-            rows addressable as [B, H, S, 64] views); returns False to leave the group to its own kernels."""
+            """Emits one attention call for the group that starts at `st` when the operands allow it (head dim 64, or
+            32 or 128 in the 16-bit types; rows addressable as [B, H, S, D] views); returns False to leave the group to
+            its own kernels."""
             grp = attention_group(st)
             if grp is None:
                 return False
@@ -436,7 +438,8 @@ class Instance:
                 return False
             k4 = k4.transpose(-1, -2)
             for t in (q4, k4, v4):
-                if t.shape[3] != 64 or t.stride(3) != 1 or any(s % 8 for s in t.stride()[:3]) or t.data_ptr() % 16:
+                dims = (64,) if t.dtype == torch.float32 else (32, 64, 128)
+                if t.shape[3] not in dims or t.stride(3) != 1 or any(s % 8 for s in t.stride()[:3]) or t.data_ptr() % 16:
                     return False
             if k4.shape[2] != v4.shape[2] or k4.shape[2] != nat[2] or q4.shape[2] != nat[1] or k4.shape[2] == 0:
                 return False
@@ -445,12 +448,12 @@ class Instance:
                 mask = materialise(val[id(e["bias"])])
                 mask = contiguous(mask.reshape(-1) if mask.is_contiguous() else mask).reshape(-1).view(b0, nat[2])
             out = new_tensor(second.output)
-            sq = nat[1]
-            o4 = out.view(b0, b1, sq, 64)
-            hm = head_merge(second, b0 * b1, sq, 64)
+            sq, hd = nat[1], q4.shape[3]
+            o4 = out.view(b0, b1, sq, hd)
+            hm = head_merge(second, b0 * b1, sq, hd)
             if hm is not None and (hm[1], hm[2]) == (b0, b1):
-                # the head merge that follows, [B, H, S, 64] -> [B, S, H, 64], is done by the kernel's stores
-                o4 = out.view(-1).view(b0, sq, b1, 64).permute(0, 2, 1, 3)
+                # the head merge that follows, [B, H, S, D] -> [B, S, H, D], is done by the kernel's stores
+                o4 = out.view(-1).view(b0, sq, b1, hd).permute(0, 2, 1, 3)
                 val[id(hm[0].output)] = o4
                 skip.add(id(hm[0]))
             if out.numel():

@@ -278,8 +278,8 @@ def convert(x, dtype, out=None, defer=False):
 
 
 def attention(q, k, v, mask=None, scale=1.0, out=None, defer=False):
-    """softmax(scale * q k^T + mask) v.  q, out: [B, H, Sq, 64]; k, v: [B, H, Skv, 64] (strided views allowed, last
-    dim contiguous); mask: None or [B, Skv]."""
+    """softmax(scale * q k^T + mask) v.  q, out: [B, H, Sq, D]; k, v: [B, H, Skv, D] (strided views allowed, last
+    dim contiguous; D = 64, or 32 or 128 in bf16 / f16); mask: None or [B, Skv]."""
     dev = _dev(q)
     if out is None:
         out = torch.empty(tuple(q.shape), dtype=q.dtype, device=dev)

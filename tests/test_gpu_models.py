@@ -265,6 +265,28 @@ def test_attention_group_becomes_one_kernel_bf16():
     assert_as_close_as_eager(ub, eager_b, want_b, BF16_RTOL, BF16_ATOL, "bert bf16, unfused")
 
 
+@pytest.mark.parametrize("heads,head_dim", [(8, 32), (3, 128), (4, 96)])
+def test_attention_group_at_other_head_dims_bf16(heads, head_dim):
+    """Encoder blocks with heads of 32 and 128 run their attention group as llc_hip_attention too; a head dim the
+    kernel does not take (96) keeps the three kernels of the group.  Against the float64 evaluation either way."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
+    hidden = heads * head_dim
+    enc = EncoderBlock(hidden=hidden, heads=heads, ffn=2 * hidden).eval().to(torch.bfloat16)
+    (x,) = make_encoder_inputs(2, 192, hidden, dtype=torch.bfloat16)
+    with torch.no_grad():
+        cm = compile_module(copy.deepcopy(enc).cuda(), (x.cuda(),))
+        got = cm(x.cuda()).float().cpu().numpy()
+        names = _kernel_names(cm.engine)[0]
+        want = copy.deepcopy(enc).double()(x.double()).numpy()
+        eager = copy.deepcopy(enc).cuda()(x.cuda()).float().cpu().numpy()
+    if head_dim == 96:
+        assert names.count("llc_hip_attention") == 0 and names.count("llc_hip_batch_matmul") == 2 and names.count("llc_hip_softmax") == 1
+    else:
+        assert names.count("llc_hip_attention") == 1 and names.count("llc_hip_batch_matmul") == 0 and names.count("llc_hip_softmax") == 0
+    assert_as_close_as_eager(got, eager, want, BF16_RTOL, BF16_ATOL, "encoder with %d heads of %d" % (heads, head_dim))
+
+
 def test_dynamic_torch_compile_reuses_one_engine():
     from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
     enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()

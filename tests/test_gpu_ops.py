@@ -699,6 +699,41 @@ def test_attention(ops, oracle, B, H, Sq, Skv, masked):
         close(host(merged).transpose(0, 2, 1, 3), want, "attention on head-split views %s" % dt)
 
 
+@pytest.mark.parametrize("D", [32, 128])
+@pytest.mark.parametrize("B,H,Sq,Skv,masked", [(1, 1, 128, 128, False), (2, 3, 100, 200, True), (3, 2, 33, 77, False),
+                                             (1, 1, 1, 1, True), (2, 12, 256, 256, True), (1, 2, 130, 448, False)])
+def test_attention_head_dims_32_and_128(ops, oracle, D, B, H, Sq, Skv, masked):
+    """The fused kernel in the 16-bit types at the other two head dims it takes (half a 128-byte row per key, and two
+    64-wide tiles side by side), contiguous operands and head-split views; fp32 operands of those head dims are refused."""
+    r = rng(D * 7 + B * 1000 + H * 100 + Sq + Skv)
+    q = bf16_round(r.uniform(-1, 1, (B, H, Sq, D)))
+    k = bf16_round(r.uniform(-1, 1, (B, H, Skv, D)))
+    v = bf16_round(r.uniform(-1, 1, (B, H, Skv, D)))
+    mask = None
+    if masked:
+        mask = np.zeros((B, Skv), np.float32)
+        for b in range(B):
+            mask[b, int(r.integers(Skv // 2, Skv)) + 1:] = -1e4
+        mask = bf16_round(mask)
+    scale = float(D) ** -0.5
+    for dt, rnd in ((torch.bfloat16, bf16_round), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+        want = _attention_oracle(oracle, q, k, v, mask, scale, rnd)
+        got = ops.attention(dev(q, dt), dev(k, dt), dev(v, dt), dev(mask, dt) if masked else None, scale)
+        assert_close_bf16(host(got), want, "attention head dim %d %s" % (D, dt))
+    qs = dev(np.ascontiguousarray(q.transpose(0, 2, 1, 3)).reshape(B, Sq, H * D), torch.bfloat16)
+    ks = dev(np.ascontiguousarray(k.transpose(0, 2, 1, 3)).reshape(B, Skv, H * D), torch.bfloat16)
+    vs = dev(np.ascontiguousarray(v.transpose(0, 2, 1, 3)).reshape(B, Skv, H * D), torch.bfloat16)
+    merged = torch.zeros((B, Sq, H, D), dtype=torch.bfloat16, device="cuda")
+    ops.attention(qs.view(B, Sq, H, D).permute(0, 2, 1, 3), ks.view(B, Skv, H, D).permute(0, 2, 1, 3),
+                  vs.view(B, Skv, H, D).permute(0, 2, 1, 3), dev(mask, torch.bfloat16) if masked else None, scale,
+                  out=merged.permute(0, 2, 1, 3))
+    assert_close_bf16(host(merged).transpose(0, 2, 1, 3), _attention_oracle(oracle, q, k, v, mask, scale, bf16_round),
+                      "attention on head-split views, head dim %d" % D)
+    from llcompiler_amd._capi import LlcHipError
+    with pytest.raises(LlcHipError):
+        ops.attention(dev(q), dev(k), dev(v), None, scale)
+
+
 @pytest.mark.parametrize("seed", range(3))
 def test_random_bmm_attention_pool_gather_cases(ops, oracle, seed):
     """Randomly drawn batched products (rank 3 and the rank-4 head-split form, either operand a transposed view,
