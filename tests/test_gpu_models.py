@@ -706,6 +706,28 @@ def test_resnet18_stays_channels_last_from_the_stem_on(dtype):
         assert torch.equal(cm(x.cuda()), got)
 
 
+def test_resnet18_bf16_at_the_benchmark_size():
+    """The bf16 line of the ResNet configuration at the size bench.py times (batch 16, 224 x 224): the 16-bit first-layer
+    kernel on 224-wide rows, channels-last pools, every body layer on its benchmark shape.  The yardstick is torch's
+    fp32 evaluation of the same bf16-valued weights on the GPU (a float64 evaluation of 58 GFLOP on the host would
+    take minutes; fp32 is 2^15 times finer than the bar), the reference evaluation torch's own bf16 kernels."""
+    from llcompiler_amd.compiler.aot import compile_module
+    from llcompiler_amd.test_models import ResNet18Folded, make_resnet_inputs
+    m = ResNet18Folded().eval().to(torch.bfloat16)
+    (x,) = make_resnet_inputs(16, 224)
+    x = x.to(torch.bfloat16)
+    with torch.no_grad():
+        mg = copy.deepcopy(m).cuda()
+        want32 = copy.deepcopy(m).float().cuda()(x.float().cuda()).double().cpu().numpy()
+        eager = mg(x.cuda()).float().cpu().numpy()
+        cm = compile_module(copy.deepcopy(m).cuda(), (x.cuda(),))
+        got = cm(x.cuda())
+        names = [c.fn.__name__ for c in list(cm.engine.instances.values())[0].calls]
+        assert names.count("llc_hip_copy") == 0 and names.count("llc_hip_conv2d") == 20, names
+        _assert_as_close_as_eager(got.float().cpu().numpy(), eager, want32, BF16_RTOL, BF16_ATOL, "resnet18 bf16 16x3x224x224")
+        assert torch.equal(cm(x.cuda()), got)
+
+
 def _plan_file_round_trip(cm, args, path):
     """Saves the plan of the (single) instance of an export-compiled module, loads it back and runs it on the
     tensors the engine passes for `args`; returns the outputs of that run."""
