@@ -110,6 +110,50 @@ def is_float(e):
     return any(is_float(a) for a in e.args)
 
 
+def _affine(e, scale, terms, order):
+    """Adds scale * e to the integer-affine form (terms: atom -> coefficient, terms[None]: the constant); returns
+    False when e holds a float constant (real-valued trees are left as they are written)."""
+    if isinstance(e, int):
+        terms[None] = terms.get(None, 0) + scale * e
+        return True
+    if not isinstance(e, Expr):
+        return False
+    if e.kind in ("add", "sub"):
+        return _affine(e.args[0], scale, terms, order) and _affine(e.args[1], scale if e.kind == "add" else -scale, terms, order)
+    if e.kind == "mul" and isinstance(e.args[0], int):
+        return _affine(e.args[1], scale * e.args[0], terms, order)
+    if e.kind == "mul" and isinstance(e.args[1], int):
+        return _affine(e.args[0], scale * e.args[1], terms, order)
+    if e not in terms:
+        order.append(e)
+    terms[e] = terms.get(e, 0) + scale
+    return True
+
+
+def _normal_sum(e):
+    """An integer sum / difference / multiple in one canonical form: atoms in order of first appearance, each with
+    its collected coefficient, then the collected constant.  (H + 2) - 3 + 1 becomes H, so that the extent of a
+    padded stride-1 window equals the extent it was computed from, structurally.)"""
+    terms, order = {}, []
+    if is_float(e) or not _affine(e, 1, terms, order):
+        return e
+    out = None
+    for atom in order:
+        c = terms[atom]
+        if c == 0:
+            continue
+        t = atom if c == 1 else Expr("mul", (c, atom))
+        out = t if out is None else Expr("add", (out, t))
+    c = terms.get(None, 0)
+    if out is None:
+        return c
+    if c > 0:
+        return Expr("add", (out, c))
+    if c < 0:
+        return Expr("sub", (out, -c))
+    return out
+
+
 def simplify(e):
     if not isinstance(e, Expr) or e.kind == "sym":
         return e
@@ -117,6 +161,8 @@ def simplify(e):
     if all(isinstance(x, _NUM) for x in a):
         return evaluate(Expr(e.kind, a), {})
     k = e.kind
+    if k in ("add", "sub") or (k == "mul" and (isinstance(a[0], int) or isinstance(a[1], int))):
+        return _normal_sum(Expr(k, a))
     if k == "add":
         if a[0] == 0: return a[1]
         if a[1] == 0: return a[0]

@@ -287,6 +287,82 @@ def test_attention_group_at_other_head_dims_bf16(heads, head_dim):
     assert_as_close_as_eager(got, eager, want, BF16_RTOL, BF16_ATOL, "encoder with %d heads of %d" % (heads, head_dim))
 
 
+@pytest.mark.parametrize("dynamic", [True, False])
+def test_the_reference_driver_example_multihead_attention(dynamic):
+    """What the reference's own driver script runs (main.py:63-69): its MultiHeadedAttention test model, which forwards
+    to torch.nn.MultiheadAttention(8, 2) (llcompiler/test_models/models/multi_head_attention.py:35-55), on three
+    [2, 24, 8] inputs through torch.compile(backend=LLCompiler(...), dynamic=True, fullgraph=False), both results
+    (the attention output and the head-averaged weights) held against eager as its check_same does.  Everything is
+    compiled: one engine, no node left to eager."""
+    from llcompiler_amd import LLCompiler
+
+    class MultiHeadedAttention(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attention = torch.nn.MultiheadAttention(8, 2)
+
+        def forward(self, query, key, value, mask=None):
+            return self.attention(query, key, value, mask)
+
+    torch.manual_seed(0)
+    m = MultiHeadedAttention().eval()
+    ins = [torch.randn(2, 24, 8) for _ in range(3)]
+    with torch.no_grad():
+        want = m(*ins)
+        torch._dynamo.reset()
+        comp = LLCompiler(mode="inference", target="gfx950", pipeline="hip")
+        opt = torch.compile(copy.deepcopy(m).cuda(), backend=comp, dynamic=dynamic, fullgraph=False)
+        got = opt(*[t.cuda() for t in ins])
+        again = opt(*[t.cuda() for t in ins])
+    assert len(comp.engines) == 1
+    kinds = [s.kind for s in comp.engines[0].steps]
+    assert kinds.count("matmul") == 4 and kinds.count("batch_matmul") == 2 and kinds.count("softmax") == 1
+    assert len(got) == 2
+    for g, a, w, what in zip(got, again, want, ("attention output", "averaged attention weights")):
+        assert tuple(g.shape) == tuple(w.shape)
+        assert_close(g.cpu().numpy(), w.numpy(), F32_RTOL, F32_ATOL, "nn.MultiheadAttention(8, 2): " + what)
+        assert torch.equal(g, a)
+
+
+def test_the_reference_resnet_test_model():
+    """The reference's Resnet test model (llcompiler/test_models/models/resnet.py:18-40, on the [1, 3, 64, 64] input of
+    main.py:70): torchvision's resnet18 with 10 classes run up to layer3, its average pool replaced by
+    Flatten + Linear(4096, 512), then the fc layer.  torchvision is not importable here, so the same graph is spelt
+    with this package's torchvision-style units (Conv2d without bias + BatchNorm2d, randomised statistics); through
+    torch.compile with dynamic shapes and fullgraph=False, as the driver script does."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.test_models import ResNet18BN
+
+    class Resnet(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.resnet = ResNet18BN(num_classes=10)
+            self.resnet.fc = torch.nn.Linear(512, 10)
+            self.head = torch.nn.Sequential(torch.nn.Flatten(1), torch.nn.Linear(4096, 512))
+
+        def forward(self, x):
+            r = self.resnet
+            x = torch.nn.functional.max_pool2d(r.stem(x), 3, 2, 1)
+            x = r.blocks[:6](x)          # layer1 .. layer3
+            x = self.head(x)
+            x = torch.flatten(x, 1)
+            return r.fc(x)
+
+    torch.manual_seed(0)
+    m = Resnet().eval()
+    x = torch.randn(1, 3, 64, 64)
+    with torch.no_grad():
+        want = m(x)
+        torch._dynamo.reset()
+        comp = LLCompiler(mode="inference", target="gfx950", pipeline="hip")
+        opt = torch.compile(copy.deepcopy(m).cuda(), backend=comp, dynamic=True, fullgraph=False)
+        got = opt(x.cuda())
+    assert len(comp.engines) == 1
+    kinds = [s.kind for s in comp.engines[0].steps if not s.attrs.get("prepared") and s.kind not in ("view", "constant")]
+    assert kinds.count("conv") == 15 and kinds.count("ew") == 0 and kinds.count("matmul") == 2, kinds
+    assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "the reference's Resnet test model")
+
+
 def test_dynamic_torch_compile_reuses_one_engine():
     from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
     enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()

@@ -559,3 +559,40 @@ def test_softmax_half_to_float_widens_before_the_softmax():
     assert names.index("convert_to") < names.index("softmax")
     sm = next(op for op in g.ops if op.name == "softmax")
     assert sm.operands[0].dtype == f32 and sm.results[0].dtype == f32
+
+
+def test_integer_sums_of_extents_have_one_form():
+    """Extents are compared structurally (a same-shape add behind a convolution becomes its residual only if the two
+    shapes are equal), so sums, differences and integer multiples collapse to one canonical form: the extent of a
+    padded stride-1 window is the extent it was computed from."""
+    h, w = Expr.sym("s0"), Expr.sym("s1")
+    assert (h + 1 + 1 - 2 - 1) // 1 + 1 == h           # 3x3 window, pad 1, stride 1
+    assert (h + 3 + 3 - 6 - 1) // 1 + 1 == h           # 7x7 window, pad 3
+    assert 2 * (h + 1) - 2 == 2 * h and h * 2 - h == h and (3 - h) + h == 3 and h - h == 0
+    pooled = (h + 1 + 1 - 2 - 1) // 2 + 1              # 3x3 window, pad 1, stride 2: stays a quotient
+    assert pooled == (h - 1) // 2 + 1 and (pooled + 2 - 3) // 1 + 1 == pooled
+    assert (h + w) - w == h and (h * w + 4) - 4 == h * w
+    for e, want in (((h + 1 + 1 - 2 - 1) // 2 + 1, 4), (2 * (h + 1) - 2 + w, 17), ((3 - h) * 2 + w, -5)):
+        assert evaluate(e, {"s0": 7, "s1": 3}) == want
+    assert repr(h / 2 + 1.5) == "((s0 / 2) + 1.5)"     # real-valued trees stay as written
+
+
+def test_residual_adds_fuse_under_symbolic_image_extents():
+    """A basic block traced with symbolic height and width: conv(3x3, pad 1) of a [N, C, H', W'] tensor has the shape
+    of the block's input, and the add + relu behind it become the convolution's epilogue."""
+    from llcompiler_amd.llh.passes import run_llh_pipeline
+    g = Graph()
+    n, hh, ww = Expr.sym("s0"), Expr.sym("s1"), Expr.sym("s2")
+    x = g.add_input((n, 8, hh, ww), f32)
+    w1 = g.add_input((8, 8, 3, 3), f32)
+    w2 = g.add_input((8, 8, 3, 3), f32)
+    attrs = {"dilation": (1, 1), "kernel_shape": (3, 3), "pad": (1, 1, 1, 1), "stride": (1, 1), "group": 1}
+    y = g.add_op("relu", [g.add_op("conv", [x, w1], dict(attrs))])
+    c2 = g.add_op("conv", [y, w2], dict(attrs))
+    assert tuple(c2.shape) == tuple(x.shape)
+    z = g.add_op("relu", [g.add_op("add", [c2, x])])
+    g.set_outputs([z])
+    run_llh_pipeline(g)
+    steps = [s for s in make_plan(g) if s.kind not in ("view", "constant")]
+    assert [s.kind for s in steps] == ["conv", "conv"]
+    assert steps[1].attrs["epilogue"]["residual"] is not None and steps[1].attrs["epilogue"]["act"] == "relu"
