@@ -1028,7 +1028,66 @@ class Torch_ExecutionEngine(ExecutionEngine):
             env[name] = v
         for name, (i, d) in g.symbol_sources.items():
             env.setdefault(name, inputs[i].shape[d])
+        derived = self._derived_symbols()
+        if derived[0]:
+            self._solve_derived(env, inputs, derived)
         return env
+
+    def _derived_symbols(self):
+        """Symbols the graph uses that no int argument and no input dim states directly: a partition of a dynamically
+        shaped graph may see a symbol only inside its inputs' extents (every tensor it gets is a strided convolution's
+        result, of extent (s - 1) // 2 + 1).  Returns (names, [(input index, dim, extent expression)]), computed once."""
+        d = getattr(self, "_derived", None)
+        if d is None:
+            g = self.graph
+            known = set(g.symbol_args) | set(g.symbol_sources)
+            names = sorted(n for n in g.symbols() if n not in known)
+            eqs = []
+            if names:
+                for i, v in enumerate(g.inputs):
+                    for k, e in enumerate(v.shape):
+                        if isinstance(e, Expr) and e.kind != "sym" and any(n in names for n in e.symbols()):
+                            eqs.append((i, k, e))
+            d = self._derived = (names, eqs, {})
+        return d
+
+    def _solve_derived(self, env, inputs, derived):
+        """Values for the derived symbols from the extents that contain them.  The graph's other extents are functions
+        of its inputs' extents, so ANY value that reproduces those gives the right shapes everywhere; extents are
+        non-decreasing in their symbols (window arithmetic: sums, products and floor divisions by positive numbers),
+        so each is found by bisection on an equation with one unknown left, and every equation is checked at the end."""
+        names, eqs, cache = derived
+        key = tuple(inputs[i].shape[k] for i, k, _ in eqs)
+        found = cache.get(key)
+        if found is None:
+            trial = dict(env)
+            left = [n for n in names if n not in trial]
+            progress = True
+            while left and progress:
+                progress = False
+                for (i, k, e), want in zip(eqs, key):
+                    unknown = [n for n in e.symbols() if n not in trial]
+                    if len(unknown) != 1:
+                        continue
+                    n, lo, hi = unknown[0], 0, 1
+                    while evaluate(e, dict(trial, **{n: hi})) < want and hi < (1 << 40):
+                        hi *= 2
+                    while lo < hi:  # smallest value whose extent reaches `want`
+                        mid = (lo + hi) // 2
+                        if evaluate(e, dict(trial, **{n: mid})) < want:
+                            lo = mid + 1
+                        else:
+                            hi = mid
+                    trial[n] = lo
+                    left.remove(n)
+                    progress = True
+            ok = not left and all(evaluate(e, trial) == want for (_, _, e), want in zip(eqs, key))
+            found = cache[key] = {n: trial[n] for n in names} if ok else False
+        if found is False:
+            missing = [n for n in names if n not in env]
+            raise KeyError("symbol %s is not bound by any input of this call" % ", ".join(missing))
+        for n, v in found.items():
+            env.setdefault(n, v)
 
     def save_plan(self, path, *args):
         """Runs the graph for `args` (so that the plan for those extents exists and is recorded), writes that plan

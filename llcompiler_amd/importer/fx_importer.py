@@ -763,6 +763,25 @@ def is_supported(node):
         return False
 
 
+def _as_traced(ctx, v, node):
+    """The translated value with the rank torch traced.  Python scalars enter the graph as tensor<1xT> constants
+    (TorchToLLH keeps them that way), so an op between a 0-d tensor and a number comes out as tensor<1xT> where torch
+    has a 0-d tensor (`num_batches_tracked + 1` of a batch norm in training mode, whose result aot autograd copies back
+    into the 0-d buffer): same elements, a reshape to the traced shape."""
+    val = node.meta.get("val")
+    if not isinstance(v, Value) or not isinstance(val, torch.Tensor):
+        return v
+    want = meta_shape(val)
+    if len(want) == v.rank or any(not isinstance(d, int) for d in tuple(want) + tuple(v.shape)):
+        return v
+    n_want = n_have = 1
+    for d in want:
+        n_want *= d
+    for d in v.shape:
+        n_have *= d
+    return _reshape_to(ctx, v, want) if n_want == n_have else v
+
+
 def torch_translate_to_llh_graph(gm, weight_files=None):
     """Counterpart of torch_translate_to_mlir_module (llcompiler/importer/fx_translate.py:517-521).
 
@@ -803,7 +822,7 @@ def torch_translate_to_llh_graph(gm, weight_files=None):
             tr = TORCH_FUNCTION_TRANSLATE.get(node.target)
             if tr is None:
                 raise NotImplementedError("no LLH translation for %s" % (node.target,))
-            ctx.env[node] = tr(ctx, node)
+            ctx.env[node] = _as_traced(ctx, tr(ctx, node), node)
         elif node.op == "output":
             outs = node.args[0]
             single = not isinstance(outs, (tuple, list))

@@ -363,6 +363,51 @@ def test_the_reference_resnet_test_model():
     assert_close(got.cpu().numpy(), want.numpy(), F32_RTOL, F32_ATOL, "the reference's Resnet test model")
 
 
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_training_mode_resnet_units_with_batch_statistics(dynamic):
+    """The first units of the torchvision-style ResNet in TRAINING mode (batch statistics, running statistics and the
+    0-d num_batches_tracked counters updated in place), static and dynamic shapes, fullgraph=False as the reference's
+    driver runs its models: forward, parameter gradients and the updated buffers against eager.  Batch-norm training
+    and the convolution backward stay in eager (torch_compile_config.py:29-62 has neither); the partitions between them
+    see the image-size symbol only inside strided extents."""
+    from llcompiler_amd import LLCompiler
+    from llcompiler_amd.test_models import ResNet18BN
+
+    class Units(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.r = ResNet18BN(num_classes=10)
+
+        def forward(self, x):
+            r = self.r
+            x = torch.nn.functional.max_pool2d(r.stem(x), 3, 2, 1)
+            return r.blocks[:2](x).mean(dim=(2, 3))
+
+    torch.manual_seed(0)
+    base = Units()
+    x = torch.randn(4, 3, 64, 64)
+    torch._dynamo.reset()
+    ref, mg = copy.deepcopy(base).train(), copy.deepcopy(base).train().cuda()
+    comp = LLCompiler(mode="training", target="gfx950", pipeline="hip")
+    opt = torch.compile(mg, backend=comp, dynamic=dynamic, fullgraph=False)
+    out = opt(x.cuda())
+    out.sum().backward()
+    want = ref(x)
+    want.sum().backward()
+    assert comp.compile_count >= 1
+    assert_close(out.detach().cpu().numpy(), want.detach().numpy(), F32_RTOL, F32_ATOL, "training-mode units, forward")
+    for (name, a), b in zip(mg.named_parameters(), ref.parameters()):
+        if b.grad is not None:
+            scale = max(1.0, float(b.grad.abs().max()))
+            assert_close(a.grad.cpu().numpy(), b.grad.numpy(), F32_RTOL, F32_ATOL * scale, "gradient of " + name)
+    for (name, a), b in zip(mg.named_buffers(), ref.buffers()):
+        assert a.shape == b.shape, name
+        if b.dtype == torch.long:
+            assert torch.equal(a.cpu(), b), name
+        else:
+            assert_close(a.cpu().numpy(), b.numpy(), F32_RTOL, F32_ATOL, "buffer " + name)
+
+
 def test_dynamic_torch_compile_reuses_one_engine():
     from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
     enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()

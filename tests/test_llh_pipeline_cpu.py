@@ -596,3 +596,29 @@ def test_residual_adds_fuse_under_symbolic_image_extents():
     steps = [s for s in make_plan(g) if s.kind not in ("view", "constant")]
     assert [s.kind for s in steps] == ["conv", "conv"]
     assert steps[1].attrs["epilogue"]["residual"] is not None and steps[1].attrs["epilogue"]["act"] == "relu"
+
+
+def test_symbols_seen_only_inside_input_extents_are_solved_for():
+    """A partition of a dynamically shaped graph whose inputs are all results of strided windows: the symbol of the
+    image size appears only inside their extents.  Any value that reproduces the given extents serves (the other
+    extents are functions of those), an inconsistent set of extents is refused."""
+    from llcompiler_amd.executor.engine import Torch_ExecutionEngine
+
+    class FakeInput:
+        def __init__(self, shape):
+            self.shape = shape
+    g = Graph()
+    s, b = Expr.sym("s7"), Expr.sym("s0")
+    half = (s - 1) // 2 + 1
+    quarter = (half - 1) // 2 + 1
+    x = g.add_input((b, 8, half, half), f32)
+    y = g.add_input((b, 8, quarter, quarter), f32)
+    g.set_outputs([g.add_op("relu", [x])])
+    eng = Torch_ExecutionEngine.__new__(Torch_ExecutionEngine)
+    eng.graph = g
+    env = eng.bind_symbols((), [FakeInput((4, 8, 32, 32)), FakeInput((4, 8, 16, 16))])
+    assert env["s0"] == 4 and evaluate(half, env) == 32 and evaluate(quarter, env) == 16
+    env = eng.bind_symbols((), [FakeInput((2, 8, 29, 29)), FakeInput((2, 8, 15, 15))])
+    assert evaluate(half, env) == 29 and evaluate(quarter, env) == 15
+    with pytest.raises(KeyError):
+        eng.bind_symbols((), [FakeInput((2, 8, 29, 29)), FakeInput((2, 8, 11, 11))])
