@@ -206,6 +206,18 @@ class Instance:
         for k, o in enumerate(g.outputs):
             if isinstance(o, Value):
                 out_ids.setdefault(id(o), []).append(k)
+        # A graph output that is a chain of views of a kernel's result (the [B S, N] product of a Linear layer seen as
+        # [B, S, N]): the kernel writes into an output buffer and the output is that view, with no copy at the end.
+        made_by = {id(st.output): st for st in steps}
+        out_roots = set()
+        for o in g.outputs:
+            st = made_by.get(id(o)) if isinstance(o, Value) else None
+            hops = 0
+            while st is not None and st.kind == "view" and hops < 16:
+                root, hops = st.inputs[0], hops + 1
+                st = made_by.get(id(root))
+                if st is not None and st.kind not in ("view", "constant") and not st.attrs.get("prepared"):
+                    out_roots.add(id(root))
         # liveness per backing buffer: a value and every view derived from it share one root; the
         # root's buffer returns to the pool after the last step that reads any of them
         root_of = {}
@@ -234,7 +246,7 @@ class Instance:
         def new_tensor(v, shape=None):
             nonlocal n_out_bufs
             shape = _concrete(v.shape if shape is None else shape, self.env)
-            if id(v) in out_ids:
+            if id(v) in out_ids or (id(v) in out_roots and self._preparing is None):
                 t = torch.empty(shape, dtype=v.dtype, device=dev)
                 self._register_root("out", n_out_bufs, t)
                 self.out_buffers.append(t)

@@ -514,6 +514,51 @@ def _softmax(ctx, node):
     return ctx.g.add_op("softmax", [x], {"axis": x.rank - 1})
 
 
+def _sdpa_args(node):
+    """(q, k, v, bias, dropout, causal, scale) of the two fused-attention ops aot autograd puts in place of
+    F.scaled_dot_product_attention on a GPU."""
+    a, kw = list(node.args), node.kwargs
+    if node.target is aten._scaled_dot_product_efficient_attention.default:
+        a += [None] * (7 - len(a))
+        return a[0], a[1], a[2], a[3], (a[5] if a[5] is not None else 0.0), bool(a[6]), kw.get("scale")
+    a += [None] * (6 - len(a))
+    return a[0], a[1], a[2], None, (a[3] if a[3] is not None else 0.0), bool(a[4]), kw.get("scale")
+
+
+def _sdpa_ok(node):
+    q, k, v, bias, dropout, causal, scale = _sdpa_args(node)
+    if bias is not None or dropout != 0.0 or causal or not _first_result_only(node):
+        return False  # masks, dropout and the statistics a backward graph reads stay with torch's kernel
+    shapes = [t.meta["val"].shape for t in (q, k, v)]
+    return all(len(sh) == 4 and isinstance(sh[3], int) for sh in shapes) and shapes[0][3] == shapes[1][3] == shapes[2][3] and \
+        tuple(shapes[0][:2]) == tuple(shapes[1][:2]) == tuple(shapes[2][:2])
+
+
+@TORCH_FUNCTION_TRANSLATE_REGISTER(aten._scaled_dot_product_flash_attention.default,
+                                   aten._scaled_dot_product_efficient_attention.default, check=_sdpa_ok)
+def _sdpa(ctx, node):
+    """F.scaled_dot_product_attention without mask or dropout, spelt as the group the reference's importer gets from an
+    attention layer written out by hand (llcompiler/test_models/models/multi_head_attention.py:20-33): batch_matmul of
+    q with the transposed keys, the scale, softmax over the keys, batch_matmul with v.  The planner folds the scale
+    into the first product and the engine runs the group as one fused kernel where the head dim allows."""
+    q, k, v, _, _, _, scale = _sdpa_args(node)
+    g = ctx.g
+    qv, kv, vv = ctx.val(q), ctx.val(k), ctx.val(v)
+    b, h, sq, d = qv.shape
+    skv = kv.shape[2]
+    if scale is None:
+        scale = float(d) ** -0.5
+    q3, v3 = (_reshape_to(ctx, t, (b * h, t.shape[2], d)) for t in (qv, vv))
+    # the keys are transposed as the rank-4 tensor they are, then flattened (what torch.matmul(q, k.transpose(-2, -1))
+    # decomposes to): a transpose of the flattened view would have to be made in memory first
+    kt3 = _reshape_to(ctx, g.add_op("transpose", [kv], {"perms": (0, 1, 3, 2)}), (b * h, d, skv))
+    scores = g.add_op("batch_matmul", [q3, kt3])
+    scores = g.add_op("mul", [scores, g.constant(float(scale), scores.dtype)])
+    probs = g.add_op("softmax", [scores], {"axis": 2})
+    out = _reshape_to(ctx, g.add_op("batch_matmul", [probs, v3]), (b, h, sq, d))
+    return (out,) + (None,) * (len(node.meta["val"]) - 1)
+
+
 def _first_result_only(node):
     """The translators of multi-result ATen ops produce the first result only (the output; not the saved
     statistics or pooling indices a backward graph asks for): a node whose other results are used stays in eager."""

@@ -408,6 +408,48 @@ def test_training_mode_resnet_units_with_batch_statistics(dynamic):
             assert_close(a.cpu().numpy(), b.numpy(), F32_RTOL, F32_ATOL, "buffer " + name)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_scaled_dot_product_attention_becomes_the_fused_kernel(dtype, dynamic):
+    """An attention layer written with F.scaled_dot_product_attention (what aot autograd hands over is torch's fused
+    flash / memory-efficient op): imported as the score product, scale, softmax and context product of the reference's
+    hand-written attention (multi_head_attention.py:20-33), which the engine runs as llc_hip_attention.  With a causal
+    mask the op stays in eager and the result is still right."""
+    from llcompiler_amd import LLCompiler
+
+    class Attn(torch.nn.Module):
+        def __init__(self, hidden, heads, causal=False):
+            super().__init__()
+            self.h, self.causal = heads, causal
+            self.qkv, self.o = torch.nn.Linear(hidden, 3 * hidden), torch.nn.Linear(hidden, hidden)
+
+        def forward(self, x):
+            B, S, E = x.shape
+            q, k, v = self.qkv(x).view(B, S, 3, self.h, E // self.h).permute(2, 0, 3, 1, 4)
+            y = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=self.causal)
+            return self.o(y.transpose(1, 2).reshape(B, S, E))
+
+    torch.manual_seed(0)
+    x = torch.randn(3, 96, 256).to(dtype)
+    rtol, atol = (F32_RTOL, F32_ATOL) if dtype == torch.float32 else (BF16_RTOL, BF16_ATOL)
+    for causal in (False, True):
+        torch._dynamo.reset()
+        m = Attn(256, 4, causal).eval().to(dtype)
+        comp = LLCompiler(mode="inference", target="gfx950", pipeline="hip")
+        opt = torch.compile(copy.deepcopy(m).cuda(), backend=comp, dynamic=dynamic, fullgraph=False)
+        with torch.no_grad():
+            want = copy.deepcopy(m).double()(x.double()).numpy()
+            got = opt(x.cuda()).float().cpu().numpy()
+        names = [c.fn.__name__ for e in comp.engines for inst in e.instances.values() for c in inst.calls]
+        assert names.count("llc_hip_attention") == (0 if causal else 1), names
+        assert names.count("llc_hip_matmul") == 2 and names.count("llc_hip_batch_matmul") == 0, names
+        if not causal:
+            # q, k and v are read in place from the packed projection, the head merge is done by the kernel's stores and
+            # the last product writes the output buffer (the [B, S, E] result is a view of its [B S, E] rows)
+            assert names == ["llc_hip_matmul", "llc_hip_attention", "llc_hip_matmul"], names
+        assert_close(got, want, rtol, atol, "scaled_dot_product_attention, causal=%s %s" % (causal, dtype))
+
+
 def test_dynamic_torch_compile_reuses_one_engine():
     from llcompiler_amd.test_models import EncoderBlock, make_encoder_inputs
     enc = EncoderBlock(hidden=64, heads=4, ffn=128).eval()
