@@ -24,7 +24,9 @@ from ..llh.passes import run_llh_pipeline
 from .torch_compile_config import LLC_DECOMPOSITIONS, LLCOperatorSupport
 
 TARGETS = ("gfx950",)
-PIPELINES = ("hip",)
+# "transform" is the reference's name for its one pipeline (include/llcompiler/Support/Enums.td:28-34; what its driver
+# passes, main.py:98): here it names the same thing, the LLH passes followed by this backend's kernel plan
+PIPELINES = ("hip", "transform")
 
 
 class LLCompiler:
@@ -38,8 +40,8 @@ class LLCompiler:
     def __init__(self, mode: str = "inference", target: str = "gfx950", pipeline: str = "hip", index_bit_width: int = 64,
                  symbol_infer=True, target_layout="NCHW", vebose_first_ir=False, log_root: str = "", log_level: str = "debug",
                  log_llvm: bool = True, cpu="", mtriple="", **kwargs) -> None:
-        # the reference accepts x86 / x86_64 and the "transform" pipeline only
-        # (include/llcompiler/Support/Enums.td:28-34, src/Compiler/Compiler.cpp:144-148)
+        # the reference generates code for x86 / x86_64 (include/llcompiler/Support/Enums.td:28-34,
+        # src/Compiler/Compiler.cpp:144-148); nothing here runs on the host, so those targets are an error
         if target not in TARGETS:
             raise ValueError("target %r: this backend generates code for %s only" % (target, ", ".join(TARGETS)))
         if pipeline not in PIPELINES:

@@ -228,8 +228,11 @@ def test_compiler_rejects_other_targets_and_pipelines():
     with pytest.raises(ValueError):
         LLCompiler(target="x86_64")
     with pytest.raises(ValueError):
-        LLCompiler(pipeline="transform")
+        LLCompiler(pipeline="basic")
     LLCompiler(mode="inference", target="gfx950", pipeline="hip", symbol_infer=True, target_layout="NCHW", log_level="debug")
+    # the keyword arguments of the reference's driver script (main.py:82-99), whose pipeline is called "transform"
+    LLCompiler(mode="inference", ir_tree_dir="ir_tree", log_root="", log_level="debug", symbol_infer=True, target_layout="NCHW",
+               pipeline="transform")
 
 
 def test_engine_argument_convention_and_errors():
