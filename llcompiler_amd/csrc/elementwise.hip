@@ -48,25 +48,32 @@ struct EwKernelParams {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// N bytes, naturally aligned, optionally with the non-temporal hint
+// N bytes, naturally aligned, optionally with the non-temporal hint.  The hint is a template argument: with a run-time
+// choice between the two forms of an access the compiler folds them into one plain instruction and the hint is lost.
 template <int N>
 struct Bytes {
   alignas(N >= 16 ? 16 : N) unsigned char b[N];
 };
-template <int N>
-__device__ __forceinline__ Bytes<N> ld_bytes(const char* p, bool nt) {
+template <int N, bool NT>
+__device__ __forceinline__ Bytes<N> ld_bytes(const char* p) {
   Bytes<N> r;
   if constexpr (N >= 16) {
 #pragma unroll
     for (int i = 0; i < N / 16; ++i) {
-      u32x4 v = nt ? __builtin_nontemporal_load((const u32x4*)p + i) : ((const u32x4*)p)[i];
+      u32x4 v;
+      if constexpr (NT) v = __builtin_nontemporal_load((const u32x4*)p + i);
+      else v = ((const u32x4*)p)[i];
       __builtin_memcpy(r.b + 16 * i, &v, 16);
     }
   } else if constexpr (N == 8) {
-    u32x2 v = nt ? __builtin_nontemporal_load((const u32x2*)p) : *(const u32x2*)p;
+    u32x2 v;
+    if constexpr (NT) v = __builtin_nontemporal_load((const u32x2*)p);
+    else v = *(const u32x2*)p;
     __builtin_memcpy(r.b, &v, 8);
   } else if constexpr (N == 4) {
-    uint32_t v = nt ? __builtin_nontemporal_load((const uint32_t*)p) : *(const uint32_t*)p;
+    uint32_t v;
+    if constexpr (NT) v = __builtin_nontemporal_load((const uint32_t*)p);
+    else v = *(const uint32_t*)p;
     __builtin_memcpy(r.b, &v, 4);
   } else if constexpr (N == 2) {
     uint16_t v = *(const uint16_t*)p;
@@ -76,25 +83,25 @@ __device__ __forceinline__ Bytes<N> ld_bytes(const char* p, bool nt) {
   }
   return r;
 }
-template <int N>
-__device__ __forceinline__ void st_bytes(char* p, const Bytes<N>& r, bool nt) {
+template <int N, bool NT>
+__device__ __forceinline__ void st_bytes(char* p, const Bytes<N>& r) {
   if constexpr (N >= 16) {
 #pragma unroll
     for (int i = 0; i < N / 16; ++i) {
       u32x4 v;
       __builtin_memcpy(&v, r.b + 16 * i, 16);
-      if (nt) __builtin_nontemporal_store(v, (u32x4*)p + i);
+      if constexpr (NT) __builtin_nontemporal_store(v, (u32x4*)p + i);
       else ((u32x4*)p)[i] = v;
     }
   } else if constexpr (N == 8) {
     u32x2 v;
     __builtin_memcpy(&v, r.b, 8);
-    if (nt) __builtin_nontemporal_store(v, (u32x2*)p);
+    if constexpr (NT) __builtin_nontemporal_store(v, (u32x2*)p);
     else *(u32x2*)p = v;
   } else if constexpr (N == 4) {
     uint32_t v;
     __builtin_memcpy(&v, r.b, 4);
-    if (nt) __builtin_nontemporal_store(v, (uint32_t*)p);
+    if constexpr (NT) __builtin_nontemporal_store(v, (uint32_t*)p);
     else *(uint32_t*)p = v;
   } else if constexpr (N == 2) {
     uint16_t v;
@@ -105,21 +112,21 @@ __device__ __forceinline__ void st_bytes(char* p, const Bytes<N>& r, bool nt) {
   }
 }
 
-template <typename S, int VEC>
-__device__ __forceinline__ void ld_elems(const char* base, uint32_t off, bool nt, S* dst) {
-  Bytes<(int)sizeof(S) * VEC> r = ld_bytes<(int)sizeof(S) * VEC>(base + (size_t)off * sizeof(S), nt);
+template <typename S, int VEC, bool NT>
+__device__ __forceinline__ void ld_elems(const char* base, uint32_t off, S* dst) {
+  Bytes<(int)sizeof(S) * VEC> r = ld_bytes<(int)sizeof(S) * VEC, NT>(base + (size_t)off * sizeof(S));
   __builtin_memcpy(dst, r.b, sizeof(S) * VEC);
 }
-template <typename S, int VEC>
-__device__ __forceinline__ void st_elems(char* base, uint32_t off, bool nt, const S* src) {
+template <typename S, int VEC, bool NT>
+__device__ __forceinline__ void st_elems(char* base, uint32_t off, const S* src) {
   Bytes<(int)sizeof(S) * VEC> r;
   __builtin_memcpy(r.b, src, sizeof(S) * VEC);
-  st_bytes<(int)sizeof(S) * VEC>(base + (size_t)off * sizeof(S), r, nt);
+  st_bytes<(int)sizeof(S) * VEC, NT>(base + (size_t)off * sizeof(S), r);
 }
 
 // ---- typed loads: VEC consecutive elements (inner stride 1) or one element repeated (stride 0) ----
-template <int VEC, typename CT>
-__device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t off, int inner_stride, bool nt, CT* dst) {
+template <int VEC, typename CT, bool NT>
+__device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t off, int inner_stride, CT* dst) {
   if (inner_stride == 0) {
     CT v;
     switch (dtype) {
@@ -137,87 +144,87 @@ __device__ __forceinline__ void load_vec(const char* base, int dtype, uint32_t o
   switch (dtype) {
     case LLC_FLOAT32: {
       float t[VEC];
-      ld_elems<float, VEC>(base, off, nt, t);
+      ld_elems<float, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     case LLC_BFLOAT16: {
       uint16_t t[VEC];
-      ld_elems<uint16_t, VEC>(base, off, nt, t);
+      ld_elems<uint16_t, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)bf16_bits_to_f32(t[j]);
     } break;
     case LLC_FLOAT16: {
       uint16_t t[VEC];
-      ld_elems<uint16_t, VEC>(base, off, nt, t);
+      ld_elems<uint16_t, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)f16_bits_to_f32(t[j]);
     } break;
     case LLC_INT64: {
       int64_t t[VEC];
-      ld_elems<int64_t, VEC>(base, off, nt, t);
+      ld_elems<int64_t, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     case LLC_INT32: {
       int32_t t[VEC];
-      ld_elems<int32_t, VEC>(base, off, nt, t);
+      ld_elems<int32_t, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
     default: {
       uint8_t t[VEC];
-      ld_elems<uint8_t, VEC>(base, off, nt, t);
+      ld_elems<uint8_t, VEC, NT>(base, off, t);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) dst[j] = (CT)t[j];
     } break;
   }
 }
 
-template <int VEC, typename CT>
-__device__ __forceinline__ void store_vec(char* base, int dtype, uint32_t off, bool nt, const CT* src) {
+template <int VEC, typename CT, bool NT>
+__device__ __forceinline__ void store_vec(char* base, int dtype, uint32_t off, const CT* src) {
   switch (dtype) {
     case LLC_FLOAT32: {
       float t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = (float)src[j];
-      st_elems<float, VEC>(base, off, nt, t);
+      st_elems<float, VEC, NT>(base, off, t);
     } break;
     case LLC_BFLOAT16: {
       uint16_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = f32_to_bf16_bits((float)src[j]);
-      st_elems<uint16_t, VEC>(base, off, nt, t);
+      st_elems<uint16_t, VEC, NT>(base, off, t);
     } break;
     case LLC_FLOAT16: {
       uint16_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = f32_to_f16_bits((float)src[j]);
-      st_elems<uint16_t, VEC>(base, off, nt, t);
+      st_elems<uint16_t, VEC, NT>(base, off, t);
     } break;
     case LLC_INT64: {
       int64_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = (int64_t)src[j];
-      st_elems<int64_t, VEC>(base, off, nt, t);
+      st_elems<int64_t, VEC, NT>(base, off, t);
     } break;
     case LLC_INT32: {
       int32_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = (int32_t)src[j];
-      st_elems<int32_t, VEC>(base, off, nt, t);
+      st_elems<int32_t, VEC, NT>(base, off, t);
     } break;
     case LLC_INT1: {
       uint8_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = src[j] != (CT)0 ? 1 : 0;
-      st_elems<uint8_t, VEC>(base, off, nt, t);
+      st_elems<uint8_t, VEC, NT>(base, off, t);
     } break;
     default: {
       uint8_t t[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) t[j] = (uint8_t)(int8_t)src[j];
-      st_elems<uint8_t, VEC>(base, off, nt, t);
+      st_elems<uint8_t, VEC, NT>(base, off, t);
     } break;
   }
 }
@@ -342,7 +349,7 @@ __device__ __forceinline__ void fetch(const RegFile<E, CT>& f, int sel, CT imm, 
   }
 }
 
-template <int VEC, int U, int MAXIN, typename CT>
+template <int VEC, int U, int MAXIN, typename CT, bool NT>
 __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
   constexpr int E = VEC * U;
   const EwHot h = p.hot;
@@ -350,7 +357,6 @@ __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
   const uint32_t v0 = blockIdx.x * (256u * U) + threadIdx.x;
   if (v0 >= h.n_vec) return;
   RegFile<E, CT> f;
-  const bool nt = h.streaming != 0;
   // ---- phase 1: issue every load ----
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -373,7 +379,7 @@ __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
     if (!h.flat)                                                                                        \
       off += idx0 * (uint32_t)p.in_stride[K][0] + idx1 * (uint32_t)p.in_stride[K][1] +                  \
              idx2 * (uint32_t)p.in_stride[K][2];                                                        \
-    load_vec<VEC, CT>(p.in[K], h.in_dtype[K], off, h.in_inner[K], nt, &ARR[u * VEC]);                   \
+    load_vec<VEC, CT, NT>(p.in[K], h.in_dtype[K], off, h.in_inner[K], &ARR[u * VEC]);                   \
   }
     LLC_LOAD_INPUT(0, f.i0)
     LLC_LOAD_INPUT(1, f.i1)
@@ -405,7 +411,7 @@ __global__ __launch_bounds__(256) void ew_kernel(const EwKernelParams p) {
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const uint32_t v = v0 + u * 256u;
-    if (v < h.n_vec) store_vec<VEC, CT>(p.out, h.out_dtype, v * VEC, nt, res + u * VEC);
+    if (v < h.n_vec) store_vec<VEC, CT, NT>(p.out, h.out_dtype, v * VEC, res + u * VEC);
   }
 }
 #undef LLC_COPY
@@ -487,13 +493,12 @@ __device__ __forceinline__ void chain_binary_imm(int op, float* acc, float imm) 
 #undef LLC_CH_BINARY_CASES
 
 // insts[i]: op (with the swapped forms above), b = operand kind, imm
-template <int VEC, int NIN>
+template <int VEC, int NIN, bool NT>
 __global__ __launch_bounds__(256) void ew_chain_kernel(const EwKernelParams p) {
   constexpr int E = VEC;
   const EwHot h = p.hot;
   const uint32_t v = blockIdx.x * 256u + threadIdx.x;
   if (v >= h.n_vec) return;
-  const bool nt = h.streaming != 0;
   const uint32_t e = v * VEC;
   uint32_t idx0 = 0, idx1 = 0, idx2 = 0, idx3 = e;
   if (!h.flat) {
@@ -512,7 +517,7 @@ __global__ __launch_bounds__(256) void ew_chain_kernel(const EwKernelParams p) {
     if (!h.flat)                                                                                        \
       off += idx0 * (uint32_t)p.in_stride[K][0] + idx1 * (uint32_t)p.in_stride[K][1] +                  \
              idx2 * (uint32_t)p.in_stride[K][2];                                                        \
-    load_vec<VEC, float>(p.in[K], h.in_dtype[K], off, h.in_inner[K], nt, ARR);                          \
+    load_vec<VEC, float, NT>(p.in[K], h.in_dtype[K], off, h.in_inner[K], ARR);                          \
   }
   LLC_LOAD_INPUT(0, acc)
   LLC_LOAD_INPUT(1, x1)
@@ -530,7 +535,7 @@ __global__ __launch_bounds__(256) void ew_chain_kernel(const EwKernelParams p) {
       default: if constexpr (NIN > 2) chain_binary<E>(op, acc, x3); break;
     }
   }
-  store_vec<VEC, float>(p.out, h.out_dtype, e, nt, acc);
+  store_vec<VEC, float, NT>(p.out, h.out_dtype, e, acc);
 }
 
 // Rewrites a program into accumulator form if it is a straight line.  On success fills chain[] (op, b = kind,
@@ -645,10 +650,13 @@ template <int VEC, int U, typename CT>
 void launch_vec(const EwKernelParams& p, hipStream_t stream) {
   const uint32_t per_block = 256u * U;
   const uint32_t blocks = (p.hot.n_vec + per_block - 1) / per_block;  // exact cover, no grid-stride loop
-  if (p.hot.n_inputs <= 2)
-    hipLaunchKernelGGL((ew_kernel<VEC, U, 2, CT>), dim3(blocks), dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((ew_kernel<VEC, U, LLC_EW_MAX_INPUTS, CT>), dim3(blocks), dim3(256), 0, stream, p);
+  if (p.hot.streaming) {
+    if (p.hot.n_inputs <= 2) hipLaunchKernelGGL((ew_kernel<VEC, U, 2, CT, true>), dim3(blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((ew_kernel<VEC, U, LLC_EW_MAX_INPUTS, CT, true>), dim3(blocks), dim3(256), 0, stream, p);
+  } else {
+    if (p.hot.n_inputs <= 2) hipLaunchKernelGGL((ew_kernel<VEC, U, 2, CT, false>), dim3(blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((ew_kernel<VEC, U, LLC_EW_MAX_INPUTS, CT, false>), dim3(blocks), dim3(256), 0, stream, p);
+  }
 }
 
 template <typename CT>
@@ -668,21 +676,27 @@ int launch(const EwKernelParams& p, int vec, hipStream_t stream) {
   return check_launch("ew_kernel");
 }
 
-template <int VEC>
+template <int VEC, bool NT>
 void launch_chain_vec(const EwKernelParams& p, hipStream_t stream) {
   const uint32_t blocks = (p.hot.n_vec + 255u) / 256u;  // exact cover: one vector per lane
-  if (p.hot.n_inputs <= 1) hipLaunchKernelGGL((ew_chain_kernel<VEC, 1>), dim3(blocks), dim3(256), 0, stream, p);
-  else if (p.hot.n_inputs == 2) hipLaunchKernelGGL((ew_chain_kernel<VEC, 2>), dim3(blocks), dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL((ew_chain_kernel<VEC, 4>), dim3(blocks), dim3(256), 0, stream, p);
+  if (p.hot.n_inputs <= 1) hipLaunchKernelGGL((ew_chain_kernel<VEC, 1, NT>), dim3(blocks), dim3(256), 0, stream, p);
+  else if (p.hot.n_inputs == 2) hipLaunchKernelGGL((ew_chain_kernel<VEC, 2, NT>), dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((ew_chain_kernel<VEC, 4, NT>), dim3(blocks), dim3(256), 0, stream, p);
+}
+
+template <bool NT>
+void launch_chain_nt(const EwKernelParams& p, int vec, hipStream_t stream) {
+  switch (vec) {
+    case 8: launch_chain_vec<8, NT>(p, stream); break;
+    case 4: launch_chain_vec<4, NT>(p, stream); break;
+    case 2: launch_chain_vec<2, NT>(p, stream); break;
+    default: launch_chain_vec<1, NT>(p, stream); break;
+  }
 }
 
 int launch_chain(const EwKernelParams& p, int vec, hipStream_t stream) {
-  switch (vec) {
-    case 8: launch_chain_vec<8>(p, stream); break;
-    case 4: launch_chain_vec<4>(p, stream); break;
-    case 2: launch_chain_vec<2>(p, stream); break;
-    default: launch_chain_vec<1>(p, stream); break;
-  }
+  if (p.hot.streaming) launch_chain_nt<true>(p, vec, stream);
+  else launch_chain_nt<false>(p, vec, stream);
   return check_launch("ew_chain_kernel");
 }
 
