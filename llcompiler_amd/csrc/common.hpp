@@ -142,6 +142,41 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   }
 }
 
+typedef uint32_t raw16_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes of storage type DT as fp32 values, and back (DT known when compiling: no branch between the loads and their use)
+template <int DT>
+__device__ __forceinline__ void unpack_typed(const raw16_t& raw, float* dst) {
+  if constexpr (DT == LLC_FLOAT32) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dst[j] = __uint_as_float(raw[j]);
+  } else if constexpr (DT == LLC_BFLOAT16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      dst[2 * j] = __uint_as_float(raw[j] << 16);
+      dst[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      dst[2 * j] = f16_bits_to_f32((uint16_t)(raw[j] & 0xffffu));
+      dst[2 * j + 1] = f16_bits_to_f32((uint16_t)(raw[j] >> 16));
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ raw16_t pack_typed(const float* src) {
+  raw16_t r;
+  if constexpr (DT == LLC_FLOAT32) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = __float_as_uint(src[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = pack_pair<DT>(src[2 * j], src[2 * j + 1]);
+  }
+  return r;
+}
+
 // erf-based GELU, 0.5 x (1 + erf(x / sqrt 2)).  erf comes from the rational approximation 7.1.26 of
 // Abramowitz & Stegun (absolute error below 1.5e-7) on the hardware reciprocal and exp2: the result stays
 // within 5e-7 of the exactly rounded one over the whole range, a fortieth of the fp32 tolerance, at a third

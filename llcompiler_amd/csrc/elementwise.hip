@@ -538,6 +538,44 @@ __global__ __launch_bounds__(256) void ew_chain_kernel(const EwKernelParams p) {
   store_vec<VEC, float, NT>(p.out, h.out_dtype, e, acc);
 }
 
+// The chain kernel for the plain case: every operand and the result are contiguous tensors of one floating storage type DT
+// and move 16 bytes per lane.  ew_chain_kernel picks the storage type of each operand in a switch, and a value a switch
+// defines must have arrived where the switch ends: its operands travel one after the other.  Here the NIN loads leave
+// back to back (operands beyond the program's own repeat operand 0 and are ignored), then the chain runs.
+template <int DT, int NIN, bool NT>
+__global__ __launch_bounds__(256) void ew_chain_typed_kernel(const EwKernelParams p) {
+  // one vector per lane: two and four per lane were slower at every size (64 Mi fp32 elements 124 | 130 | 127 us)
+  constexpr int E = DT == LLC_FLOAT32 ? 4 : 8;
+  const EwHot h = p.hot;
+  const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+  if (v >= h.n_vec) return;
+  u32x4 raw[NIN];
+#pragma unroll
+  for (int k = 0; k < NIN; ++k) {
+    const u32x4* src = (const u32x4*)p.in[k < h.n_inputs ? k : 0] + v;
+    if constexpr (NT) raw[k] = __builtin_nontemporal_load(src);
+    else raw[k] = *src;
+  }
+  float acc[E], x[NIN > 1 ? NIN - 1 : 1][E];
+  unpack_typed<DT>(raw[0], acc);
+#pragma unroll
+  for (int k = 1; k < NIN; ++k) unpack_typed<DT>(raw[k], x[k - 1]);
+  for (int i = 0; i < h.n_insts; ++i) {
+    const int op = p.insts[i].op, kind = p.insts[i].b;
+    switch (kind) {
+      case kKindNone: chain_unary<E>(op, acc); break;
+      case kKindImm: chain_binary_imm<E>(op, acc, p.insts[i].imm); break;
+      case kKindAcc: chain_binary<E>(op, acc, acc); break;
+      case kKindIn1: if constexpr (NIN > 1) chain_binary<E>(op, acc, x[0]); break;
+      case kKindIn1 + 1: if constexpr (NIN > 2) chain_binary<E>(op, acc, x[1]); break;
+      default: if constexpr (NIN > 3) chain_binary<E>(op, acc, x[2]); break;
+    }
+  }
+  u32x4* dst = (u32x4*)p.out + v;
+  if constexpr (NT) __builtin_nontemporal_store(pack_typed<DT>(acc), dst);
+  else *dst = pack_typed<DT>(acc);
+}
+
 // Rewrites a program into accumulator form if it is a straight line.  On success fills chain[] (op, b = kind,
 // imm), slot[] (original input index held by each slot) and the counts.
 bool linearize(const llc_ew_program* prog, size_t n_inputs, llc_ew_inst* chain, int* n_chain, int* slot, int* n_slots) {
@@ -694,7 +732,38 @@ void launch_chain_nt(const EwKernelParams& p, int vec, hipStream_t stream) {
   }
 }
 
+template <int DT, bool NT>
+void launch_chain_typed(const EwKernelParams& p, hipStream_t stream) {
+  const uint32_t blocks = (p.hot.n_vec + 255u) / 256u;
+  switch (p.hot.n_inputs) {
+    case 0:
+    case 1: hipLaunchKernelGGL((ew_chain_typed_kernel<DT, 1, NT>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((ew_chain_typed_kernel<DT, 2, NT>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((ew_chain_typed_kernel<DT, 3, NT>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((ew_chain_typed_kernel<DT, 4, NT>), dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+}
+
+// Whether the typed chain kernel takes this launch: same-shape contiguous operands of the result's floating type, 16 bytes a lane
+bool chain_typed_ok(const EwKernelParams& p, int vec) {
+  const int dt = p.hot.out_dtype;
+  if (dt != LLC_FLOAT32 && dt != LLC_BFLOAT16 && dt != LLC_FLOAT16) return false;
+  if (!p.hot.flat || p.hot.n_inputs < 1 || p.hot.n_inputs > 4 || vec != (dt == LLC_FLOAT32 ? 4 : 8)) return false;
+  for (int k = 0; k < p.hot.n_inputs; ++k)
+    if (p.hot.in_dtype[k] != dt || p.hot.in_inner[k] != 1) return false;
+  return true;
+}
+
 int launch_chain(const EwKernelParams& p, int vec, hipStream_t stream) {
+  if (chain_typed_ok(p, vec)) {
+    const bool nt = p.hot.streaming != 0;
+    switch (p.hot.out_dtype) {
+      case LLC_FLOAT32: nt ? launch_chain_typed<LLC_FLOAT32, true>(p, stream) : launch_chain_typed<LLC_FLOAT32, false>(p, stream); break;
+      case LLC_BFLOAT16: nt ? launch_chain_typed<LLC_BFLOAT16, true>(p, stream) : launch_chain_typed<LLC_BFLOAT16, false>(p, stream); break;
+      default: nt ? launch_chain_typed<LLC_FLOAT16, true>(p, stream) : launch_chain_typed<LLC_FLOAT16, false>(p, stream); break;
+    }
+    return check_launch("ew_chain_typed_kernel");
+  }
   if (p.hot.streaming) launch_chain_nt<true>(p, vec, stream);
   else launch_chain_nt<false>(p, vec, stream);
   return check_launch("ew_chain_kernel");

@@ -346,39 +346,6 @@ __global__ __launch_bounds__(256) void row_kernel(const RowParams p) {
   }
 }
 
-// 16 bytes of storage type DT as fp32 values, and back (DT known when compiling: no branch between the loads and their use)
-template <int DT>
-__device__ __forceinline__ void unpack_typed(const u32x4& raw, float* dst) {
-  if constexpr (DT == LLC_FLOAT32) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) dst[j] = __uint_as_float(raw[j]);
-  } else if constexpr (DT == LLC_BFLOAT16) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      dst[2 * j] = __uint_as_float(raw[j] << 16);
-      dst[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      dst[2 * j] = f16_bits_to_f32((uint16_t)(raw[j] & 0xffffu));
-      dst[2 * j + 1] = f16_bits_to_f32((uint16_t)(raw[j] >> 16));
-    }
-  }
-}
-template <int DT>
-__device__ __forceinline__ u32x4 pack_typed(const float* src) {
-  u32x4 r;
-  if constexpr (DT == LLC_FLOAT32) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = __float_as_uint(src[j]);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = pack_pair<DT>(src[2 * j], src[2 * j + 1]);
-  }
-  return r;
-}
-
 template <int DT, bool NT>
 __device__ __forceinline__ void store_typed(char* dst, const float* src) {
   if constexpr (NT) __builtin_nontemporal_store(pack_typed<DT>(src), (u32x4*)dst);
