@@ -700,28 +700,8 @@ __global__ __launch_bounds__(256) void nhwc_split_reduce_kernel(const ConvParams
   const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   const int64_t total = (int64_t)p.ncols * p.F;
   if (i4 >= total) return;  // F % 4 == 0: a vector never straddles the end
-  const float* part = (const float*)p.partial + i4;
-  f32x4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int k = 0; k < p.splits; ++k) s += *(const f32x4_t*)(part + (int64_t)k * total);
   const int f = (int)(i4 % p.F);
-  if constexpr (sizeof(T) == 4) {
-    f32x4_t b = {0.0f, 0.0f, 0.0f, 0.0f}, r = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (p.bias) b = *(const f32x4_t*)((const float*)p.bias + f);
-    if (p.residual) r = *(const f32x4_t*)((const float*)p.residual + i4);
-    f32x4_t o;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = s[e] * p.alpha + b[e] + r[e];
-      if (p.act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;
-      else if (p.act == LLC_ACT_GELU) v = gelu_exact(v);
-      o[e] = v;
-    }
-    *(f32x4_t*)((float*)p.Y + i4) = o;
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      epilogue_store<T>((T*)p.Y, i4 + e, s[e], p.alpha, p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, f + e) : 0.0f, p.residual, p.act);
-  }
+  gemm::split_epilogue4<T>((const float*)p.partial, p.splits, total, i4, f, p.alpha, p.bias, p.residual, p.act, (T*)p.Y);
 }
 
 template <typename T, int BM, int BN, int WM, int WN>

@@ -772,16 +772,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
                                                             const char* __restrict__ residual, int act, T* __restrict__ out) {
   const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i4 >= mn) return;
-  f32x4_t acc = *(const f32x4_t*)(part + i4);
-  for (int z = 1; z < splits; ++z) {
-    const f32x4_t v = *(const f32x4_t*)(part + (int64_t)z * mn + i4);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] += v[j];
-  }
   const int col = (int)(i4 % n);  // n is a multiple of 4: the four values share a row
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    epilogue_store<T>(out, i4 + j, acc[j], alpha, bias ? load_as_f32(bias, Elem<T>::kDtype, col + j) : 0.0f, residual, act);
+  split_epilogue4<T>(part, splits, mn, i4, col, alpha, bias, residual, act, out);
 }
 
 // Number of reduction chunks, 1 = no split; bk = elements of a k-tile (32 for fp32, 64 for the 16-bit types).  A

@@ -317,5 +317,49 @@ __device__ __forceinline__ void epilogue_store(T* C, int64_t o, float acc, float
   else ((uint16_t*)C)[o] = f32_to_f16_bits(v);
 }
 
+// The pass over the partial sums of a split reduction, four consecutive outputs of one row per lane:
+// out[i4 .. i4 + 3] = act(alpha * (part[0] + part[1] + ...) + bias[col ..] + residual[i4 ..]), the partial sums `stride`
+// floats apart and added in split order (the same order on every run).  Written as a loop of load-and-add, each load waits
+// for the one before it, nine to eighteen trips to memory in a row on every lane, and bias and residual follow after the
+// last; here bias and residual are requested first (unconditionally: an absent operand reads the first partial sum's
+// memory and is ignored) and the partial sums eight at a time.
+template <typename T>
+__device__ __forceinline__ void split_epilogue4(const float* part, int splits, int64_t stride, int64_t i4, int col, float alpha,
+                                                const char* bias, const char* residual, int act, T* out) {
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  constexpr int dt = Elem<T>::kDtype;
+  const char* bsrc = bias ? bias + (int64_t)col * sizeof(T) : (const char*)part;
+  const char* rsrc = residual ? residual + i4 * (int64_t)sizeof(T) : (const char*)part;
+  float b[4], r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b[j] = load_as_f32(bsrc, dt, j);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = load_as_f32(rsrc, dt, j);
+  const float* src = part + i4;
+  v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k0 = 0; k0 < splits; k0 += 8) {
+    v4f v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = *(const v4f*)(src + (int64_t)(k0 + j < splits ? k0 + j : splits - 1) * stride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (k0 + j < splits) acc = k0 + j == 0 ? v[j] : acc + v[j];
+  }
+  float o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float v = acc[j] * alpha + (bias ? b[j] : 0.0f);
+    if (residual) v += r[j];
+    if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
+    else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
+    o[j] = v;
+  }
+  if constexpr (dt == LLC_FLOAT32) {
+    *(v4f*)((float*)out + i4) = v4f{o[0], o[1], o[2], o[3]};
+  } else {
+    *(uint2*)((uint16_t*)out + i4) = uint2{pack_pair<dt>(o[0], o[1]), pack_pair<dt>(o[2], o[3])};
+  }
+}
+
 }  // namespace gemm
 }  // namespace llc
