@@ -172,14 +172,25 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
     const int n = col / ohw, pix = col - n * ohw;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      int64_t o[16];
+      bool ok[16];
+      float b16[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        if (row >= p.Fg) continue;
-        const int f = g * p.Fg + row;
-        const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, f) : 0.0f;
-        epilogue_store<T>(Y, ((int64_t)n * p.F + f) * ohw + pix, acc[i][j][r], p.alpha, bv, p.residual, p.act);
+        ok[r] = row < p.Fg;
+        const int f = g * p.Fg + (ok[r] ? row : p.Fg - 1);
+        o[r] = ((int64_t)n * p.F + f) * ohw + pix;
+        b16[r] = 0.0f;
       }
+      if (p.bias) {  // one test around the sixteen loads: they travel together
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
+          b16[r] = load_as_f32(p.bias, Elem<T>::kDtype, g * p.Fg + (ok[r] ? row : p.Fg - 1));
+        }
+      }
+      epilogue_block16<T>(Y, p.residual, o, ok, acc[i][j], p.alpha, b16, p.act);
     }
   }
 }
@@ -682,15 +693,25 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_kernel(const ConvParam
     if (!BFULL && col >= p.F) continue;
     const float bv = (p.bias && p.splits == 1) ? load_as_f32(p.bias, Elem<T>::kDtype, col) : 0.0f;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+      int64_t o[16];
+      bool ok[16];
+      float b16[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        if (row >= p.ncols) continue;
-        const int64_t o = (int64_t)row * p.F + col;
-        if (p.splits > 1) part[o] = acc[i][j][r];
-        else epilogue_store<T>((T*)p.Y, o, acc[i][j][r], p.alpha, bv, res, p.act);
+        ok[r] = row < p.ncols;
+        o[r] = (int64_t)(ok[r] ? row : p.ncols - 1) * p.F + col;
+        b16[r] = bv;
       }
+      if (p.splits > 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (ok[r]) part[o[r]] = acc[i][j][r];
+      } else {
+        epilogue_block16<T>((T*)p.Y, res, o, ok, acc[i][j], p.alpha, b16, p.act);
+      }
+    }
   }
 }
 

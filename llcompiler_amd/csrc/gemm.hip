@@ -150,12 +150,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, (int64_t)z0 * p.bias_sb + col) : 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      int64_t o[16];
+      bool ok[16];
+      float b16[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        if (!FULL && row >= p.M) continue;
-        if (sizeof(T) != 4 && p.c_f32) ((float*)p.C)[c_off + (int64_t)row * p.c_sm + col] = acc[i][j][r];
-        else epilogue_store<T>(C, (int64_t)row * p.c_sm + col, acc[i][j][r], p.alpha, bv, res, p.act);
+        ok[r] = FULL || row < p.M;
+        o[r] = (int64_t)(ok[r] ? row : p.M - 1) * p.c_sm + col;
+        b16[r] = bv;
+      }
+      if (sizeof(T) != 4 && p.c_f32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (ok[r]) ((float*)p.C)[c_off + o[r]] = acc[i][j][r];
+      } else {
+        epilogue_block16<T>(C, res, o, ok, acc[i][j], p.alpha, b16, p.act);
       }
     }
   }

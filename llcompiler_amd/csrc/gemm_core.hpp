@@ -317,6 +317,35 @@ __device__ __forceinline__ void epilogue_store(T* C, int64_t o, float acc, float
   else ((uint16_t*)C)[o] = f32_to_f16_bits(v);
 }
 
+// A lane's sixteen values of one 32x32 accumulator block through the epilogue: C[o[r]] = act(alpha * acc[r] + bias[r] +
+// residual[o[r]]) where ok[r]; o[r] is a valid offset also where ok[r] is false (clamped by the caller), so the residual loads
+// are unconditional.  All sixteen residual values are requested before the first result is stored: written element by
+// element (load, add, store), every load waits for the store before it, which may alias it, and every store for its load:
+// thirty-two trips to memory in a row on each lane.  A residual that is the output tensor itself (an in-place add) stays
+// correct: a lane reads exactly the elements it writes.
+template <typename T>
+__device__ __forceinline__ void epilogue_block16(T* C, const char* res, const int64_t (&o)[16], const bool (&ok)[16],
+                                                 const f32x16_t& acc, float alpha, const float (&bias)[16], int act) {
+  constexpr int dt = Elem<T>::kDtype;
+  float rv[16];
+  if (res) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) rv[r] = load_as_f32(res, dt, o[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v = acc[r] * alpha + bias[r];
+    if (res) v += rv[r];
+    if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
+    else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
+    if (ok[r]) {
+      if constexpr (dt == LLC_FLOAT32) C[o[r]] = v;
+      else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o[r]] = f32_to_bf16_bits(v);
+      else ((uint16_t*)C)[o[r]] = f32_to_f16_bits(v);
+    }
+  }
+}
+
 // The pass over the partial sums of a split reduction, four consecutive outputs of one row per lane:
 // out[i4 .. i4 + 3] = act(alpha * (part[0] + part[1] + ...) + bias[col ..] + residual[i4 ..]), the partial sums `stride`
 // floats apart and added in split order (the same order on every run).  Written as a loop of load-and-add, each load waits
