@@ -186,8 +186,26 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const ConvParams p, int
   constexpr int EPV = 16 / ES;           // outputs per 16-byte store
   constexpr int CPR = 64 / EPV;          // stores per pixel
   const int64_t img_off = (int64_t)n * ohw;
+  // bias and residual of every pass are requested before the first pass stores: inside the loop each pass's loads waited
+  // behind the stores of the pass before, which may alias them (a lane's filters are the same in every pass; rows past
+  // the image read its last pixel and are not stored)
+  constexpr int NIT = 128 * CPR / 256;
+  u32x4_t bq_all = {0, 0, 0, 0}, rq_all[NIT];
 #pragma unroll
-  for (int it = 0; it < 128 * CPR / 256; ++it) {
+  for (int it = 0; it < NIT; ++it) rq_all[it] = u32x4_t{0, 0, 0, 0};
+  {
+    const int lc0 = (threadIdx.x % CPR) * EPV;
+    if (p.bias) bq_all = *(const u32x4_t*)((const char*)p.bias + (int64_t)(f0 + lc0) * ES);
+    if (p.residual) {
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int prow = p0 + it * (256 / CPR) + threadIdx.x / CPR;
+        rq_all[it] = *(const u32x4_t*)((const char*)p.residual + ((img_off + (prow < ohw ? prow : ohw - 1)) * p.F + f0 + lc0) * ES);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
     const int vid = it * 256 + threadIdx.x;
     const int row = vid / CPR, c0 = (vid % CPR) * EPV;
     if (p0 + row >= ohw) continue;
@@ -195,9 +213,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const ConvParams p, int
     const int64_t o = (img_off + p0 + row) * p.F + f0 + c0;
     if constexpr (ES == 4) {
       const f32x4_t x = *(const f32x4_t*)s0;
-      f32x4_t b = {0.0f, 0.0f, 0.0f, 0.0f}, rr = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (p.bias) b = *(const f32x4_t*)((const float*)p.bias + f0 + c0);
-      if (p.residual) rr = *(const f32x4_t*)((const float*)p.residual + o);
+      const f32x4_t b = __builtin_bit_cast(f32x4_t, bq_all), rr = __builtin_bit_cast(f32x4_t, rq_all[it]);
       f32x4_t outv;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -210,9 +226,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(const ConvParams p, int
     } else {
       const f32x4_t x0 = *(const f32x4_t*)s0, x1 = *(const f32x4_t*)(s0 + 4);
       const float v[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-      u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-      if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + f0 + c0);
-      if (p.residual) rq = *(const u32x4_t*)((const T*)p.residual + o);
+      const u32x4_t bq = bq_all, rq = rq_all[it];
       float xs[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {

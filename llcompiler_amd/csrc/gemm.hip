@@ -403,6 +403,15 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
+  // bias and residual of all four passes are requested before the first pass stores: inside the loop each pass's loads
+  // waited behind the stores of the pass before, which may alias them (a lane's eight columns are the same in every pass)
+  u32x4_t bq_all = {0, 0, 0, 0}, rq_all[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+  if (p.bias) bq_all = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + (threadIdx.x % 16) * 8);
+  if (res) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      rq_all[it] = *(const u32x4_t*)(res + (int64_t)(m0 + it * 32 + threadIdx.x / 16) * p.c_sm + n0 + (threadIdx.x % 16) * 8);
+  }
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int vid = it * 512 + threadIdx.x;
@@ -419,9 +428,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const GemmParams p) {
       v[4 * h + 3] = x.w + y.w;
     }
     const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
-    u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
-    if (res) rq = *(const u32x4_t*)(res + o);
+    const u32x4_t bq = bq_all, rq = rq_all[it];
     float xs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -591,6 +598,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
+  // bias and residual of all four passes are requested before the first pass stores: inside the loop each pass's loads
+  // waited behind the stores of the pass before, which may alias them (a lane's eight columns are the same in every pass)
+  u32x4_t bq_all = {0, 0, 0, 0}, rq_all[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+  if (p.bias) bq_all = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + (threadIdx.x % 16) * 8);
+  if (res) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      rq_all[it] = *(const u32x4_t*)(res + (int64_t)(m0 + it * 32 + threadIdx.x / 16) * p.c_sm + n0 + (threadIdx.x % 16) * 8);
+  }
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int vid = it * 512 + threadIdx.x;
@@ -606,9 +622,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       v[4 * h + 3] = x[3];
     }
     const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
-    u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
-    if (res) rq = *(const u32x4_t*)(res + o);
+    const u32x4_t bq = bq_all, rq = rq_all[it];
     float xs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {

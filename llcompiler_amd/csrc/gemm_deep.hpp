@@ -127,6 +127,15 @@ __global__ __launch_bounds__(256) void gemm_deep_kernel(const GemmParams p) {
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const T* res = p.residual ? (const T*)p.residual + c_off : nullptr;
+  // bias and residual of both passes are requested before the first pass stores (inside the loop the second pass's loads
+  // waited behind the first pass's stores, which may alias them); a lane's eight columns are the same in both passes
+  u32x4_t bq_all = {0, 0, 0, 0}, rq_all[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  if (p.bias) bq_all = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + (threadIdx.x % 8) * 8);
+  if (res) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+      rq_all[it] = *(const u32x4_t*)(res + (int64_t)(m0 + it * 32 + threadIdx.x / 8) * p.c_sm + n0 + (threadIdx.x % 8) * 8);
+  }
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int vid = it * 256 + threadIdx.x;
@@ -135,9 +144,7 @@ __global__ __launch_bounds__(256) void gemm_deep_kernel(const GemmParams p) {
     const float4 x0 = *(const float4*)s0, x1 = *(const float4*)(s0 + 4);
     const float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
     const int64_t o = (int64_t)(m0 + row) * p.c_sm + n0 + c0;
-    u32x4_t bq = {0, 0, 0, 0}, rq = {0, 0, 0, 0};
-    if (p.bias) bq = *(const u32x4_t*)((const T*)p.bias + (int64_t)z0 * p.bias_sb + n0 + c0);
-    if (res) rq = *(const u32x4_t*)(res + o);
+    const u32x4_t bq = bq_all, rq = rq_all[it];
     float xs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
