@@ -687,11 +687,19 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_kernel(const ConvParam
   //      filters of one pixel ----
   float* part = (float*)p.partial + (int64_t)split * p.ncols * p.F;
   const char* res = p.splits > 1 ? nullptr : p.residual;
+  // the bias of every column block is requested before the first block stores (behind a store, which may alias it, the
+  // next block's bias would wait for that store)
+  float bvs[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * WTN + j * 32 + li;
+    bvs[j] = (p.bias && p.splits == 1) ? load_as_f32(p.bias, Elem<T>::kDtype, BFULL || col < p.F ? col : p.F - 1) : 0.0f;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
     if (!BFULL && col >= p.F) continue;
-    const float bv = (p.bias && p.splits == 1) ? load_as_f32(p.bias, Elem<T>::kDtype, col) : 0.0f;
+    const float bv = bvs[j];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       int64_t o[16];

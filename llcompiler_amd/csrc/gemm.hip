@@ -143,11 +143,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
   const int64_t c_off = (int64_t)z0 * p.c_sb + (int64_t)z1 * p.c_sb1;
   T* C = (T*)p.C + c_off;
   const char* res = p.residual ? p.residual + c_off * (int64_t)sizeof(T) : nullptr;
+  // the bias of every column block is requested before the first block stores (behind a store, which may alias it, the
+  // next block's bias would wait for that store)
+  float bvs[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * WTN + j * 32 + li;
+    bvs[j] = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, (int64_t)z0 * p.bias_sb + (FULL || col < p.N ? col : p.N - 1)) : 0.0f;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn * WTN + j * 32 + li;
     if (!FULL && col >= p.N) continue;
-    const float bv = p.bias ? load_as_f32(p.bias, Elem<T>::kDtype, (int64_t)z0 * p.bias_sb + col) : 0.0f;
+    const float bv = bvs[j];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       int64_t o[16];
