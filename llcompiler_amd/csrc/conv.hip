@@ -172,25 +172,21 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvParams p) {
     const int n = col / ohw, pix = col - n * ohw;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      int64_t o[16];
-      bool ok[16];
+      const int row0 = m0 + wm * WTM + i * 32 + lh * 4;  // the lane's first filter (inside the group) of this block
+      const int rows_left = p.Fg - row0;
+      const int f0 = g * p.Fg + (rows_left > 0 ? row0 : p.Fg - 1);
       float b16[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        ok[r] = row < p.Fg;
-        const int f = g * p.Fg + (ok[r] ? row : p.Fg - 1);
-        o[r] = ((int64_t)n * p.F + f) * ohw + pix;
-        b16[r] = 0.0f;
-      }
+      for (int r = 0; r < 16; ++r) b16[r] = 0.0f;
       if (p.bias) {  // one test around the sixteen loads: they travel together
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-          b16[r] = load_as_f32(p.bias, Elem<T>::kDtype, g * p.Fg + (ok[r] ? row : p.Fg - 1));
+          const int ro = (r / 4) * 8 + (r % 4);
+          b16[r] = load_as_f32(p.bias, Elem<T>::kDtype, f0 + (ro < rows_left ? ro : 0));
         }
       }
-      epilogue_block16<T>(Y, p.residual, o, ok, acc[i][j], p.alpha, b16, p.act);
+      epilogue_block16<T, true>(Y, p.residual, ((int64_t)n * p.F + f0) * ohw + pix, ohw, rows_left, acc[i][j], p.alpha,
+                                [&](int r) { return b16[r]; }, p.act);
     }
   }
 }
@@ -702,22 +698,17 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_nhwc_kernel(const ConvParam
     const float bv = bvs[j];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      int64_t o[16];
-      bool ok[16];
-      float b16[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        ok[r] = row < p.ncols;
-        o[r] = (int64_t)(ok[r] ? row : p.ncols - 1) * p.F + col;
-        b16[r] = bv;
-      }
+      const int row0 = m0 + wm * WTM + i * 32 + lh * 4;  // the lane's first pixel of this block
+      const int rows_left = p.ncols - row0;
+      const int64_t base = (int64_t)(rows_left > 0 ? row0 : p.ncols - 1) * p.F + col;
       if (p.splits > 1) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (ok[r]) part[o[r]] = acc[i][j][r];
+        for (int r = 0; r < 16; ++r) {
+          const int ro = (r / 4) * 8 + (r % 4);
+          if (ro < rows_left) part[base + (int64_t)ro * p.F] = acc[i][j][r];
+        }
       } else {
-        epilogue_block16<T>((T*)p.Y, res, o, ok, acc[i][j], p.alpha, b16, p.act);
+        epilogue_block16<T, true>((T*)p.Y, res, base, p.F, rows_left, acc[i][j], p.alpha, [&](int) { return bv; }, p.act);
       }
     }
   }

@@ -158,22 +158,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const GemmParams p) 
     const float bv = bvs[j];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      int64_t o[16];
-      bool ok[16];
-      float b16[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * WTM + i * 32 + (r / 4) * 8 + lh * 4 + (r % 4);
-        ok[r] = FULL || row < p.M;
-        o[r] = (int64_t)(ok[r] ? row : p.M - 1) * p.c_sm + col;
-        b16[r] = bv;
-      }
+      const int row0 = m0 + wm * WTM + i * 32 + lh * 4;  // the lane's first row of this block
+      const int rows_left = p.M - row0;
+      const int64_t base = (int64_t)(FULL || rows_left > 0 ? row0 : p.M - 1) * p.c_sm + col;
       if (sizeof(T) != 4 && p.c_f32) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (ok[r]) ((float*)p.C)[c_off + o[r]] = acc[i][j][r];
+        for (int r = 0; r < 16; ++r) {
+          const int ro = (r / 4) * 8 + (r % 4);
+          if (FULL || ro < rows_left) ((float*)p.C)[c_off + base + (int64_t)ro * p.c_sm] = acc[i][j][r];
+        }
       } else {
-        epilogue_block16<T>(C, res, o, ok, acc[i][j], p.alpha, b16, p.act);
+        epilogue_block16<T, !FULL>(C, res, base, p.c_sm, rows_left, acc[i][j], p.alpha, [&](int) { return bv; }, p.act);
       }
     }
   }

@@ -317,31 +317,40 @@ __device__ __forceinline__ void epilogue_store(T* C, int64_t o, float acc, float
   else ((uint16_t*)C)[o] = f32_to_f16_bits(v);
 }
 
-// A lane's sixteen values of one 32x32 accumulator block through the epilogue: C[o[r]] = act(alpha * acc[r] + bias[r] +
-// residual[o[r]]) where ok[r]; o[r] is a valid offset also where ok[r] is false (clamped by the caller), so the residual loads
-// are unconditional.  All sixteen residual values are requested before the first result is stored: written element by
-// element (load, add, store), every load waits for the store before it, which may alias it, and every store for its load:
-// thirty-two trips to memory in a row on each lane.  A residual that is the output tensor itself (an in-place add) stays
-// correct: a lane reads exactly the elements it writes.
-template <typename T>
-__device__ __forceinline__ void epilogue_block16(T* C, const char* res, const int64_t (&o)[16], const bool (&ok)[16],
-                                                 const f32x16_t& acc, float alpha, const float (&bias)[16], int act) {
+// A lane's sixteen values of one 32x32 accumulator block through the epilogue.  Value r belongs to row 8 (r / 4) + r % 4 of
+// the lane's sixteen (its first row and its column are in `base`, an element offset into C and the residual; rows are `ld`
+// elements apart): C[..] = act(alpha * acc[r] + bias_of(r) + residual[..]).  GUARD: only the first `rows_left` of those
+// row numbers exist (base then points at an existing row; rows_left may be <= 0); what does not exist is computed from
+// the lane's first row and not stored.  All sixteen residual values are requested before the first result is stored:
+// written element by element (load, add, store), every load waits for the store before it, which may alias it, and
+// every store for its load: thirty-two trips to memory in a row on each lane.  A residual that is the output tensor
+// itself (an in-place add) stays correct: a lane reads exactly the elements it writes.  The row offsets are multiples
+// of `ld` known when compiling, so they live in scalar registers: sixteen 64-bit offsets per lane had cost the
+// 128 x 128 four-wave configuration half its waves (272 registers against 240).
+template <typename T, bool GUARD, typename BiasFn>
+__device__ __forceinline__ void epilogue_block16(T* C, const char* res, int64_t base, int64_t ld, int rows_left,
+                                                 const f32x16_t& acc, float alpha, BiasFn bias_of, int act) {
   constexpr int dt = Elem<T>::kDtype;
   float rv[16];
   if (res) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) rv[r] = load_as_f32(res, dt, o[r]);
+    for (int r = 0; r < 16; ++r) {
+      const int ro = (r / 4) * 8 + (r % 4);
+      rv[r] = load_as_f32(res, dt, base + (int64_t)((!GUARD || ro < rows_left) ? ro : 0) * ld);
+    }
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    float v = acc[r] * alpha + bias[r];
+    const int ro = (r / 4) * 8 + (r % 4);
+    float v = acc[r] * alpha + bias_of(r);
     if (res) v += rv[r];
     if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
     else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
-    if (ok[r]) {
-      if constexpr (dt == LLC_FLOAT32) C[o[r]] = v;
-      else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o[r]] = f32_to_bf16_bits(v);
-      else ((uint16_t*)C)[o[r]] = f32_to_f16_bits(v);
+    if (!GUARD || ro < rows_left) {
+      const int64_t o = base + (int64_t)ro * ld;
+      if constexpr (dt == LLC_FLOAT32) C[o] = v;
+      else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o] = f32_to_bf16_bits(v);
+      else ((uint16_t*)C)[o] = f32_to_f16_bits(v);
     }
   }
 }
