@@ -342,11 +342,11 @@ __device__ __forceinline__ void epilogue_block16(T* C, const char* res, int64_t 
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int ro = (r / 4) * 8 + (r % 4);
-    float v = acc[r] * alpha + bias_of(r);
-    if (res) v += rv[r];
-    if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
-    else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
-    if (!GUARD || ro < rows_left) {
+    if (!GUARD || ro < rows_left) {  // nothing is computed for rows that do not exist (grouped convolutions: most of a block)
+      float v = acc[r] * alpha + bias_of(r);
+      if (res) v += rv[r];
+      if (act == LLC_ACT_RELU) v = v < 0.0f ? 0.0f : v;  // NaN passes through, like torch.relu
+      else if (act == LLC_ACT_GELU) v = gelu_for<T>(v);
       const int64_t o = base + (int64_t)ro * ld;
       if constexpr (dt == LLC_FLOAT32) C[o] = v;
       else if constexpr (dt == LLC_BFLOAT16) ((uint16_t*)C)[o] = f32_to_bf16_bits(v);
