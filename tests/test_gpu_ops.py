@@ -941,6 +941,26 @@ def test_matmul_epilogue(ops, oracle):
         assert_close_f32(host(ops.matmul(dev(a), dev(b), epi)), want, "epilogue " + act)
 
 
+@pytest.mark.parametrize("M,N,K,dt", [(70, 136, 200, torch.float32), (256, 256, 64, torch.float32), (384, 256, 128, torch.bfloat16),
+                                      (128, 192, 128, torch.bfloat16), (1024, 768, 256, torch.bfloat16), (448, 768, 3072, torch.float32)])
+def test_matmul_residual_may_be_the_output(ops, oracle, M, N, K, dt):
+    """An in-place residual add (the residual operand is the result tensor): every kernel family reads a lane's residual
+    values before it stores that lane's results, so the product is the same as with a separate result."""
+    r = rng(77 + M + K)
+    a = bf16_round(r.uniform(-1, 1, (M, K)) * 0.25)  # sums of 3072 products stay near the residual's size
+    b = bf16_round(r.uniform(-1, 1, (K, N)) * 0.25)
+    res = bf16_round(r.standard_normal((M, N)))
+    bias = bf16_round(r.standard_normal(N))
+    want = oracle.matmul(a, b, "mkn") + bias[None, :] + res
+    inout = dev(res, dt)
+    got = ops.matmul(dev(a, dt), dev(b, dt), ops.Epilogue(bias=dev(bias, dt), residual=inout), out=inout)
+    assert got.data_ptr() == inout.data_ptr()
+    if dt == torch.float32:
+        assert_close_f32(host(got), want, "in-place residual f32 %dx%dx%d" % (M, N, K))
+    else:
+        assert_close_bf16(host(got), bf16_round(want.astype(np.float32)), "in-place residual bf16 %dx%dx%d" % (M, N, K))
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_matmul_cases(ops, oracle, seed):
     """Randomly drawn products: extents on both sides of every dispatch threshold (16 rows, complete 128-tiles,
@@ -1142,6 +1162,27 @@ NHWC_CASES = [
     (2, 128, 28, 28, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),    # 1568 pixels: 64-pixel tiles, no split
     (1, 192, 6, 9, 36, 3, 3, (1, 0, 2, 1), (1, 1), (1, 1)),       # 16-bit k-tiles of 64 in 192 channels, partial filter tile
 ]
+
+
+@pytest.mark.parametrize("case", [NHWC_CASES[0], NHWC_CASES[5], NHWC_CASES[7]])
+def test_conv2d_channels_last_residual_may_be_the_output(ops, oracle, case):
+    """A residual block's add done in place (the residual operand is the result tensor), on the tile kernel, the split
+    reduction and, in bf16, the input-patch kernel: a lane reads its residual values before it stores its results."""
+    N, C, H, W, Fo, KH, KW, pad, s, d = case
+    r = rng(sum(case[:7]) + 5)
+    x = bf16_round(r.standard_normal((N, C, H, W)))
+    w = bf16_round(r.standard_normal((Fo, C, KH, KW)) / np.sqrt(C * KH * KW))
+    b = bf16_round(r.standard_normal(Fo))
+    conv = oracle.conv2d(x, w, b, pad=pad, stride=s, dilation=d)
+    res = bf16_round(r.standard_normal(conv.shape))
+    want = oracle.unary("relu", conv + res)
+    cl = torch.channels_last
+    for dt, close in ((torch.float32, assert_close_f32), (torch.bfloat16, assert_close_bf16)):
+        inout = dev(res, dt).contiguous(memory_format=cl)
+        got = ops.conv2d(dev(x, dt).contiguous(memory_format=cl), dev(w, dt).contiguous(memory_format=cl), pad=pad, stride=s,
+                         dilation=d, epilogue=ops.Epilogue(bias=dev(b, dt), residual=inout, act="relu"), out=inout)
+        assert got.data_ptr() == inout.data_ptr()
+        close(host(got), want if dt == torch.float32 else bf16_round(want), "in-place residual conv %s %s" % (dt, case))
 
 
 @pytest.mark.parametrize("case", NHWC_CASES)
