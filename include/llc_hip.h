@@ -106,7 +106,9 @@ typedef struct llc_epilogue {
   const llc_tensor* bias;     /* rank 1, one value per output column / filter; may be NULL.  batch_matmul with two
                                  batch dims also takes rank 2, [B0, N]: one row per outer batch (an attention
                                  mask [B,1,1,S] added to scores [B,H,S,S]) */
-  const llc_tensor* residual; /* same shape as the output, contiguous; may be NULL */
+  const llc_tensor* residual; /* same shape as the output, contiguous; may be NULL.  It may be the output tensor itself
+                                 (an in-place add: every kernel reads an element's residual before it stores that
+                                 element); any other overlap with the output is undefined */
   int act;                    /* llc_activation */
 } llc_epilogue;
 
