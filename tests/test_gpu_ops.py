@@ -942,7 +942,8 @@ def test_matmul_epilogue(ops, oracle):
 
 
 @pytest.mark.parametrize("M,N,K,dt", [(70, 136, 200, torch.float32), (256, 256, 64, torch.float32), (384, 256, 128, torch.bfloat16),
-                                      (128, 192, 128, torch.bfloat16), (1024, 768, 256, torch.bfloat16), (448, 768, 3072, torch.float32)])
+                                      (128, 192, 128, torch.bfloat16), (1024, 768, 256, torch.bfloat16), (448, 768, 3072, torch.float32),
+                                      (4096, 3072, 128, torch.bfloat16)])
 def test_matmul_residual_may_be_the_output(ops, oracle, M, N, K, dt):
     """An in-place residual add (the residual operand is the result tensor): every kernel family reads a lane's residual
     values before it stores that lane's results, so the product is the same as with a separate result."""
@@ -959,6 +960,22 @@ def test_matmul_residual_may_be_the_output(ops, oracle, M, N, K, dt):
         assert_close_f32(host(got), want, "in-place residual f32 %dx%dx%d" % (M, N, K))
     else:
         assert_close_bf16(host(got), bf16_round(want.astype(np.float32)), "in-place residual bf16 %dx%dx%d" % (M, N, K))
+
+
+def test_batch_matmul_residual_may_be_the_output(ops, oracle):
+    """The same for the batched product with K = 64 (its kernel transposes a tile through LDS between reading the residual
+    and storing the result)."""
+    r = rng(91)
+    B, M, K, N = 16, 512, 64, 512
+    a = bf16_round(r.uniform(-1, 1, (B, M, K)) * 0.25)
+    b = bf16_round(r.uniform(-1, 1, (B, K, N)) * 0.25)
+    res = bf16_round(r.standard_normal((B, M, N)))
+    want = np.stack([oracle.matmul(a[i], b[i], "mkn") for i in range(B)]) + res
+    for dt, close in ((torch.float32, assert_close_f32), (torch.bfloat16, assert_close_bf16)):
+        inout = dev(res, dt)
+        got = ops.batch_matmul(dev(a, dt), dev(b, dt), ops.Epilogue(residual=inout), out=inout)
+        assert got.data_ptr() == inout.data_ptr()
+        close(host(got), want if dt == torch.float32 else bf16_round(want.astype(np.float32)), "in-place residual bmm %s" % dt)
 
 
 @pytest.mark.parametrize("seed", range(4))
